@@ -1,0 +1,287 @@
+// The four gather maps behind Conv2d / DeConv2d: im2col, col2im, and DeConv2d's col2im / im2col.
+// All are HBM-bandwidth bound; every output element is written exactly once, every launch is a
+// grid-stride loop over 16-byte vectors along the contiguous axis wherever the geometry allows.
+//
+// Replaces Conv2dIm2ColKernel / Conv2dCol2ImKernel (deep8/src/math/Conv2d.cu:10-118) and
+// DeConv2dCol2ImKernel / DeConv2dIm2ColKernel (deep8/src/math/DeConv2d.cu:11-58,310-351).
+#include "common.h"
+
+namespace d8 {
+
+struct MapGeom {
+    int B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, pt, pl;
+};
+
+static inline int grid_for(long work, int block) {
+    long blocks = (work + block - 1) / block;
+    const long cap = (long)cu_count() * 32;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return (int)blocks;
+}
+
+// ---- im2col: pure copy, V is the raw vector moved per thread (bit-exact) -------------------
+template <typename V>
+__global__ __launch_bounds__(256) void im2col_kernel(const V *__restrict__ im, V *__restrict__ col,
+                                                     MapGeom g, int CV, long total) {
+    const int taps = g.FH * g.FW;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int cv = (int)(idx % CV);
+        const long t = idx / CV;
+        const int tap = (int)(t % taps);
+        const long r = t / taps;
+        const int fx = tap % g.FW, fy = tap / g.FW;
+        const int ox = (int)(r % g.OW);
+        const long q = r / g.OW;
+        const int oy = (int)(q % g.OH), b = (int)(q / g.OH);
+        const int iy = oy * g.sy + fy * g.dy - g.pt;
+        const int ix = ox * g.sx + fx * g.dx - g.pl;
+        V v;
+        memset(&v, 0, sizeof(V));
+        if (iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW)
+            v = im[(((long)b * g.IH + iy) * g.IW + ix) * CV + cv];
+        col[idx] = v;
+    }
+}
+
+// ---- col2im: one thread owns VEC channels of one image pixel; taps are added in (fy, fx)
+// ascending order into registers, then the pixel is written once. -----------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void col2im_kernel(const T *__restrict__ col, T *__restrict__ im,
+                                                     MapGeom g, long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    const int CV = g.C / VEC;
+    const long K = (long)g.FH * g.FW * g.C;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int cv = (int)(idx % CV);
+        const long p = idx / CV;
+        const int ix = (int)(p % g.IW);
+        const long q = p / g.IW;
+        const int iy = (int)(q % g.IH), b = (int)(q / g.IH);
+        T *dst = im + p * g.C + (long)cv * VEC;
+        float acc[VEC];
+        {
+            VT v = *(const VT *)dst;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = (float)v[e];
+        }
+        for (int fy = 0; fy < g.FH; ++fy) {
+            const int ty = iy + g.pt - fy * g.dy;
+            if (ty < 0 || ty % g.sy) continue;
+            const int oy = ty / g.sy;
+            if (oy >= g.OH) continue;
+            for (int fx = 0; fx < g.FW; ++fx) {
+                const int tx = ix + g.pl - fx * g.dx;
+                if (tx < 0 || tx % g.sx) continue;
+                const int ox = tx / g.sx;
+                if (ox >= g.OW) continue;
+                const VT v = *(const VT *)(col + (((long)b * g.OH + oy) * g.OW + ox) * K +
+                                           (long)(fy * g.FW + fx) * g.C + (long)cv * VEC);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] += (float)v[e];
+            }
+        }
+        VT o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = (T)acc[e];
+        *(VT *)dst = o;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void col2im_scalar_kernel(const T *__restrict__ col, T *__restrict__ im,
+                                                            MapGeom g, long total) {
+    const long K = (long)g.FH * g.FW * g.C;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int c = (int)(idx % g.C);
+        const long p = idx / g.C;
+        const int ix = (int)(p % g.IW);
+        const long q = p / g.IW;
+        const int iy = (int)(q % g.IH), b = (int)(q / g.IH);
+        float acc = (float)im[idx];
+        for (int fy = 0; fy < g.FH; ++fy) {
+            const int ty = iy + g.pt - fy * g.dy;
+            if (ty < 0 || ty % g.sy) continue;
+            const int oy = ty / g.sy;
+            if (oy >= g.OH) continue;
+            for (int fx = 0; fx < g.FW; ++fx) {
+                const int tx = ix + g.pl - fx * g.dx;
+                if (tx < 0 || tx % g.sx) continue;
+                const int ox = tx / g.sx;
+                if (ox >= g.OW) continue;
+                acc += (float)col[(((long)b * g.OH + oy) * g.OW + ox) * K + (long)(fy * g.FW + fx) * g.C + c];
+            }
+        }
+        im[idx] = (T)acc;
+    }
+}
+
+// ---- DeConv2d col2im (gather, overwrite) -------------------------------------------------------
+// In MapGeom for the two DeConv2d maps: C = OC, (IH,IW) = deconv input, (OH,OW) = deconv output.
+template <typename T>
+__global__ __launch_bounds__(256) void deconv_col2im_kernel(const T *__restrict__ zmat, T *__restrict__ z,
+                                                            MapGeom g, long total) {
+    const int taps = g.FH * g.FW;
+    const long N = (long)g.C * taps;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int oc = (int)(idx % g.C);
+        const long p = idx / g.C;
+        const int ox = (int)(p % g.OW);
+        const long q = p / g.OW;
+        const int oy = (int)(q % g.OH), b = (int)(q / g.OH);
+        float acc = 0.f;
+        for (int fy = 0; fy < g.FH; ++fy) {
+            const int ty = oy - g.pt + fy;
+            if (ty < 0 || ty % g.sy) continue;
+            const int iy = ty / g.sy;
+            if (iy >= g.IH) continue;
+            for (int fx = 0; fx < g.FW; ++fx) {
+                const int tx = ox - g.pl + fx;
+                if (tx < 0 || tx % g.sx) continue;
+                const int ix = tx / g.sx;
+                if (ix >= g.IW) continue;
+                acc += (float)zmat[(((long)b * g.IH + iy) * g.IW + ix) * N + (long)oc * taps + fy * g.FW + fx];
+            }
+        }
+        z[idx] = (T)acc;
+    }
+}
+
+// ---- DeConv2d im2col (pure copy) ------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void deconv_im2col_kernel(const T *__restrict__ dz, T *__restrict__ dzmat,
+                                                            MapGeom g, long total) {
+    const int taps = g.FH * g.FW;
+    const int N = g.C * taps;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int col = (int)(idx % N);
+        const long r = idx / N;
+        const int ix = (int)(r % g.IW);
+        const long q = r / g.IW;
+        const int iy = (int)(q % g.IH), b = (int)(q / g.IH);
+        const int oc = col / taps, tap = col % taps;
+        const int fy = tap / g.FW, fx = tap % g.FW;
+        const int oy = iy * g.sy + g.pt - fy;
+        const int ox = ix * g.sx + g.pl - fx;
+        T v = (T)0;
+        if (oy >= 0 && oy < g.OH && ox >= 0 && ox < g.OW)
+            v = dz[(((long)b * g.OH + oy) * g.OW + ox) * g.C + oc];
+        dzmat[idx] = v;
+    }
+}
+
+static int check_geom(const char *who, int dtype, const void *a, const void *b, const MapGeom &g) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
+    D8_REQUIRE(g.B >= 0 && g.IH > 0 && g.IW > 0 && g.C > 0 && g.OH > 0 && g.OW > 0 && g.FH > 0 && g.FW > 0,
+               "%s: sizes must be positive", who);
+    D8_REQUIRE(g.sy >= 1 && g.sx >= 1 && g.dy >= 1 && g.dx >= 1, "%s: stride and dilation must be >= 1", who);
+    D8_REQUIRE(g.pt >= 0 && g.pl >= 0, "%s: padding must be >= 0", who);
+    D8_REQUIRE(g.B == 0 || (a && b), "%s: null pointer", who);
+    return 0;
+}
+
+static inline bool aligned16(const void *p) { return ((size_t)p & 15) == 0; }
+
+}  // namespace d8
+
+using namespace d8;
+
+extern "C" {
+
+int d8_im2col(int dtype, const void *im, void *col,
+              int B, int IH, int IW, int C, int OH, int OW, int FH, int FW,
+              int sy, int sx, int dy, int dx, int padTop, int padLeft, void *stream) {
+    MapGeom g = {B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft};
+    if (int rc = check_geom("d8_im2col", dtype, im, col, g)) return rc;
+    if (B == 0) return 0;
+    const size_t es = dtype_bytes(dtype);
+    const long elems = (long)B * OH * OW * FH * FW * C;
+    const size_t row_bytes = (size_t)C * es;
+    hipStream_t s = as_stream(stream);
+    if (row_bytes % 16 == 0 && aligned16(im) && aligned16(col)) {
+        const int CV = (int)(row_bytes / 16);
+        const long total = elems / (16 / es);
+        hipLaunchKernelGGL((im2col_kernel<uint4>), dim3(grid_for(total, 256)), dim3(256), 0, s,
+                           (const uint4 *)im, (uint4 *)col, g, CV, total);
+    } else if (es == 4) {
+        hipLaunchKernelGGL((im2col_kernel<unsigned>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned *)im, (unsigned *)col, g, C, elems);
+    } else {
+        hipLaunchKernelGGL((im2col_kernel<unsigned short>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned short *)im, (unsigned short *)col, g, C, elems);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int d8_col2im(int dtype, const void *col, void *im,
+              int B, int IH, int IW, int C, int OH, int OW, int FH, int FW,
+              int sy, int sx, int dy, int dx, int padTop, int padLeft, void *stream) {
+    MapGeom g = {B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft};
+    if (int rc = check_geom("d8_col2im", dtype, col, im, g)) return rc;
+    if (B == 0) return 0;
+    const long elems = (long)B * IH * IW * C;
+    hipStream_t s = as_stream(stream);
+    const bool al = aligned16(im) && aligned16(col);
+    if (dtype == D8_FLOAT32) {
+        if (C % 4 == 0 && al)
+            hipLaunchKernelGGL((col2im_kernel<float, 4>), dim3(grid_for(elems / 4, 256)), dim3(256), 0, s,
+                               (const float *)col, (float *)im, g, elems / 4);
+        else
+            hipLaunchKernelGGL((col2im_scalar_kernel<float>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                               (const float *)col, (float *)im, g, elems);
+    } else {
+        if (C % 8 == 0 && al)
+            hipLaunchKernelGGL((col2im_kernel<f16, 8>), dim3(grid_for(elems / 8, 256)), dim3(256), 0, s,
+                               (const f16 *)col, (f16 *)im, g, elems / 8);
+        else
+            hipLaunchKernelGGL((col2im_scalar_kernel<f16>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                               (const f16 *)col, (f16 *)im, g, elems);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int d8_deconv_col2im(int dtype, const void *zmat, void *z,
+                     int B, int IH, int IW, int OH, int OW, int OC, int FH, int FW,
+                     int sy, int sx, int padTop, int padLeft, void *stream) {
+    MapGeom g = {B, IH, IW, OC, OH, OW, FH, FW, sy, sx, 1, 1, padTop, padLeft};
+    if (int rc = check_geom("d8_deconv_col2im", dtype, zmat, z, g)) return rc;
+    if (B == 0) return 0;
+    const long elems = (long)B * OH * OW * OC;
+    hipStream_t s = as_stream(stream);
+    if (dtype == D8_FLOAT32)
+        hipLaunchKernelGGL((deconv_col2im_kernel<float>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const float *)zmat, (float *)z, g, elems);
+    else
+        hipLaunchKernelGGL((deconv_col2im_kernel<f16>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const f16 *)zmat, (f16 *)z, g, elems);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
+                     int B, int IH, int IW, int OH, int OW, int OC, int FH, int FW,
+                     int sy, int sx, int padTop, int padLeft, void *stream) {
+    MapGeom g = {B, IH, IW, OC, OH, OW, FH, FW, sy, sx, 1, 1, padTop, padLeft};
+    if (int rc = check_geom("d8_deconv_im2col", dtype, dz, dzmat, g)) return rc;
+    if (B == 0) return 0;
+    const long elems = (long)B * IH * IW * OC * FH * FW;
+    hipStream_t s = as_stream(stream);
+    if (dtype == D8_FLOAT32)
+        hipLaunchKernelGGL((deconv_im2col_kernel<unsigned>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned *)dz, (unsigned *)dzmat, g, elems);
+    else
+        hipLaunchKernelGGL((deconv_im2col_kernel<unsigned short>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned short *)dz, (unsigned short *)dzmat, g, elems);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,314 @@
+// Row-major GEMM for gfx950 on MFMA: C_b = op(A_b) op(B_b) + beta C_b, fp32 and fp16 (fp32
+// accumulate), NN / NT / TN, strided batch with broadcast operands, optional summation of the
+// whole batch into one C, and a deterministic split of the reduction through a workspace.
+//
+// Replaces the cuBLAS calls of deep8/src/math/MatrixMultiply.cu, Conv2d.cu and DeConv2d.cu
+// (call sites listed in include/deep8_hip.h).
+//
+// MFMA operand layouts used throughout (wave64):
+//   v_mfma_f32_32x32x16_f16 : lane l supplies A[row l%32][8 consecutive k of group l/32] and
+//                             B[8 consecutive k of group l/32][col l%32]
+//   v_mfma_f32_32x32x2_f32  : lane l supplies A[row l%32][k = l/32], B[k = l/32][col l%32]
+//   accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32]
+// Both LDS tiles are kept K-contiguous ([row][k]), so one 16-byte LDS read feeds an MFMA
+// operand; the transposed-operand cases differ only in how the tile loader walks global memory.
+#include "common.h"
+
+namespace d8 {
+
+struct GemmArgs {
+    const void *A;
+    const void *B;
+    void *C;
+    float *ws;
+    int M, N, K;
+    int lda, ldb, ldc;
+    long sA, sB, sC;
+    int batch;            // independent outputs
+    int red;              // products summed into each output (1 unless strideC == 0)
+    int splits;           // pieces the extended reduction (red x K tiles) is cut into
+    int tiles_per_split;  // K tiles per piece
+    float beta;
+};
+
+template <typename T>
+struct Tile;
+template <>
+struct Tile<f16> {
+    static constexpr int BK = 32, LD = 40;
+};
+template <>
+struct Tile<float> {
+    static constexpr int BK = 16, LD = 20;
+};
+
+__device__ inline float to_f32(float v) { return v; }
+__device__ inline float to_f32(f16 v) { return (float)v; }
+
+// One wave multiplies its (TM*32) x (TN*32) sub-tile over one K tile held in LDS.
+template <int TM, int TN, int LD, int BK>
+__device__ inline void wave_mma(const f16 *As, const f16 *Bs, int arow, int brow, int lane,
+                                f32x16 (&acc)[TM][TN]) {
+    const int l32 = lane & 31, kg = (lane >> 5) * 8;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 16) {
+        f16x8 a[TM], b[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = *(const f16x8 *)&As[(arow + i * 32 + l32) * LD + kk + kg];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = *(const f16x8 *)&Bs[(brow + j * 32 + l32) * LD + kk + kg];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+}
+
+// fp32: an 8-wide K chunk is read as two float4 per operand row (lanes 0-31 take k 0..3,
+// lanes 32-63 take k 4..7); MFMA q of the chunk then pairs k = q with k = 4 + q.  A and B use
+// the same assignment, so every k is multiplied exactly once.
+template <int TM, int TN, int LD, int BK>
+__device__ inline void wave_mma(const float *As, const float *Bs, int arow, int brow, int lane,
+                                f32x16 (&acc)[TM][TN]) {
+    const int l32 = lane & 31, kg = (lane >> 5) * 4;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 8) {
+        f32x4 a[TM], b[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = *(const f32x4 *)&As[(arow + i * 32 + l32) * LD + kk + kg];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = *(const f32x4 *)&Bs[(brow + j * 32 + l32) * LD + kk + kg];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][q], b[j][q], acc[i][j], 0, 0, 0);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// General kernel: any M, N, K, leading dimension and alignment.  128 x 128 tile, 4 waves in a
+// 2 x 2 arrangement, 64 x 64 per wave; element-wise, bounds-checked tile loads.
+// ------------------------------------------------------------------------------------------
+template <typename T, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_general_kernel(GemmArgs g) {
+    constexpr int BM = 128, BN = 128, BK = Tile<T>::BK, LD = Tile<T>::LD;
+    __shared__ __attribute__((aligned(16))) T As[BM * LD];
+    __shared__ __attribute__((aligned(16))) T Bs[BN * LD];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int b = blockIdx.z / g.splits, s = blockIdx.z % g.splits;
+
+    const int ktiles = (g.K + BK - 1) / BK;
+    const int total = g.red * ktiles;
+    const int t0 = s * g.tiles_per_split;
+    const int t1 = min(total, t0 + g.tiles_per_split);
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    for (int t = t0; t < t1; ++t) {
+        const int r = t / ktiles, k0 = (t - r * ktiles) * BK;
+        const T *Ap = (const T *)g.A + (long)(b + r) * g.sA;
+        const T *Bp = (const T *)g.B + (long)(b + r) * g.sB;
+
+        for (int i = tid; i < BM * BK; i += 256) {
+            int m, k;
+            if (!TA) {
+                m = i / BK;
+                k = i % BK;
+            } else {
+                k = i / BM;
+                m = i % BM;
+            }
+            const int gm = m0 + m, gk = k0 + k;
+            T v = (T)0;
+            if (gm < g.M && gk < g.K) v = TA ? Ap[(long)gk * g.lda + gm] : Ap[(long)gm * g.lda + gk];
+            As[m * LD + k] = v;
+        }
+        for (int i = tid; i < BN * BK; i += 256) {
+            int n, k;
+            if (TB) {
+                n = i / BK;
+                k = i % BK;
+            } else {
+                k = i / BN;
+                n = i % BN;
+            }
+            const int gn = n0 + n, gk = k0 + k;
+            T v = (T)0;
+            if (gn < g.N && gk < g.K) v = TB ? Bp[(long)gn * g.ldb + gk] : Bp[(long)gk * g.ldb + gn];
+            Bs[n * LD + k] = v;
+        }
+        __syncthreads();
+        wave_mma<2, 2, LD, BK>(As, Bs, wm * 64, wn * 64, lane, acc);
+        __syncthreads();
+    }
+
+    const int l32 = lane & 31, lhi = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + wn * 64 + j * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+                if (m < g.M && n < g.N) {
+                    if (g.splits == 1) {
+                        T *c = (T *)g.C + (long)b * g.sC + (long)m * g.ldc + n;
+                        float v = acc[i][j][r];
+                        if (g.beta != 0.f) v += to_f32(*c);
+                        *c = (T)v;
+                    } else {
+                        g.ws[((long)(b * g.splits + s) * g.M + m) * g.N + n] = acc[i][j][r];
+                    }
+                }
+            }
+        }
+}
+
+// C[b][m][n] = beta * C + sum_s ws[b][s][m][n]; partials are added in split order.
+template <typename T>
+__global__ void gemm_split_reduce_kernel(GemmArgs g) {
+    const long mn = (long)g.M * g.N;
+    const long total = mn * g.batch;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int b = (int)(i / mn);
+        const long e = i - (long)b * mn;
+        const int m = (int)(e / g.N), n = (int)(e - (long)m * g.N);
+        const float *p = g.ws + (long)b * g.splits * mn + e;
+        float v = 0.f;
+        for (int s = 0; s < g.splits; ++s) v += p[(long)s * mn];
+        T *c = (T *)g.C + (long)b * g.sC + (long)m * g.ldc + n;
+        if (g.beta != 0.f) v += to_f32(*c);
+        *c = (T)v;
+    }
+}
+
+// How many pieces to cut the reduction into.  Splitting is only worth a second pass when the
+// output alone gives the 256 CUs too few tiles; long reductions are also split to keep each
+// fp32 accumulation chain short.
+static int plan_splits(int dtype, int M, int N, int K, int batch, int red, int *tiles_per_split) {
+    const int BK = dtype == D8_FLOAT16 ? 32 : 16;
+    const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
+    const long total = (long)red * ceil_div(K, BK);
+    const int cus = cu_count();
+    long splits = 1;
+    if (tiles < cus) splits = (2L * cus + tiles - 1) / tiles;
+    const long max_by_len = total / 8 > 0 ? total / 8 : 1;  // at least 8 K tiles per piece
+    if (splits > max_by_len) splits = max_by_len;
+    if (splits > 128) splits = 128;
+    if (splits < 1) splits = 1;
+    long tps = (total + splits - 1) / splits;
+    splits = (total + tps - 1) / tps;
+    *tiles_per_split = (int)tps;
+    return (int)splits;
+}
+
+template <typename T>
+static int launch(GemmArgs &g, int transA, int transB, hipStream_t stream) {
+    dim3 grid(ceil_div(g.N, 128), ceil_div(g.M, 128), g.batch * g.splits);
+    if (!transA && !transB)
+        hipLaunchKernelGGL((gemm_general_kernel<T, false, false>), grid, dim3(256), 0, stream, g);
+    else if (!transA && transB)
+        hipLaunchKernelGGL((gemm_general_kernel<T, false, true>), grid, dim3(256), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemm_general_kernel<T, true, false>), grid, dim3(256), 0, stream, g);
+    D8_LAUNCH_CHECK();
+    if (g.splits > 1) {
+        const long total = (long)g.M * g.N * g.batch;
+        int blocks = (int)((total + 255) / 256);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL((gemm_split_reduce_kernel<T>), dim3(blocks), dim3(256), 0, stream, g);
+        D8_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+}  // namespace d8
+
+using namespace d8;
+
+extern "C" {
+
+size_t d8_gemm_workspace_bytes(int dtype, int transA, int transB, int M, int N, int K,
+                               int batch, long strideC) {
+    (void)transA;
+    (void)transB;
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
+    const int red = (strideC == 0 && batch > 1) ? batch : 1;
+    const int outs = red > 1 ? 1 : batch;
+    int tps = 0;
+    const int splits = plan_splits(dtype, M, N, K, outs, red, &tps);
+    return splits > 1 ? (size_t)splits * outs * M * N * sizeof(float) : 0;
+}
+
+int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
+            const void *A, int lda, long strideA,
+            const void *B, int ldb, long strideB,
+            float beta, void *C, int ldc, long strideC, int batch,
+            void *workspace, size_t workspace_bytes, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_gemm: element type %d is not supported", dtype);
+    D8_REQUIRE(!(transA && transB), "d8_gemm: transA and transB together are not supported");
+    D8_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "d8_gemm: negative size");
+    D8_REQUIRE(beta == 0.f || beta == 1.f, "d8_gemm: beta must be 0 or 1");
+    if (M == 0 || N == 0 || batch == 0) return 0;
+    D8_REQUIRE(A && B && C, "d8_gemm: null operand");
+    D8_REQUIRE(lda >= (transA ? M : K), "d8_gemm: lda %d too small", lda);
+    D8_REQUIRE(ldb >= (transB ? K : N), "d8_gemm: ldb %d too small", ldb);
+    D8_REQUIRE(ldc >= N, "d8_gemm: ldc %d too small", ldc);
+    D8_REQUIRE(strideA >= 0 && strideB >= 0 && strideC >= 0, "d8_gemm: negative stride");
+    D8_REQUIRE((long)ceil_div(M, 128) < 65536 && (long)batch * 128 < 65536, "d8_gemm: grid too large");
+
+    GemmArgs g;
+    g.A = A;
+    g.B = B;
+    g.C = C;
+    g.ws = (float *)workspace;
+    g.M = M;
+    g.N = N;
+    g.K = K;
+    g.lda = lda;
+    g.ldb = ldb;
+    g.ldc = ldc;
+    g.sA = strideA;
+    g.sB = strideB;
+    g.sC = strideC;
+    g.beta = beta;
+    g.red = (strideC == 0 && batch > 1) ? batch : 1;
+    g.batch = g.red > 1 ? 1 : batch;
+    if (K == 0) {
+        // empty reduction: C = beta * C
+        g.splits = 1;
+        g.tiles_per_split = 0;
+    } else {
+        g.splits = plan_splits(dtype, M, N, K, g.batch, g.red, &g.tiles_per_split);
+        const size_t per_split = (size_t)g.batch * M * N * sizeof(float);
+        if (g.splits > 1 && (!workspace || workspace_bytes < per_split * g.splits)) {
+            // use as many pieces as the caller's workspace holds
+            long fit = workspace ? (long)(workspace_bytes / per_split) : 1;
+            if (fit < 2) fit = 1;
+            const int BK = dtype == D8_FLOAT16 ? 32 : 16;
+            const long total = (long)g.red * ceil_div(K, BK);
+            long tps = (total + fit - 1) / fit;
+            g.tiles_per_split = (int)tps;
+            g.splits = (int)((total + tps - 1) / tps);
+        }
+    }
+    return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, as_stream(stream))
+                               : launch<float>(g, transA, transB, as_stream(stream));
+}
+
+}  // extern "C"

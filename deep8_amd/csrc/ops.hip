@@ -1,0 +1,290 @@
+// Whole-operator entry points: the shape cases, pad formulas, scratch layout and
+// overwrite / accumulate semantics of Deep8's MatrixMultiply, Conv2d and DeConv2d GPU paths,
+// expressed as d8_gemm plus the four gather maps.
+//
+//   MatrixMultiply   deep8/src/math/MatrixMultiply.cu:21-57 (fwd), :193-232 (GradX), :381-420 (GradY)
+//   Conv2d           deep8/src/math/Conv2d.cu:145-196, :440-492, :750-802, pads :332-336
+//   DeConv2d         deep8/src/math/DeConv2d.cu:76-131, :371-429, :642-700, pads :99-100
+#include "common.h"
+
+namespace d8 {
+
+static inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+struct Gemm {
+    int ta, tb, M, N, K;
+    const void *A;
+    int lda;
+    long sA;
+    const void *B;
+    int ldb;
+    long sB;
+    float beta;
+    void *C;
+    int ldc;
+    long sC;
+    int batch;
+};
+
+static size_t gemm_ws(int dtype, const Gemm &g) {
+    return d8_gemm_workspace_bytes(dtype, g.ta, g.tb, g.M, g.N, g.K, g.batch, g.sC);
+}
+
+static int run(int dtype, const Gemm &g, void *ws, size_t ws_bytes, void *stream) {
+    return d8_gemm(dtype, g.ta, g.tb, g.M, g.N, g.K, g.A, g.lda, g.sA, g.B, g.ldb, g.sB, g.beta,
+                   g.C, g.ldc, g.sC, g.batch, ws, ws_bytes, stream);
+}
+
+static int check_mm(const char *who, int dtype, int xb, int xr, int xc, int yb, int yr, int yc) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
+    D8_REQUIRE(xb > 0 && xr > 0 && xc > 0 && yb > 0 && yr > 0 && yc > 0, "%s: sizes must be positive", who);
+    D8_REQUIRE(xb == yb || xb == 1 || yb == 1, "%s: batch %d vs %d", who, xb, yb);
+    D8_REQUIRE(xc == yr, "%s: inner dimensions %d vs %d", who, xc, yr);
+    return 0;
+}
+
+// which: 0 forward, 1 gradient of x, 2 gradient of y.  Pointers may be null when only the
+// shape is wanted (workspace query).
+static Gemm mm_plan(int which, const void *x, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
+                    const void *z) {
+    const int zb = xb > yb ? xb : yb;
+    const long xs = (long)xr * xc, ys = (long)yr * yc, zs = (long)xr * yc;
+    Gemm g;
+    if (which == 0) {
+        if (yb == 1) g = {0, 0, xb * xr, yc, xc, x, xc, 0, y, yc, 0, 0.f, (void *)z, yc, 0, 1};
+        else if (xb == 1 && yc == 1) g = {0, 1, yb, xr, xc, y, xc, 0, x, xc, 0, 0.f, (void *)z, xr, 0, 1};
+        else g = {0, 0, xr, yc, xc, x, xc, xb == 1 ? 0 : xs, y, yc, ys, 0.f, (void *)z, yc, zs, zb};
+    } else if (which == 1) {  // x plays dx (output), z plays dz
+        if (yb == 1) g = {0, 1, xb * xr, xc, yc, z, yc, 0, y, yc, 0, 1.f, (void *)x, xc, 0, 1};
+        else if (xb == 1 && yc == 1) g = {1, 0, xr, xc, yb, z, xr, 0, y, xc, 0, 1.f, (void *)x, xc, 0, 1};
+        else g = {0, 1, xr, xc, yc, z, yc, zs, y, yc, ys, 1.f, (void *)x, xc, xb == 1 ? 0 : xs, zb};
+    } else {  // y plays dy (output), z plays dz
+        if (yb == 1) g = {1, 0, yr, yc, xb * xr, x, xc, 0, z, yc, 0, 1.f, (void *)y, yc, 0, 1};
+        else if (xb == 1 && yc == 1) g = {0, 0, yb, xc, xr, z, xr, 0, x, xc, 0, 1.f, (void *)y, xc, 0, 1};
+        else g = {1, 0, yr, yc, xr, x, xc, xb == 1 ? 0 : xs, z, yc, zs, 1.f, (void *)y, yc, ys, zb};
+    }
+    return g;
+}
+
+static int check_conv(const char *who, int dtype, int B, int IH, int IW, int IC, int OC, int FH, int FW,
+                      int sy, int sx, int dy, int dx) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
+    D8_REQUIRE(B > 0 && IH > 0 && IW > 0 && IC > 0 && OC > 0 && FH > 0 && FW > 0, "%s: sizes must be positive", who);
+    D8_REQUIRE(sy >= 1 && sx >= 1 && dy >= 1 && dx >= 1, "%s: the stride and dilation must >= 1", who);
+    return 0;
+}
+
+}  // namespace d8
+
+using namespace d8;
+
+extern "C" {
+
+// ---------------------------------------------------------------------------------------------
+size_t d8_matmul_scratch_bytes(int dtype, int which, int xb, int xr, int xc, int yb, int yr, int yc) {
+    if (check_mm("d8_matmul_scratch_bytes", dtype, xb, xr, xc, yb, yr, yc)) return 0;
+    return gemm_ws(dtype, mm_plan(which, nullptr, xb, xr, xc, nullptr, yb, yr, yc, nullptr));
+}
+
+int d8_matmul(int dtype, const void *x, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
+              void *z, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_mm("d8_matmul", dtype, xb, xr, xc, yb, yr, yc)) return rc;
+    D8_REQUIRE(x && y && z, "d8_matmul: null tensor");
+    return run(dtype, mm_plan(0, x, xb, xr, xc, y, yb, yr, yc, z), scratch, scratch_bytes, stream);
+}
+
+int d8_matmul_grad_x(int dtype, void *dx, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
+                     const void *dz, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_mm("d8_matmul_grad_x", dtype, xb, xr, xc, yb, yr, yc)) return rc;
+    D8_REQUIRE(dx && y && dz, "d8_matmul_grad_x: null tensor");
+    return run(dtype, mm_plan(1, dx, xb, xr, xc, y, yb, yr, yc, dz), scratch, scratch_bytes, stream);
+}
+
+int d8_matmul_grad_y(int dtype, const void *x, int xb, int xr, int xc, void *dy, int yb, int yr, int yc,
+                     const void *dz, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_mm("d8_matmul_grad_y", dtype, xb, xr, xc, yb, yr, yc)) return rc;
+    D8_REQUIRE(x && dy && dz, "d8_matmul_grad_y: null tensor");
+    return run(dtype, mm_plan(2, x, xb, xr, xc, dy, yb, yr, yc, dz), scratch, scratch_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+int d8_conv2d_geometry(int IH, int IW, int FH, int FW, int covered, int sy, int sx, int dy, int dx, int *out) {
+    D8_REQUIRE(out, "d8_conv2d_geometry: out is null");
+    D8_REQUIRE(IH > 0 && IW > 0 && FH > 0 && FW > 0 && sy >= 1 && sx >= 1 && dy >= 1 && dx >= 1,
+               "d8_conv2d_geometry: bad geometry");
+    const int rfh = FH + (FH - 1) * (dy - 1), rfw = FW + (FW - 1) * (dx - 1);
+    int OH, OW;
+    if (!covered) {
+        OH = (IH - rfh) / sy + 1;
+        OW = (IW - rfw) / sx + 1;
+        D8_REQUIRE(rfh <= IH && rfw <= IW, "d8_conv2d_geometry: the filter is larger than the input");
+    } else {
+        OH = (IH - 1) / sy + 1;
+        OW = (IW - 1) / sx + 1;
+    }
+    out[0] = OH;
+    out[1] = OW;
+    const int py = (OH - 1) * sy + rfh - IH, px = (OW - 1) * sx + rfw - IW;
+    out[2] = (py > 0 ? py : 0) / 2;
+    out[3] = (px > 0 ? px : 0) / 2;
+    return 0;
+}
+
+int d8_deconv2d_geometry(int IH, int IW, int FH, int FW, int covered, int sy, int sx, int *out) {
+    D8_REQUIRE(out, "d8_deconv2d_geometry: out is null");
+    D8_REQUIRE(IH > 0 && IW > 0 && FH > 0 && FW > 0 && sy >= 1 && sx >= 1, "d8_deconv2d_geometry: bad geometry");
+    int OH, OW;
+    if (!covered) {
+        OH = (IH - 1) * sy + FH;
+        OW = (IW - 1) * sx + FW;
+    } else {
+        OH = (IH - 1) * sy + 1;
+        OW = (IW - 1) * sx + 1;
+    }
+    out[0] = OH;
+    out[1] = OW;
+    const int py = OH + FH - (IH - 1) * sy - 2, px = OW + FW - (IW - 1) * sx - 2;
+    out[2] = (py > 0 ? py : 0) / 2;
+    out[3] = (px > 0 ? px : 0) / 2;
+    return 0;
+}
+
+// Conv2d GEMMs on the patch matrix [M x K], M = B*OH*OW, K = FH*FW*IC.
+static Gemm conv_plan(int which, int M, int K, int OC, const void *col, const void *w, const void *zz) {
+    if (which == 0) return {0, 1, M, OC, K, col, K, 0, w, K, 0, 0.f, (void *)zz, OC, 0, 1};   // z = xcol W^T
+    if (which == 1) return {0, 0, M, K, OC, zz, OC, 0, w, K, 0, 0.f, (void *)col, K, 0, 1};   // dxcol = dz W
+    return {1, 0, OC, K, M, zz, OC, 0, col, K, 0, 1.f, (void *)w, K, 0, 1};                   // dW += dz^T xcol
+}
+
+size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
+                               int OC, int FH, int FW, int covered, int sy, int sx, int dy, int dx) {
+    int g[4];
+    if (check_conv("d8_conv2d_scratch_bytes", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return 0;
+    if (d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return 0;
+    const int M = B * g[0] * g[1], K = FH * FW * IC;
+    const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
+    return col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
+}
+
+int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
+              const void *w, int OC, int FH, int FW, void *z,
+              int covered, int sy, int sx, int dy, int dx,
+              void *scratch, size_t scratch_bytes, void *stream) {
+    int g[4];
+    if (int rc = check_conv("d8_conv2d", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return rc;
+    if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
+    const int M = B * g[0] * g[1], K = FH * FW * IC;
+    const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
+    D8_REQUIRE(x && w && z && scratch, "d8_conv2d: null tensor");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d: scratch too small");
+    if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
+        return rc;
+    const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
+    return run(dtype, conv_plan(0, M, K, OC, scratch, w, z), ws ? (char *)scratch + col : nullptr, ws, stream);
+}
+
+int d8_conv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
+                     const void *w, int OC, int FH, int FW, const void *gz,
+                     int covered, int sy, int sx, int dy, int dx,
+                     void *scratch, size_t scratch_bytes, void *stream) {
+    int g[4];
+    if (int rc = check_conv("d8_conv2d_grad_x", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return rc;
+    if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
+    const int M = B * g[0] * g[1], K = FH * FW * IC;
+    const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
+    D8_REQUIRE(gx && w && gz && scratch, "d8_conv2d_grad_x: null tensor");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_x: scratch too small");
+    const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
+    if (int rc = run(dtype, conv_plan(1, M, K, OC, scratch, w, gz), ws ? (char *)scratch + col : nullptr, ws, stream))
+        return rc;
+    return d8_col2im(dtype, scratch, gx, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream);
+}
+
+int d8_conv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
+                     void *gw, int OC, int FH, int FW, const void *gz,
+                     int covered, int sy, int sx, int dy, int dx,
+                     void *scratch, size_t scratch_bytes, void *stream) {
+    int g[4];
+    if (int rc = check_conv("d8_conv2d_grad_y", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return rc;
+    if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
+    const int M = B * g[0] * g[1], K = FH * FW * IC;
+    const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
+    D8_REQUIRE(x && gw && gz && scratch, "d8_conv2d_grad_y: null tensor");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_y: scratch too small");
+    if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
+        return rc;
+    const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
+    return run(dtype, conv_plan(2, M, K, OC, scratch, gw, gz), ws ? (char *)scratch + col : nullptr, ws, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// DeConv2d GEMMs on zmat / dzmat [M x NP], M = B*IH*IW, NP = OC*FH*FW, filter viewed [NP x IC].
+static Gemm deconv_plan(int which, int M, int NP, int IC, const void *mat, const void *w, const void *xx) {
+    if (which == 0) return {0, 1, M, NP, IC, xx, IC, 0, w, IC, 0, 0.f, (void *)mat, NP, 0, 1};  // zmat = x W^T
+    if (which == 1) return {0, 0, M, IC, NP, mat, NP, 0, w, IC, 0, 1.f, (void *)xx, IC, 0, 1};  // dx += dzmat W
+    return {1, 0, NP, IC, M, mat, NP, 0, xx, IC, 0, 1.f, (void *)w, IC, 0, 1};                  // dW += dzmat^T x
+}
+
+size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
+                                 int OC, int FH, int FW, int covered, int sy, int sx) {
+    (void)covered;
+    if (check_conv("d8_deconv2d_scratch_bytes", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return 0;
+    const int M = B * IH * IW, NP = OC * FH * FW;
+    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
+    return mat + gemm_ws(dtype, deconv_plan(which, M, NP, IC, nullptr, nullptr, nullptr));
+}
+
+int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
+                const void *w, int OC, int FH, int FW, void *z,
+                int covered, int sy, int sx,
+                void *scratch, size_t scratch_bytes, void *stream) {
+    int g[4];
+    if (int rc = check_conv("d8_deconv2d", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+    const int M = B * IH * IW, NP = OC * FH * FW;
+    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
+    D8_REQUIRE(x && w && z && scratch, "d8_deconv2d: null tensor");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * NP * dtype_bytes(dtype), "d8_deconv2d: scratch too small");
+    const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
+    if (int rc = run(dtype, deconv_plan(0, M, NP, IC, scratch, w, x), ws ? (char *)scratch + mat : nullptr, ws, stream))
+        return rc;
+    return d8_deconv_col2im(dtype, scratch, z, B, IH, IW, g[0], g[1], OC, FH, FW, sy, sx, g[2], g[3], stream);
+}
+
+int d8_deconv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
+                       const void *w, int OC, int FH, int FW, const void *gz,
+                       int covered, int sy, int sx,
+                       void *scratch, size_t scratch_bytes, void *stream) {
+    int g[4];
+    if (int rc = check_conv("d8_deconv2d_grad_x", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+    const int M = B * IH * IW, NP = OC * FH * FW;
+    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
+    D8_REQUIRE(gx && w && gz && scratch, "d8_deconv2d_grad_x: null tensor");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * NP * dtype_bytes(dtype), "d8_deconv2d_grad_x: scratch too small");
+    if (int rc = d8_deconv_im2col(dtype, gz, scratch, B, IH, IW, g[0], g[1], OC, FH, FW, sy, sx, g[2], g[3], stream))
+        return rc;
+    const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
+    return run(dtype, deconv_plan(1, M, NP, IC, scratch, w, gx), ws ? (char *)scratch + mat : nullptr, ws, stream);
+}
+
+int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
+                       void *gw, int OC, int FH, int FW, const void *gz,
+                       int covered, int sy, int sx,
+                       void *scratch, size_t scratch_bytes, void *stream) {
+    int g[4];
+    if (int rc = check_conv("d8_deconv2d_grad_y", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+    const int M = B * IH * IW, NP = OC * FH * FW;
+    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
+    D8_REQUIRE(x && gw && gz && scratch, "d8_deconv2d_grad_y: null tensor");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * NP * dtype_bytes(dtype), "d8_deconv2d_grad_y: scratch too small");
+    if (int rc = d8_deconv_im2col(dtype, gz, scratch, B, IH, IW, g[0], g[1], OC, FH, FW, sy, sx, g[2], g[3], stream))
+        return rc;
+    const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
+    return run(dtype, deconv_plan(2, M, NP, IC, scratch, gw, x), ws ? (char *)scratch + mat : nullptr, ws, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,258 @@
+"""numpy-in / numpy-out drivers of the C ABI, used by the parity tests, smoke() and bench.py.
+
+Every function copies its operands to the GPU, calls one entry point of libdeep8_hip.so and copies
+the result back.  Tensors follow Deep8's layout: first axis = Shape::batch, then Shape::dims
+(matrix: (batch, rows[, cols]); image: (B, H, W, C); filter: (OC, FH, FW, IC)).
+float32 and float16 arrays are accepted; all operands of one call must share the dtype.
+"""
+import ctypes
+
+import numpy as np
+
+from . import capi
+from .capi import DeviceArray, check
+
+
+def _same_dtype(*arrays):
+    dt = arrays[0].dtype
+    for a in arrays:
+        if a.dtype != dt:
+            raise ValueError("the data type must be same")
+    return capi.dtype_id(dt)
+
+
+def _mat(a):
+    if a.ndim == 2:
+        return a.shape[0], a.shape[1], 1
+    if a.ndim == 3:
+        return a.shape
+    raise ValueError("the shape is error")
+
+
+def matmul_out_shape(x, y):
+    xb, xr, xc = _mat(x)
+    yb, yr, yc = _mat(y)
+    if not (xb == yb or xb == 1 or yb == 1) or xc != yr:
+        raise ValueError("the shape is error")
+    return (max(xb, yb), xr) if y.ndim == 2 else (max(xb, yb), xr, yc)
+
+
+def _scratch(nbytes):
+    return DeviceArray((max(int(nbytes), 16),), np.uint8)
+
+
+def gemm(ta, tb, A, B, C=None, beta=0.0, use_workspace=True):
+    """C = op(A) op(B) + beta C for 2-D (or batched 3-D, broadcast by a leading 1) arrays."""
+    lib = capi.init()
+    A, B = np.ascontiguousarray(A), np.ascontiguousarray(B)
+    dt = _same_dtype(A, B)
+    A3 = A if A.ndim == 3 else A[None]
+    B3 = B if B.ndim == 3 else B[None]
+    K, M = (A3.shape[1], A3.shape[2]) if ta else (A3.shape[2], A3.shape[1])
+    N = B3.shape[1] if tb else B3.shape[2]
+    batch = max(A3.shape[0], B3.shape[0])
+    if C is None:
+        C3 = np.zeros((batch, M, N), A.dtype)
+    else:
+        C3 = np.ascontiguousarray(C)
+        C3 = C3 if C3.ndim == 3 else C3[None]
+    sA = 0 if A3.shape[0] == 1 else A3.shape[1] * A3.shape[2]
+    sB = 0 if B3.shape[0] == 1 else B3.shape[1] * B3.shape[2]
+    sC = 0 if C3.shape[0] == 1 else M * N
+    dA, dB, dC = DeviceArray.from_numpy(A3), DeviceArray.from_numpy(B3), DeviceArray.from_numpy(C3)
+    wsb = lib.d8_gemm_workspace_bytes(dt, ta, tb, M, N, K, batch, sC) if use_workspace else 0
+    ws = _scratch(wsb) if wsb else None
+    check(lib.d8_gemm(dt, ta, tb, M, N, K, dA.ptr, A3.shape[2], sA, dB.ptr, B3.shape[2], sB, beta,
+                      dC.ptr, N, sC, batch, ws.ptr if ws else None, wsb, None))
+    out = dC.numpy()
+    squeeze = (np.ndim(C) == 2) if C is not None else (A.ndim == 2 and B.ndim == 2)
+    return out[0] if squeeze else out
+
+
+# ---- MatrixMultiply ----------------------------------------------------------------------------
+def _mm(which, x, y, z):
+    lib = capi.init()
+    dt = _same_dtype(x, y, z)
+    xb, xr, xc = _mat(x)
+    yb, yr, yc = _mat(y)
+    dx_, dy_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray.from_numpy(z)
+    nb = lib.d8_matmul_scratch_bytes(dt, which, xb, xr, xc, yb, yr, yc)
+    ws = _scratch(nb) if nb else None
+    fn = (lib.d8_matmul, lib.d8_matmul_grad_x, lib.d8_matmul_grad_y)[which]
+    check(fn(dt, dx_.ptr, xb, xr, xc, dy_.ptr, yb, yr, yc, dz_.ptr, ws.ptr if ws else None, nb, None))
+    return (dz_, dx_, dy_)[which].numpy()
+
+
+def matmul(x, y):
+    x, y = np.ascontiguousarray(x), np.ascontiguousarray(y)
+    z = np.zeros(matmul_out_shape(x, y), x.dtype)
+    return _mm(0, x, y, z)
+
+
+def matmul_grad_x(x, y, dz, dx=None):
+    """returns dx + dz * y^T (dx defaults to zeros of x's shape; x only supplies the shape)"""
+    y, dz = np.ascontiguousarray(y), np.ascontiguousarray(dz)
+    dx = np.zeros(np.shape(x), y.dtype) if dx is None else np.ascontiguousarray(dx)
+    return _mm(1, dx, y, dz)
+
+
+def matmul_grad_y(x, y, dz, dy=None):
+    x, dz = np.ascontiguousarray(x), np.ascontiguousarray(dz)
+    dy = np.zeros(np.shape(y), x.dtype) if dy is None else np.ascontiguousarray(dy)
+    return _mm(2, x, dy, dz)
+
+
+# ---- geometry -------------------------------------------------------------------------------------
+def conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx):
+    out = (ctypes.c_int * 4)()
+    check(capi.load().d8_conv2d_geometry(IH, IW, FH, FW, int(covered), sy, sx, dy, dx, out))
+    return tuple(out)
+
+
+def deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx):
+    out = (ctypes.c_int * 4)()
+    check(capi.load().d8_deconv2d_geometry(IH, IW, FH, FW, int(covered), sy, sx, out))
+    return tuple(out)
+
+
+# ---- Conv2d ------------------------------------------------------------------------------------------
+def _filt(w):
+    w = np.ascontiguousarray(w)
+    return w[0] if w.ndim == 5 else w
+
+
+def conv2d(x, w, covered=True, sy=1, sx=1, dy=1, dx=1):
+    lib = capi.init()
+    x, w = np.ascontiguousarray(x), _filt(w)
+    dt = _same_dtype(x, w)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = w.shape
+    OH, OW, _, _ = conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx)
+    dx_, dw_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w)
+    dz_ = DeviceArray((B, OH, OW, OC), x.dtype)
+    nb = lib.d8_conv2d_scratch_bytes(dt, 0, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx)
+    ws = _scratch(nb)
+    check(lib.d8_conv2d(dt, dx_.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dz_.ptr, int(covered), sy, sx, dy, dx,
+                        ws.ptr, nb, None))
+    return dz_.numpy()
+
+
+def conv2d_grad_x(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None):
+    lib = capi.init()
+    w, gz = _filt(w), np.ascontiguousarray(gz)
+    dt = _same_dtype(w, gz)
+    B, IH, IW, IC = np.shape(x)
+    OC, FH, FW, _ = w.shape
+    gx = np.zeros((B, IH, IW, IC), w.dtype) if gx is None else np.ascontiguousarray(gx)
+    dgx, dw_, dgz = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
+    nb = lib.d8_conv2d_scratch_bytes(dt, 1, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx)
+    ws = _scratch(nb)
+    check(lib.d8_conv2d_grad_x(dt, dgx.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dgz.ptr, int(covered),
+                               sy, sx, dy, dx, ws.ptr, nb, None))
+    return dgx.numpy()
+
+
+def conv2d_grad_y(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None):
+    lib = capi.init()
+    x, gz = np.ascontiguousarray(x), np.ascontiguousarray(gz)
+    dt = _same_dtype(x, gz)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = np.shape(_filt(w)) if not isinstance(w, tuple) else w
+    gw = np.zeros((OC, FH, FW, IC), x.dtype) if gw is None else _filt(gw)
+    dx_, dgw, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(gw), DeviceArray.from_numpy(gz)
+    nb = lib.d8_conv2d_scratch_bytes(dt, 2, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx)
+    ws = _scratch(nb)
+    check(lib.d8_conv2d_grad_y(dt, dx_.ptr, B, IH, IW, IC, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
+                               sy, sx, dy, dx, ws.ptr, nb, None))
+    return dgw.numpy()
+
+
+# ---- DeConv2d -----------------------------------------------------------------------------------------
+def deconv2d(x, w, covered=False, sy=1, sx=1):
+    lib = capi.init()
+    x, w = np.ascontiguousarray(x), _filt(w)
+    dt = _same_dtype(x, w)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = w.shape
+    OH, OW, _, _ = deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx)
+    dx_, dw_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w)
+    dz_ = DeviceArray((B, OH, OW, OC), x.dtype)
+    nb = lib.d8_deconv2d_scratch_bytes(dt, 0, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx)
+    ws = _scratch(nb)
+    check(lib.d8_deconv2d(dt, dx_.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dz_.ptr, int(covered), sy, sx,
+                          ws.ptr, nb, None))
+    return dz_.numpy()
+
+
+def deconv2d_grad_x(x, w, gz, covered=False, sy=1, sx=1, gx=None):
+    lib = capi.init()
+    w, gz = _filt(w), np.ascontiguousarray(gz)
+    dt = _same_dtype(w, gz)
+    B, IH, IW, IC = np.shape(x)
+    OC, FH, FW, _ = w.shape
+    gx = np.zeros((B, IH, IW, IC), w.dtype) if gx is None else np.ascontiguousarray(gx)
+    dgx, dw_, dgz = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
+    nb = lib.d8_deconv2d_scratch_bytes(dt, 1, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx)
+    ws = _scratch(nb)
+    check(lib.d8_deconv2d_grad_x(dt, dgx.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dgz.ptr, int(covered),
+                                 sy, sx, ws.ptr, nb, None))
+    return dgx.numpy()
+
+
+def deconv2d_grad_y(x, w, gz, covered=False, sy=1, sx=1, gw=None):
+    lib = capi.init()
+    x, gz = np.ascontiguousarray(x), np.ascontiguousarray(gz)
+    dt = _same_dtype(x, gz)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = np.shape(_filt(w))
+    gw = np.zeros((OC, FH, FW, IC), x.dtype) if gw is None else _filt(gw)
+    dx_, dgw, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(gw), DeviceArray.from_numpy(gz)
+    nb = lib.d8_deconv2d_scratch_bytes(dt, 2, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx)
+    ws = _scratch(nb)
+    check(lib.d8_deconv2d_grad_y(dt, dx_.ptr, B, IH, IW, IC, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
+                                 sy, sx, ws.ptr, nb, None))
+    return dgw.numpy()
+
+
+# ---- the four maps ---------------------------------------------------------------------------------------
+def im2col(im, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft):
+    lib = capi.init()
+    im = np.ascontiguousarray(im)
+    B, IH, IW, C = im.shape
+    dim_ = DeviceArray.from_numpy(im)
+    col = DeviceArray((B * OH * OW, FH * FW * C), im.dtype)
+    check(lib.d8_im2col(capi.dtype_id(im.dtype), dim_.ptr, col.ptr, B, IH, IW, C, OH, OW, FH, FW,
+                        sy, sx, dy, dx, padTop, padLeft, None))
+    return col.numpy()
+
+
+def col2im(col, im, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft):
+    """returns im + col2im(col)"""
+    lib = capi.init()
+    col, im = np.ascontiguousarray(col), np.ascontiguousarray(im)
+    dt = _same_dtype(col, im)
+    B, IH, IW, C = im.shape
+    dcol, dim_ = DeviceArray.from_numpy(col), DeviceArray.from_numpy(im)
+    check(lib.d8_col2im(dt, dcol.ptr, dim_.ptr, B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft, None))
+    return dim_.numpy()
+
+
+def deconv_col2im(zmat, B, IH, IW, OH, OW, OC, FH, FW, sy, sx, padTop, padLeft):
+    lib = capi.init()
+    zmat = np.ascontiguousarray(zmat)
+    dzm = DeviceArray.from_numpy(zmat)
+    z = DeviceArray((B, OH, OW, OC), zmat.dtype)
+    check(lib.d8_deconv_col2im(capi.dtype_id(zmat.dtype), dzm.ptr, z.ptr, B, IH, IW, OH, OW, OC, FH, FW,
+                               sy, sx, padTop, padLeft, None))
+    return z.numpy()
+
+
+def deconv_im2col(dz, IH, IW, FH, FW, sy, sx, padTop, padLeft):
+    lib = capi.init()
+    dz = np.ascontiguousarray(dz)
+    B, OH, OW, OC = dz.shape
+    ddz = DeviceArray.from_numpy(dz)
+    m = DeviceArray((B * IH * IW, OC * FH * FW), dz.dtype)
+    check(lib.d8_deconv_im2col(capi.dtype_id(dz.dtype), ddz.ptr, m.ptr, B, IH, IW, OH, OW, OC, FH, FW,
+                               sy, sx, padTop, padLeft, None))
+    return m.numpy()

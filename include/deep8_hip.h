@@ -1,0 +1,170 @@
+/*
+ * deep8_hip.h -- C ABI of libdeep8_hip.so: the MI355X (gfx950) kernels behind Deep8's
+ * MatrixMultiply / Conv2d / DeConv2d GPU entry points.
+ *
+ * Plain pointers and integers only.  Every function returns 0 on success or a non-zero code
+ * (a hipError_t value, or D8_ERR_* below); d8_last_error() gives the text.  Nothing throws
+ * across this boundary; the C++ host layer turns a non-zero code into the same
+ * std::runtime_error Deep8's CUDA_CHECK raises (deep8/include/basic/GPUException.h:15-24).
+ *
+ * All matrices are row-major (deep8/src/model/Shape.cpp:86-96).  Device pointers unless said
+ * otherwise.  `stream` is a hipStream_t passed as void* (NULL = the default stream, which is
+ * what Deep8 uses everywhere).  All launches are asynchronous.
+ */
+#ifndef DEEP8_HIP_H
+#define DEEP8_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types: the ids of Deep8's DType (deep8/include/model/ElementType.h:8-22) */
+#define D8_FLOAT16 10
+#define D8_FLOAT32 11
+
+#define D8_ERR_ARGUMENT 10001 /* bad shape / leading dimension / null pointer */
+#define D8_ERR_DTYPE    10002 /* element type not supported by this build     */
+#define D8_ERR_ARCH     10003 /* the device is not gfx950                      */
+
+const char *d8_last_error(void);
+
+/* ---- device plumbing -------------------------------------------------------------------
+ * Replaces what GPUDevice / GPUMemoryAllocator do through the CUDA runtime
+ * (deep8/src/model/GPUDevice.cu:10-12, deep8/src/model/GPUMemoryAllocator.cu:17-56).      */
+int d8_device_init(int device_id);                /* hipSetDevice + arch check (gfx950)    */
+int d8_device_count(int *count);
+int d8_device_info(int *cu_count, int *clock_khz, size_t *hbm_bytes, char *name, int name_len);
+int d8_malloc(void **ptr, size_t bytes);          /* cudaMalloc      GPUMemoryAllocator.cu:17 */
+int d8_free(void *ptr);                           /* cudaFree        GPUMemoryAllocator.cu:27 */
+int d8_host_malloc(void **ptr, size_t bytes);     /* pinned host memory                    */
+int d8_host_free(void *ptr);
+int d8_memset(void *ptr, int value, size_t bytes, void *stream);   /* cudaMemset  :34      */
+int d8_memcpy_h2d(void *dst, const void *src, size_t bytes);       /* cudaMemcpy  :46      */
+int d8_memcpy_d2h(void *dst, const void *src, size_t bytes);       /* cudaMemcpy  :50      */
+int d8_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);  /* :40,:54     */
+int d8_stream_create(void **stream);
+int d8_stream_destroy(void *stream);
+int d8_stream_sync(void *stream);
+int d8_event_create(void **event);
+int d8_event_destroy(void *event);
+int d8_event_record(void *event, void *stream);
+int d8_event_elapsed_ms(void *start, void *stop, float *ms);  /* synchronises on `stop` */
+
+/* ---- GEMM ------------------------------------------------------------------------------
+ * C_b = op(A_b) * op(B_b) + beta * C_b,   b = 0 .. batch-1,  beta in {0, 1}
+ *
+ * op(A) is M x K, op(B) is K x N.  transA != 0: A is stored K x M (lda >= M); otherwise M x K
+ * (lda >= K).  transB != 0: B is stored N x K (ldb >= K); otherwise K x N (ldb >= N).
+ * transA and transB both set is rejected (Deep8 never issues it).  Strides are in elements;
+ * strideA/strideB 0 broadcasts that operand over the batch.  strideC == 0 with batch > 1
+ * sums all batch products into the one C (Deep8's gradient of a batch-1 operand).
+ * fp16 operands accumulate in fp32 and are rounded once; beta = 1 adds the old C in fp32.
+ *
+ * `workspace` (may be NULL) lets the kernel split the reduction (long K / summed batch, small
+ * M x N) over more workgroups; d8_gemm_workspace_bytes says how much it can use.
+ *
+ * Replaces the 27 cublas{S,H}gemm call sites in deep8/src/math/MatrixMultiply.cu:36-55,
+ * 75-94,115-134 (forward), :211-230,253-272,296-315 (GradX), :399-418,441-460,484-503
+ * (GradY) and the 18 in deep8/src/math/Conv2d.cu:195,473,801 / DeConv2d.cu:109,428,699
+ * (+ their half twins).                                                                    */
+size_t d8_gemm_workspace_bytes(int dtype, int transA, int transB, int M, int N, int K,
+                               int batch, long strideC);
+int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
+            const void *A, int lda, long strideA,
+            const void *B, int ldb, long strideB,
+            float beta, void *C, int ldc, long strideC, int batch,
+            void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- Conv2d gather / scatter -------------------------------------------------------------
+ * Geometry is explicit; padTop/padLeft >= 0 count the zero rows/columns before the image
+ * (Deep8 passes the same numbers negated, deep8/src/math/Conv2d.cu:335-336).
+ *
+ * d8_im2col:  col[(b,oy,ox)][(fy,fx,c)] = im[b, oy*sy + fy*dy - padTop, ox*sx + fx*dx - padLeft, c]
+ *             or +0 outside.  col is [B*OH*OW, FH*FW*C].   Replaces Conv2dIm2ColKernel
+ *             (deep8/src/math/Conv2d.cu:10-61, launched :170,:776).
+ * d8_col2im:  im += transpose of that map applied to col; taps added in (fy,fx) ascending
+ *             order.  Replaces Conv2dCol2ImKernel (Conv2d.cu:64-118, launched :475).       */
+int d8_im2col(int dtype, const void *im, void *col,
+              int B, int IH, int IW, int C, int OH, int OW, int FH, int FW,
+              int sy, int sx, int dy, int dx, int padTop, int padLeft, void *stream);
+int d8_col2im(int dtype, const void *col, void *im,
+              int B, int IH, int IW, int C, int OH, int OW, int FH, int FW,
+              int sy, int sx, int dy, int dx, int padTop, int padLeft, void *stream);
+
+/* ---- DeConv2d gather maps ------------------------------------------------------------------
+ * zmat / dzmat are [B*IH*IW, OC*FH*FW] with column index oc*FH*FW + fy*FW + fx.
+ *
+ * d8_deconv_col2im: z[b,oy,ox,oc] = sum over taps (fy,fx) with iy*sy == oy - padTop + fy,
+ *             ix*sx == ox - padLeft + fx inside the input, of zmat[(b,iy,ix)][oc,fy,fx];
+ *             overwrites z.  Replaces DeConv2dCol2ImKernel (deep8/src/math/DeConv2d.cu:11-58,
+ *             launched :115).
+ * d8_deconv_im2col: dzmat[(b,iy,ix)][oc,fy,fx] = dz[b, iy*sy + padTop - fy, ix*sx + padLeft - fx, oc]
+ *             or +0 outside.  Replaces DeConv2dIm2ColKernel (DeConv2d.cu:310-351, launched
+ *             :405,:675).                                                                   */
+int d8_deconv_col2im(int dtype, const void *zmat, void *z,
+                     int B, int IH, int IW, int OH, int OW, int OC, int FH, int FW,
+                     int sy, int sx, int padTop, int padLeft, void *stream);
+int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
+                     int B, int IH, int IW, int OH, int OW, int OC, int FH, int FW,
+                     int sy, int sx, int padTop, int padLeft, void *stream);
+
+/* ---- whole-operator entry points -----------------------------------------------------------
+ * What Math::*GPU call (deep8/include/math/MatrixMultiply.h:17,26,35, Conv2d.h:23,33,45,
+ * DeConv2d.h:18,28,38): shape cases, pad formulas, scratch use and accumulate-vs-overwrite
+ * semantics are Deep8's.  A matrix operand is (batch, rows, cols) with cols = 1 for a 1-D
+ * tensor.  `scratch` is the interim buffer the node allocates (size from the *_scratch_bytes
+ * function, which already includes any split-reduction workspace).                          */
+size_t d8_matmul_scratch_bytes(int dtype, int which /*0 fwd, 1 gradX, 2 gradY*/,
+                               int xb, int xr, int xc, int yb, int yr, int yc);
+int d8_matmul(int dtype, const void *x, int xb, int xr, int xc,
+              const void *y, int yb, int yr, int yc, void *z,
+              void *scratch, size_t scratch_bytes, void *stream);
+int d8_matmul_grad_x(int dtype, void *dx, int xb, int xr, int xc,
+                     const void *y, int yb, int yr, int yc, const void *dz,
+                     void *scratch, size_t scratch_bytes, void *stream);
+int d8_matmul_grad_y(int dtype, const void *x, int xb, int xr, int xc,
+                     void *dy, int yb, int yr, int yc, const void *dz,
+                     void *scratch, size_t scratch_bytes, void *stream);
+
+/* out[0..3] = OH, OW, padTop, padLeft (deep8/src/math/Conv2d.cpp:20-32, Conv2d.cu:332-336;
+ * deep8/src/math/DeConv2d.cpp:23-29, DeConv2d.cu:99-100) */
+int d8_conv2d_geometry(int IH, int IW, int FH, int FW, int covered,
+                       int sy, int sx, int dy, int dx, int *out);
+int d8_deconv2d_geometry(int IH, int IW, int FH, int FW, int covered, int sy, int sx, int *out);
+
+size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
+                               int OC, int FH, int FW, int covered, int sy, int sx, int dy, int dx);
+int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
+              const void *w, int OC, int FH, int FW, void *z,
+              int covered, int sy, int sx, int dy, int dx,
+              void *scratch, size_t scratch_bytes, void *stream);
+int d8_conv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
+                     const void *w, int OC, int FH, int FW, const void *gz,
+                     int covered, int sy, int sx, int dy, int dx,
+                     void *scratch, size_t scratch_bytes, void *stream);
+int d8_conv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
+                     void *gw, int OC, int FH, int FW, const void *gz,
+                     int covered, int sy, int sx, int dy, int dx,
+                     void *scratch, size_t scratch_bytes, void *stream);
+
+size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
+                                 int OC, int FH, int FW, int covered, int sy, int sx);
+int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
+                const void *w, int OC, int FH, int FW, void *z,
+                int covered, int sy, int sx,
+                void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
+                       const void *w, int OC, int FH, int FW, const void *gz,
+                       int covered, int sy, int sx,
+                       void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
+                       void *gw, int OC, int FH, int FW, const void *gz,
+                       int covered, int sy, int sx,
+                       void *scratch, size_t scratch_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEP8_HIP_H */

@@ -1,0 +1,332 @@
+"""CPU checkers for the Deep8 dense-contraction hot path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests/, ``__graft_entry__.smoke()`` and ``bench.py``'s ``cpu_baseline`` leg may import this
+package; the product (``deep8_amd``) never does.
+
+Two checkers with the same numpy-level interface:
+
+* ``port``  -- ``libdeep8_oracle.so``, the plain-C restatement in ``deep8_oracle.c``.
+* ``ref``   -- ``_ref/libdeep8_ref.so``, Deep8's own CPU (Eigen) sources compiled unmodified and
+  wrapped by ``ref_shim.cpp``; ``None`` when it has not been built.
+
+Tensors are numpy float32 arrays whose first axis is Deep8's ``Shape::batch`` and whose remaining
+axes are ``Shape::dims`` (deep8/include/model/Shape.h:32-83): a matrix operand is ``(batch, rows)``
+or ``(batch, rows, cols)``, an image ``(B, H, W, C)``, a filter ``(1, OC, FH, FW, IC)`` or
+``(OC, FH, FW, IC)``.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+PORT_PATH = os.path.join(_HERE, "libdeep8_oracle.so")
+REF_PATH = os.path.join(_HERE, "_ref", "libdeep8_ref.so")
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_i = ctypes.c_int
+
+
+def build(with_ref=True):
+    """Compile the checkers (the reference build only where /root/reference exists)."""
+    subprocess.check_call(["make", "-s", "-C", _HERE, "oracle"])
+    if with_ref:
+        subprocess.check_call(["make", "-s", "-j8", "-C", _HERE, "ref"])
+
+
+def _p(a):
+    return a.ctypes.data_as(_f32p)
+
+
+def _c(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a
+
+
+def _mat(a):
+    """(batch, nDims, rows, cols) of a matrix operand."""
+    if a.ndim == 2:
+        return a.shape[0], 1, a.shape[1], 1
+    if a.ndim == 3:
+        return a.shape[0], 2, a.shape[1], a.shape[2]
+    raise ValueError("matrix operand must be (batch, rows[, cols])")
+
+
+def matmul_out_shape(x, y):
+    """deep8/src/nodes/MatrixMultiply.cpp:10-28"""
+    xb, _, xr, xc = _mat(x)
+    yb, _, yr, yc = _mat(y)
+    if not (xb == yb or xb == 1 or yb == 1) or xc != yr:
+        raise ValueError("shape error")
+    return (max(xb, yb), xr) if yc == 1 else (max(xb, yb), xr, yc)
+
+
+def _filt(w):
+    w = _c(w)
+    if w.ndim == 5:
+        assert w.shape[0] == 1
+        w = w[0]
+    return w
+
+
+class _Port:
+    name = "port"
+
+    def __init__(self, path):
+        self.lib = ctypes.CDLL(path)
+        self.lib.orc_threads.restype = _i
+
+    def threads(self):
+        return self.lib.orc_threads()
+
+    # -- MatrixMultiply ------------------------------------------------------------------
+    def matmul(self, x, y):
+        x, y = _c(x), _c(y)
+        z = np.zeros(matmul_out_shape(x, y), np.float32)
+        xb, _, xr, xc = _mat(x)
+        yb, _, yr, yc = _mat(y)
+        self.lib.orc_matmul(_p(x), _i(xb), _i(xr), _i(xc), _p(y), _i(yb), _i(yr), _i(yc), _p(z))
+        return z
+
+    def matmul_grad_x(self, x, y, dz, dx=None):
+        x, y, dz = _c(x), _c(y), _c(dz)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        xb, _, xr, xc = _mat(x)
+        yb, _, yr, yc = _mat(y)
+        self.lib.orc_matmul_grad_x(_p(dx), _i(xb), _i(xr), _i(xc), _p(y), _i(yb), _i(yr), _i(yc), _p(dz))
+        return dx
+
+    def matmul_grad_y(self, x, y, dz, dy=None):
+        x, y, dz = _c(x), _c(y), _c(dz)
+        dy = np.zeros_like(y) if dy is None else _c(dy).copy()
+        xb, _, xr, xc = _mat(x)
+        yb, _, yr, yc = _mat(y)
+        self.lib.orc_matmul_grad_y(_p(x), _i(xb), _i(xr), _i(xc), _p(dy), _i(yb), _i(yr), _i(yc), _p(dz))
+        return dy
+
+    def gemm(self, ta, tb, A, B, C=None, beta=0.0):
+        A, B = _c(A), _c(B)
+        M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+        N = B.shape[0] if tb else B.shape[1]
+        C = np.zeros((M, N), np.float32) if C is None else _c(C).copy()
+        self.lib.orc_gemm(_i(ta), _i(tb), _i(M), _i(N), _i(K), _p(A), _i(A.shape[1]), _p(B), _i(B.shape[1]),
+                          ctypes.c_float(beta), _p(C), _i(N))
+        return C
+
+    # -- geometry --------------------------------------------------------------------------
+    def conv2d_geometry(self, IH, IW, FH, FW, covered, sy, sx, dy, dx):
+        out = (ctypes.c_int * 4)()
+        self.lib.orc_conv2d_geometry(IH, IW, FH, FW, int(covered), sy, sx, dy, dx, out)
+        return tuple(out)
+
+    def deconv2d_geometry(self, IH, IW, FH, FW, covered, sy, sx):
+        out = (ctypes.c_int * 4)()
+        self.lib.orc_deconv2d_geometry(IH, IW, FH, FW, int(covered), sy, sx, out)
+        return tuple(out)
+
+    # -- Conv2d ----------------------------------------------------------------------------
+    def conv2d(self, x, w, covered=True, sy=1, sx=1, dy=1, dx=1):
+        x, w = _c(x), _filt(w)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        OH, OW, _, _ = self.conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx)
+        z = np.zeros((B, OH, OW, OC), np.float32)
+        self.lib.orc_conv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), int(covered), sy, sx, dy, dx)
+        return z
+
+    def conv2d_grad_x(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
+        self.lib.orc_conv2d_grad_x(_p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(gz), int(covered), sy, sx, dy, dx)
+        return gx
+
+    def conv2d_grad_y(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
+        self.lib.orc_conv2d_grad_y(_p(x), B, IH, IW, IC, _p(gw), OC, FH, FW, _p(gz), int(covered), sy, sx, dy, dx)
+        return gw
+
+    # -- DeConv2d --------------------------------------------------------------------------
+    def deconv2d(self, x, w, covered=False, sy=1, sx=1):
+        x, w = _c(x), _filt(w)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        OH, OW, _, _ = self.deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx)
+        z = np.zeros((B, OH, OW, OC), np.float32)
+        self.lib.orc_deconv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), int(covered), sy, sx)
+        return z
+
+    def deconv2d_grad_x(self, x, w, gz, covered=False, sy=1, sx=1, gx=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
+        self.lib.orc_deconv2d_grad_x(_p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(gz), int(covered), sy, sx)
+        return gx
+
+    def deconv2d_grad_y(self, x, w, gz, covered=False, sy=1, sx=1, gw=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
+        self.lib.orc_deconv2d_grad_y(_p(x), B, IH, IW, IC, _p(gw), OC, FH, FW, _p(gz), int(covered), sy, sx)
+        return gw
+
+    # -- gather / scatter maps ---------------------------------------------------------------
+    def im2col(self, im, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft):
+        im = _c(im)
+        B, IH, IW, C = im.shape
+        col = np.empty((B * OH * OW, FH * FW * C), np.float32)
+        self.lib.orc_im2col(_p(im), _p(col), B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft)
+        return col
+
+    def col2im(self, col, im, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft):
+        """returns im + col2im(col)"""
+        col, im = _c(col), _c(im).copy()
+        B, IH, IW, C = im.shape
+        self.lib.orc_col2im(_p(col), _p(im), B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft)
+        return im
+
+    def deconv_col2im(self, zmat, B, IH, IW, OH, OW, OC, FH, FW, sy, sx, padTop, padLeft):
+        zmat = _c(zmat)
+        z = np.empty((B, OH, OW, OC), np.float32)
+        self.lib.orc_deconv_col2im(_p(zmat), _p(z), B, IH, IW, OH, OW, OC, FH, FW, sy, sx, padTop, padLeft)
+        return z
+
+    def deconv_im2col(self, dz, IH, IW, FH, FW, sy, sx, padTop, padLeft):
+        dz = _c(dz)
+        B, OH, OW, OC = dz.shape
+        m = np.empty((B * IH * IW, OC * FH * FW), np.float32)
+        self.lib.orc_deconv_im2col(_p(dz), _p(m), B, IH, IW, OH, OW, OC, FH, FW, sy, sx, padTop, padLeft)
+        return m
+
+
+class _Ref:
+    """Deep8's own CPU path (float only)."""
+    name = "reference"
+
+    def __init__(self, path):
+        self.lib = ctypes.CDLL(path)
+        self.lib.ref_last_error.restype = ctypes.c_char_p
+        self.lib.ref_threads.restype = _i
+
+    def threads(self):
+        return self.lib.ref_threads()
+
+    def _chk(self, rc):
+        if rc == 1:
+            raise ValueError(self.lib.ref_last_error().decode())
+        if rc:
+            raise RuntimeError(self.lib.ref_last_error().decode())
+
+    def matmul(self, x, y, z_shape=None):
+        x, y = _c(x), _c(y)
+        z = np.zeros(matmul_out_shape(x, y) if z_shape is None else z_shape, np.float32)
+        self._chk(self.lib.ref_matmul(_p(x), *map(_i, _mat(x)), _p(y), *map(_i, _mat(y)), _p(z), *map(_i, _mat(z))))
+        return z
+
+    def matmul_grad_x(self, x, y, dz, dx=None):
+        x, y, dz = _c(x), _c(y), _c(dz)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        z = np.zeros_like(dz)
+        self._chk(self.lib.ref_matmul_grad_x(_p(x), _p(dx), *map(_i, _mat(x)), _p(y), *map(_i, _mat(y)),
+                                             _p(z), _p(dz), *map(_i, _mat(dz))))
+        return dx
+
+    def matmul_grad_y(self, x, y, dz, dy=None):
+        x, y, dz = _c(x), _c(y), _c(dz)
+        dy = np.zeros_like(y) if dy is None else _c(dy).copy()
+        z = np.zeros_like(dz)
+        self._chk(self.lib.ref_matmul_grad_y(_p(x), *map(_i, _mat(x)), _p(y), _p(dy), *map(_i, _mat(y)),
+                                             _p(z), _p(dz), *map(_i, _mat(dz))))
+        return dy
+
+    def conv2d(self, x, w, covered=True, sy=1, sx=1, dy=1, dx=1, out_hw=None):
+        x, w = _c(x), _filt(w)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        OH, OW = out_hw if out_hw else port.conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx)[:2]
+        z = np.zeros((B, OH, OW, OC), np.float32)
+        self._chk(self.lib.ref_conv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), OH, OW,
+                                      int(covered), sy, sx, dy, dx))
+        return z
+
+    def conv2d_grad_x(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        _, OH, OW, _ = gz.shape
+        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
+        z = np.zeros_like(gz)
+        self._chk(self.lib.ref_conv2d_grad_x(_p(x), _p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), _p(gz),
+                                             OH, OW, int(covered), sy, sx, dy, dx))
+        return gx
+
+    def conv2d_grad_y(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        _, OH, OW, _ = gz.shape
+        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
+        z = np.zeros_like(gz)
+        self._chk(self.lib.ref_conv2d_grad_y(_p(x), B, IH, IW, IC, _p(w), _p(gw), OC, FH, FW, _p(z), _p(gz),
+                                             OH, OW, int(covered), sy, sx, dy, dx))
+        return gw
+
+    def deconv2d(self, x, w, covered=False, sy=1, sx=1, out_hw=None):
+        x, w = _c(x), _filt(w)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        OH, OW = out_hw if out_hw else port.deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx)[:2]
+        z = np.zeros((B, OH, OW, OC), np.float32)
+        self._chk(self.lib.ref_deconv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), OH, OW,
+                                        int(covered), sy, sx))
+        return z
+
+    def deconv2d_grad_x(self, x, w, gz, covered=False, sy=1, sx=1, gx=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        _, OH, OW, _ = gz.shape
+        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
+        z = np.zeros_like(gz)
+        self._chk(self.lib.ref_deconv2d_grad_x(_p(x), _p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), _p(gz),
+                                               OH, OW, int(covered), sy, sx))
+        return gx
+
+    def deconv2d_grad_y(self, x, w, gz, covered=False, sy=1, sx=1, gw=None):
+        x, w, gz = _c(x), _filt(w), _c(gz)
+        B, IH, IW, IC = x.shape
+        OC, FH, FW, _ = w.shape
+        _, OH, OW, _ = gz.shape
+        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
+        z = np.zeros_like(gz)
+        self._chk(self.lib.ref_deconv2d_grad_y(_p(x), B, IH, IW, IC, _p(w), _p(gw), OC, FH, FW, _p(z), _p(gz),
+                                               OH, OW, int(covered), sy, sx))
+        return gw
+
+    def image_patches(self, im, FH, FW, sy, sx, dy, dx, iy, ix, pt, pb, pl, pr, OH, OW):
+        """Materialised Eigen extract_image_patches(...).reshape([B*OH*OW, FH*FW*C])."""
+        im = _c(im)
+        B, H, W, C = im.shape
+        out = np.empty((B * OH * OW, FH * FW * C), np.float32)
+        self._chk(self.lib.ref_image_patches(_p(im), B, H, W, C, FH, FW, sy, sx, dy, dx, iy, ix,
+                                             pt, pb, pl, pr, OH, OW, _p(out)))
+        return out
+
+
+port = _Port(PORT_PATH) if os.path.exists(PORT_PATH) else None
+ref = _Ref(REF_PATH) if os.path.exists(REF_PATH) else None
+
+
+def rel_fro(got, want):
+    """||got - want||_F / ||want||_F in double."""
+    g = np.asarray(got, np.float64).ravel()
+    w = np.asarray(want, np.float64).ravel()
+    d = np.linalg.norm(w)
+    return float(np.linalg.norm(g - w) / d) if d else float(np.linalg.norm(g))

@@ -1,0 +1,80 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU restatement (plain C) of Deep8's dense-contraction hot path.
+ * Only tests, the smoke check and the benchmark's cpu_baseline leg may load this library; the
+ * product path (the HIP library) never does.
+ *
+ * Conventions: every matrix is row-major; images are [B,H,W,C]; filters are [OC,FH,FW,IC].
+ * All sums are carried in double and rounded to float once, so for integer-valued inputs the
+ * results are exact and for real inputs they are at least as accurate as the reference's Eigen
+ * float accumulation (the parity tests compare against both).
+ *
+ * Pin status (which independent check fixes each function) is recorded in deep8_oracle.c.
+ */
+#ifndef DEEP8_ORACLE_H
+#define DEEP8_ORACLE_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- MatrixMultiply: x (xb,[xr,xc]), y (yb,[yr,yc]), z (max(xb,yb),[xr,yc]) -------------- */
+void orc_matmul(const float *x, int xb, int xr, int xc,
+                const float *y, int yb, int yr, int yc, float *z);
+void orc_matmul_grad_x(float *dx, int xb, int xr, int xc,
+                       const float *y, int yb, int yr, int yc, const float *dz);
+void orc_matmul_grad_y(const float *x, int xb, int xr, int xc,
+                       float *dy, int yb, int yr, int yc, const float *dz);
+
+/* ---- generic row-major GEMM, C = op(A) op(B) + beta*C, beta in {0,1} ---------------------- */
+void orc_gemm(int transA, int transB, int M, int N, int K,
+              const float *A, int lda, const float *B, int ldb, float beta, float *C, int ldc);
+
+/* ---- Deep8 geometry ------------------------------------------------------------------------ */
+/* out[0..3] = OH, OW, padTop, padLeft (pads >= 0, rows/cols of zeros before the image) */
+void orc_conv2d_geometry(int IH, int IW, int FH, int FW, int covered,
+                         int sy, int sx, int dy, int dx, int *out);
+void orc_deconv2d_geometry(int IH, int IW, int FH, int FW, int covered,
+                           int sy, int sx, int *out);
+
+/* ---- Conv2d, direct loops ------------------------------------------------------------------- */
+void orc_conv2d(const float *x, int B, int IH, int IW, int IC,
+                const float *w, int OC, int FH, int FW, float *z,
+                int covered, int sy, int sx, int dy, int dx);
+void orc_conv2d_grad_x(float *gx, int B, int IH, int IW, int IC,
+                       const float *w, int OC, int FH, int FW, const float *gz,
+                       int covered, int sy, int sx, int dy, int dx);
+void orc_conv2d_grad_y(const float *x, int B, int IH, int IW, int IC,
+                       float *gw, int OC, int FH, int FW, const float *gz,
+                       int covered, int sy, int sx, int dy, int dx);
+
+/* ---- DeConv2d, direct loops ----------------------------------------------------------------- */
+void orc_deconv2d(const float *x, int B, int IH, int IW, int IC,
+                  const float *w, int OC, int FH, int FW, float *z,
+                  int covered, int sy, int sx);
+void orc_deconv2d_grad_x(float *gx, int B, int IH, int IW, int IC,
+                         const float *w, int OC, int FH, int FW, const float *gz,
+                         int covered, int sy, int sx);
+void orc_deconv2d_grad_y(const float *x, int B, int IH, int IW, int IC,
+                         float *gw, int OC, int FH, int FW, const float *gz,
+                         int covered, int sy, int sx);
+
+/* ---- the four gather/scatter maps, explicit geometry ---------------------------------------- */
+/* col[(b,oy,ox)][(fy,fx,c)] = im[b, oy*sy + fy*dy - padTop, ox*sx + fx*dx - padLeft, c] or +0 */
+void orc_im2col(const float *im, float *col, int B, int IH, int IW, int C, int OH, int OW,
+                int FH, int FW, int sy, int sx, int dy, int dx, int padTop, int padLeft);
+/* im[...] += the same map transposed */
+void orc_col2im(const float *col, float *im, int B, int IH, int IW, int C, int OH, int OW,
+                int FH, int FW, int sy, int sx, int dy, int dx, int padTop, int padLeft);
+/* z[b,oy,ox,oc] = sum_{fy,fx : (oy-padTop+fy) = iy*sy, ...} zmat[(b,iy,ix)][oc*FH*FW+fy*FW+fx] */
+void orc_deconv_col2im(const float *zmat, float *z, int B, int IH, int IW, int OH, int OW, int OC,
+                       int FH, int FW, int sy, int sx, int padTop, int padLeft);
+/* dzmat[(b,iy,ix)][oc*FH*FW+fy*FW+fx] = dz[b, iy*sy+padTop-fy, ix*sx+padLeft-fx, oc] or +0 */
+void orc_deconv_im2col(const float *dz, float *dzmat, int B, int IH, int IW, int OH, int OW, int OC,
+                       int FH, int FW, int sy, int sx, int padTop, int padLeft);
+
+int orc_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,123 @@
+"""d8_gemm against the oracle's GEMM: integer inputs must match bit for bit (every partial sum is
+an exactly representable integer, so summation order cannot matter -- the reference tests' own
+trick, test/MatrixMultiplyTest.h:25-41); seeded real inputs must match within the tolerance."""
+import numpy as np
+import pytest
+
+from util import FP16_TOL, FP32_TOL, f, h, ints, rel_fro, rng, uni
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(64, 256, 128), (128, 128, 32), (1, 1, 1), (7, 5, 3), (130, 70, 33), (257, 129, 65), (33, 300, 17),
+          (300, 1, 100), (1, 300, 100), (512, 512, 512)]
+TRANS = [(0, 0), (0, 1), (1, 0)]
+
+
+def _ab(r, ta, tb, M, N, K, gen):
+    A = gen(r, (K, M) if ta else (M, K))
+    B = gen(r, (N, K) if tb else (K, N))
+    return A, B
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_gemm_f32_integer_exact(oracle_port, ta, tb, M, N, K):
+    from deep8_amd import ops
+    r = rng(M * 7 + N * 3 + K)
+    A, B = _ab(r, ta, tb, M, N, K, lambda r, s: ints(r, s, 50))
+    C0 = ints(r, (M, N), 50)
+    for beta, C in ((0.0, None), (1.0, C0)):
+        want = oracle_port.gemm(ta, tb, A, B, C, beta)
+        got = ops.gemm(ta, tb, A, B, C, beta)
+        assert np.array_equal(got, want), (ta, tb, M, N, K, beta)
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_gemm_f16_integer_exact(oracle_port, ta, tb, M, N, K):
+    from deep8_amd import ops
+    r = rng(M * 7 + N * 3 + K + 1)
+    hi = 4 if K <= 128 else 2  # keep every result below 2048 so fp16 holds it exactly
+    A, B = _ab(r, ta, tb, M, N, K, lambda r, s: ints(r, s, hi))
+    C0 = ints(r, (M, N), 4)
+    for beta, C in ((0.0, None), (1.0, C0)):
+        want = oracle_port.gemm(ta, tb, A, B, C, beta)
+        assert want.max() < 2048
+        got = ops.gemm(ta, tb, h(A), h(B), None if C is None else h(C), beta)
+        assert got.dtype == np.float16
+        assert np.array_equal(f(got), want), (ta, tb, M, N, K, beta)
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("M,N,K", [(64, 256, 128), (257, 129, 65), (512, 512, 512), (96, 80, 4099)])
+def test_gemm_real_tolerance(oracle_port, ta, tb, M, N, K):
+    from deep8_amd import ops
+    r = rng(11 + M + N + K)
+    A, B = _ab(r, ta, tb, M, N, K, uni)
+    C0 = uni(r, (M, N))
+    want = oracle_port.gemm(ta, tb, A, B, C0, 1.0)
+    assert rel_fro(ops.gemm(ta, tb, A, B, C0, 1.0), want) <= FP32_TOL
+    Ah, Bh, Ch = h(A), h(B), h(C0)
+    want_h = oracle_port.gemm(ta, tb, f(Ah), f(Bh), f(Ch), 1.0)
+    assert rel_fro(f(ops.gemm(ta, tb, Ah, Bh, Ch, 1.0)), want_h) <= FP16_TOL
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_gemm_batched_and_broadcast(oracle_port, ta, tb):
+    from deep8_amd import ops
+    r = rng(5)
+    M, N, K, nb = 70, 45, 50, 5
+    for abatch, bbatch in ((nb, nb), (1, nb), (nb, 1)):
+        A = ints(r, (abatch,) + ((K, M) if ta else (M, K)))
+        B = ints(r, (bbatch,) + ((N, K) if tb else (K, N)))
+        C0 = ints(r, (nb, M, N))
+        got = ops.gemm(ta, tb, A, B, C0, 1.0)
+        for b in range(nb):
+            want = oracle_port.gemm(ta, tb, A[b % abatch], B[b % bbatch], C0[b], 1.0)
+            assert np.array_equal(got[b], want)
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("use_ws", [True, False])
+def test_gemm_batch_summed_into_one_output(oracle_port, ta, tb, use_ws):
+    """strideC == 0: all batch products accumulate into the single C (gradient of a batch-1 operand)."""
+    from deep8_amd import ops
+    r = rng(6)
+    M, N, K, nb = 40, 33, 70, 6
+    A = ints(r, (nb,) + ((K, M) if ta else (M, K)), 20)
+    B = ints(r, (nb,) + ((N, K) if tb else (K, N)), 20)
+    C0 = ints(r, (M, N))
+    want = C0.copy()
+    for b in range(nb):
+        want = oracle_port.gemm(ta, tb, A[b], B[b], want, 1.0)
+    got = ops.gemm(ta, tb, A, B, C0, 1.0, use_workspace=use_ws)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("use_ws", [True, False])
+def test_gemm_long_reduction_split(oracle_port, use_ws):
+    """Skinny output, long K: the split path (with workspace) and the single-pass path agree with the oracle."""
+    from deep8_amd import ops
+    r = rng(7)
+    M, N, K = 64, 96, 20000
+    A, B = ints(r, (K, M), 8), ints(r, (K, N), 8)
+    C0 = ints(r, (M, N))
+    want = oracle_port.gemm(1, 0, A, B, C0, 1.0)
+    assert np.array_equal(ops.gemm(1, 0, A, B, C0, 1.0, use_workspace=use_ws), want)
+    Ar, Br = uni(r, (K, M)), uni(r, (K, N))
+    want = oracle_port.gemm(1, 0, Ar, Br, C0, 1.0)
+    assert rel_fro(ops.gemm(1, 0, Ar, Br, C0, 1.0, use_workspace=use_ws), want) <= FP32_TOL
+
+
+def test_gemm_argument_errors():
+    from deep8_amd import capi
+    lib = capi.init()
+    a = capi.DeviceArray((16, 16), np.float32, zero=True)
+    rc = lib.d8_gemm(capi.FLOAT32, 1, 1, 16, 16, 16, a.ptr, 16, 0, a.ptr, 16, 0, 0.0, a.ptr, 16, 0, 1, None, 0, None)
+    assert rc == 10001 and b"transA" in lib.d8_last_error()
+    rc = lib.d8_gemm(12, 0, 0, 16, 16, 16, a.ptr, 16, 0, a.ptr, 16, 0, 0.0, a.ptr, 16, 0, 1, None, 0, None)
+    assert rc == 10002
+    rc = lib.d8_gemm(capi.FLOAT32, 0, 0, 16, 16, 16, a.ptr, 8, 0, a.ptr, 16, 0, 0.0, a.ptr, 16, 0, 1, None, 0, None)
+    assert rc == 10001 and b"lda" in lib.d8_last_error()
+    rc = lib.d8_gemm(capi.FLOAT32, 0, 0, 16, 16, 16, a.ptr, 16, 0, a.ptr, 16, 0, 0.5, a.ptr, 16, 0, 1, None, 0, None)
+    assert rc == 10001 and b"beta" in lib.d8_last_error()

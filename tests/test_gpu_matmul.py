@@ -1,0 +1,122 @@
+"""MatrixMultiply forward / GradX / GradY through the C ABI against the oracle: the three shape
+cases of deep8/src/math/MatrixMultiply.cpp:94-116 (collapsed batch, vector-by-batch, batched with
+broadcast), the reference's own test shapes (test/MatrixMultiplyTest.h), and BASELINE configs."""
+import numpy as np
+import pytest
+
+from util import FP16_TOL, FP32_TOL, f, h, ints, nrm, rel_fro, rng, uni
+
+pytestmark = pytest.mark.gpu
+
+# (x shape, y shape): first axis is the batch
+CASES = [
+    ((10, 400, 200), (1, 200, 300)),   # forwardCPU / GPU1: y.batch == 1 (F1/X1/Y1)
+    ((1, 300, 100), (10, 100)),        # forwardCPU2 / GPU2: x.batch == 1, y is a batch of vectors (F2/X2/Y2)
+    ((6, 40, 30), (6, 30, 50)),        # batched both (F3/X3/Y3)
+    ((1, 40, 30), (6, 30, 50)),        # x broadcast: dX sums over the batch
+    ((6, 40, 30), (6, 30)),            # batched matrix-vector (1-D y, both batched)
+    ((1, 64, 128), (1, 128, 256)),     # BASELINE config 1
+    ((3, 17), (1, 1, 9)),              # 1-D x (column vector) times a row: outer products
+]
+
+
+@pytest.mark.parametrize("xs,ys", CASES)
+def test_matmul_integer_exact(oracle_port, xs, ys):
+    from deep8_amd import ops
+    r = rng(sum(xs) + sum(ys))
+    x, y = ints(r, xs), ints(r, ys)
+    z = ops.matmul(x, y)
+    want = oracle_port.matmul(x, y)
+    assert z.shape == want.shape and np.array_equal(z, want)
+    dz = ints(r, z.shape)
+    dx0, dy0 = ints(r, xs), ints(r, ys)
+    assert np.array_equal(ops.matmul_grad_x(x, y, dz, dx0), oracle_port.matmul_grad_x(x, y, dz, dx0))
+    assert np.array_equal(ops.matmul_grad_y(x, y, dz, dy0), oracle_port.matmul_grad_y(x, y, dz, dy0))
+
+
+@pytest.mark.parametrize("xs,ys", CASES)
+def test_matmul_half_integer_exact(oracle_port, xs, ys):
+    from deep8_amd import ops
+    r = rng(sum(xs) + sum(ys) + 1)
+    x, y = ints(r, xs, 2), ints(r, ys, 2)
+    z = ops.matmul(h(x), h(y))
+    assert z.dtype == np.float16 and np.array_equal(f(z), oracle_port.matmul(x, y))
+    dz = ints(r, z.shape, 2)
+    want_dx, want_dy = oracle_port.matmul_grad_x(x, y, dz), oracle_port.matmul_grad_y(x, y, dz)
+    assert max(want_dx.max(), want_dy.max()) < 2048
+    assert np.array_equal(f(ops.matmul_grad_x(h(x), h(y), h(dz))), want_dx)
+    assert np.array_equal(f(ops.matmul_grad_y(h(x), h(y), h(dz))), want_dy)
+
+
+@pytest.mark.parametrize("xs,ys", CASES)
+def test_matmul_real_tolerance(oracle_port, xs, ys):
+    from deep8_amd import ops
+    r = rng(sum(xs) + sum(ys) + 2)
+    x, y = uni(r, xs), uni(r, ys)
+    want = oracle_port.matmul(x, y)
+    assert rel_fro(ops.matmul(x, y), want) <= FP32_TOL
+    dz = uni(r, want.shape)
+    assert rel_fro(ops.matmul_grad_x(x, y, dz), oracle_port.matmul_grad_x(x, y, dz)) <= FP32_TOL
+    assert rel_fro(ops.matmul_grad_y(x, y, dz), oracle_port.matmul_grad_y(x, y, dz)) <= FP32_TOL
+    xh, yh, dzh = h(x), h(y), h(dz)
+    assert rel_fro(f(ops.matmul(xh, yh)), oracle_port.matmul(f(xh), f(yh))) <= FP16_TOL
+    assert rel_fro(f(ops.matmul_grad_x(xh, yh, dzh)), oracle_port.matmul_grad_x(f(xh), f(yh), f(dzh))) <= FP16_TOL
+    assert rel_fro(f(ops.matmul_grad_y(xh, yh, dzh)), oracle_port.matmul_grad_y(f(xh), f(yh), f(dzh))) <= FP16_TOL
+
+
+def test_grad_accumulates_running_twice_doubles(oracle_port):
+    """Every Grad routine adds into its destination (MatrixMultiply.cpp:147, MatrixMultiply.cu:203)."""
+    from deep8_amd import ops
+    r = rng(3)
+    x, y = ints(r, (4, 20, 10)), ints(r, (1, 10, 30))
+    dz = ints(r, (4, 20, 30))
+    once = ops.matmul_grad_y(x, y, dz)
+    twice = ops.matmul_grad_y(x, y, dz, once)
+    assert np.array_equal(twice, 2 * once)
+    once = ops.matmul_grad_x(x, y, dz)
+    assert np.array_equal(ops.matmul_grad_x(x, y, dz, once), 2 * once)
+
+
+def _against_reference_or_port(oracle_port, name, *args):
+    import oracle
+    src = oracle.ref if oracle.ref is not None else oracle_port
+    return getattr(src, name)(*args)
+
+
+@pytest.mark.parametrize("yb", [32, 1])
+def test_config2_batched_fp32(oracle_port, yb):
+    """BASELINE config 2: batch 32 of 512x512x512 (and the shared-weight broadcast case), uniform(-1,1)."""
+    from deep8_amd import ops
+    r = rng(2024)
+    x, y, dz = uni(r, (32, 512, 512)), uni(r, (yb, 512, 512)), uni(r, (32, 512, 512))
+    assert rel_fro(ops.matmul(x, y), _against_reference_or_port(oracle_port, "matmul", x, y)) <= FP32_TOL
+    assert rel_fro(ops.matmul_grad_x(x, y, dz),
+                   _against_reference_or_port(oracle_port, "matmul_grad_x", x, y, dz)) <= FP32_TOL
+    assert rel_fro(ops.matmul_grad_y(x, y, dz),
+                   _against_reference_or_port(oracle_port, "matmul_grad_y", x, y, dz)) <= FP32_TOL
+
+
+def test_config3_large_half_properties(oracle_port):
+    """BASELINE config 3 (4096^3 half) at full size, checked through size-independent properties:
+    sampled rows/columns against the oracle's GEMM on the half-rounded inputs, and linearity."""
+    from deep8_amd import ops
+    r = rng(4096)
+    n = 4096
+    A, B = h(nrm(r, (1, n, n), 1 / 64.0)), h(nrm(r, (1, n, n), 1 / 64.0))
+    dC = h(nrm(r, (1, n, n), 1.0))
+    C = ops.matmul(A, B)
+    dA = ops.matmul_grad_x(A, B, dC)
+    dB = ops.matmul_grad_y(A, B, dC)
+    rows = r.choice(n, 24, replace=False)
+    Af, Bf, dCf = f(A[0]), f(B[0]), f(dC[0])
+    want = oracle_port.gemm(0, 0, Af[rows], Bf)
+    assert rel_fro(f(C[0][rows]), want) <= FP16_TOL
+    want = oracle_port.gemm(0, 1, dCf[rows], Bf)            # dA = dC B^T
+    assert rel_fro(f(dA[0][rows]), want) <= FP16_TOL
+    want = oracle_port.gemm(1, 0, np.ascontiguousarray(Af[:, rows]), dCf)   # dB = A^T dC, sampled rows of dB
+    assert rel_fro(f(dB[0][rows]), want) <= FP16_TOL
+    # <C, dC> == <A, dA> == <B, dB> (adjoint identity of the three products), in double
+    ip = lambda u, v: float(np.sum(u.astype(np.float64) * v.astype(np.float64)))
+    t = ip(f(C), f(dC))
+    assert abs(ip(f(A), f(dA)) - t) <= 2e-3 * abs(t) + 1.0
+    assert abs(ip(f(B), f(dB)) - t) <= 2e-3 * abs(t) + 1.0
