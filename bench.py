@@ -1,0 +1,333 @@
+#!/usr/bin/env python3
+"""Benchmark of the Deep8 dense-contraction hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--no-cpu] [--no-others]
+
+A step is one forward + both backward passes of the workload over one batch of synthetic input that
+already sits in HBM.  The headline workload is BASELINE config 3 (MatrixMultiply, half,
+4096 x 4096 x 4096); the other configs are timed briefly and reported under "others".
+Prints ONE JSON line.
+
+  value          whole-step throughput: algorithmic FLOPs of fwd + dX + dY / wall time of a step
+                 (gradient destinations are zeroed inside the step, as Deep8's executor does)
+  roofline       the slowest of the step's GEMM launches, timed alone with HIP events on the stream
+                 it runs on, against the dense FP16 MFMA peak
+  cpu_baseline   Deep8's own CPU (Eigen) path from oracle/_ref -- or the C restatement when that was
+                 not built -- on a bounded sample of the same workload, on this host's cores
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"f16": 2500.0, "f32": 157.3}   # dense MFMA TFLOP/s, MI355X
+HBM_PEAK = 8000.0                      # GB/s
+
+
+def _dev(a):
+    from deep8_amd.capi import DeviceArray
+    return DeviceArray.from_numpy(a)
+
+
+def _time_steps(fn, steps, warmup):
+    """wall-clock ms per step over exactly `steps` calls, device idle on both sides"""
+    from deep8_amd import capi
+    for _ in range(warmup):
+        fn()
+    capi.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    capi.sync()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def _time_events(fn, reps):
+    """average ms per call measured with HIP events on the launch stream"""
+    from deep8_amd import capi
+    fn()
+    capi.sync()
+    t = capi.Timer(None)
+    t.start()
+    for _ in range(reps):
+        fn()
+    return t.stop_ms() / reps
+
+
+class MatMulWorkload:
+    """MatrixMultiply forward + GradX + GradY through d8_matmul* (Math::MatrixMultiply*GPU)."""
+
+    def __init__(self, name, dtype, xs, ys, gen, seed):
+        from deep8_amd import capi
+        self.name, self.dtype = name, np.dtype(dtype)
+        self.lib = capi.init()
+        self.dt = capi.dtype_id(self.dtype)
+        r = np.random.default_rng(seed)
+        self.xs, self.ys = xs, ys
+        zb = max(xs[0], ys[0])
+        self.zs = (zb, xs[1], ys[2])
+        self.x, self.y, self.dz = _dev(gen["x"](r, xs).astype(dtype)), _dev(gen["y"](r, ys).astype(dtype)), \
+            _dev(gen["dz"](r, self.zs).astype(dtype))
+        self.z = capi.DeviceArray(self.zs, dtype)
+        self.dx = capi.DeviceArray(xs, dtype)
+        self.dy = capi.DeviceArray(ys, dtype)
+        nb = max(self.lib.d8_matmul_scratch_bytes(self.dt, w, *xs, *ys) for w in range(3))
+        self.ws_bytes = nb
+        self.ws = capi.DeviceArray((max(nb, 16),), np.uint8)
+        m, k, n = xs[1], xs[2], ys[2]
+        self.flops = 3 * 2.0 * zb * m * k * n
+        es = self.dtype.itemsize
+        nx, ny, nz = np.prod(xs), np.prod(ys), np.prod(self.zs)
+        # fwd reads x,y writes z; dX reads dz,y and read-modify-writes dx; dY likewise
+        self.bytes = es * ((nx + ny + nz) + (nz + ny + 2 * nx) + (nx + nz + 2 * ny))
+
+    def fwd(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_matmul(self.dt, self.x.ptr, *self.xs, self.y.ptr, *self.ys, self.z.ptr,
+                                 self.ws.ptr, self.ws_bytes, None))
+
+    def grad_x(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_matmul_grad_x(self.dt, self.dx.ptr, *self.xs, self.y.ptr, *self.ys, self.dz.ptr,
+                                        self.ws.ptr, self.ws_bytes, None))
+
+    def grad_y(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_matmul_grad_y(self.dt, self.x.ptr, *self.xs, self.dy.ptr, *self.ys, self.dz.ptr,
+                                        self.ws.ptr, self.ws_bytes, None))
+
+    def step(self):
+        self.fwd()
+        self.dx.zero_()
+        self.dy.zero_()
+        self.grad_x()
+        self.grad_y()
+
+    def parts(self):
+        f = self.flops / 3
+        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
+
+
+class ConvWorkload:
+    """Conv2d or DeConv2d forward + GradX + GradY through d8_conv2d* / d8_deconv2d*."""
+
+    def __init__(self, name, dtype, deconv, B, IH, IW, IC, OC, FH, FW, covered, sy, sx, seed):
+        from deep8_amd import capi, ops
+        self.name, self.dtype, self.deconv = name, np.dtype(dtype), deconv
+        self.lib = capi.init()
+        self.dt = capi.dtype_id(self.dtype)
+        self.B = B
+        r = np.random.default_rng(seed)
+        if deconv:
+            OH, OW, _, _ = ops.deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx)
+            self.geo = (int(covered), sy, sx)
+        else:
+            OH, OW, _, _ = ops.conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, 1, 1)
+            self.geo = (int(covered), sy, sx, 1, 1)
+        self.xd, self.wd = (B, IH, IW, IC), (OC, FH, FW, IC)
+        self.x = _dev(r.standard_normal((B, IH, IW, IC)).astype(np.float32).astype(dtype))
+        self.w = _dev((r.standard_normal((OC, FH, FW, IC)) * np.sqrt(2.0 / (FH * FW * IC))).astype(np.float32).astype(dtype))
+        self.gz = _dev(r.standard_normal((B, OH, OW, OC)).astype(np.float32).astype(dtype))
+        self.z = capi.DeviceArray((B, OH, OW, OC), dtype)
+        self.gx = capi.DeviceArray((B, IH, IW, IC), dtype)
+        self.gw = capi.DeviceArray((OC, FH, FW, IC), dtype)
+        q = self.lib.d8_deconv2d_scratch_bytes if deconv else self.lib.d8_conv2d_scratch_bytes
+        self.ws_bytes = max(q(self.dt, w, B, IH, IW, IC, OC, FH, FW, *self.geo) for w in range(3))
+        self.ws = capi.DeviceArray((self.ws_bytes,), np.uint8)
+        if deconv:
+            self.flops = 3 * 2.0 * (B * IH * IW) * IC * (OC * FH * FW)
+            mat = B * IH * IW * OC * FH * FW
+        else:
+            self.flops = 3 * 2.0 * (B * OH * OW) * (FH * FW * IC) * OC
+            mat = B * OH * OW * FH * FW * IC
+        es = self.dtype.itemsize
+        nx, nw, nz = B * IH * IW * IC, OC * FH * FW * IC, B * OH * OW * OC
+        self.mat_bytes = mat * es
+        # per pass: gather map (read source, write matrix) + GEMM (read matrix, operand, write result)
+        self.bytes = es * ((nx + mat) + (mat + nw + nz)        # fwd
+                           + (nz + nw + mat) + (mat + 2 * nx)  # grad x
+                           + (nx + mat) + (mat + nz + 2 * nw)) if not deconv else \
+            es * ((nx + nw + mat) + (mat + nz) + (nz + mat) + (mat + nw + 2 * nx) + (nz + mat) + (mat + nx + 2 * nw))
+
+    def _call(self, fn, a, b, c):
+        from deep8_amd.capi import check
+        B, IH, IW, IC = self.xd
+        OC, FH, FW, _ = self.wd
+        check(fn(self.dt, a, B, IH, IW, IC, b, OC, FH, FW, c, *self.geo, self.ws.ptr, self.ws_bytes, None))
+
+    def fwd(self):
+        self._call(self.lib.d8_deconv2d if self.deconv else self.lib.d8_conv2d, self.x.ptr, self.w.ptr, self.z.ptr)
+
+    def grad_x(self):
+        self._call(self.lib.d8_deconv2d_grad_x if self.deconv else self.lib.d8_conv2d_grad_x,
+                   self.gx.ptr, self.w.ptr, self.gz.ptr)
+
+    def grad_y(self):
+        self._call(self.lib.d8_deconv2d_grad_y if self.deconv else self.lib.d8_conv2d_grad_y,
+                   self.x.ptr, self.gw.ptr, self.gz.ptr)
+
+    def step(self):
+        self.fwd()
+        self.gx.zero_()
+        self.gw.zero_()
+        self.grad_x()
+        self.grad_y()
+
+    def parts(self):
+        f = self.flops / 3
+        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
+
+
+def _uni(r, s):
+    return r.uniform(-1, 1, s).astype(np.float32)
+
+
+def make_workload(key):
+    U = {"x": _uni, "y": _uni, "dz": _uni}
+    if key == "c1":
+        return MatMulWorkload("c1: MatrixMultiply fwd+dX+dY fp32 [64x128]x[128x256]", np.float32,
+                              (1, 64, 128), (1, 128, 256), U, 1)
+    if key == "c2a":
+        return MatMulWorkload("c2a: MatrixMultiply fwd+dX+dY fp32 batch 32 of [512x512]x[512x512]", np.float32,
+                              (32, 512, 512), (32, 512, 512), U, 2)
+    if key == "c2b":
+        return MatMulWorkload("c2b: MatrixMultiply fwd+dX+dY fp32 A batch 32 [512x512], B batch 1 (shared)",
+                              np.float32, (32, 512, 512), (1, 512, 512), U, 3)
+    if key == "c3":
+        g = {"x": lambda r, s: (r.standard_normal(s) / 64.0).astype(np.float32),
+             "y": lambda r, s: (r.standard_normal(s) / 64.0).astype(np.float32),
+             "dz": lambda r, s: r.standard_normal(s).astype(np.float32)}
+        return MatMulWorkload("c3: MatrixMultiply fwd+dX+dY half [4096x4096]x[4096x4096]", np.float16,
+                              (1, 4096, 4096), (1, 4096, 4096), g, 4)
+    if key == "c4":
+        return ConvWorkload("c4: Conv2d fwd+dX+dW fp32 B32 56x56x64 3x3x64->64 s1 same", np.float32, False,
+                            32, 56, 56, 64, 64, 3, 3, True, 1, 1, 5)
+    if key == "c5":
+        return ConvWorkload("c5: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 58x58x64 (Deep8 covered=false)",
+                            np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
+    raise SystemExit("unknown workload %r" % key)
+
+
+def cpu_baseline(key):
+    """Deep8's CPU path on a bounded sample of the workload (forward + both gradients)."""
+    import oracle
+    src = oracle.ref if oracle.ref is not None else oracle.port
+    kind = "reference" if oracle.ref is not None else "port"
+    r = np.random.default_rng(9)
+    if key in ("c4", "c5"):
+        # the reference runs Conv2d/DeConv2d on Eigen's thread pool: all host cores
+        B = 2
+        if key == "c4":
+            x, w = r.standard_normal((B, 56, 56, 64)).astype(np.float32), r.standard_normal((64, 3, 3, 64)).astype(np.float32)
+            args, f3 = (True, 1, 1, 1, 1), (src.conv2d, src.conv2d_grad_x, src.conv2d_grad_y)
+            flops = 3 * 2.0 * B * 56 * 56 * 576 * 64
+        else:
+            x, w = r.standard_normal((B, 28, 28, 128)).astype(np.float32), r.standard_normal((64, 4, 4, 128)).astype(np.float32)
+            args, f3 = (False, 2, 2), (src.deconv2d, src.deconv2d_grad_x, src.deconv2d_grad_y)
+            flops = 3 * 2.0 * B * 28 * 28 * 128 * 1024
+        z = f3[0](x, w, *args)
+        gz = r.standard_normal(z.shape).astype(np.float32)
+        t0 = time.perf_counter()
+        f3[0](x, w, *args)
+        f3[1](x, w, gz, *args)
+        f3[2](x, w, gz, *args)
+        dt = time.perf_counter() - t0
+        return {"value": B / dt, "unit": "images/s", "cores": src.threads(), "kind": kind,
+                "sample": "%s fwd+dX+dW on %d images (fp32 CPU path), %.2f s" % (key, B, dt),
+                "tflops": flops / dt / 1e12}
+    # MatrixMultiply: Eigen's dense product is single-threaded in the reference build
+    if key == "c3":
+        m, k, n, b = 256, 4096, 4096, 1
+    elif key in ("c2a", "c2b"):
+        m, k, n, b = 512, 512, 512, 8
+    else:
+        m, k, n, b = 64, 128, 256, 1
+    x, y = r.uniform(-1, 1, (b, m, k)).astype(np.float32), r.uniform(-1, 1, (1 if key != "c2a" else b, k, n)).astype(np.float32)
+    dz = r.uniform(-1, 1, (b, m, n)).astype(np.float32)
+    src.matmul(x[:, :8], y)  # warm the library
+    t0 = time.perf_counter()
+    src.matmul(x, y)
+    src.matmul_grad_x(x, y, dz)
+    src.matmul_grad_y(x, y, dz)
+    dt = time.perf_counter() - t0
+    flops = 3 * 2.0 * b * m * k * n
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1 if kind == "reference" else src.threads(),
+            "kind": kind,
+            "sample": "fwd+dX+dY of %d x [%dx%d]x[%dx%d] fp32 (the reference has no CPU half), %.2f s" % (b, m, k, k, n, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-others", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
+                         "no second device anywhere in the path)" % a.gpus)
+
+    from deep8_amd import capi
+    capi.init()
+
+    wl = make_workload(a.workload)
+    ms = _time_steps(wl.step, a.steps, a.warmup)
+    dtype = "f16" if wl.dtype == np.float16 else "f32"
+    is_conv = isinstance(wl, ConvWorkload)
+    tflops = wl.flops / (ms * 1e-3) / 1e12
+
+    parts = {}
+    for pname, (fn, fl) in wl.parts().items():
+        pms = _time_events(fn, max(5, a.steps))
+        parts[pname] = {"ms": round(pms, 4), "tflops": round(fl / (pms * 1e-3) / 1e12, 2)}
+    slow = max(parts, key=lambda p: parts[p]["ms"])
+    roof = {"bound": "mfma", "kernel": "%s GEMM launch (%s)" % (a.workload, slow),
+            "achieved": parts[slow]["tflops"], "peak": PEAK[dtype], "unit": "TFLOP/s",
+            "frac": round(parts[slow]["tflops"] / PEAK[dtype], 4), "traffic": None}
+    if is_conv:
+        roof = {"bound": "hbm", "kernel": "%s whole step (gather maps + GEMMs)" % a.workload,
+                "achieved": round(wl.bytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK, "unit": "GB/s",
+                "frac": round(wl.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK, 4), "traffic": None}
+
+    out = {
+        "metric": "Conv2d fwd+bwd images/s" if is_conv else "MatrixMultiply fwd+bwd TFLOP/s",
+        "value": round(wl.B / (ms * 1e-3), 1) if is_conv else round(tflops, 2),
+        "unit": "images/s" if is_conv else "TFLOP/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic (seeded numpy generators, resident in HBM before timing)",
+        "config": {"workload": wl.name},
+        "pct_mfma_peak": round(100.0 * tflops / PEAK[dtype], 2),
+        "tflops": round(tflops, 2),
+        "parts": parts,
+        "roofline": roof,
+    }
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(a.workload)
+    if not a.no_others:
+        others = {}
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5"):
+            if key == a.workload:
+                continue
+            del wl
+            wl = make_workload(key)
+            oms = _time_steps(wl.step, 5, 2)
+            o = {"ms_per_step": round(oms, 4), "tflops": round(wl.flops / (oms * 1e-3) / 1e12, 2),
+                 "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
+            if isinstance(wl, ConvWorkload):
+                o["images_per_s"] = round(wl.B / (oms * 1e-3), 1)
+            others[key] = o
+        out["others"] = others
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

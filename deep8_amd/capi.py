@@ -29,6 +29,7 @@ SIGNATURES = {
     "d8_host_malloc": (_I, [_PP, _Z]),
     "d8_host_free": (_I, [_P]),
     "d8_memset": (_I, [_P, _I, _Z, _P]),
+    "d8_fill": (_I, [_I, _P, _Z, _F, _P]),
     "d8_memcpy_h2d": (_I, [_P, _P, _Z]),
     "d8_memcpy_d2h": (_I, [_P, _P, _Z]),
     "d8_memcpy_d2d": (_I, [_P, _P, _Z, _P]),

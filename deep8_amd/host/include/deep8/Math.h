@@ -1,0 +1,60 @@
+// Math:: dispatchers and their GPU implementations for the dense-contraction path, with the
+// reference's signatures:
+//   MatrixMultiply   deep8/include/math/MatrixMultiply.h:12-36, checks deep8/src/math/MatrixMultiply.cpp:7-91
+//   Conv2d           deep8/include/math/Conv2d.h:17-47,         checks deep8/src/math/Conv2d.cpp:6-290
+//   DeConv2d         deep8/include/math/DeConv2d.h:11-40,       checks deep8/src/math/DeConv2d.cpp:6-243
+//   Constant         deep8/include/math/Constant.h (zeroGradient / oneGradient)
+// Forward routines overwrite their output; every Grad routine adds into its destination.
+// The *GPU functions call libdeep8_hip.so through its C ABI (include/deep8_hip.h).  Tensors on
+// DeviceType::CPU are refused with std::runtime_error: there is no CPU path in this build.
+#ifndef DEEP8_HOST_MATH_H
+#define DEEP8_HOST_MATH_H
+
+#include "deep8/Model.h"
+
+namespace Deep8 {
+namespace Math {
+
+void Constant(Tensor &x, float scalar);
+void ConstantGPU(Tensor &x, float scalar);
+
+/** z = x * y */
+void MatrixMultiply(const Tensor &x, const Tensor &y, Tensor &z);
+void MatrixMultiplyGPU(const Tensor &x, const Tensor &y, Tensor &z);
+/** dx += dz * y^T */
+void MatrixMultiplyGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz);
+void MatrixMultiplyGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz);
+/** dy += x^T * dz */
+void MatrixMultiplyGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+void MatrixMultiplyGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+
+/** x [B,IH,IW,IC], y [OC,FH,FW,IC] (batch 1), z [B,OH,OW,OC]; the *InterimSize functions give
+ *  the bytes of device scratch the caller must pass as the last argument. */
+size_t Conv2dInterimSize(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, int dilationY, int dilationX);
+void Conv2d(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *interimPtr);
+void Conv2dGPU(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *xcol);
+
+size_t Conv2dGradXInterimSize(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX);
+void Conv2dGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *interimPtr);
+void Conv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *dxcol);
+
+size_t Conv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX);
+void Conv2dGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *interimPtr);
+void Conv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *xcol);
+
+size_t DeConv2dInterimSize(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX);
+void DeConv2d(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, void *interimPtr);
+void DeConv2dGPU(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, void *interimPtr);
+
+size_t DeConv2dGradXInterimSize(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX);
+void DeConv2dGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
+void DeConv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
+
+size_t DeConv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX);
+void DeConv2dGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
+void DeConv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
+
+}  // namespace Math
+}  // namespace Deep8
+
+#endif

@@ -1,0 +1,154 @@
+// Graph nodes: Node, Variable, Function and the three Function subclasses on the dense-contraction
+// path.  Same public surface as the reference:
+//   Node / OutputEntry   deep8/include/nodes/Node.h:29-80, deep8/include/model/OutputEntry.h:10-30
+//   Variable             deep8/include/nodes/Variable.h:9-53 (+ feed/fetch and the three op builders)
+//   Function             deep8/include/nodes/Function.h:46-65, deep8/src/nodes/Function.cpp:41-102
+//   MatrixMultiply       deep8/src/nodes/MatrixMultiply.cpp:6-52
+//   Conv2d               deep8/src/nodes/Conv2d.cpp:6-152
+//   DeConv2d             deep8/src/nodes/DeConv2d.cpp:6-126
+#ifndef DEEP8_HOST_NODES_H
+#define DEEP8_HOST_NODES_H
+
+#include <unordered_map>
+
+#include "deep8/Model.h"
+
+namespace Deep8 {
+
+class Executor;
+class Node;
+
+enum class NodeType { Unknow = 0, Variable, Function };
+
+class OutputEntry {
+public:
+    std::unordered_map<Node *, size_t> entries;  // consumer -> which of its inputs this node is
+    void add(Node *node, size_t i);
+    void remove(Node *node);
+    void clear();
+    size_t size();
+    Node *first();
+};
+
+class Node {
+public:
+    NodeType type;
+    int64_t id;
+    std::string name;
+    Executor *executor;  // may be nullptr (nodes built by hand, as the tests do)
+    std::vector<Node *> inputs;
+    OutputEntry outputs;
+
+protected:
+    Node();
+    explicit Node(Node *input);
+    explicit Node(std::vector<Node *> &inputs);
+    Node(int64_t id, std::string name, Executor *exe);
+    Node(int64_t id, std::string name, Executor *exe, Node *input);
+    Node(int64_t id, std::string name, Executor *exe, std::vector<Node *> &inputs);
+
+public:
+    virtual ~Node();
+    virtual void forward();
+    virtual void backward();
+    virtual std::string toString();
+};
+
+class Variable : public Node {
+public:
+    Tensor value;
+    Tensor gradient;
+    bool updateGradient;
+
+protected:
+    Variable(int64_t id, std::string name, Executor *exe);
+
+public:
+    Variable(int64_t id, std::string name, Executor *exe, Tensor &v);
+    Variable(int64_t id, std::string name, Executor *exe, Tensor &v, Tensor &g);
+    Variable(int64_t id, std::string name, Executor *exe, Node *input);
+    Variable(int64_t id, std::string name, Executor *exe, Node *input, Tensor &v);
+    Variable(int64_t id, std::string name, Executor *exe, Node *input, Tensor &v, Tensor &g);
+
+    Shape shape();
+    ElementType elementType();
+    DeviceType deviceType();
+    bool isScalar();
+    void zeroGradient();
+    void oneGradient();
+    void removeGradient();
+    void forward() override;   // nothing to do
+    void backward() override;  // nothing to do
+    std::string valueStr();
+
+    Variable &feed(const void *hostPtr);  // host -> value
+    Variable &fetch(void *hostPtr);       // value -> host (blocking)
+    Variable &constant(float scalar = 0);
+    Variable &zero();
+    Variable &one();
+
+    // graph builders of the dense-contraction path (need an executor)
+    Variable &matrixMultiply(Variable &y);
+    Variable &conv2d(Variable &filter, bool covered = true, int strideY = 1, int strideX = 1, int dilationY = 1, int dilationX = 1);
+    Variable &deConv2d(Variable &filter, bool covered = false, int strideY = 1, int strideX = 1);
+};
+
+enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply };
+
+class Function : public Node {
+protected:
+    explicit Function(std::vector<Node *> &inputs);
+
+public:
+    virtual bool isShared();
+    virtual Shape checkShape(std::vector<Shape> &inputShapes);
+    virtual ElementType checkElementType(std::vector<ElementType> &inputTypes);
+
+    virtual void forward(const std::vector<const Tensor *> &inputs, Tensor *output);
+    virtual void backward(const std::vector<const Tensor *> &inputs, const Tensor *output,
+                          const Tensor *outputGradient, size_t index, Tensor *iGradient);
+
+    void forward() override;   // gathers the input Variables' values, writes the output Variable
+    void backward() override;  // one backward(..., i, ...) per input that wants a gradient
+};
+
+class MatrixMultiply : public Function {
+public:
+    explicit MatrixMultiply(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+class Conv2d : public Function {
+public:
+    bool covered;
+    int strideY, strideX, dilationY, dilationX;
+
+    explicit Conv2d(std::vector<Node *> &inputs, bool covered = true, int strideY = 1, int strideX = 1,
+                    int dilationY = 1, int dilationX = 1);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+class DeConv2d : public Function {
+public:
+    bool forwardCovered;
+    int forwardStrideY, forwardStrideX;
+
+    explicit DeConv2d(std::vector<Node *> &inputs, bool covered = false, int strideY = 1, int strideX = 1);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+}  // namespace Deep8
+
+#endif

@@ -1,0 +1,307 @@
+// Math:: dispatchers (argument checks as in the reference) and their GPU bodies, which hand the
+// raw pointers and sizes to libdeep8_hip.so.  See deep8/Math.h for the reference line numbers.
+#include "deep8/Math.h"
+
+#include "deep8_hip.h"
+
+namespace Deep8 {
+namespace Math {
+
+namespace {
+
+int dtypeOf(const Tensor &t) {
+    switch (t.elementType.id) {
+    case DType::Float32: return D8_FLOAT32;
+    case DType::Float16: return D8_FLOAT16;
+    default: DEEP8_RUNTIME_ERROR("type " << t.elementType.name << " is not support");
+    }
+}
+
+void requireGPU(const Tensor &t) {
+    if (DeviceType::GPU != t.deviceType())
+        DEEP8_RUNTIME_ERROR("this build carries the GPU path only: CPU tensors are not supported");
+}
+
+// Device scratch taken from the tensor's pool for the duration of one call.  Freed as soon as
+// the launches are queued: the pool never returns memory to the driver while it lives and all
+// work runs on the one default stream, the same rule Deep8's nodes rely on for their interim
+// buffers (deep8/src/nodes/Conv2d.cpp:77-82).
+struct PoolScratch {
+    Device *device;
+    void *ptr;
+    size_t bytes;
+    PoolScratch(Device *d, size_t n) : device(d), ptr(n ? d->malloc(n) : nullptr), bytes(n) {}
+    ~PoolScratch() {
+        if (ptr) device->free(ptr);
+    }
+};
+
+struct MM {
+    int xb, xr, xc, yb, yr, yc;
+};
+
+MM mmDims(const Tensor &x, const Tensor &y) {
+    return MM{(int)x.batch(), (int)x.row(), (int)x.col(), (int)y.batch(), (int)y.row(), (int)y.col()};
+}
+
+void checkMatrixMultiplyShapes(const Tensor &x, const Tensor &y, const Tensor &z) {
+    const Shape &xs = x.shape, &ys = y.shape, &zs = z.shape;
+    DEEP8_ARGUMENT_CHECK(1 == xs.batch || xs.batch == zs.batch, "the shape is error");
+    DEEP8_ARGUMENT_CHECK(1 == ys.batch || ys.batch == zs.batch, "the shape is error");
+    DEEP8_ARGUMENT_CHECK((1 == xs.nDims || 2 == xs.nDims) && (1 == ys.nDims || 2 == ys.nDims) &&
+                             (1 == zs.nDims || 2 == zs.nDims),
+                         "the shape is error");
+    DEEP8_ARGUMENT_CHECK(xs.row() == zs.row() && ys.col() == zs.col() && xs.col() == ys.row(), "the shape is error");
+}
+
+struct ConvDims {
+    int B, IH, IW, IC, OC, FH, FW, OH, OW;
+};
+
+ConvDims convDims(const Tensor &x, const Tensor &y, const Tensor &z) {
+    return ConvDims{(int)x.batch(), (int)x.dim(0), (int)x.dim(1), (int)x.dim(2), (int)y.dim(0),
+                    (int)y.dim(1),  (int)y.dim(2), (int)z.dim(0), (int)z.dim(1)};
+}
+
+// shared by Conv2d / GradX / GradY and their InterimSize twins (deep8/src/math/Conv2d.cpp:6-38)
+ConvDims checkConv(const Tensor &x, const Tensor &y, const Tensor &z, bool covered, int strideY, int strideX,
+                   int dilationY, int dilationX) {
+    DEEP8_ARGUMENT_CHECK(strideY >= 1 && strideX >= 1 && dilationY >= 1 && dilationX >= 1,
+                         "the stride and dilation must >= 1");
+    DEEP8_ARGUMENT_CHECK(3 == x.nDims() && 4 == y.nDims() && 3 == z.nDims(), "the shape is error");
+    ConvDims d = convDims(x, y, z);
+    int g[4];
+    const int rc = d8_conv2d_geometry(d.IH, d.IW, d.FH, d.FW, covered, strideY, strideX, dilationY, dilationX, g);
+    DEEP8_ARGUMENT_CHECK(0 == rc, "the shape is error: " << d8_last_error());
+    DEEP8_ARGUMENT_CHECK(d.B == (int)z.batch() && g[0] == d.OH && g[1] == d.OW && d.OC == (int)z.dim(2),
+                         "the z shape is error");
+    DEEP8_ARGUMENT_CHECK(1 == y.batch() && d.IC == (int)y.dim(3), "the filter shape is error");
+    return d;
+}
+
+// deep8/src/math/DeConv2d.cpp:6-35
+ConvDims checkDeConv(const Tensor &x, const Tensor &y, const Tensor &z, bool covered, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(strideY >= 1 && strideX >= 1, "the stride must >= 1");
+    DEEP8_ARGUMENT_CHECK(3 == x.nDims() && 4 == y.nDims() && 3 == z.nDims(), "the shape is error");
+    ConvDims d = convDims(x, y, z);
+    int g[4];
+    const int rc = d8_deconv2d_geometry(d.IH, d.IW, d.FH, d.FW, covered, strideY, strideX, g);
+    DEEP8_ARGUMENT_CHECK(0 == rc, "the shape is error: " << d8_last_error());
+    DEEP8_ARGUMENT_CHECK(d.B == (int)z.batch() && g[0] == d.OH && g[1] == d.OW && d.OC == (int)z.dim(2),
+                         "the z shape is error");
+    DEEP8_ARGUMENT_CHECK(1 == y.batch() && d.IC == (int)y.dim(3), "the filter shape is error");
+    return d;
+}
+
+}  // namespace
+
+// ---- Constant ---------------------------------------------------------------------------------------------
+void Constant(Tensor &x, float scalar) {
+    requireGPU(x);
+    ConstantGPU(x, scalar);
+}
+
+void ConstantGPU(Tensor &x, float scalar) { D8_CHECK(d8_fill(dtypeOf(x), x.raw(), x.size(), scalar, nullptr)); }
+
+// ---- MatrixMultiply -------------------------------------------------------------------------------------------
+void MatrixMultiply(const Tensor &x, const Tensor &y, Tensor &z) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType() && x.deviceType() == z.deviceType(), "the device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the data type must be same");
+    checkMatrixMultiplyShapes(x, y, z);
+    requireGPU(x);
+    MatrixMultiplyGPU(x, y, z);
+}
+
+void MatrixMultiplyGPU(const Tensor &x, const Tensor &y, Tensor &z) {
+    const MM d = mmDims(x, y);
+    const int dt = dtypeOf(x);
+    PoolScratch ws(x.device(), d8_matmul_scratch_bytes(dt, 0, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
+    D8_CHECK(d8_matmul(dt, x.raw(), d.xb, d.xr, d.xc, y.raw(), d.yb, d.yr, d.yc, z.raw(), ws.ptr, ws.bytes, nullptr));
+}
+
+void MatrixMultiplyGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == dx.deviceType() && x.deviceType() == y.deviceType() &&
+                             x.deviceType() == z.deviceType() && x.deviceType() == dz.deviceType(),
+                         "the device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && z.shape == dz.shape, "the shape is error");
+    checkMatrixMultiplyShapes(x, y, z);
+    requireGPU(x);
+    MatrixMultiplyGradXGPU(x, dx, y, z, dz);
+}
+
+void MatrixMultiplyGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &, const Tensor &dz) {
+    const MM d = mmDims(x, y);
+    const int dt = dtypeOf(x);
+    PoolScratch ws(x.device(), d8_matmul_scratch_bytes(dt, 1, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
+    D8_CHECK(d8_matmul_grad_x(dt, dx.raw(), d.xb, d.xr, d.xc, y.raw(), d.yb, d.yr, d.yc, dz.raw(), ws.ptr, ws.bytes, nullptr));
+}
+
+void MatrixMultiplyGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType() && x.deviceType() == dy.deviceType() &&
+                             x.deviceType() == z.deviceType() && x.deviceType() == dz.deviceType(),
+                         "the device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == dy.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    checkMatrixMultiplyShapes(x, y, z);
+    requireGPU(x);
+    MatrixMultiplyGradYGPU(x, y, dy, z, dz);
+}
+
+void MatrixMultiplyGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &, const Tensor &dz) {
+    const MM d = mmDims(x, y);
+    const int dt = dtypeOf(x);
+    PoolScratch ws(x.device(), d8_matmul_scratch_bytes(dt, 2, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
+    D8_CHECK(d8_matmul_grad_y(dt, x.raw(), d.xb, d.xr, d.xc, dy.raw(), d.yb, d.yr, d.yc, dz.raw(), ws.ptr, ws.bytes, nullptr));
+}
+
+// ---- Conv2d -------------------------------------------------------------------------------------------------------
+#define CONV_ARGS covered, strideY, strideX, dilationY, dilationX
+
+size_t Conv2dInterimSize(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the data type must be same");
+    const ConvDims d = checkConv(x, y, z, CONV_ARGS);
+    requireGPU(x);
+    return d8_conv2d_scratch_bytes(dtypeOf(x), 0, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
+}
+
+void Conv2d(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *interimPtr) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the data type must be same");
+    checkConv(x, y, z, CONV_ARGS);
+    requireGPU(x);
+    Conv2dGPU(x, y, z, CONV_ARGS, interimPtr);
+}
+
+void Conv2dGPU(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *xcol) {
+    const ConvDims d = convDims(x, y, z);
+    const int dt = dtypeOf(x);
+    const size_t bytes = d8_conv2d_scratch_bytes(dt, 0, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
+    D8_CHECK(d8_conv2d(dt, x.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, z.raw(), CONV_ARGS, xcol, bytes, nullptr));
+}
+
+size_t Conv2dGradXInterimSize(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && z.shape == dz.shape, "the shape is error");
+    const ConvDims d = checkConv(x, y, z, CONV_ARGS);
+    requireGPU(x);
+    return d8_conv2d_scratch_bytes(dtypeOf(x), 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
+}
+
+void Conv2dGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *interimPtr) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && z.shape == dz.shape, "the shape is error");
+    checkConv(x, y, z, CONV_ARGS);
+    requireGPU(x);
+    Conv2dGradXGPU(x, dx, y, z, dz, CONV_ARGS, interimPtr);
+}
+
+void Conv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *dxcol) {
+    const ConvDims d = convDims(x, y, z);
+    const int dt = dtypeOf(x);
+    const size_t bytes = d8_conv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
+    D8_CHECK(d8_conv2d_grad_x(dt, dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS, dxcol, bytes, nullptr));
+}
+
+size_t Conv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == dy.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    const ConvDims d = checkConv(x, y, z, CONV_ARGS);
+    requireGPU(x);
+    return d8_conv2d_scratch_bytes(dtypeOf(x), 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
+}
+
+void Conv2dGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *interimPtr) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == dy.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    checkConv(x, y, z, CONV_ARGS);
+    requireGPU(x);
+    Conv2dGradYGPU(x, y, dy, z, dz, CONV_ARGS, interimPtr);
+}
+
+void Conv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *xcol) {
+    const ConvDims d = convDims(x, y, z);
+    const int dt = dtypeOf(x);
+    const size_t bytes = d8_conv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
+    D8_CHECK(d8_conv2d_grad_y(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS, xcol, bytes, nullptr));
+}
+
+#undef CONV_ARGS
+
+// ---- DeConv2d -------------------------------------------------------------------------------------------------------
+#define DECONV_ARGS covered, strideY, strideX
+
+size_t DeConv2dInterimSize(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the data type must be same");
+    const ConvDims d = checkDeConv(x, y, z, DECONV_ARGS);
+    requireGPU(x);
+    return d8_deconv2d_scratch_bytes(dtypeOf(x), 0, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
+}
+
+void DeConv2d(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, void *interimPtr) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the data type must be same");
+    checkDeConv(x, y, z, DECONV_ARGS);
+    requireGPU(x);
+    DeConv2dGPU(x, y, z, DECONV_ARGS, interimPtr);
+}
+
+void DeConv2dGPU(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, void *interimPtr) {
+    const ConvDims d = convDims(x, y, z);
+    const int dt = dtypeOf(x);
+    const size_t bytes = d8_deconv2d_scratch_bytes(dt, 0, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
+    D8_CHECK(d8_deconv2d(dt, x.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, z.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
+}
+
+size_t DeConv2dGradXInterimSize(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && z.shape == dz.shape, "the shape is error");
+    const ConvDims d = checkDeConv(x, y, z, DECONV_ARGS);
+    requireGPU(x);
+    return d8_deconv2d_scratch_bytes(dtypeOf(x), 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
+}
+
+void DeConv2dGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && z.shape == dz.shape, "the shape is error");
+    checkDeConv(x, y, z, DECONV_ARGS);
+    requireGPU(x);
+    DeConv2dGradXGPU(x, dx, y, z, dz, DECONV_ARGS, interimPtr);
+}
+
+void DeConv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr) {
+    const ConvDims d = convDims(x, y, z);
+    const int dt = dtypeOf(x);
+    const size_t bytes = d8_deconv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
+    D8_CHECK(d8_deconv2d_grad_x(dt, dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
+}
+
+size_t DeConv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == dy.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    const ConvDims d = checkDeConv(x, y, z, DECONV_ARGS);
+    requireGPU(x);
+    return d8_deconv2d_scratch_bytes(dtypeOf(x), 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
+}
+
+void DeConv2dGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == dy.elementType && x.elementType == z.elementType && x.elementType == dz.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    checkDeConv(x, y, z, DECONV_ARGS);
+    requireGPU(x);
+    DeConv2dGradYGPU(x, y, dy, z, dz, DECONV_ARGS, interimPtr);
+}
+
+void DeConv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr) {
+    const ConvDims d = convDims(x, y, z);
+    const int dt = dtypeOf(x);
+    const size_t bytes = d8_deconv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
+    D8_CHECK(d8_deconv2d_grad_y(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
+}
+
+#undef DECONV_ARGS
+
+}  // namespace Math
+}  // namespace Deep8

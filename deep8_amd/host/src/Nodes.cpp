@@ -1,0 +1,367 @@
+// Node, Variable, Function and the MatrixMultiply / Conv2d / DeConv2d functions (see deep8/Nodes.h).
+#include "deep8/Nodes.h"
+
+#include <algorithm>
+
+#include "deep8/Executor.h"
+#include "deep8/Math.h"
+
+namespace Deep8 {
+
+// ---- OutputEntry ---------------------------------------------------------------------------------------
+void OutputEntry::add(Node *node, size_t i) {
+    DEEP8_ARGUMENT_CHECK(nullptr != node, "the node can not be nullptr");
+    entries[node] = i;
+}
+void OutputEntry::remove(Node *node) { entries.erase(node); }
+void OutputEntry::clear() { entries.clear(); }
+size_t OutputEntry::size() { return entries.size(); }
+Node *OutputEntry::first() {
+    DEEP8_ARGUMENT_CHECK(!entries.empty(), "the outputs is empty");
+    return entries.begin()->first;
+}
+
+// ---- Node ---------------------------------------------------------------------------------------------------
+Node::Node() : type(NodeType::Unknow), id(-1), executor(nullptr) {}
+
+Node::Node(Node *input) : Node() {
+    inputs.push_back(input);
+    input->outputs.add(this, 0);
+}
+
+Node::Node(std::vector<Node *> &in) : Node() {
+    inputs = in;
+    for (size_t i = 0; i < inputs.size(); ++i) inputs[i]->outputs.add(this, i);
+}
+
+Node::Node(int64_t i, std::string n, Executor *exe) : type(NodeType::Unknow), id(i), name(std::move(n)), executor(exe) {}
+
+Node::Node(int64_t i, std::string n, Executor *exe, Node *input) : Node(i, std::move(n), exe) {
+    inputs.push_back(input);
+    input->outputs.add(this, 0);
+}
+
+Node::Node(int64_t i, std::string n, Executor *exe, std::vector<Node *> &in) : Node(i, std::move(n), exe) {
+    inputs = in;
+    for (size_t k = 0; k < inputs.size(); ++k) inputs[k]->outputs.add(this, k);
+}
+
+Node::~Node() {}
+void Node::forward() { DEEP8_RUNTIME_ERROR("Can not call this function from Node"); }
+void Node::backward() { DEEP8_RUNTIME_ERROR("Can not call this function from Node"); }
+std::string Node::toString() { return "Node: the Base class of Function and Variable"; }
+
+// ---- Variable --------------------------------------------------------------------------------------------------
+static void checkPair(const Tensor &value, const Tensor &gradient) {
+    DEEP8_ARGUMENT_CHECK(value.deviceType() == gradient.deviceType(), "the values and gradient must be the same type");
+    DEEP8_ARGUMENT_CHECK(value.elementType == gradient.elementType, "the values and gradient data type must be the same");
+    DEEP8_ARGUMENT_CHECK(value.shape == gradient.shape, "the shape of Value and Gradient must be same");
+}
+
+Variable::Variable(int64_t id, std::string name, Executor *exe) : Node(id, std::move(name), exe), updateGradient(false) {
+    type = NodeType::Variable;
+}
+
+Variable::Variable(int64_t id, std::string name, Executor *exe, Tensor &v)
+    : Node(id, std::move(name), exe), value(v), updateGradient(false) {
+    type = NodeType::Variable;
+}
+
+Variable::Variable(int64_t id, std::string name, Executor *exe, Tensor &v, Tensor &g)
+    : Node(id, std::move(name), exe), value(v), gradient(g), updateGradient(true) {
+    checkPair(value, gradient);
+    type = NodeType::Variable;
+}
+
+Variable::Variable(int64_t id, std::string name, Executor *exe, Node *input)
+    : Node(id, std::move(name), exe, input), updateGradient(false) {
+    type = NodeType::Variable;
+}
+
+Variable::Variable(int64_t id, std::string name, Executor *exe, Node *input, Tensor &v)
+    : Node(id, std::move(name), exe, input), value(v), updateGradient(false) {
+    type = NodeType::Variable;
+}
+
+Variable::Variable(int64_t id, std::string name, Executor *exe, Node *input, Tensor &v, Tensor &g)
+    : Node(id, std::move(name), exe, input), value(v), gradient(g), updateGradient(true) {
+    checkPair(value, gradient);
+    type = NodeType::Variable;
+}
+
+Shape Variable::shape() {
+    if (updateGradient) DEEP8_ARGUMENT_CHECK(value.shape == gradient.shape, "the value and gradient shape must be same");
+    return value.shape;
+}
+
+ElementType Variable::elementType() {
+    if (updateGradient)
+        DEEP8_ARGUMENT_CHECK(value.elementType == gradient.elementType, "the value and gradient elementType must be same");
+    return value.elementType;
+}
+
+DeviceType Variable::deviceType() {
+    if (updateGradient)
+        DEEP8_ARGUMENT_CHECK(value.deviceType() == gradient.deviceType(), "the value and gradient deviceType must be same");
+    return value.deviceType();
+}
+
+bool Variable::isScalar() { return updateGradient ? value.isScalar() && gradient.isScalar() : value.isScalar(); }
+
+void Variable::zeroGradient() {
+    DEEP8_ARGUMENT_CHECK(updateGradient, "this variable does not have gradient");
+    Math::Constant(gradient, 0);
+}
+
+void Variable::oneGradient() {
+    DEEP8_ARGUMENT_CHECK(updateGradient, "this variable does not have gradient");
+    Math::Constant(gradient, 1);
+}
+
+void Variable::removeGradient() {
+    if (updateGradient) {
+        gradient = Tensor();
+        updateGradient = false;
+    }
+}
+
+void Variable::forward() {}
+void Variable::backward() {}
+std::string Variable::valueStr() { return value.valueStr(); }
+
+Variable &Variable::feed(const void *ptr) {
+    DEEP8_ARGUMENT_CHECK(nullptr != ptr, "the pointer can not be null");
+    value.device()->copyFromCPUToGPU(ptr, value.raw(), value.byteCount());
+    return *this;
+}
+
+Variable &Variable::fetch(void *ptr) {
+    DEEP8_ARGUMENT_CHECK(nullptr != ptr, "the pointer can not be null");
+    value.device()->copyFromGPUToCPU(value.raw(), ptr, value.byteCount());
+    return *this;
+}
+
+Variable &Variable::constant(float scalar) {
+    Math::Constant(value, scalar);
+    return *this;
+}
+Variable &Variable::zero() { return constant(0); }
+Variable &Variable::one() { return constant(1); }
+
+Variable &Variable::matrixMultiply(Variable &y) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this, &y};
+    return *executor->addFunction(new MatrixMultiply(in));
+}
+
+Variable &Variable::conv2d(Variable &filter, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this, &filter};
+    return *executor->addFunction(new Conv2d(in, covered, strideY, strideX, dilationY, dilationX));
+}
+
+Variable &Variable::deConv2d(Variable &filter, bool covered, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this, &filter};
+    return *executor->addFunction(new DeConv2d(in, covered, strideY, strideX));
+}
+
+// ---- Function -----------------------------------------------------------------------------------------------------
+Function::Function(std::vector<Node *> &in) : Node(in) { type = NodeType::Function; }
+
+bool Function::isShared() { return false; }
+Shape Function::checkShape(std::vector<Shape> &) { return Shape(); }
+
+ElementType Function::checkElementType(std::vector<ElementType> &inputTypes) {
+    if (inputTypes.empty()) return ElementType::unknown();
+    for (size_t i = 1; i < inputTypes.size(); ++i)
+        DEEP8_ARGUMENT_CHECK(inputTypes[0] == inputTypes[i], "the input's ElementType must be same");
+    return inputTypes[0];
+}
+
+void Function::forward(const std::vector<const Tensor *> &, Tensor *) {
+    DEEP8_RUNTIME_ERROR("can not call this forward by Function class");
+}
+
+void Function::backward(const std::vector<const Tensor *> &, const Tensor *, const Tensor *, size_t, Tensor *) {
+    DEEP8_RUNTIME_ERROR("can not call this backward by Function class");
+}
+
+// Collect the input Variables' value tensors, all on the output's device.
+static std::vector<const Tensor *> gatherInputs(Function *f, Variable *&outputVar) {
+    for (Node *n : f->inputs) DEEP8_ARGUMENT_CHECK(NodeType::Variable == n->type, "the inputs must be a Variable type");
+    DEEP8_ARGUMENT_CHECK(1 == f->outputs.size(), "the output size must be 1");
+    DEEP8_ARGUMENT_CHECK(NodeType::Variable == f->outputs.first()->type, "the output must be a Variable type");
+    outputVar = (Variable *)f->outputs.first();
+    const DeviceType dev = outputVar->deviceType();
+    std::vector<const Tensor *> values;
+    for (Node *n : f->inputs) {
+        Variable *v = (Variable *)n;
+        DEEP8_ARGUMENT_CHECK(dev == v->deviceType(), "the device of input must be same with output");
+        values.push_back(&v->value);
+    }
+    return values;
+}
+
+void Function::forward() {
+    Variable *out = nullptr;
+    std::vector<const Tensor *> values = gatherInputs(this, out);
+    this->forward(values, &out->value);
+}
+
+void Function::backward() {
+    Variable *out = nullptr;
+    std::vector<const Tensor *> values = gatherInputs(this, out);
+    for (size_t i = 0; i < inputs.size(); ++i) {
+        Variable *in = (Variable *)inputs[i];
+        if (in->updateGradient) this->backward(values, &out->value, &out->gradient, i, &in->gradient);
+    }
+}
+
+// ---- MatrixMultiply ---------------------------------------------------------------------------------------------------
+MatrixMultiply::MatrixMultiply(std::vector<Node *> &in) : Function(in) {
+    DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the MatrixMultiply Function needs 2 input");
+}
+
+Shape MatrixMultiply::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputShapes.size(), "the input count must be 2");
+    const Shape &x = inputShapes[0], &y = inputShapes[1];
+    DEEP8_ARGUMENT_CHECK(x.batch == y.batch || 1 == x.batch || 1 == y.batch, "the batch of input is error");
+    DEEP8_ARGUMENT_CHECK((1 == x.nDims || 2 == x.nDims) && (1 == y.nDims || 2 == y.nDims), "the inputs dimensions is error");
+    DEEP8_ARGUMENT_CHECK(x.col() == y.row(), "the col of input1 must same to the row of input2");
+    const size_t batch = std::max(x.batch, y.batch);
+    if (1 == y.col()) return Shape(batch, {x.row()});  // a 1-D result
+    return Shape(batch, {x.row(), y.col()});
+}
+
+ElementType MatrixMultiply::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputTypes.size(), "the input count must be 2");
+    return Function::checkElementType(inputTypes);
+}
+
+void MatrixMultiply::forward(const std::vector<const Tensor *> &in, Tensor *output) {
+    Math::MatrixMultiply(*in[0], *in[1], *output);
+}
+
+void MatrixMultiply::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient,
+                              size_t index, Tensor *iGradient) {
+    if (0 == index) Math::MatrixMultiplyGradX(*in[0], *iGradient, *in[1], *output, *outputGradient);
+    else if (1 == index) Math::MatrixMultiplyGradY(*in[0], *in[1], *iGradient, *output, *outputGradient);
+    else DEEP8_RUNTIME_ERROR("the index is error");
+}
+
+// ---- Conv2d / DeConv2d ---------------------------------------------------------------------------------------------------
+// An interim buffer from the device pool for one Math call; freed as soon as the call has
+// queued its kernels (single stream + a pool that never gives memory back while alive).
+namespace {
+struct Interim {
+    Device *device;
+    void *ptr;
+    Interim(Device *d, size_t bytes) : device(d), ptr(d->malloc(bytes)) {}
+    ~Interim() { device->free(ptr); }
+};
+
+void checkConvInputs(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputShapes.size(), "the input count must be 2");
+    const Shape &in = inputShapes[0], &filter = inputShapes[1];
+    DEEP8_ARGUMENT_CHECK(3 == in.nDims, "Conv2d needs inputs nDims is 3");
+    DEEP8_ARGUMENT_CHECK(4 == filter.nDims && 1 == filter.batch, "Conv2d needs filter nDims is 4, the batch must be 1");
+    DEEP8_ARGUMENT_CHECK(in.dim(2) == filter.dim(3), "the inputs dimension is error");
+    DEEP8_ARGUMENT_CHECK(filter.dim(1) > 0 && filter.dim(2) > 0, "the filter width and height must bigger than 0");
+}
+}  // namespace
+
+Conv2d::Conv2d(std::vector<Node *> &in, bool cov, int sy, int sx, int dy, int dx)
+    : Function(in), covered(cov), strideY(sy), strideX(sx), dilationY(dy), dilationX(dx) {
+    DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the Conv2d Function needs 2 input");
+    DEEP8_ARGUMENT_CHECK(strideY >= 1 && strideX >= 1, "the stride can not smaller than 1");
+    DEEP8_ARGUMENT_CHECK(dilationY >= 1 && dilationX >= 1, "the dilation can not smaller than 1");
+}
+
+Shape Conv2d::checkShape(std::vector<Shape> &inputShapes) {
+    checkConvInputs(inputShapes);
+    const Shape &in = inputShapes[0], &filter = inputShapes[1];
+    const int FH = (int)filter.dim(1), FW = (int)filter.dim(2), IH = (int)in.dim(0), IW = (int)in.dim(1);
+    if (!covered)
+        DEEP8_ARGUMENT_CHECK(FH <= IH && FW <= IW, "the not covered mode Padding type needs filter smaller than input");
+    const int realFH = FH + (FH - 1) * (dilationY - 1), realFW = FW + (FW - 1) * (dilationX - 1);
+    const int OH = covered ? (IH - 1) / strideY + 1 : (IH - realFH) / strideY + 1;
+    const int OW = covered ? (IW - 1) / strideX + 1 : (IW - realFW) / strideX + 1;
+    DEEP8_ARGUMENT_CHECK(OH > 0 && OW > 0, "the output height or width must > 0");
+    return Shape(in.batch, {(size_t)OH, (size_t)OW, filter.dim(0)});
+}
+
+ElementType Conv2d::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputTypes.size(), "the input count must be 2");
+    return Function::checkElementType(inputTypes);
+}
+
+void Conv2d::forward(const std::vector<const Tensor *> &in, Tensor *output) {
+    Interim buf(output->device(),
+                Math::Conv2dInterimSize(*in[0], *in[1], *output, covered, strideY, strideX, dilationY, dilationX));
+    Math::Conv2d(*in[0], *in[1], *output, covered, strideY, strideX, dilationY, dilationX, buf.ptr);
+}
+
+void Conv2d::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient,
+                      size_t index, Tensor *iGradient) {
+    if (0 == index) {
+        Interim buf(iGradient->device(), Math::Conv2dGradXInterimSize(*in[0], *iGradient, *in[1], *output, *outputGradient,
+                                                                      covered, strideY, strideX, dilationY, dilationX));
+        Math::Conv2dGradX(*in[0], *iGradient, *in[1], *output, *outputGradient, covered, strideY, strideX, dilationY,
+                          dilationX, buf.ptr);
+    } else if (1 == index) {
+        Interim buf(iGradient->device(), Math::Conv2dGradYInterimSize(*in[0], *in[1], *iGradient, *output, *outputGradient,
+                                                                      covered, strideY, strideX, dilationY, dilationX));
+        Math::Conv2dGradY(*in[0], *in[1], *iGradient, *output, *outputGradient, covered, strideY, strideX, dilationY,
+                          dilationX, buf.ptr);
+    } else {
+        DEEP8_RUNTIME_ERROR("the index is error");
+    }
+}
+
+DeConv2d::DeConv2d(std::vector<Node *> &in, bool cov, int sy, int sx)
+    : Function(in), forwardCovered(cov), forwardStrideY(sy), forwardStrideX(sx) {
+    DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the DeConv2d Function needs 2 input");
+    DEEP8_ARGUMENT_CHECK(forwardStrideY >= 1 && forwardStrideX >= 1, "the stride is error");
+}
+
+Shape DeConv2d::checkShape(std::vector<Shape> &inputShapes) {
+    checkConvInputs(inputShapes);
+    const Shape &in = inputShapes[0], &filter = inputShapes[1];
+    const int FH = (int)filter.dim(1), FW = (int)filter.dim(2), IH = (int)in.dim(0), IW = (int)in.dim(1);
+    // the inverse of Conv2d's size rule
+    const int OH = (IH - 1) * forwardStrideY + (forwardCovered ? 1 : FH);
+    const int OW = (IW - 1) * forwardStrideX + (forwardCovered ? 1 : FW);
+    DEEP8_ARGUMENT_CHECK(OH > 0 && OW > 0, "the output height/width must > 0");
+    return Shape(in.batch, {(size_t)OH, (size_t)OW, filter.dim(0)});
+}
+
+ElementType DeConv2d::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputTypes.size(), "the input count must be 2");
+    return Function::checkElementType(inputTypes);
+}
+
+void DeConv2d::forward(const std::vector<const Tensor *> &in, Tensor *output) {
+    Interim buf(output->device(),
+                Math::DeConv2dInterimSize(*in[0], *in[1], *output, forwardCovered, forwardStrideY, forwardStrideX));
+    Math::DeConv2d(*in[0], *in[1], *output, forwardCovered, forwardStrideY, forwardStrideX, buf.ptr);
+}
+
+void DeConv2d::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient,
+                        size_t index, Tensor *iGradient) {
+    if (0 == index) {
+        Interim buf(iGradient->device(), Math::DeConv2dGradXInterimSize(*in[0], *iGradient, *in[1], *output, *outputGradient,
+                                                                        forwardCovered, forwardStrideY, forwardStrideX));
+        Math::DeConv2dGradX(*in[0], *iGradient, *in[1], *output, *outputGradient, forwardCovered, forwardStrideY,
+                            forwardStrideX, buf.ptr);
+    } else if (1 == index) {
+        Interim buf(iGradient->device(), Math::DeConv2dGradYInterimSize(*in[0], *in[1], *iGradient, *output, *outputGradient,
+                                                                        forwardCovered, forwardStrideY, forwardStrideX));
+        Math::DeConv2dGradY(*in[0], *in[1], *iGradient, *output, *outputGradient, forwardCovered, forwardStrideY,
+                            forwardStrideX, buf.ptr);
+    } else {
+        DEEP8_RUNTIME_ERROR("the index of DeConv2d backward is error");
+    }
+}
+
+}  // namespace Deep8

@@ -1,0 +1,543 @@
+// Test driver of the C++ host layer.  Node-level tests in the style of the reference's
+// test/MatrixMultiplyTest.h, test/Conv2dTest.h and test/DeConv2dTest.h: build a node over two
+// placeholder Variables, call the explicit-tensor forward/backward, and compare with naive host
+// loops on small non-negative integer inputs, for which float results are exact.
+//
+//   deep8_host_tests            run everything (needs a GPU)
+//   deep8_host_tests --cpu      run only the tests that touch no device
+//   deep8_host_tests --list     list test names
+// Prints "PASS <name>" / "FAIL <name>: <why>" per test; exit code = number of failures.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <iostream>
+#include <random>
+
+#include "deep8/Deep8.h"
+
+using namespace Deep8;
+
+namespace {
+
+struct Failure : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+#define EXPECT(cond)                                                                      \
+    do {                                                                                  \
+        if (!(cond)) throw Failure(std::string(#cond) + " at line " + std::to_string(__LINE__)); \
+    } while (0)
+
+template <typename E, typename F>
+bool throws(F f) {
+    try {
+        f();
+    } catch (const E &) {
+        return true;
+    } catch (...) {
+        return false;
+    }
+    return false;
+}
+
+std::mt19937 rng(12345);
+float randInt(int hi) { return (float)(rng() % hi); }
+
+struct Test {
+    const char *name;
+    bool needsGpu;
+    std::function<void()> body;
+};
+std::vector<Test> &tests() {
+    static std::vector<Test> t;
+    return t;
+}
+struct Reg {
+    Reg(const char *n, bool gpu, std::function<void()> b) { tests().push_back({n, gpu, std::move(b)}); }
+};
+#define TEST_CPU(name) \
+    void name();       \
+    Reg reg_##name(#name, false, name); \
+    void name()
+#define TEST_GPU(name) \
+    void name();       \
+    Reg reg_##name(#name, true, name); \
+    void name()
+
+GPUDevice &gpu() {
+    static GPUDevice *d = new GPUDevice();
+    return *d;
+}
+
+// A device tensor plus its host mirror (float values; stored as float or half on the device).
+struct HostTensor {
+    Tensor t;
+    std::vector<float> host;
+};
+
+Tensor makeTensor(GPUDevice &dev, ElementType type, size_t batch, std::vector<size_t> dims) {
+    Shape shape(batch, dims);
+    const size_t bytes = type.byteWidth * shape.size();
+    void *ptr = dev.malloc(bytes);
+    size_t *ref = (size_t *)dev.mallocCPU(sizeof(size_t));
+    TensorStorage storage(ptr, ref, bytes, &dev);
+    return Tensor(storage, 0, shape, type);
+}
+
+void upload(HostTensor &h) {
+    if (h.t.elementType.id == DType::Float32) {
+        h.t.device()->copyFromCPUToGPU(h.host.data(), h.t.raw(), h.t.byteCount());
+    } else {
+        std::vector<half> tmp(h.host.begin(), h.host.end());
+        h.t.device()->copyFromCPUToGPU(tmp.data(), h.t.raw(), h.t.byteCount());
+    }
+}
+
+void download(HostTensor &h) {
+    if (h.t.elementType.id == DType::Float32) {
+        h.t.device()->copyFromGPUToCPU(h.t.raw(), h.host.data(), h.t.byteCount());
+    } else {
+        std::vector<half> tmp(h.host.size());
+        h.t.device()->copyFromGPUToCPU(h.t.raw(), tmp.data(), h.t.byteCount());
+        for (size_t i = 0; i < tmp.size(); ++i) h.host[i] = (float)tmp[i];
+    }
+}
+
+HostTensor randomTensor(ElementType type, size_t batch, std::vector<size_t> dims, int hi) {
+    HostTensor h;
+    h.t = makeTensor(gpu(), type, batch, dims);
+    h.host.resize(h.t.size());
+    for (float &v : h.host) v = hi ? randInt(hi) : 0.f;
+    upload(h);
+    return h;
+}
+
+Variable placeholder(ElementType type) {
+    Tensor v = makeTensor(gpu(), type, 1, {1});
+    Tensor g = makeTensor(gpu(), type, 1, {1});
+    return Variable(0, "", nullptr, v, g);
+}
+
+// ---------------------------------------------------------------------------------------------
+TEST_CPU(half_conversion) {
+    EXPECT(half(1.0f).bits == 0x3c00);
+    EXPECT(half(-2.0f).bits == 0xc000);
+    EXPECT(half(65504.0f).bits == 0x7bff);
+    EXPECT(half(65520.0f).bits == 0x7c00);
+    EXPECT(half(5.9604645e-8f).bits == 0x0001);
+    EXPECT(half(2.9802322e-8f).bits == 0x0000);  // tie to even
+    EXPECT(half(1.0009766f).bits == 0x3c01);
+    EXPECT(half(1.00048828125f).bits == 0x3c00);  // tie to even
+    EXPECT(half(1.00146484375f).bits == 0x3c02);  // tie to even, upwards
+    for (uint32_t b = 0; b < 65536; ++b) {
+        const uint32_t exp = (b >> 10) & 31, man = b & 1023;
+        if (exp == 31 && man) continue;  // NaN
+        EXPECT(half(half::toFloat((uint16_t)b)).bits == b);
+    }
+}
+
+TEST_CPU(shape_basics) {
+    Shape s(5, {2, 3, 4});
+    EXPECT(s.batch == 5 && s.nDims == 3 && s.size() == 120 && s.batchSize() == 24);
+    EXPECT(s.stride(0) == 12 && s.stride(1) == 4 && s.stride(2) == 1);
+    EXPECT(s.row() == 2 && s.col() == 3);
+    Shape v(3, {7});
+    EXPECT(v.row() == 7 && v.col() == 1);
+    EXPECT(Shape(5, {2, 3, 4}) == s && Shape(4, {2, 3, 4}) != s);
+    EXPECT(s.equalExceptBatch(Shape(1, {2, 3, 4})));
+    EXPECT(throws<std::invalid_argument>([] { Shape bad(1, {2, 0}); }));
+    EXPECT(throws<std::invalid_argument>([] { Shape bad(1, {1, 2, 3, 4, 5}); }));
+    EXPECT(throws<std::invalid_argument>([&] { s.dim(3); }));
+    EXPECT(ElementType::from<float>().byteWidth == 4 && ElementType::from<half>().byteWidth == 2);
+    EXPECT(ElementType::from(DType::Float16).id == DType::Float16);
+}
+
+TEST_CPU(node_shape_inference) {
+    // checkShape needs no device
+    std::vector<Node *> none;
+    struct Probe : Variable {
+        Probe() : Variable(0, "", nullptr) {}
+    } a, b;
+    std::vector<Node *> in = {&a, &b};
+    MatrixMultiply mm(in);
+    std::vector<Shape> s = {Shape(10, {400, 200}), Shape(1, {200, 300})};
+    EXPECT(mm.checkShape(s) == Shape(10, {400, 300}));
+    s = {Shape(1, {300, 100}), Shape(10, {100})};
+    EXPECT(mm.checkShape(s) == Shape(10, {300}));
+    s = {Shape(2, {3, 4}), Shape(3, {4, 5})};
+    EXPECT(throws<std::invalid_argument>([&] { mm.checkShape(s); }));
+    s = {Shape(1, {3, 4}), Shape(1, {5, 5})};
+    EXPECT(throws<std::invalid_argument>([&] { mm.checkShape(s); }));
+
+    Conv2d same(in, true, 1, 1, 1, 1);
+    s = {Shape(32, {56, 56, 64}), Shape(1, {64, 3, 3, 64})};
+    EXPECT(same.checkShape(s) == Shape(32, {56, 56, 64}));
+    Conv2d strided(in, true, 2, 2, 2, 2);
+    s = {Shape(2, {32, 32, 64}), Shape(1, {32, 4, 4, 64})};
+    EXPECT(strided.checkShape(s) == Shape(2, {16, 16, 32}));
+    Conv2d valid(in, false, 1, 1, 1, 1);
+    EXPECT(valid.checkShape(s) == Shape(2, {29, 29, 32}));
+    s = {Shape(2, {3, 3, 64}), Shape(1, {32, 4, 4, 64})};
+    EXPECT(throws<std::invalid_argument>([&] { valid.checkShape(s); }));
+    EXPECT(throws<std::invalid_argument>([&] { Conv2d bad(in, true, 0, 1, 1, 1); }));
+
+    DeConv2d up(in, false, 2, 2), upCovered(in, true, 2, 2);
+    s = {Shape(16, {28, 28, 128}), Shape(1, {64, 4, 4, 128})};
+    EXPECT(up.checkShape(s) == Shape(16, {58, 58, 64}));
+    EXPECT(upCovered.checkShape(s) == Shape(16, {55, 55, 64}));
+    s = {Shape(16, {28, 28, 128}), Shape(1, {64, 4, 4, 100})};
+    EXPECT(throws<std::invalid_argument>([&] { up.checkShape(s); }));
+}
+
+TEST_GPU(memory_pool) {
+    GPUMemoryPool pool(0, size_t(1) << 24);  // 16 MiB blocks
+    void *a = pool.malloc(1000);
+    void *b = pool.malloc(1000);
+    EXPECT(a && b && a != b);
+    EXPECT(pool.blockCount() == 1 && pool.bytesInUse() == 2048);
+    pool.free(a);
+    void *c = pool.malloc(600);  // reuses the 1 KiB chunk just freed
+    EXPECT(c == a);
+    pool.free(b);
+    pool.free(c);
+    EXPECT(pool.bytesInUse() == 0);
+    void *whole = pool.malloc(size_t(1) << 24);  // everything merged back: the whole block is free
+    EXPECT(whole && pool.blockCount() == 1);
+    void *more = pool.malloc(5 << 20);  // needs a second block
+    EXPECT(more && pool.blockCount() == 2);
+    pool.free(whole);
+    pool.free(more);
+    EXPECT(pool.malloc(0) == nullptr);
+    EXPECT(throws<std::invalid_argument>([&] { pool.malloc((size_t(1) << 24) + 1); }));
+    int onStack = 0;
+    EXPECT(throws<std::runtime_error>([&] { pool.free(&onStack); }));
+    void *d = pool.malloc(4096);
+    pool.free(d);
+    EXPECT(throws<std::runtime_error>([&] { pool.free(d); }));  // double free
+    // the default pool refuses more than 512 MiB in one piece, like the reference's
+    EXPECT(throws<std::invalid_argument>([&] { gpu().malloc((size_t(512) << 20) + 1); }));
+}
+
+TEST_GPU(tensor_storage_refcount) {
+    const size_t before = gpu().memoryPool->bytesInUse();
+    {
+        Tensor t = makeTensor(gpu(), ElementType::from<float>(), 2, {8, 8});
+        EXPECT(t.refCount() == 1 && t.byteCount() == 512);
+        {
+            Tensor u = t;
+            EXPECT(t.refCount() == 2 && u.raw() == t.raw());
+        }
+        EXPECT(t.refCount() == 1);
+        t.zero();
+        std::vector<float> h(128, 1.f);
+        gpu().copyFromGPUToCPU(t.raw(), h.data(), 512);
+        for (float v : h) EXPECT(v == 0.f);
+        EXPECT(throws<std::invalid_argument>([&] { t.data<half>(); }));
+        EXPECT(t.data<float>() == t.raw());
+    }
+    EXPECT(gpu().memoryPool->bytesInUse() == before);
+    Tensor s = makeTensor(gpu(), ElementType::from<half>(), 1, {1});
+    s.one();
+    half one;
+    gpu().copyFromGPUToCPU(s.raw(), &one, 2);
+    EXPECT(one.bits == 0x3c00);
+}
+
+// ---- MatrixMultiply ---------------------------------------------------------------------------------------
+void matmulCase(ElementType type, size_t xb, std::vector<size_t> xd, size_t yb, std::vector<size_t> yd, int hi) {
+    HostTensor x = randomTensor(type, xb, xd, hi), y = randomTensor(type, yb, yd, hi);
+    Variable v0 = placeholder(type), v1 = placeholder(type);
+    std::vector<Node *> in = {&v0, &v1};
+    MatrixMultiply mm(in);
+    std::vector<Shape> shapes = {x.t.shape, y.t.shape};
+    Shape zs = mm.checkShape(shapes);
+    HostTensor z = randomTensor(type, zs.batch, std::vector<size_t>(zs.dims, zs.dims + zs.nDims), 0);
+    HostTensor dz = randomTensor(type, zs.batch, std::vector<size_t>(zs.dims, zs.dims + zs.nDims), hi);
+    HostTensor dx = randomTensor(type, xb, xd, 0), dy = randomTensor(type, yb, yd, 0);
+
+    std::vector<const Tensor *> tin = {&x.t, &y.t};
+    mm.forward(tin, &z.t);
+    mm.backward(tin, &z.t, &dz.t, 0, &dx.t);
+    mm.backward(tin, &z.t, &dz.t, 1, &dy.t);
+    download(z);
+    download(dx);
+    download(dy);
+
+    const size_t M = x.t.row(), K = x.t.col(), N = y.t.col(), B = zs.batch;
+    std::vector<float> wz(z.host.size(), 0.f), wdx(dx.host.size(), 0.f), wdy(dy.host.size(), 0.f);
+    for (size_t b = 0; b < B; ++b) {
+        const float *xp = x.host.data() + (b % xb) * M * K, *yp = y.host.data() + (b % yb) * K * N;
+        const float *gp = dz.host.data() + b * M * N;
+        float *zp = wz.data() + b * M * N, *dxp = wdx.data() + (b % xb) * M * K, *dyp = wdy.data() + (b % yb) * K * N;
+        for (size_t m = 0; m < M; ++m)
+            for (size_t n = 0; n < N; ++n) {
+                float acc = 0;
+                for (size_t k = 0; k < K; ++k) {
+                    acc += xp[m * K + k] * yp[k * N + n];
+                    dxp[m * K + k] += gp[m * N + n] * yp[k * N + n];
+                    dyp[k * N + n] += xp[m * K + k] * gp[m * N + n];
+                }
+                zp[m * N + n] = acc;
+            }
+    }
+    EXPECT(z.host == wz);
+    EXPECT(dx.host == wdx);
+    EXPECT(dy.host == wdy);
+}
+
+TEST_GPU(matrix_multiply_float_collapsed_batch) {  // MatrixMultiplyTest GPU1_float shape, reduced
+    matmulCase(ElementType::from<float>(), 10, {40, 20}, 1, {20, 30}, 50);
+}
+TEST_GPU(matrix_multiply_float_vector_batch) {  // GPU2_float: x batch 1, y a batch of vectors
+    matmulCase(ElementType::from<float>(), 1, {30, 10}, 10, {10}, 50);
+}
+TEST_GPU(matrix_multiply_float_batched) {
+    matmulCase(ElementType::from<float>(), 6, {33, 17}, 6, {17, 29}, 50);
+    matmulCase(ElementType::from<float>(), 1, {33, 17}, 6, {17, 29}, 50);  // dX sums over the batch
+}
+TEST_GPU(matrix_multiply_half) {
+    matmulCase(ElementType::from<half>(), 4, {24, 16}, 1, {16, 40}, 3);
+    matmulCase(ElementType::from<half>(), 1, {24, 16}, 5, {16}, 3);
+    matmulCase(ElementType::from<half>(), 3, {24, 16}, 3, {16, 8}, 3);
+}
+
+TEST_GPU(matrix_multiply_errors) {
+    ElementType f32 = ElementType::from<float>();
+    HostTensor x = randomTensor(f32, 1, {4, 5}, 5), y = randomTensor(f32, 1, {5, 6}, 5);
+    HostTensor z = randomTensor(f32, 1, {4, 6}, 0), bad = randomTensor(f32, 1, {4, 7}, 0);
+    HostTensor zh = randomTensor(ElementType::from<half>(), 1, {4, 6}, 0);
+    EXPECT(throws<std::invalid_argument>([&] { Math::MatrixMultiply(x.t, y.t, bad.t); }));
+    EXPECT(throws<std::invalid_argument>([&] { Math::MatrixMultiply(x.t, y.t, zh.t); }));
+    EXPECT(throws<std::invalid_argument>([&] { Math::MatrixMultiplyGradX(x.t, bad.t, y.t, z.t, z.t); }));
+    Tensor d64 = makeTensor(gpu(), ElementType::from<double>(), 1, {4, 4});
+    EXPECT(throws<std::runtime_error>([&] { Math::MatrixMultiply(d64, d64, d64); }));
+    Variable v0 = placeholder(f32);
+    std::vector<Node *> one = {&v0};
+    EXPECT(throws<std::invalid_argument>([&] { MatrixMultiply mm(one); }));
+    Variable v1 = placeholder(f32);
+    std::vector<Node *> two = {&v0, &v1};
+    MatrixMultiply mm(two);
+    std::vector<const Tensor *> tin = {&x.t, &y.t};
+    EXPECT(throws<std::runtime_error>([&] { mm.backward(tin, &z.t, &z.t, 2, &z.t); }));
+}
+
+// ---- Conv2d ---------------------------------------------------------------------------------------------------
+void convCase(ElementType type, int B, int IH, int IW, int IC, int OC, int FH, int FW, bool covered, int sy, int sx,
+              int dy, int dx, int hi) {
+    HostTensor x = randomTensor(type, B, {(size_t)IH, (size_t)IW, (size_t)IC}, hi);
+    HostTensor w = randomTensor(type, 1, {(size_t)OC, (size_t)FH, (size_t)FW, (size_t)IC}, hi);
+    Variable v0 = placeholder(type), v1 = placeholder(type);
+    std::vector<Node *> in = {&v0, &v1};
+    Conv2d conv(in, covered, sy, sx, dy, dx);
+    std::vector<Shape> shapes = {x.t.shape, w.t.shape};
+    Shape zs = conv.checkShape(shapes);
+    const int OH = (int)zs.dim(0), OW = (int)zs.dim(1);
+    HostTensor z = randomTensor(type, B, {(size_t)OH, (size_t)OW, (size_t)OC}, 0);
+    HostTensor gz = randomTensor(type, B, {(size_t)OH, (size_t)OW, (size_t)OC}, hi);
+    HostTensor gx = randomTensor(type, B, {(size_t)IH, (size_t)IW, (size_t)IC}, 0);
+    HostTensor gw = randomTensor(type, 1, {(size_t)OC, (size_t)FH, (size_t)FW, (size_t)IC}, 0);
+
+    std::vector<const Tensor *> tin = {&x.t, &w.t};
+    conv.forward(tin, &z.t);
+    conv.backward(tin, &z.t, &gz.t, 0, &gx.t);
+    conv.backward(tin, &z.t, &gz.t, 1, &gw.t);
+    download(z);
+    download(gx);
+    download(gw);
+
+    const int rfh = FH + (FH - 1) * (dy - 1), rfw = FW + (FW - 1) * (dx - 1);
+    const int padTop = std::max(0, (OH - 1) * sy + rfh - IH) / 2, padLeft = std::max(0, (OW - 1) * sx + rfw - IW) / 2;
+    std::vector<float> wz(z.host.size(), 0.f), wgx(gx.host.size(), 0.f), wgw(gw.host.size(), 0.f);
+    for (int b = 0; b < B; ++b)
+        for (int oy = 0; oy < OH; ++oy)
+            for (int ox = 0; ox < OW; ++ox)
+                for (int oc = 0; oc < OC; ++oc) {
+                    const size_t zi = (((size_t)b * OH + oy) * OW + ox) * OC + oc;
+                    for (int fy = 0; fy < FH; ++fy)
+                        for (int fx = 0; fx < FW; ++fx) {
+                            const int iy = oy * sy + fy * dy - padTop, ix = ox * sx + fx * dx - padLeft;
+                            if (iy < 0 || iy >= IH || ix < 0 || ix >= IW) continue;
+                            for (int ic = 0; ic < IC; ++ic) {
+                                const size_t xi = (((size_t)b * IH + iy) * IW + ix) * IC + ic;
+                                const size_t wi = (((size_t)oc * FH + fy) * FW + fx) * IC + ic;
+                                wz[zi] += x.host[xi] * w.host[wi];
+                                wgx[xi] += gz.host[zi] * w.host[wi];
+                                wgw[wi] += gz.host[zi] * x.host[xi];
+                            }
+                        }
+                }
+    EXPECT(z.host == wz);
+    EXPECT(gx.host == wgx);
+    EXPECT(gw.host == wgw);
+}
+
+TEST_GPU(conv2d_float_covered_stride_dilation) {  // Conv2dTest forwardCPU_float geometry, smaller tensors
+    convCase(ElementType::from<float>(), 2, 16, 16, 8, 6, 4, 4, true, 2, 2, 2, 2, 20);
+}
+TEST_GPU(conv2d_float_covered_5x5) { convCase(ElementType::from<float>(), 2, 12, 12, 4, 4, 5, 5, true, 1, 1, 1, 1, 20); }
+TEST_GPU(conv2d_float_not_covered) { convCase(ElementType::from<float>(), 2, 13, 11, 5, 3, 3, 3, false, 1, 1, 1, 1, 20); }
+TEST_GPU(conv2d_half) { convCase(ElementType::from<half>(), 2, 8, 8, 8, 8, 3, 3, true, 1, 1, 1, 1, 2); }
+
+// ---- DeConv2d -----------------------------------------------------------------------------------------------------
+void deconvCase(ElementType type, int B, int IH, int IW, int IC, int OC, int FH, int FW, bool covered, int sy, int sx, int hi) {
+    HostTensor x = randomTensor(type, B, {(size_t)IH, (size_t)IW, (size_t)IC}, hi);
+    HostTensor w = randomTensor(type, 1, {(size_t)OC, (size_t)FH, (size_t)FW, (size_t)IC}, hi);
+    Variable v0 = placeholder(type), v1 = placeholder(type);
+    std::vector<Node *> in = {&v0, &v1};
+    DeConv2d deconv(in, covered, sy, sx);
+    std::vector<Shape> shapes = {x.t.shape, w.t.shape};
+    Shape zs = deconv.checkShape(shapes);
+    const int OH = (int)zs.dim(0), OW = (int)zs.dim(1);
+    HostTensor z = randomTensor(type, B, {(size_t)OH, (size_t)OW, (size_t)OC}, 0);
+    HostTensor gz = randomTensor(type, B, {(size_t)OH, (size_t)OW, (size_t)OC}, hi);
+    HostTensor gx = randomTensor(type, B, {(size_t)IH, (size_t)IW, (size_t)IC}, 0);
+    HostTensor gw = randomTensor(type, 1, {(size_t)OC, (size_t)FH, (size_t)FW, (size_t)IC}, 0);
+
+    std::vector<const Tensor *> tin = {&x.t, &w.t};
+    deconv.forward(tin, &z.t);
+    deconv.backward(tin, &z.t, &gz.t, 0, &gx.t);
+    deconv.backward(tin, &z.t, &gz.t, 1, &gw.t);
+    download(z);
+    download(gx);
+    download(gw);
+
+    const int padTop = std::max(0, OH + FH - (IH - 1) * sy - 2) / 2, padLeft = std::max(0, OW + FW - (IW - 1) * sx - 2) / 2;
+    std::vector<float> wz(z.host.size(), 0.f), wgx(gx.host.size(), 0.f), wgw(gw.host.size(), 0.f);
+    for (int b = 0; b < B; ++b)
+        for (int oy = 0; oy < OH; ++oy)
+            for (int ox = 0; ox < OW; ++ox)
+                for (int oc = 0; oc < OC; ++oc) {
+                    const size_t zi = (((size_t)b * OH + oy) * OW + ox) * OC + oc;
+                    for (int fy = 0; fy < FH; ++fy)
+                        for (int fx = 0; fx < FW; ++fx) {
+                            const int ty = oy - padTop + fy, tx = ox - padLeft + fx;
+                            if (ty < 0 || tx < 0 || ty % sy || tx % sx) continue;
+                            const int iy = ty / sy, ix = tx / sx;
+                            if (iy >= IH || ix >= IW) continue;
+                            for (int ic = 0; ic < IC; ++ic) {
+                                const size_t xi = (((size_t)b * IH + iy) * IW + ix) * IC + ic;
+                                const size_t wi = (((size_t)oc * FH + fy) * FW + fx) * IC + ic;
+                                wz[zi] += x.host[xi] * w.host[wi];
+                                wgx[xi] += gz.host[zi] * w.host[wi];
+                                wgw[wi] += gz.host[zi] * x.host[xi];
+                            }
+                        }
+                }
+    EXPECT(z.host == wz);
+    EXPECT(gx.host == wgx);
+    EXPECT(gw.host == wgw);
+}
+
+TEST_GPU(deconv2d_float_not_covered_stride3) { deconvCase(ElementType::from<float>(), 2, 8, 8, 8, 4, 4, 4, false, 3, 3, 20); }
+TEST_GPU(deconv2d_float_covered_stride3) { deconvCase(ElementType::from<float>(), 2, 8, 8, 8, 4, 4, 4, true, 3, 3, 20); }
+TEST_GPU(deconv2d_float_stride2) { deconvCase(ElementType::from<float>(), 2, 7, 6, 4, 6, 4, 4, false, 2, 2, 20); }
+TEST_GPU(deconv2d_half) { deconvCase(ElementType::from<half>(), 2, 6, 6, 8, 8, 4, 4, false, 2, 2, 2); }
+
+TEST_GPU(conv2d_errors) {
+    ElementType f32 = ElementType::from<float>();
+    HostTensor x = randomTensor(f32, 2, {8, 8, 4}, 5), w = randomTensor(f32, 1, {3, 3, 3, 4}, 5);
+    HostTensor z = randomTensor(f32, 2, {8, 8, 3}, 0), bad = randomTensor(f32, 2, {7, 8, 3}, 0);
+    EXPECT(Math::Conv2dInterimSize(x.t, w.t, z.t, true, 1, 1, 1, 1) >= sizeof(float) * 2 * 8 * 8 * 3 * 3 * 4);
+    EXPECT(throws<std::invalid_argument>([&] { Math::Conv2dInterimSize(x.t, w.t, bad.t, true, 1, 1, 1, 1); }));
+    EXPECT(throws<std::invalid_argument>([&] { Math::Conv2d(x.t, w.t, z.t, true, 0, 1, 1, 1, nullptr); }));
+    EXPECT(throws<std::invalid_argument>([&] { Math::DeConv2dInterimSize(x.t, w.t, z.t, false, 1, 1); }));
+}
+
+// ---- through the executor ---------------------------------------------------------------------------------------------
+TEST_GPU(eager_executor_matmul_chain) {
+    EagerExecutor executor(DeviceType::GPU);
+    const size_t K = 48, N = 40;
+    Variable &x = inputParameter(&executor, {1, K});
+    Variable &W = parameter(&executor, {K, N});
+    Variable &v = parameter(&executor, {N});
+    std::vector<float> hx(K), hW(K * N), hv(N);
+    for (float &f : hx) f = randInt(10);
+    for (float &f : hW) f = randInt(10);
+    for (float &f : hv) f = randInt(10);
+    x.feed(hx.data());
+    W.feed(hW.data());
+    v.feed(hv.data());
+
+    Variable &h = x * W;  // [1 x N]
+    Variable &loss = h * v;  // scalar
+    EXPECT(h.shape() == Shape(1, {1, N}) && loss.isScalar());
+    float got = 0;
+    loss.fetch(&got);
+    std::vector<float> hh(N, 0.f);
+    float want = 0;
+    for (size_t n = 0; n < N; ++n) {
+        for (size_t k = 0; k < K; ++k) hh[n] += hx[k] * hW[k * N + n];
+        want += hh[n] * hv[n];
+    }
+    EXPECT(got == want);
+
+    const std::string interimName = h.name;
+    backward(loss);
+    std::vector<float> gW(K * N), gv(N);
+    gpu().copyFromGPUToCPU(W.gradient.raw(), gW.data(), gW.size() * 4);
+    gpu().copyFromGPUToCPU(v.gradient.raw(), gv.data(), gv.size() * 4);
+    for (size_t n = 0; n < N; ++n) {
+        EXPECT(gv[n] == hh[n]);
+        for (size_t k = 0; k < K; ++k) EXPECT(gW[k * N + n] == hx[k] * hv[n]);
+    }
+    EXPECT(executor.trainableParameters().size() == 2);
+    EXPECT(executor.nodeByName(interimName) == nullptr);  // interim nodes are gone after backward
+}
+
+TEST_GPU(eager_executor_conv_to_scalar) {
+    EagerExecutor executor(DeviceType::GPU);
+    Variable &x = parameter(&executor, 1, {3, 3, 2});
+    Variable &w = parameter(&executor, {1, 3, 3, 2});
+    std::vector<float> hx(18), hw(18);
+    for (float &f : hx) f = randInt(10);
+    for (float &f : hw) f = randInt(10);
+    x.feed(hx.data());
+    w.feed(hw.data());
+    Variable &z = x.conv2d(w, false);  // 3x3 filter over a 3x3 image, no padding: one number
+    EXPECT(z.isScalar());
+    float got = 0, want = 0;
+    z.fetch(&got);
+    for (int i = 0; i < 18; ++i) want += hx[i] * hw[i];
+    EXPECT(got == want);
+    backward(z);
+    std::vector<float> gx(18), gw(18);
+    gpu().copyFromGPUToCPU(x.gradient.raw(), gx.data(), 72);
+    gpu().copyFromGPUToCPU(w.gradient.raw(), gw.data(), 72);
+    EXPECT(gx == hw && gw == hx);
+
+    EXPECT(throws<std::runtime_error>([] { EagerExecutor cpu(DeviceType::CPU); }));
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+    bool cpuOnly = false, list = false;
+    std::string only;
+    for (int i = 1; i < argc; ++i) {
+        if (!strcmp(argv[i], "--cpu")) cpuOnly = true;
+        else if (!strcmp(argv[i], "--list")) list = true;
+        else only = argv[i];
+    }
+    int failures = 0, ran = 0;
+    for (Test &t : tests()) {
+        if (list) {
+            printf("%s %s\n", t.needsGpu ? "gpu" : "cpu", t.name);
+            continue;
+        }
+        if ((cpuOnly && t.needsGpu) || (!only.empty() && only != t.name)) continue;
+        printf("RUN  %s\n", t.name);
+        fflush(stdout);
+        try {
+            t.body();
+            printf("PASS %s\n", t.name);
+        } catch (const std::exception &e) {
+            printf("FAIL %s: %s\n", t.name, e.what());
+            ++failures;
+        }
+        fflush(stdout);
+        ++ran;
+    }
+    if (!list) printf("%d test(s), %d failure(s)\n", ran, failures);
+    return failures;
+}

@@ -44,6 +44,9 @@ int d8_memset(void *ptr, int value, size_t bytes, void *stream);   /* cudaMemset
 int d8_memcpy_h2d(void *dst, const void *src, size_t bytes);       /* cudaMemcpy  :46      */
 int d8_memcpy_d2h(void *dst, const void *src, size_t bytes);       /* cudaMemcpy  :50      */
 int d8_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);  /* :40,:54     */
+/* value[i] = scalar for n elements.  Replaces ConstantKernel (deep8/src/math/Constant.cu:10-44),
+ * which Variable::zeroGradient / oneGradient use (deep8/src/nodes/Variable.cpp:119-130).   */
+int d8_fill(int dtype, void *ptr, size_t n, float scalar, void *stream);
 int d8_stream_create(void **stream);
 int d8_stream_destroy(void *stream);
 int d8_stream_sync(void *stream);

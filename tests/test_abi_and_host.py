@@ -1,0 +1,59 @@
+"""No-GPU checks of the boundary: the shared library loads and exports every symbol the header
+declares, the Python signature table covers them all, and the C++ host layer's device-free tests pass."""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST_TESTS = os.path.join(ROOT, "deep8_amd", "host", "deep8_host_tests")
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "deep8_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(d8_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    import ctypes
+    from deep8_amd import capi
+    names = _declared()
+    assert len(names) >= 40
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(capi.SIGNATURES) == names
+    capi.load()
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from deep8_amd import capi
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", os.path.join(ROOT, "deep8_amd", "no_such_library.so"))
+    with pytest.raises(capi.Deep8HipError):
+        capi.load()
+
+
+def test_product_never_imports_the_oracle():
+    """Nothing under deep8_amd/ or include/ may refer to the CPU checkers."""
+    for base, _, files in os.walk(os.path.join(ROOT, "deep8_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")) or f == "Makefile":
+                text = open(os.path.join(base, f), errors="ignore").read()
+                assert "oracle" not in text.lower(), os.path.join(base, f)
+
+
+def test_host_layer_device_free_tests():
+    assert os.path.exists(HOST_TESTS), "build the host layer first (__graft_entry__.build())"
+    out = subprocess.run([HOST_TESTS, "--cpu"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "PASS half_conversion" in out.stdout and "PASS node_shape_inference" in out.stdout
+    listed = subprocess.run([HOST_TESTS, "--list"], capture_output=True, text=True, timeout=60).stdout
+    assert "gpu matrix_multiply_float_collapsed_batch" in listed and "gpu eager_executor_matmul_chain" in listed
+
+
+def test_bench_refuses_more_than_one_gpu():
+    out = subprocess.run(["python", os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert out.returncode != 0 and "ONE GPU" in out.stderr

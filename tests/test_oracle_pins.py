@@ -1,0 +1,290 @@
+"""Pins of the CPU oracle (oracle/deep8_oracle.c).  No GPU.
+
+Every oracle function is fixed by something that is not a retyping of its own formula:
+  * golden vectors written by Deep8's own CPU (Eigen) build (tests/golden/deep8_cpu_reference.npz),
+  * the same library live, on integer inputs, when oracle/_ref is present,
+  * numpy / torch CPU routines (matmul, conv2d + autograd, conv_transpose2d),
+  * identities: adjointness of the gather maps, 1x1 conv == GEMM, outer product, accumulate twice.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from util import ints, nrm, rel_fro, rng, uni
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "deep8_cpu_reference.npz"))
+TOL = 2e-6  # oracle (double accumulation) vs Eigen (float accumulation) on O(10..100)-term sums
+
+
+def _n(prefix):
+    return sorted({int(k[len(prefix):].split("_")[0]) for k in GOLD.files if k.startswith(prefix) and k[len(prefix)].isdigit()})
+
+
+# ---- golden vectors -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("i", _n("mm"))
+def test_matmul_against_golden(oracle_port, i):
+    g = lambda k: GOLD["mm%d_%s" % (i, k)]
+    z = oracle_port.matmul(g("x"), g("y"))
+    assert z.shape == g("z").shape and rel_fro(z, g("z")) <= TOL
+    assert rel_fro(oracle_port.matmul_grad_x(g("x"), g("y"), g("dz"), g("dx0")), g("dx")) <= TOL
+    assert rel_fro(oracle_port.matmul_grad_y(g("x"), g("y"), g("dz"), g("dy0")), g("dy")) <= TOL
+
+
+@pytest.mark.parametrize("i", _n("conv"))
+def test_conv2d_against_golden(oracle_port, i):
+    g = lambda k: GOLD["conv%d_%s" % (i, k)]
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = (int(v) for v in g("cfg"))
+    a = (bool(cov), sy, sx, dy, dx)
+    z = oracle_port.conv2d(g("x"), g("w"), *a)
+    assert z.shape == g("z").shape and rel_fro(z, g("z")) <= TOL
+    assert rel_fro(oracle_port.conv2d_grad_x(g("x"), g("w"), g("gz"), *a, gx=g("gx0")), g("gx")) <= TOL
+    assert rel_fro(oracle_port.conv2d_grad_y(g("x"), g("w"), g("gz"), *a, gw=g("gw0")), g("gw")) <= TOL
+    # im2col == the patch matrix Eigen builds, bit for bit
+    OH, OW, pt, pl = oracle_port.conv2d_geometry(IH, IW, FH, FW, cov, sy, sx, dy, dx)
+    col = oracle_port.im2col(g("x"), OH, OW, FH, FW, sy, sx, dy, dx, pt, pl)
+    assert np.array_equal(col.view(np.uint32), g("patches").view(np.uint32))
+
+
+@pytest.mark.parametrize("i", _n("deconv"))
+def test_deconv2d_against_golden(oracle_port, i):
+    g = lambda k: GOLD["deconv%d_%s" % (i, k)]
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = (int(v) for v in g("cfg"))
+    a = (bool(cov), sy, sx)
+    z = oracle_port.deconv2d(g("x"), g("w"), *a)
+    assert z.shape == g("z").shape and rel_fro(z, g("z")) <= TOL
+    assert rel_fro(oracle_port.deconv2d_grad_x(g("x"), g("w"), g("gz"), *a, gx=g("gx0")), g("gx")) <= TOL
+    assert rel_fro(oracle_port.deconv2d_grad_y(g("x"), g("w"), g("gz"), *a, gw=g("gw0")), g("gw")) <= TOL
+    # deconv im2col is a pure permutation of the patches Eigen extracts from dz with the flipped filter:
+    # dzmat[r, oc*FH*FW + fy*FW + fx] == patches[r, ((FH-1-fy)*FW + (FW-1-fx))*OC + oc]
+    OH, OW, pt, pl = oracle_port.deconv2d_geometry(IH, IW, FH, FW, cov, sy, sx)
+    m = oracle_port.deconv_im2col(g("gz"), IH, IW, FH, FW, sy, sx, pt, pl).reshape(-1, OC, FH, FW)
+    p = g("gpatches").reshape(-1, FH, FW, OC)[:, ::-1, ::-1, :].transpose(0, 3, 1, 2)
+    assert np.array_equal(m.view(np.uint32), np.ascontiguousarray(p).view(np.uint32))
+
+
+# ---- the reference library, live -------------------------------------------------------------------------
+MM_SHAPES = [((10, 40, 20), (1, 20, 30)), ((1, 30, 10), (10, 10)), ((4, 8, 6), (4, 6, 5)), ((1, 8, 6), (4, 6, 5)),
+             ((4, 8, 6), (4, 6)), ((3, 17), (1, 1, 9))]
+
+
+@pytest.mark.parametrize("xs,ys", MM_SHAPES)
+def test_matmul_against_reference_live(oracle_port, oracle_ref, xs, ys):
+    r = rng(1)
+    x, y = ints(r, xs), ints(r, ys)
+    z = oracle_ref.matmul(x, y)
+    assert np.array_equal(oracle_port.matmul(x, y), z)
+    dz = ints(r, z.shape)
+    assert np.array_equal(oracle_port.matmul_grad_x(x, y, dz), oracle_ref.matmul_grad_x(x, y, dz))
+    assert np.array_equal(oracle_port.matmul_grad_y(x, y, dz), oracle_ref.matmul_grad_y(x, y, dz))
+
+
+@pytest.mark.parametrize("cov", [True, False])
+@pytest.mark.parametrize("s,d,F", [(1, 1, 3), (2, 2, 4), (2, 1, 3), (1, 2, 3), (3, 1, 5)])
+def test_conv2d_against_reference_live(oracle_port, oracle_ref, cov, s, d, F):
+    r = rng(2)
+    x, w = ints(r, (2, 17, 17, 5)), ints(r, (6, F, F, 5))
+    a = (cov, s, s, d, d)
+    z = oracle_ref.conv2d(x, w, *a)
+    assert np.array_equal(oracle_port.conv2d(x, w, *a), z)
+    gz = ints(r, z.shape)
+    assert np.array_equal(oracle_port.conv2d_grad_x(x, w, gz, *a), oracle_ref.conv2d_grad_x(x, w, gz, *a))
+    assert np.array_equal(oracle_port.conv2d_grad_y(x, w, gz, *a), oracle_ref.conv2d_grad_y(x, w, gz, *a))
+
+
+@pytest.mark.parametrize("cov", [True, False])
+@pytest.mark.parametrize("s,F", [(1, 3), (2, 4), (3, 4), (2, 3), (3, 2)])
+def test_deconv2d_against_reference_live(oracle_port, oracle_ref, cov, s, F):
+    r = rng(3)
+    x, w = ints(r, (2, 9, 9, 5)), ints(r, (6, F, F, 5))
+    a = (cov, s, s)
+    z = oracle_ref.deconv2d(x, w, *a)
+    assert np.array_equal(oracle_port.deconv2d(x, w, *a), z)
+    gz = ints(r, z.shape)
+    assert np.array_equal(oracle_port.deconv2d_grad_x(x, w, gz, *a), oracle_ref.deconv2d_grad_x(x, w, gz, *a))
+    assert np.array_equal(oracle_port.deconv2d_grad_y(x, w, gz, *a), oracle_ref.deconv2d_grad_y(x, w, gz, *a))
+
+
+def test_reference_rejects_bad_shapes(oracle_ref):
+    with pytest.raises(ValueError):
+        oracle_ref.matmul(np.zeros((1, 3, 4), np.float32), np.zeros((1, 4, 5), np.float32), z_shape=(1, 3, 6))
+
+
+# ---- numpy / torch -------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("xs,ys", MM_SHAPES)
+def test_matmul_against_numpy(oracle_port, xs, ys):
+    r = rng(4)
+    x, y = uni(r, xs), uni(r, ys)
+    x3 = x.astype(np.float64).reshape(xs[0], xs[1], xs[2] if len(xs) == 3 else 1)
+    y3 = y.astype(np.float64).reshape(ys[0], ys[1], ys[2] if len(ys) == 3 else 1)
+    zb = max(xs[0], ys[0])
+    X, Y = np.broadcast_to(x3, (zb,) + x3.shape[1:]), np.broadcast_to(y3, (zb,) + y3.shape[1:])
+    z = oracle_port.matmul(x, y)
+    want = np.matmul(X, Y)
+    assert rel_fro(z.reshape(want.shape), want) <= 1e-6
+    dz = uni(r, z.shape)
+    DZ = dz.astype(np.float64).reshape(want.shape)
+    dX = np.matmul(DZ, Y.transpose(0, 2, 1))
+    dY = np.matmul(X.transpose(0, 2, 1), DZ)
+    if xs[0] == 1:
+        dX = dX.sum(0, keepdims=True)
+    if ys[0] == 1:
+        dY = dY.sum(0, keepdims=True)
+    assert rel_fro(oracle_port.matmul_grad_x(x, y, dz).reshape(dX.shape), dX) <= 1e-6
+    assert rel_fro(oracle_port.matmul_grad_y(x, y, dz).reshape(dY.shape), dY) <= 1e-6
+
+
+CONV = [(2, 12, 12, 4, 5, 3, 3, True, 1, 1, 1, 1), (2, 13, 12, 3, 4, 4, 4, True, 2, 2, 2, 2),
+        (1, 11, 11, 3, 2, 3, 3, False, 2, 2, 1, 1), (1, 10, 9, 2, 3, 5, 3, True, 1, 2, 1, 1),
+        (2, 9, 9, 4, 4, 2, 2, True, 3, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("cfg", CONV)
+def test_conv2d_against_torch(oracle_port, cfg):
+    torch = pytest.importorskip("torch")
+    F = torch.nn.functional
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    r = rng(5)
+    x, w = nrm(r, (B, IH, IW, IC)), nrm(r, (OC, FH, FW, IC))
+    OH, OW, pt, pl = oracle_port.conv2d_geometry(IH, IW, FH, FW, cov, sy, sx, dy, dx)
+    rfh, rfw = FH + (FH - 1) * (dy - 1), FW + (FW - 1) * (dx - 1)
+    py, px = max(0, (OH - 1) * sy + rfh - IH), max(0, (OW - 1) * sx + rfw - IW)
+    tx = torch.tensor(x, dtype=torch.float64).permute(0, 3, 1, 2).requires_grad_(True)
+    tw = torch.tensor(w, dtype=torch.float64).permute(0, 3, 1, 2).requires_grad_(True)
+    tz = F.conv2d(F.pad(tx, (pl, px - pl, pt, py - pt)), tw, stride=(sy, sx), dilation=(dy, dx))
+    a = (cov, sy, sx, dy, dx)
+    z = oracle_port.conv2d(x, w, *a)
+    assert z.shape == (B, OH, OW, OC) == tuple(tz.permute(0, 2, 3, 1).shape)
+    assert rel_fro(z, tz.detach().permute(0, 2, 3, 1).numpy()) <= 1e-6
+    gz = nrm(r, z.shape)
+    tz.backward(torch.tensor(gz, dtype=torch.float64).permute(0, 3, 1, 2))
+    assert rel_fro(oracle_port.conv2d_grad_x(x, w, gz, *a), tx.grad.permute(0, 2, 3, 1).numpy()) <= 1e-6
+    assert rel_fro(oracle_port.conv2d_grad_y(x, w, gz, *a), tw.grad.permute(0, 2, 3, 1).numpy()) <= 1e-6
+
+
+DECONV = [(2, 5, 5, 3, 4, 4, 4, False, 2, 2), (2, 5, 5, 3, 4, 4, 4, True, 2, 2), (1, 6, 4, 2, 3, 3, 3, True, 3, 3),
+          (1, 4, 6, 2, 3, 4, 4, False, 3, 3), (2, 5, 5, 2, 2, 3, 3, False, 1, 1), (2, 5, 5, 2, 2, 4, 4, True, 1, 1)]
+
+
+@pytest.mark.parametrize("cfg", DECONV)
+def test_deconv2d_against_torch(oracle_port, cfg):
+    """Deep8's DeConv2d == conv_transpose2d with the spatially flipped filter, cropped at FH-1-padTop."""
+    torch = pytest.importorskip("torch")
+    F = torch.nn.functional
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = cfg
+    r = rng(6)
+    x, w = nrm(r, (B, IH, IW, IC)), nrm(r, (OC, FH, FW, IC))
+    OH, OW, pt, pl = oracle_port.deconv2d_geometry(IH, IW, FH, FW, cov, sy, sx)
+    tx = torch.tensor(x, dtype=torch.float64).permute(0, 3, 1, 2).requires_grad_(True)
+    tw = torch.tensor(w, dtype=torch.float64).requires_grad_(True)
+    wt = torch.flip(tw, (1, 2)).permute(3, 0, 1, 2)  # [IC, OC, FH, FW]
+    full = F.conv_transpose2d(tx, wt, stride=(sy, sx))
+    oy, ox = FH - 1 - pt, FW - 1 - pl
+    tz = full[:, :, oy:oy + OH, ox:ox + OW]
+    a = (cov, sy, sx)
+    z = oracle_port.deconv2d(x, w, *a)
+    assert z.shape == (B, OH, OW, OC) == tuple(tz.permute(0, 2, 3, 1).shape)
+    assert rel_fro(z, tz.detach().permute(0, 2, 3, 1).numpy()) <= 1e-6
+    gz = nrm(r, z.shape)
+    tz.backward(torch.tensor(gz, dtype=torch.float64).permute(0, 3, 1, 2))
+    assert rel_fro(oracle_port.deconv2d_grad_x(x, w, gz, *a), tx.grad.permute(0, 2, 3, 1).numpy()) <= 1e-6
+    assert rel_fro(oracle_port.deconv2d_grad_y(x, w, gz, *a), tw.grad.numpy()) <= 1e-6
+
+
+# ---- identities ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("cfg", CONV)
+def test_im2col_brute_force_and_adjoint(oracle_port, cfg):
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    OH, OW, pt, pl = oracle_port.conv2d_geometry(IH, IW, FH, FW, cov, sy, sx, dy, dx)
+    r = rng(7)
+    im = ints(r, (B, IH, IW, IC))
+    col = oracle_port.im2col(im, OH, OW, FH, FW, sy, sx, dy, dx, pt, pl)
+    # brute force through a zero-padded copy and numpy fancy indexing
+    big = np.zeros((B, IH + 2 * 64, IW + 2 * 64, IC), np.float32)
+    big[:, 64:64 + IH, 64:64 + IW] = im
+    want = np.empty((B, OH, OW, FH, FW, IC), np.float32)
+    for fy in range(FH):
+        for fx in range(FW):
+            ys = 64 - pt + fy * dy + sy * np.arange(OH)
+            xs = 64 - pl + fx * dx + sx * np.arange(OW)
+            want[:, :, :, fy, fx, :] = big[:, ys][:, :, xs]
+    assert np.array_equal(col, want.reshape(col.shape))
+    # <im2col(im), c> == <im, col2im(c)> exactly on integers
+    c = ints(r, col.shape, 10)
+    back = oracle_port.col2im(c, np.zeros_like(im), OH, OW, FH, FW, sy, sx, dy, dx, pt, pl)
+    assert float(np.sum(col.astype(np.float64) * c)) == float(np.sum(im.astype(np.float64) * back))
+    # col2im adds into its destination
+    twice = oracle_port.col2im(c, back, OH, OW, FH, FW, sy, sx, dy, dx, pt, pl)
+    assert np.array_equal(twice, 2 * back)
+
+
+@pytest.mark.parametrize("cfg", DECONV)
+def test_deconv_maps_adjoint(oracle_port, cfg):
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = cfg
+    OH, OW, pt, pl = oracle_port.deconv2d_geometry(IH, IW, FH, FW, cov, sy, sx)
+    r = rng(8)
+    zmat = ints(r, (B * IH * IW, OC * FH * FW), 10)
+    dz = ints(r, (B, OH, OW, OC), 10)
+    z = oracle_port.deconv_col2im(zmat, B, IH, IW, OH, OW, OC, FH, FW, sy, sx, pt, pl)
+    m = oracle_port.deconv_im2col(dz, IH, IW, FH, FW, sy, sx, pt, pl)
+    assert float(np.sum(z.astype(np.float64) * dz)) == float(np.sum(zmat.astype(np.float64) * m))
+
+
+@pytest.mark.parametrize("cfg", CONV)
+def test_conv2d_equals_im2col_gemm_col2im(oracle_port, cfg):
+    """The direct loops and the lowering the GPU path uses agree (integers: exactly)."""
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    OH, OW, pt, pl = oracle_port.conv2d_geometry(IH, IW, FH, FW, cov, sy, sx, dy, dx)
+    r = rng(9)
+    x, w, gz = ints(r, (B, IH, IW, IC), 20), ints(r, (OC, FH, FW, IC), 20), ints(r, (B, OH, OW, OC), 20)
+    a = (cov, sy, sx, dy, dx)
+    g = (OH, OW, FH, FW, sy, sx, dy, dx, pt, pl)
+    col = oracle_port.im2col(x, *g)
+    wm = w.reshape(OC, -1)
+    assert np.array_equal(oracle_port.gemm(0, 1, col, wm).reshape(B, OH, OW, OC), oracle_port.conv2d(x, w, *a))
+    dxcol = oracle_port.gemm(0, 0, gz.reshape(-1, OC), wm)
+    assert np.array_equal(oracle_port.col2im(dxcol, np.zeros_like(x), *g), oracle_port.conv2d_grad_x(x, w, gz, *a))
+    assert np.array_equal(oracle_port.gemm(1, 0, gz.reshape(-1, OC), col).reshape(w.shape),
+                          oracle_port.conv2d_grad_y(x, w, gz, *a))
+
+
+@pytest.mark.parametrize("cfg", DECONV)
+def test_deconv2d_equals_gemm_and_maps(oracle_port, cfg):
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = cfg
+    OH, OW, pt, pl = oracle_port.deconv2d_geometry(IH, IW, FH, FW, cov, sy, sx)
+    r = rng(10)
+    x, w, gz = ints(r, (B, IH, IW, IC), 20), ints(r, (OC, FH, FW, IC), 20), ints(r, (B, OH, OW, OC), 20)
+    a = (cov, sy, sx)
+    wm = w.reshape(OC * FH * FW, IC)
+    zmat = oracle_port.gemm(0, 1, x.reshape(-1, IC), wm)
+    assert np.array_equal(oracle_port.deconv_col2im(zmat, B, IH, IW, OH, OW, OC, FH, FW, sy, sx, pt, pl),
+                          oracle_port.deconv2d(x, w, *a))
+    dzmat = oracle_port.deconv_im2col(gz, IH, IW, FH, FW, sy, sx, pt, pl)
+    assert np.array_equal(oracle_port.gemm(0, 0, dzmat, wm).reshape(x.shape), oracle_port.deconv2d_grad_x(x, w, gz, *a))
+    assert np.array_equal(oracle_port.gemm(1, 0, dzmat, x.reshape(-1, IC)).reshape(w.shape),
+                          oracle_port.deconv2d_grad_y(x, w, gz, *a))
+
+
+def test_special_cases(oracle_port):
+    r = rng(11)
+    # 1x1 filter, stride 1: conv is a GEMM over pixels
+    x, w = ints(r, (2, 5, 6, 7)), ints(r, (3, 1, 1, 7))
+    assert np.array_equal(oracle_port.conv2d(x, w).reshape(-1, 3), x.reshape(-1, 7) @ w.reshape(3, 7).T)
+    # K = 1: outer product; identity operand
+    a, b = ints(r, (1, 9, 1)), ints(r, (1, 1, 4))
+    assert np.array_equal(oracle_port.matmul(a, b)[0], np.outer(a[0, :, 0], b[0, 0]))
+    m = ints(r, (1, 6, 6))
+    assert np.array_equal(oracle_port.matmul(m, np.eye(6, dtype=np.float32)[None]), m)
+    # gradients accumulate: running twice doubles
+    y, dz = ints(r, (1, 6, 5)), ints(r, (1, 6, 5))
+    once = oracle_port.matmul_grad_x(m, y, dz)
+    assert np.array_equal(oracle_port.matmul_grad_x(m, y, dz, once), 2 * once)
+    # stride >= filter: col2im never overlaps, every element is copied once
+    im = np.zeros((1, 6, 6, 2), np.float32)
+    col = ints(r, (9, 2 * 2 * 2)) + 1
+    out = oracle_port.col2im(col, im, 3, 3, 2, 2, 2, 2, 1, 1, 0, 0)
+    assert sorted(out.ravel()) == sorted(col.ravel())
+    # geometry of the BASELINE configs
+    assert oracle_port.conv2d_geometry(56, 56, 3, 3, True, 1, 1, 1, 1) == (56, 56, 1, 1)
+    assert oracle_port.deconv2d_geometry(28, 28, 4, 4, False, 2, 2) == (58, 58, 3, 3)
+    assert oracle_port.deconv2d_geometry(28, 28, 4, 4, True, 2, 2) == (55, 55, 1, 1)
