@@ -12,24 +12,9 @@
 //   accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32]
 // Both LDS tiles are kept K-contiguous ([row][k]), so one 16-byte LDS read feeds an MFMA
 // operand; the transposed-operand cases differ only in how the tile loader walks global memory.
-#include "common.h"
+#include "gemm_args.h"
 
 namespace d8 {
-
-struct GemmArgs {
-    const void *A;
-    const void *B;
-    void *C;
-    float *ws;
-    int M, N, K;
-    int lda, ldb, ldc;
-    long sA, sB, sC;
-    int batch;            // independent outputs
-    int red;              // products summed into each output (1 unless strideC == 0)
-    int splits;           // pieces the extended reduction (red x K tiles) is cut into
-    int tiles_per_split;  // K tiles per piece
-    float beta;
-};
 
 template <typename T>
 struct Tile;
@@ -218,6 +203,9 @@ static int plan_splits(int dtype, int M, int N, int K, int batch, int red, int *
 
 template <typename T>
 static int launch(GemmArgs &g, int transA, int transB, hipStream_t stream) {
+    int rc = 0;
+    if (sizeof(T) == 2 ? gemm_f16_tiled(g, transA, transB, stream, &rc) : gemm_f32_tiled(g, transA, transB, stream, &rc))
+        return rc;
     dim3 grid(ceil_div(g.N, 128), ceil_div(g.M, 128), g.batch * g.splits);
     if (!transA && !transB)
         hipLaunchKernelGGL((gemm_general_kernel<T, false, false>), grid, dim3(256), 0, stream, g);
