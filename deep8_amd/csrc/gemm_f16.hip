@@ -72,10 +72,13 @@ __device__ __host__ constexpr int slot_of(int t, int n, int MT) { return t * MT 
 
 // One K step.  Ar/Br: this lane's operand addresses in the LDS half being multiplied; An/Bn: the
 // same in the other half (next step); Aw/Bw: where this thread's pieces of the next step go;
-// pa/pb: where its pieces of the step after that come from.
+// ra/rb: buffer descriptors of the A and B matrices; ga/gb: wave-uniform byte offset (tile origin +
+// K step) of the pieces of the step after that, a_off/b_off: this thread's byte offset in a piece.
+// Uniform parts stay in scalar registers, so a piece costs one address VGPR per operand.
 template <typename T>
 __device__ __forceinline__ void k_step(const f16 *Ar, const f16 *Br, const f16 *An, const f16 *Bn, f16 *Aw, f16 *Bw,
-                                       const f16 *pa, const f16 *pb, long a_pass, long b_pass,
+                                       __amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb, unsigned ga, unsigned gb,
+                                       unsigned a_pass, unsigned b_pass, unsigned a_off, unsigned b_off,
                                        u32x4 (&R)[T::NP], f16x8 (&fa)[2][T::TM], f16x8 (&fb)[2][T::TN],
                                        f32x16 (&acc)[T::TM][T::TN]) {
     constexpr int TM = T::TM, TN = T::TN, MT = T::MT, NP = T::NP, A_IT = T::A_IT, NF = TM + TN;
@@ -99,7 +102,8 @@ __device__ __forceinline__ void k_step(const f16 *Ar, const f16 *Br, const f16 *
             for (int t = 0; t < g_n; ++t)
                 if (slot_of(t, g_n, MT) == m) {
                     const int p = g_lo + t;
-                    R[p] = *(const u32x4 *)(p < A_IT ? pa + p * a_pass : pb + (p - A_IT) * b_pass);
+                    R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, ga + p * a_pass, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, gb + (p - A_IT) * b_pass, 0);
                 }
             // operands of the next quarter (of the next step's first quarter when q == 3)
 #pragma unroll
@@ -165,20 +169,26 @@ __global__ __launch_bounds__(T::NT) void gemm_f16_tiled_kernel(GemmArgs g, int t
     const int m_own = tm * BM, n_own = tn * BN;
     const int m0 = min(m_own, g.M - BM), n0 = min(n_own, g.N - BN);
 
-    const int b = blockIdx.z;
-    const f16 *Ag = (const f16 *)g.A + (long)b * g.sA;
-    const f16 *Bg = (const f16 *)g.B + (long)b * g.sB;
-
     // ---- the 16-byte pieces this thread moves each K step: piece `it` of an operand lies a fixed
-    // number of rows below piece 0, in global memory and in LDS alike
+    // number of rows below piece 0, in global memory and in LDS alike.  Global memory is read
+    // through buffer descriptors: byte offset = uniform part (tile origin, K step, piece; scalar
+    // registers) + per-thread part (one VGPR per operand).
+    const int b = blockIdx.z;
+    const long a_rows = A_KC ? g.M : g.K, b_rows = B_KC ? g.N : g.K;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const f16 *)g.A + (long)b * g.sA), 0, (int)(2 * a_rows * g.lda), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const f16 *)g.B + (long)b * g.sB), 0, (int)(2 * b_rows * g.ldb), 0x00020000);
+    const unsigned Au = 2u * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0);
+    const unsigned Bu = 2u * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
     const int a_r = A_KC ? tid >> 3 : tid / (BM / 8), a_c = A_KC ? tid & 7 : tid % (BM / 8);
     const int b_r = B_KC ? tid >> 3 : tid / (BN / 8), b_c = B_KC ? tid & 7 : tid % (BN / 8);
-    const f16 *a_src = A_KC ? Ag + (long)(m0 + a_r) * g.lda + a_c * 8 : Ag + (long)a_r * g.lda + m0 + a_c * 8;
-    const f16 *b_src = B_KC ? Bg + (long)(n0 + b_r) * g.ldb + b_c * 8 : Bg + (long)b_r * g.ldb + n0 + b_c * 8;
+    const unsigned a_off = 2u * ((unsigned)a_r * (unsigned)g.lda + a_c * 8);
+    const unsigned b_off = 2u * ((unsigned)b_r * (unsigned)g.ldb + b_c * 8);
     const int a_dst = a_r * A_LD + a_c * 8, b_dst = b_r * B_LD + b_c * 8;
-    const long a_pass = (long)T::A_ROWS * g.lda, b_pass = (long)T::B_ROWS * g.ldb;
-    const long a_step = A_KC ? BK : (long)BK * g.lda;
-    const long b_step = B_KC ? BK : (long)BK * g.ldb;
+    const unsigned a_pass = 2u * T::A_ROWS * g.lda, b_pass = 2u * T::B_ROWS * g.ldb;  // bytes
+    const unsigned a_step = A_KC ? 2u * BK : 2u * BK * g.lda;
+    const unsigned b_step = B_KC ? 2u * BK : 2u * BK * g.ldb;
 
     // ---- per-lane LDS offsets of its MFMA operands
     const int a_frag = A_KC ? (wm * TM * 32 + l32) * A_LD + kg
@@ -199,15 +209,19 @@ __global__ __launch_bounds__(T::NT) void gemm_f16_tiled_kernel(GemmArgs g, int t
     // ---- prologue: step 0 into LDS half 0, step 1 into registers, first operands of step 0
     const int ktiles = g.K / BK;
 #pragma unroll
-    for (int p = 0; p < NP; ++p) R[p] = *(const u32x4 *)(p < A_IT ? a_src + p * a_pass : b_src + (p - A_IT) * b_pass);
+    for (int p = 0; p < NP; ++p)
+        R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, Au + p * a_pass, 0)
+                        : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, Bu + (p - A_IT) * b_pass, 0);
 #pragma unroll
     for (int p = 0; p < NP; ++p)
         *(u32x4 *)(p < A_IT ? As0 + a_dst + p * T::A_ROWS * A_LD : Bs0 + b_dst + (p - A_IT) * T::B_ROWS * B_LD) = R[p];
     {
         const int t1 = min(1, ktiles - 1);
-        const f16 *pa = a_src + t1 * a_step, *pb = b_src + t1 * b_step;
+        const unsigned pa = Au + t1 * a_step, pb = Bu + t1 * b_step;
 #pragma unroll
-        for (int p = 0; p < NP; ++p) R[p] = *(const u32x4 *)(p < A_IT ? pa + p * a_pass : pb + (p - A_IT) * b_pass);
+        for (int p = 0; p < NP; ++p)
+            R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, pa + p * a_pass, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, pb + (p - A_IT) * b_pass, 0);
     }
     __syncthreads();
 #pragma unroll
@@ -223,12 +237,12 @@ __global__ __launch_bounds__(T::NT) void gemm_f16_tiled_kernel(GemmArgs g, int t
         {
             const int t2 = min(kt + 2, ktiles - 1);
             k_step<T>(As0 + a_frag, Bs0 + b_frag, As1 + a_frag, Bs1 + b_frag, As1 + a_dst, Bs1 + b_dst,
-                      a_src + t2 * a_step, b_src + t2 * b_step, a_pass, b_pass, R, fa, fb, acc);
+                      ra, rb, Au + t2 * a_step, Bu + t2 * b_step, a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
         }
         if (kt + 1 < ktiles) {
             const int t3 = min(kt + 3, ktiles - 1);
             k_step<T>(As1 + a_frag, Bs1 + b_frag, As0 + a_frag, Bs0 + b_frag, As0 + a_dst, Bs0 + b_dst,
-                      a_src + t3 * a_step, b_src + t3 * b_step, a_pass, b_pass, R, fa, fb, acc);
+                      ra, rb, Au + t3 * a_step, Bu + t3 * b_step, a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
         }
     }
 
@@ -270,6 +284,7 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     if (force && g.M >= 256 && g.N >= 256) {
         switch (atoi(force)) {
         case 2: return launch_tiled<256, 256, 2, 4, A_KC, B_KC>(g, stream);
+        case 4: return launch_tiled<256, 256, 2, 2, A_KC, B_KC>(g, stream);
         case 128: big = false; break;
         default: big = true;
         }
@@ -280,6 +295,8 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
 
 bool gemm_f16_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc) {
     if (g.red != 1 || g.splits != 1) return false;
+    // byte offsets inside one matrix are 32-bit
+    if ((long)(transA ? g.K : g.M) * g.lda >= (1L << 30) || (long)(transB ? g.N : g.K) * g.ldb >= (1L << 30)) return false;
     if (g.M < 128 || g.N < 128 || g.K < 64 || g.K % 64 || g.lda % 8 || g.ldb % 8 || g.sA % 8 || g.sB % 8) return false;
     if (((size_t)g.A | (size_t)g.B) & 15) return false;
     if (transA && g.M % 8) return false;
