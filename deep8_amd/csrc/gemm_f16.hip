@@ -246,9 +246,51 @@ __global__ __launch_bounds__(T::NT) void gemm_f16_tiled_kernel(GemmArgs g, int t
         }
     }
 
-    // ---- epilogue: lane holds column l32 of rows 8*(r/4) + 4*(lane/32) + r%4 of each 32x32 block
+    // ---- epilogue.  Lane holds column l32 of rows 8*(r/4) + 4*(lane/32) + r%4 of each 32x32 block.
     f16 *Cg = (f16 *)g.C + (long)b * g.sC;
     const int lhi = lane >> 5;
+    const bool vector_ok = (g.ldc % 8 == 0) && (g.sC % 8 == 0) && (((size_t)g.C & 15) == 0) && (g.N % 8 == 0);
+    if (vector_ok) {
+        // Each wave turns one 32x32 block at a time around through its own 32 x 36 float patch of
+        // LDS (the A half is free once every wave is past the last step), so that a lane ends up
+        // with 8 consecutive columns of one row: 16-byte loads of the old C and 16-byte stores.
+        static_assert((size_t)T::A_SZ * sizeof(f16) >= (size_t)T::NT / 64 * 32 * 36 * sizeof(float), "patch space");
+        __syncthreads();
+        float *patch = (float *)As0 + wave * (32 * 36);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) patch[((r >> 2) * 8 + lhi * 4 + (r & 3)) * 36 + l32] = acc[i][j][r];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int q = lane + 64 * t, row = q >> 2, cc = (q & 3) * 8;
+                    const int m = m0 + (wm * TM + i) * 32 + row, n = n0 + (wn * TN + j) * 32 + cc;
+                    const f32x4 lo = *(const f32x4 *)(patch + row * 36 + cc), hi = *(const f32x4 *)(patch + row * 36 + cc + 4);
+                    if (m >= m_own && n >= n_own) {
+                        f16 *c = Cg + (long)m * g.ldc + n;
+                        f16x8 o;
+                        if (g.beta != 0.f) {
+                            const f16x8 old = *(const f16x8 *)c;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                o[e] = (f16)(lo[e] + (float)old[e]);
+                                o[e + 4] = (f16)(hi[e] + (float)old[e + 4]);
+                            }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                o[e] = (f16)lo[e];
+                                o[e + 4] = (f16)hi[e];
+                            }
+                        }
+                        *(f16x8 *)c = o;
+                    }
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll

@@ -49,6 +49,26 @@ def test_gemm_f16_integer_exact(oracle_port, ta, tb, M, N, K):
 
 
 @pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("M,N,K", [(300, 264, 128), (136, 130, 64), (512, 520, 256), (1000, 392, 192), (304, 261, 128),
+                                   (256, 256, 64), (768, 1280, 448)])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_gemm_tiled_kernels_edge_tiles(oracle_port, ta, tb, M, N, K, dtype):
+    """Shapes that take the tiled kernels (K a multiple of 64, rows movable in 16-byte pieces) with
+    ragged last tiles in M and N: edge tiles are shifted inwards and must not double-accumulate."""
+    from deep8_amd import ops
+    r = rng(M + 3 * N + 7 * K)
+    hi = 3 if dtype == np.float16 else 50
+    A, B = _ab(r, ta, tb, M, N, K, lambda r, s: ints(r, s, hi))
+    C0 = ints(r, (M, N), hi)
+    c = (lambda a: h(a)) if dtype == np.float16 else (lambda a: a)
+    for beta, C in ((0.0, None), (1.0, C0)):
+        want = oracle_port.gemm(ta, tb, A, B, C, beta)
+        assert want.max() < 2048 or dtype == np.float32
+        got = ops.gemm(ta, tb, c(A), c(B), None if C is None else c(C), beta)
+        assert np.array_equal(f(got), want), (ta, tb, M, N, K, beta)
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
 @pytest.mark.parametrize("M,N,K", [(64, 256, 128), (257, 129, 65), (512, 512, 512), (96, 80, 4099)])
 def test_gemm_real_tolerance(oracle_port, ta, tb, M, N, K):
     from deep8_amd import ops
