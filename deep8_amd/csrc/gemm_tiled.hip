@@ -1,0 +1,425 @@
+// Tiled GEMM for gfx950, fp16 (v_mfma_f32_32x32x16_f16, fp32 accumulation) and fp32
+// (v_mfma_f32_32x32x2_f32, true fp32 operands).
+//
+// A workgroup owns a BM x BN tile of C and walks K in steps of 128 bytes of a row (64 halfs or
+// 32 floats).  While step t is multiplied out of one half of a double-buffered LDS area, the A
+// and B tiles of step t+1 are written from registers into the other half and the tiles of step
+// t+2 are fetched from global memory into those registers with 16-byte buffer loads (uniform
+// address part in scalar registers, one offset VGPR per operand).  The loop body is written, and
+// pinned with scheduling barriers, in issue order: every MFMA is followed by at most one LDS
+// write, one global load and a couple of LDS reads, so the matrix pipe never waits behind a burst
+// of memory instructions.  The one workgroup barrier per step sits before the last quarter of the
+// step's MFMAs, which then cover the latency of the first operand reads of the next step.
+//
+// Both tiles keep in LDS the layout they have in memory; the transposed-operand products differ
+// only in how the tiles are read back:
+//   * an operand contiguous along K is stored [row][k]; one 16-byte LDS read gives a lane the 8
+//     halfs (4 floats) of its row that it feeds to the next MFMA(s);
+//   * an operand contiguous along M (A of a TN product) or N (B of an NN / TN product) is stored
+//     [k][row]; fp16 reads it back with ds_read_b64_tr_b16, the transposing LDS read, which hands
+//     each lane four consecutive-k values of its row; fp32 reads one float per k, consecutive
+//     lanes reading consecutive addresses.  No transpose is ever materialised.
+// Any pairing of k values with lanes works as long as A and B use the same one, because the MFMA
+// sums over k; both element types pair lanes 0-31 with the first half of a k group and lanes
+// 32-63 with the second half.
+//
+// Workgroup ids are remapped so that the workgroups one XCD receives (ids congruent mod 8) cover
+// a compact block of tiles and share A / B panels in that XCD's L2.  The epilogue turns each
+// 32 x 32 accumulator block around through LDS so that C is read and written 16 bytes per lane.
+#include "gemm_args.h"
+
+namespace d8 {
+
+typedef __fp16 f16x4v __attribute__((ext_vector_type(4)));
+typedef __fp16 f16x8v __attribute__((ext_vector_type(8)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T *)(p))
+
+// instruction classes of __builtin_amdgcn_sched_group_barrier
+#define SG_MFMA 0x008
+#define SG_VMEM_READ 0x020
+#define SG_DS_READ 0x100
+#define SG_DS_WRITE 0x200
+
+// ---- per element type: operand fragments and how to multiply one k group --------------------
+template <typename E>
+struct Elem;
+
+template <>
+struct Elem<f16> {
+    typedef f16x8 Frag;                      // 8 k values of one row
+    static constexpr int KG = 16;            // k values one fragment pair covers (2 lane halves x 8)
+    static constexpr int MFMA_PER_FRAG = 1;  // MFMAs that consume one fragment pair
+    static constexpr int TR_READS = 2;       // LDS instructions per fragment in the [k][row] layout
+    static constexpr int TR_PAD = 64;        // bytes added to a [k][row] row: its 4 k-rows x 64 B hit different banks
+    // lane's element offset inside a [row][k] tile (row r0 + lane%32, its half of the k group)
+    __device__ static int kc_offset(int lane, int ld, int row0) { return (row0 + (lane & 31)) * ld + (lane >> 5) * 8; }
+    // ... and inside a [k][row] tile: the lane whose index within its group of 16 is i addresses
+    // k-row (i / 4), columns 4 * (i % 4) .. + 3 of its 16-column group, and receives column i
+    __device__ static int tr_offset(int lane, int ld, int row0) {
+        return ((lane >> 5) * 8 + ((lane & 15) >> 2)) * ld + row0 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    }
+    __device__ static Frag read_kc(const f16 *p) { return *(const f16x8 *)p; }
+    __device__ static Frag read_tr(const f16 *p, int ld) {
+        const f16x4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16(LDS_PTR(f16x4v, p));
+        const f16x4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4f16(LDS_PTR(f16x4v, p + 4 * ld));
+        const f16x8v both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(f16x8, both);
+    }
+    __device__ static f32x16 mfma(const Frag &a, const Frag &b, const f32x16 &c, int) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <>
+struct Elem<float> {
+    typedef f32x4 Frag;  // lanes 0-31: k 0..3 of the group of 8, lanes 32-63: k 4..7
+    static constexpr int KG = 8;
+    static constexpr int MFMA_PER_FRAG = 4;  // MFMA e pairs k = e with k = 4 + e
+    static constexpr int TR_READS = 4;
+    static constexpr int TR_PAD = 160;  // rows 4 apart (the two lane halves) land in different bank halves
+    __device__ static int kc_offset(int lane, int ld, int row0) { return (row0 + (lane & 31)) * ld + (lane >> 5) * 4; }
+    __device__ static int tr_offset(int lane, int ld, int row0) { return (lane >> 5) * 4 * ld + row0 + (lane & 31); }
+    __device__ static Frag read_kc(const float *p) { return *(const f32x4 *)p; }
+    __device__ static Frag read_tr(const float *p, int ld) {
+        Frag v;
+        v[0] = p[0];
+        v[1] = p[ld];
+        v[2] = p[2 * ld];
+        v[3] = p[3 * ld];
+        return v;
+    }
+    __device__ static f32x16 mfma(const Frag &a, const Frag &b, const f32x16 &c, int e) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+    }
+};
+
+template <typename E_, int BM_, int BN_, int WGM_, int WGN_, bool A_KC_, bool B_KC_>
+struct Tile {
+    typedef E_ E;
+    typedef Elem<E> EL;
+    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
+    static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
+    static constexpr int ES = sizeof(E), EPV = 16 / ES;  // element size, elements per 16-byte piece
+    static constexpr int BK = 128 / ES;                  // K step: 128 bytes of a row
+    static constexpr int QUARTERS = 4, KQ = BK / QUARTERS;
+    static_assert(KQ == EL::KG, "a quarter step is one k group");
+    static constexpr int NT = WGM * WGN * 64;
+    static constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32;
+    static constexpr int MQ = TM * TN * EL::MFMA_PER_FRAG;  // MFMAs per quarter step
+    // leading dimensions in elements: [row][k] rows get 16 bytes of padding so that consecutive
+    // rows start in different banks
+    static constexpr int A_LD = A_KC ? BK + EPV : BM + EL::TR_PAD / ES;
+    static constexpr int B_LD = B_KC ? BK + EPV : BN + EL::TR_PAD / ES;
+    static constexpr int A_SZ = A_KC ? BM * A_LD : BK * A_LD;
+    static constexpr int B_SZ = B_KC ? BN * B_LD : BK * B_LD;
+    // 16-byte pieces each thread moves per K step, and the rows one pass of all threads covers
+    static constexpr int A_IT = BM * 8 / NT, B_IT = BN * 8 / NT, NP = A_IT + B_IT;
+    static constexpr int A_ROWS = A_KC ? NT / 8 : NT / (BM / EPV);
+    static constexpr int B_ROWS = B_KC ? NT / 8 : NT / (BN / EPV);
+    static constexpr int A_RD = A_KC ? 1 : EL::TR_READS, B_RD = B_KC ? 1 : EL::TR_READS;
+};
+
+// Pieces [lo(q), lo(q+1)) are written to LDS during quarter q = 0, 1, 2 of a step and re-fetched
+// from global memory during quarter q + 1.
+template <int NP>
+__device__ __host__ constexpr int piece_lo(int q) { return q * NP / 3; }
+// The t-th of n events of a quarter goes right after MFMA number (t * MQ) / n.
+__device__ __host__ constexpr int slot_of(int t, int n, int MQ) { return t * MQ / n; }
+
+// One K step.  Ar/Br: this lane's operand addresses in the LDS half being multiplied; An/Bn: the
+// same in the other half (next step); Aw/Bw: where this thread's pieces of the next step go;
+// ra/rb: buffer descriptors of the A and B matrices; ga/gb: wave-uniform byte offset (tile origin +
+// K step) of the pieces of the step after that, a_off/b_off: this thread's byte offset in a piece.
+template <typename T>
+__device__ __forceinline__ void k_step(const typename T::E *Ar, const typename T::E *Br, const typename T::E *An,
+                                       const typename T::E *Bn, typename T::E *Aw, typename T::E *Bw,
+                                       __amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb, unsigned ga, unsigned gb,
+                                       unsigned a_pass, unsigned b_pass, unsigned a_off, unsigned b_off,
+                                       u32x4 (&R)[T::NP], typename T::EL::Frag (&fa)[2][T::TM],
+                                       typename T::EL::Frag (&fb)[2][T::TN], f32x16 (&acc)[T::TM][T::TN]) {
+    typedef typename T::E E;
+    typedef typename T::EL EL;
+    constexpr int TM = T::TM, TN = T::TN, MQ = T::MQ, NP = T::NP, A_IT = T::A_IT, NF = TM + TN;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        if (q == 3) __syncthreads();  // every wave has written its pieces and finished reading this half
+        const int w_lo = q < 3 ? piece_lo<NP>(q) : 0, w_n = q < 3 ? piece_lo<NP>(q + 1) - w_lo : 0;
+        const int g_lo = q > 0 ? piece_lo<NP>(q - 1) : 0, g_n = q > 0 ? piece_lo<NP>(q) - g_lo : 0;
+#pragma unroll
+        for (int m = 0; m < MQ; ++m) {
+            {
+                const int e = m / (TM * TN), ij = m % (TM * TN), i = ij / TN, j = ij % TN;
+                acc[i][j] = EL::mfma(fa[q & 1][i], fb[q & 1][j], acc[i][j], e);
+            }
+#pragma unroll
+            for (int t = 0; t < w_n; ++t)
+                if (slot_of(t, w_n, MQ) == m) {
+                    const int p = w_lo + t;
+                    E *dst = p < A_IT ? Aw + p * T::A_ROWS * T::A_LD : Bw + (p - A_IT) * T::B_ROWS * T::B_LD;
+                    *(u32x4 *)dst = R[p];
+                }
+#pragma unroll
+            for (int t = 0; t < g_n; ++t)
+                if (slot_of(t, g_n, MQ) == m) {
+                    const int p = g_lo + t;
+                    R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, ga + p * a_pass, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, gb + (p - A_IT) * b_pass, 0);
+                }
+            // operands of the next quarter (of the next step's first quarter when q == 3)
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+                if (slot_of(f, NF, MQ) == m) {
+                    const int kk = q < 3 ? (q + 1) * T::KQ : 0;
+                    const E *a_base = q < 3 ? Ar : An, *b_base = q < 3 ? Br : Bn;
+                    if (f < TM)
+                        fa[(q + 1) & 1][f] = T::A_KC ? EL::read_kc(a_base + f * 32 * T::A_LD + kk)
+                                                     : EL::read_tr(a_base + kk * T::A_LD + f * 32, T::A_LD);
+                    else
+                        fb[(q + 1) & 1][f - TM] = T::B_KC ? EL::read_kc(b_base + (f - TM) * 32 * T::B_LD + kk)
+                                                          : EL::read_tr(b_base + kk * T::B_LD + (f - TM) * 32, T::B_LD);
+                }
+        }
+        // pin the issue order to the program order above
+#pragma unroll
+        for (int m = 0; m < MQ; ++m) {
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+#pragma unroll
+            for (int t = 0; t < w_n; ++t)
+                if (slot_of(t, w_n, MQ) == m) __builtin_amdgcn_sched_group_barrier(SG_DS_WRITE, 1, 0);
+#pragma unroll
+            for (int t = 0; t < g_n; ++t)
+                if (slot_of(t, g_n, MQ) == m) __builtin_amdgcn_sched_group_barrier(SG_VMEM_READ, 1, 0);
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+                if (slot_of(f, NF, MQ) == m) {
+                    if (f < TM) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, T::A_RD, 0);
+                    else __builtin_amdgcn_sched_group_barrier(SG_DS_READ, T::B_RD, 0);
+                }
+        }
+    }
+}
+
+__device__ inline float as_f32(float v) { return v; }
+__device__ inline float as_f32(f16 v) { return (float)v; }
+
+template <typename T>
+__global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tilesM, int tilesN) {
+    typedef typename T::E E;
+    typedef typename T::EL EL;
+    typedef E EV __attribute__((ext_vector_type(T::EPV)));
+    constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN, A_LD = T::A_LD, B_LD = T::B_LD;
+    constexpr int A_IT = T::A_IT, NP = T::NP, ES = T::ES, EPV = T::EPV;
+    constexpr bool A_KC = T::A_KC, B_KC = T::B_KC;
+    // four separate arrays, so that reads of one half are known not to touch the other
+    __shared__ __attribute__((aligned(16))) E As0[T::A_SZ];
+    __shared__ __attribute__((aligned(16))) E As1[T::A_SZ];
+    __shared__ __attribute__((aligned(16))) E Bs0[T::B_SZ];
+    __shared__ __attribute__((aligned(16))) E Bs1[T::B_SZ];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / T::WGN, wn = wave % T::WGN;
+
+    // ---- which tile: ids of one XCD (same id mod 8) form a contiguous run, runs are laid out in
+    // bands of GM tile rows walked column by column
+    int id = blockIdx.x;
+    const int total = tilesM * tilesN;
+    if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    constexpr int GM = 4;
+    const int band = id / (GM * tilesN), first = band * GM;
+    const int rows_in_band = min(GM, tilesM - first);
+    const int in_band = id - band * GM * tilesN;
+    const int tm = first + in_band % rows_in_band, tn = in_band / rows_in_band;
+    // A tile that would stick out of the matrix is moved back inside; the rows / columns it then
+    // shares with its neighbour are computed twice but stored only by the neighbour.
+    const int m_own = tm * BM, n_own = tn * BN;
+    const int m0 = min(m_own, g.M - BM), n0 = min(n_own, g.N - BN);
+
+    // ---- the 16-byte pieces this thread moves each K step: piece `it` of an operand lies a fixed
+    // number of rows below piece 0, in global memory and in LDS alike.  Global memory is read
+    // through buffer descriptors: byte offset = uniform part (tile origin, K step, piece; scalar
+    // registers) + per-thread part (one VGPR per operand).
+    const int b = blockIdx.z;
+    const long a_rows = A_KC ? g.M : g.K, b_rows = B_KC ? g.N : g.K;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const E *)g.A + (long)b * g.sA), 0, (int)(ES * a_rows * g.lda), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const E *)g.B + (long)b * g.sB), 0, (int)(ES * b_rows * g.ldb), 0x00020000);
+    const unsigned Au = (unsigned)ES * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0);
+    const unsigned Bu = (unsigned)ES * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
+    const int a_r = A_KC ? tid >> 3 : tid / (BM / EPV), a_c = A_KC ? tid & 7 : tid % (BM / EPV);
+    const int b_r = B_KC ? tid >> 3 : tid / (BN / EPV), b_c = B_KC ? tid & 7 : tid % (BN / EPV);
+    const unsigned a_off = (unsigned)ES * ((unsigned)a_r * (unsigned)g.lda + a_c * EPV);
+    const unsigned b_off = (unsigned)ES * ((unsigned)b_r * (unsigned)g.ldb + b_c * EPV);
+    const int a_dst = a_r * A_LD + a_c * EPV, b_dst = b_r * B_LD + b_c * EPV;
+    const unsigned a_pass = (unsigned)ES * T::A_ROWS * g.lda, b_pass = (unsigned)ES * T::B_ROWS * g.ldb;  // bytes
+    const unsigned a_step = A_KC ? 128u : (unsigned)ES * BK * g.lda;
+    const unsigned b_step = B_KC ? 128u : (unsigned)ES * BK * g.ldb;
+
+    // ---- per-lane LDS offsets of its MFMA operands
+    const int a_frag = A_KC ? EL::kc_offset(lane, A_LD, wm * TM * 32) : EL::tr_offset(lane, A_LD, wm * TM * 32);
+    const int b_frag = B_KC ? EL::kc_offset(lane, B_LD, wn * TN * 32) : EL::tr_offset(lane, B_LD, wn * TN * 32);
+
+    u32x4 R[NP];
+    typename EL::Frag fa[2][TM], fb[2][TN];
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // ---- prologue: step 0 into LDS half 0, step 1 into registers, first operands of step 0
+    const int ktiles = g.K / BK;
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+        R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, Au + p * a_pass, 0)
+                        : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, Bu + (p - A_IT) * b_pass, 0);
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+        *(u32x4 *)(p < A_IT ? As0 + a_dst + p * T::A_ROWS * A_LD : Bs0 + b_dst + (p - A_IT) * T::B_ROWS * B_LD) = R[p];
+    {
+        const int t1 = min(1, ktiles - 1);
+        const unsigned pa = Au + t1 * a_step, pb = Bu + t1 * b_step;
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+            R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, pa + p * a_pass, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, pb + (p - A_IT) * b_pass, 0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+        fa[0][i] = A_KC ? EL::read_kc(As0 + a_frag + i * 32 * A_LD) : EL::read_tr(As0 + a_frag + i * 32, A_LD);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+        fb[0][j] = B_KC ? EL::read_kc(Bs0 + b_frag + j * 32 * B_LD) : EL::read_tr(Bs0 + b_frag + j * 32, B_LD);
+
+    // ---- main loop, two steps per trip so that the LDS half of every access is known statically;
+    // fetches past the last step re-read the last step and are never used
+    for (int kt = 0; kt < ktiles; kt += 2) {
+        {
+            const int t2 = min(kt + 2, ktiles - 1);
+            k_step<T>(As0 + a_frag, Bs0 + b_frag, As1 + a_frag, Bs1 + b_frag, As1 + a_dst, Bs1 + b_dst, ra, rb,
+                      Au + t2 * a_step, Bu + t2 * b_step, a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
+        }
+        if (kt + 1 < ktiles) {
+            const int t3 = min(kt + 3, ktiles - 1);
+            k_step<T>(As1 + a_frag, Bs1 + b_frag, As0 + a_frag, Bs0 + b_frag, As0 + a_dst, Bs0 + b_dst, ra, rb,
+                      Au + t3 * a_step, Bu + t3 * b_step, a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
+        }
+    }
+
+    // ---- epilogue.  Lane holds column lane%32 of rows 8*(r/4) + 4*(lane/32) + r%4 of each 32x32 block.
+    E *Cg = (E *)g.C + (long)b * g.sC;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const bool vector_ok = (g.ldc % EPV == 0) && (g.sC % EPV == 0) && (((size_t)g.C & 15) == 0) && (g.N % 8 == 0);
+    if (vector_ok) {
+        // Each wave turns one 32x32 block at a time around through its own 32 x 36 float patch of
+        // LDS (the A half is free once every wave is past the last step), so that a lane ends up
+        // with 8 consecutive columns of one row: 16-byte loads of the old C and 16-byte stores.
+        static_assert((size_t)T::A_SZ * ES >= (size_t)T::NT / 64 * 32 * 36 * sizeof(float), "patch space");
+        __syncthreads();
+        float *patch = (float *)As0 + wave * (32 * 36);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) patch[((r >> 2) * 8 + lhi * 4 + (r & 3)) * 36 + l32] = acc[i][j][r];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int q = lane + 64 * t, row = q >> 2, cc = (q & 3) * 8;
+                    const int m = m0 + (wm * TM + i) * 32 + row, n = n0 + (wn * TN + j) * 32 + cc;
+                    float v[8];
+                    *(f32x4 *)&v[0] = *(const f32x4 *)(patch + row * 36 + cc);
+                    *(f32x4 *)&v[4] = *(const f32x4 *)(patch + row * 36 + cc + 4);
+                    if (m >= m_own && n >= n_own) {
+                        E *c = Cg + (long)m * g.ldc + n;
+#pragma unroll
+                        for (int h = 0; h < 8 / EPV; ++h) {
+                            EV o;
+                            if (g.beta != 0.f) {
+                                const EV old = *(const EV *)(c + h * EPV);
+#pragma unroll
+                                for (int e = 0; e < EPV; ++e) o[e] = (E)(v[h * EPV + e] + as_f32(old[e]));
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < EPV; ++e) o[e] = (E)v[h * EPV + e];
+                            }
+                            *(EV *)(c + h * EPV) = o;
+                        }
+                    }
+                }
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + (wn * TN + j) * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + (wm * TM + i) * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+                if (m >= m_own && n >= n_own) {
+                    E *c = Cg + (long)m * g.ldc + n;
+                    float v = acc[i][j][r];
+                    if (g.beta != 0.f) v += as_f32(*c);
+                    *c = (E)v;
+                }
+            }
+        }
+}
+
+template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC>
+static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
+    typedef Tile<E, BM, BN, WGM, WGN, A_KC, B_KC> T;
+    const int tilesM = ceil_div(g.M, BM), tilesN = ceil_div(g.N, BN);
+    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, g.batch), dim3(T::NT), 0, stream, g, tilesM, tilesN);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename E, bool A_KC, bool B_KC>
+static int pick_tile(const GemmArgs &g, hipStream_t stream) {
+    static const char *force = getenv("D8_GEMM_TILE");  // tuning aid
+    const long big_tiles = (long)ceil_div(g.M, 256) * ceil_div(g.N, 256) * g.batch;
+    bool big = g.M >= 256 && g.N >= 256 && big_tiles >= (long)cu_count() * 3 / 4;
+    if (force && g.M >= 256 && g.N >= 256) big = atoi(force) != 128;
+    // fp32 runs 64-cycle MFMAs on a quarter of the bytes per flop: the 128 x 128 tile already
+    // keeps the matrix pipe fed, and the compiler cannot hold the 256 x 256 variant in registers
+    if constexpr (sizeof(E) == 2) {
+        if (big) return launch_tiled<E, 256, 256, 4, 2, A_KC, B_KC>(g, stream);
+    }
+    return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC>(g, stream);
+}
+
+template <typename E>
+static bool gemm_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc) {
+    constexpr int ES = sizeof(E), EPV = 16 / ES, BK = 128 / ES;
+    if (g.red != 1 || g.splits != 1) return false;
+    // byte offsets inside one matrix are 32-bit
+    if ((long)(transA ? g.K : g.M) * g.lda * ES >= (1L << 31) || (long)(transB ? g.N : g.K) * g.ldb * ES >= (1L << 31))
+        return false;
+    if (g.M < 128 || g.N < 128 || g.K < BK || g.K % BK || g.lda % EPV || g.ldb % EPV || g.sA % EPV || g.sB % EPV)
+        return false;
+    if (((size_t)g.A | (size_t)g.B) & 15) return false;
+    if (transA && g.M % EPV) return false;
+    if (!transB && g.N % EPV) return false;
+    if ((long)ceil_div(g.M, 128) * ceil_div(g.N, 128) > 0x7fffffffL || g.batch > 65535) return false;
+    if (!transA && !transB) *rc = pick_tile<E, true, false>(g, stream);
+    else if (!transA && transB) *rc = pick_tile<E, true, true>(g, stream);
+    else *rc = pick_tile<E, false, false>(g, stream);
+    return true;
+}
+
+bool gemm_f16_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc) {
+    return gemm_tiled<f16>(g, transA, transB, stream, rc);
+}
+
+bool gemm_f32_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc) {
+    return gemm_tiled<float>(g, transA, transB, stream, rc);
+}
+
+}  // namespace d8
