@@ -181,39 +181,42 @@ __global__ void gemm_split_reduce_kernel(GemmArgs g) {
     }
 }
 
-// How many pieces to cut the reduction into.  Splitting is only worth a second pass when the
-// output alone gives the 256 CUs too few tiles; long reductions are also split to keep each
-// fp32 accumulation chain short.
-static int plan_splits(int dtype, int M, int N, int K, int batch, int red, int *tiles_per_split) {
-    const int BK = dtype == D8_FLOAT16 ? 32 : 16;
+// How many pieces to cut the reduction into, for a kernel whose K step is BK.  Splitting is only
+// worth a second pass when the output alone gives the 256 CUs too few tiles; the long reductions
+// this catches are also the ones whose single fp32 accumulation chain would be longest.
+static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t workspace_bytes, int *tiles_per_split) {
     const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
     const long total = (long)red * ceil_div(K, BK);
     const int cus = cu_count();
     long splits = 1;
     if (tiles < cus) splits = (2L * cus + tiles - 1) / tiles;
-    const long max_by_len = total / 8 > 0 ? total / 8 : 1;  // at least 8 K tiles per piece
+    const long max_by_len = total / 4 > 0 ? total / 4 : 1;  // at least 4 K steps per piece
     if (splits > max_by_len) splits = max_by_len;
     if (splits > 128) splits = 128;
-    if (splits < 1) splits = 1;
-    long tps = (total + splits - 1) / splits;
-    splits = (total + tps - 1) / tps;
+    // no more pieces than the caller's workspace holds
+    const size_t per_split = (size_t)batch * M * N * sizeof(float);
+    const long fit = (long)(workspace_bytes / per_split);
+    if (splits > fit) splits = fit;
+    if (splits < 2) splits = 1;
+    const long tps = (total + splits - 1) / splits;
     *tiles_per_split = (int)tps;
-    return (int)splits;
+    return tps > 0 ? (int)((total + tps - 1) / tps) : 1;
 }
 
 template <typename T>
-static int launch(GemmArgs &g, int transA, int transB, hipStream_t stream) {
-    int rc = 0;
-    if (sizeof(T) == 2 ? gemm_f16_tiled(g, transA, transB, stream, &rc) : gemm_f32_tiled(g, transA, transB, stream, &rc))
-        return rc;
-    dim3 grid(ceil_div(g.N, 128), ceil_div(g.M, 128), g.batch * g.splits);
-    if (!transA && !transB)
-        hipLaunchKernelGGL((gemm_general_kernel<T, false, false>), grid, dim3(256), 0, stream, g);
-    else if (!transA && transB)
-        hipLaunchKernelGGL((gemm_general_kernel<T, false, true>), grid, dim3(256), 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_general_kernel<T, true, false>), grid, dim3(256), 0, stream, g);
-    D8_LAUNCH_CHECK();
+static int launch(GemmArgs &g, int transA, int transB, bool tiled, hipStream_t stream) {
+    if (tiled) {
+        if (int rc = gemm_tiled_launch(sizeof(T) == 2 ? D8_FLOAT16 : D8_FLOAT32, g, transA, transB, stream)) return rc;
+    } else {
+        dim3 grid(ceil_div(g.N, 128), ceil_div(g.M, 128), g.batch * g.splits);
+        if (!transA && !transB)
+            hipLaunchKernelGGL((gemm_general_kernel<T, false, false>), grid, dim3(256), 0, stream, g);
+        else if (!transA && transB)
+            hipLaunchKernelGGL((gemm_general_kernel<T, false, true>), grid, dim3(256), 0, stream, g);
+        else
+            hipLaunchKernelGGL((gemm_general_kernel<T, true, false>), grid, dim3(256), 0, stream, g);
+        D8_LAUNCH_CHECK();
+    }
     if (g.splits > 1) {
         const long total = (long)g.M * g.N * g.batch;
         int blocks = (int)((total + 255) / 256);
@@ -237,8 +240,11 @@ size_t d8_gemm_workspace_bytes(int dtype, int transA, int transB, int M, int N, 
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
     const int red = (strideC == 0 && batch > 1) ? batch : 1;
     const int outs = red > 1 ? 1 : batch;
+    // whichever kernel ends up running, the larger of the two plans fits
     int tps = 0;
-    const int splits = plan_splits(dtype, M, N, K, outs, red, &tps);
+    const int a = plan_splits(gemm_tiled_k_step(dtype), M, N, K, outs, red, (size_t)-1, &tps);
+    const int b = plan_splits(dtype == D8_FLOAT16 ? Tile<f16>::BK : Tile<float>::BK, M, N, K, outs, red, (size_t)-1, &tps);
+    const int splits = a > b ? a : b;
     return splits > 1 ? (size_t)splits * outs * M * N * sizeof(float) : 0;
 }
 
@@ -277,26 +283,15 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     g.beta = beta;
     g.red = (strideC == 0 && batch > 1) ? batch : 1;
     g.batch = g.red > 1 ? 1 : batch;
-    if (K == 0) {
-        // empty reduction: C = beta * C
-        g.splits = 1;
-        g.tiles_per_split = 0;
-    } else {
-        g.splits = plan_splits(dtype, M, N, K, g.batch, g.red, &g.tiles_per_split);
-        const size_t per_split = (size_t)g.batch * M * N * sizeof(float);
-        if (g.splits > 1 && (!workspace || workspace_bytes < per_split * g.splits)) {
-            // use as many pieces as the caller's workspace holds
-            long fit = workspace ? (long)(workspace_bytes / per_split) : 1;
-            if (fit < 2) fit = 1;
-            const int BK = dtype == D8_FLOAT16 ? 32 : 16;
-            const long total = (long)g.red * ceil_div(K, BK);
-            long tps = (total + fit - 1) / fit;
-            g.tiles_per_split = (int)tps;
-            g.splits = (int)((total + tps - 1) / tps);
-        }
+    g.splits = 1;
+    g.tiles_per_split = 0;
+    const bool tiled = K > 0 && gemm_tiled_eligible(dtype, g, transA, transB);
+    if (K > 0) {  // K == 0 is the empty reduction: C = beta * C
+        const int BK = tiled ? gemm_tiled_k_step(dtype) : (dtype == D8_FLOAT16 ? Tile<f16>::BK : Tile<float>::BK);
+        g.splits = plan_splits(BK, M, N, K, g.batch, g.red, workspace ? workspace_bytes : 0, &g.tiles_per_split);
     }
-    return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, as_stream(stream))
-                               : launch<float>(g, transA, transB, as_stream(stream));
+    return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, tiled, as_stream(stream))
+                               : launch<float>(g, transA, transB, tiled, as_stream(stream));
 }
 
 }  // extern "C"

@@ -21,11 +21,12 @@ struct GemmArgs {
     float beta;
 };
 
-// Tiled fp16 kernels for shapes whose operands can be moved in 16-byte pieces.  Returns false
-// when the shape does not qualify (the caller then uses the general kernel); otherwise launches
-// and stores the launch status in *rc.
-bool gemm_f16_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc);
-bool gemm_f32_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc);
+// Tiled kernels (fp16 and fp32) for shapes whose operands can be moved in 16-byte pieces.
+int gemm_tiled_k_step(int dtype);  // K elements per step: 64 (fp16) or 32 (fp32)
+// Whether the shape qualifies (g.splits / g.tiles_per_split need not be set yet).
+bool gemm_tiled_eligible(int dtype, const GemmArgs &g, int transA, int transB);
+// Launch; with g.splits > 1 the fp32 partial sums go to g.ws for the caller to reduce.
+int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipStream_t stream);
 
 }  // namespace d8
 

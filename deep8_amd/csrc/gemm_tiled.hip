@@ -203,6 +203,76 @@ __device__ __forceinline__ void k_step(const typename T::E *Ar, const typename T
 __device__ inline float as_f32(float v) { return v; }
 __device__ inline float as_f32(f16 v) { return (float)v; }
 
+struct Origin {
+    int m0, n0;        // where the computed tile starts (moved inside the matrix)
+    int m_own, n_own;  // rows / columns from here on are this workgroup's to store
+    int wm0, wn0;      // this wave's offset inside the tile
+};
+
+// Store a wave's accumulators.  Lane holds column lane%32 of rows 8*(r/4) + 4*(lane/32) + r%4 of
+// each 32x32 block.  Where rows of C can be moved 16 bytes at a time, each block is turned around
+// through the wave's own 32 x 36 float patch of LDS, so that a lane ends up with 8 consecutive
+// columns of one row: 16-byte loads of the old C and 16-byte stores.
+template <typename T, typename O>
+__device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *lds, O *C, int ldc, float beta,
+                                           bool aligned, int N, const Origin &o) {
+    constexpr int TM = T::TM, TN = T::TN, OPV = 16 / sizeof(O);
+    typedef O OV __attribute__((ext_vector_type(OPV)));
+    static_assert((size_t)T::A_SZ * T::ES >= (size_t)T::NT / 64 * 32 * 36 * sizeof(float), "patch space");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lhi = lane >> 5;
+    if (aligned && N % 8 == 0) {
+        float *patch = lds + wave * (32 * 36);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) patch[((r >> 2) * 8 + lhi * 4 + (r & 3)) * 36 + l32] = acc[i][j][r];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int q = lane + 64 * t, row = q >> 2, cc = (q & 3) * 8;
+                    const int m = o.m0 + o.wm0 + i * 32 + row, n = o.n0 + o.wn0 + j * 32 + cc;
+                    float v[8];
+                    *(f32x4 *)&v[0] = *(const f32x4 *)(patch + row * 36 + cc);
+                    *(f32x4 *)&v[4] = *(const f32x4 *)(patch + row * 36 + cc + 4);
+                    if (m >= o.m_own && n >= o.n_own) {
+                        O *c = C + (long)m * ldc + n;
+#pragma unroll
+                        for (int h = 0; h < 8 / OPV; ++h) {
+                            OV out;
+                            if (beta != 0.f) {
+                                const OV old = *(const OV *)(c + h * OPV);
+#pragma unroll
+                                for (int e = 0; e < OPV; ++e) out[e] = (O)(v[h * OPV + e] + as_f32(old[e]));
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < OPV; ++e) out[e] = (O)v[h * OPV + e];
+                            }
+                            *(OV *)(c + h * OPV) = out;
+                        }
+                    }
+                }
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = o.n0 + o.wn0 + j * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = o.m0 + o.wm0 + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
+                if (m >= o.m_own && n >= o.n_own) {
+                    O *c = C + (long)m * ldc + n;
+                    float v = acc[i][j][r];
+                    if (beta != 0.f) v += as_f32(*c);
+                    *c = (O)v;
+                }
+            }
+        }
+}
+
 template <typename T>
 __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tilesM, int tilesN) {
     typedef typename T::E E;
@@ -239,12 +309,14 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // number of rows below piece 0, in global memory and in LDS alike.  Global memory is read
     // through buffer descriptors: byte offset = uniform part (tile origin, K step, piece; scalar
     // registers) + per-thread part (one VGPR per operand).
-    const int b = blockIdx.z;
+    // blockIdx.z = output batch index * splits + piece of the reduction.  The reduction runs over
+    // `red` products (1 unless the whole batch is summed into one C) times K, cut into `splits`.
+    const int b = blockIdx.z / g.splits, split = blockIdx.z - b * g.splits;
     const long a_rows = A_KC ? g.M : g.K, b_rows = B_KC ? g.N : g.K;
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)((const E *)g.A + (long)b * g.sA), 0, (int)(ES * a_rows * g.lda), 0x00020000);
+        (void *)((const E *)g.A + (long)b * g.sA), 0, (int)(ES * ((g.red - 1) * g.sA + a_rows * g.lda)), 0x00020000);
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)((const E *)g.B + (long)b * g.sB), 0, (int)(ES * b_rows * g.ldb), 0x00020000);
+        (void *)((const E *)g.B + (long)b * g.sB), 0, (int)(ES * ((g.red - 1) * g.sB + b_rows * g.ldb)), 0x00020000);
     const unsigned Au = (unsigned)ES * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0);
     const unsigned Bu = (unsigned)ES * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
     const int a_r = A_KC ? tid >> 3 : tid / (BM / EPV), a_c = A_KC ? tid & 7 : tid % (BM / EPV);
@@ -270,18 +342,33 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // ---- prologue: step 0 into LDS half 0, step 1 into registers, first operands of step 0
+    // ---- this workgroup's steps x0 .. x0 + nsteps - 1 of the extended reduction; step x reads
+    // product x / ktiles at K offset (x % ktiles) * BK (all uniform: scalar arithmetic)
     const int ktiles = g.K / BK;
+    const int x0 = split * g.tiles_per_split, nsteps = min(g.red * ktiles, x0 + g.tiles_per_split) - x0;
+    const unsigned a_prod = (unsigned)ES * (unsigned)g.sA, b_prod = (unsigned)ES * (unsigned)g.sB;
+    auto step_a = [&](int i) {
+        const int x = x0 + min(i, nsteps - 1), r = x / ktiles;  // past the end: refetch the last step, never used
+        return Au + (g.red > 1 ? r * a_prod : 0u) + (x - r * ktiles) * a_step;
+    };
+    auto step_b = [&](int i) {
+        const int x = x0 + min(i, nsteps - 1), r = x / ktiles;
+        return Bu + (g.red > 1 ? r * b_prod : 0u) + (x - r * ktiles) * b_step;
+    };
+
+    // ---- prologue: step 0 into LDS half 0, step 1 into registers, first operands of step 0
+    {
+        const unsigned pa = step_a(0), pb = step_b(0);
 #pragma unroll
-    for (int p = 0; p < NP; ++p)
-        R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, Au + p * a_pass, 0)
-                        : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, Bu + (p - A_IT) * b_pass, 0);
+        for (int p = 0; p < NP; ++p)
+            R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, pa + p * a_pass, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, pb + (p - A_IT) * b_pass, 0);
+    }
 #pragma unroll
     for (int p = 0; p < NP; ++p)
         *(u32x4 *)(p < A_IT ? As0 + a_dst + p * T::A_ROWS * A_LD : Bs0 + b_dst + (p - A_IT) * T::B_ROWS * B_LD) = R[p];
     {
-        const int t1 = min(1, ktiles - 1);
-        const unsigned pa = Au + t1 * a_step, pb = Bu + t1 * b_step;
+        const unsigned pa = step_a(1), pb = step_b(1);
 #pragma unroll
         for (int p = 0; p < NP; ++p)
             R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, pa + p * a_pass, 0)
@@ -296,87 +383,29 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         fb[0][j] = B_KC ? EL::read_kc(Bs0 + b_frag + j * 32 * B_LD) : EL::read_tr(Bs0 + b_frag + j * 32, B_LD);
 
     // ---- main loop, two steps per trip so that the LDS half of every access is known statically;
-    // fetches past the last step re-read the last step and are never used
-    for (int kt = 0; kt < ktiles; kt += 2) {
-        {
-            const int t2 = min(kt + 2, ktiles - 1);
-            k_step<T>(As0 + a_frag, Bs0 + b_frag, As1 + a_frag, Bs1 + b_frag, As1 + a_dst, Bs1 + b_dst, ra, rb,
-                      Au + t2 * a_step, Bu + t2 * b_step, a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
-        }
-        if (kt + 1 < ktiles) {
-            const int t3 = min(kt + 3, ktiles - 1);
+    for (int i = 0; i < nsteps; i += 2) {
+        k_step<T>(As0 + a_frag, Bs0 + b_frag, As1 + a_frag, Bs1 + b_frag, As1 + a_dst, Bs1 + b_dst, ra, rb,
+                  step_a(i + 2), step_b(i + 2), a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
+        if (i + 1 < nsteps)
             k_step<T>(As1 + a_frag, Bs1 + b_frag, As0 + a_frag, Bs0 + b_frag, As0 + a_dst, Bs0 + b_dst, ra, rb,
-                      Au + t3 * a_step, Bu + t3 * b_step, a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
-        }
+                      step_a(i + 3), step_b(i + 3), a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
     }
 
-    // ---- epilogue.  Lane holds column lane%32 of rows 8*(r/4) + 4*(lane/32) + r%4 of each 32x32 block.
-    E *Cg = (E *)g.C + (long)b * g.sC;
-    const int l32 = lane & 31, lhi = lane >> 5;
-    const bool vector_ok = (g.ldc % EPV == 0) && (g.sC % EPV == 0) && (((size_t)g.C & 15) == 0) && (g.N % 8 == 0);
-    if (vector_ok) {
-        // Each wave turns one 32x32 block at a time around through its own 32 x 36 float patch of
-        // LDS (the A half is free once every wave is past the last step), so that a lane ends up
-        // with 8 consecutive columns of one row: 16-byte loads of the old C and 16-byte stores.
-        static_assert((size_t)T::A_SZ * ES >= (size_t)T::NT / 64 * 32 * 36 * sizeof(float), "patch space");
-        __syncthreads();
-        float *patch = (float *)As0 + wave * (32 * 36);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) patch[((r >> 2) * 8 + lhi * 4 + (r & 3)) * 36 + l32] = acc[i][j][r];
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const int q = lane + 64 * t, row = q >> 2, cc = (q & 3) * 8;
-                    const int m = m0 + (wm * TM + i) * 32 + row, n = n0 + (wn * TN + j) * 32 + cc;
-                    float v[8];
-                    *(f32x4 *)&v[0] = *(const f32x4 *)(patch + row * 36 + cc);
-                    *(f32x4 *)&v[4] = *(const f32x4 *)(patch + row * 36 + cc + 4);
-                    if (m >= m_own && n >= n_own) {
-                        E *c = Cg + (long)m * g.ldc + n;
-#pragma unroll
-                        for (int h = 0; h < 8 / EPV; ++h) {
-                            EV o;
-                            if (g.beta != 0.f) {
-                                const EV old = *(const EV *)(c + h * EPV);
-#pragma unroll
-                                for (int e = 0; e < EPV; ++e) o[e] = (E)(v[h * EPV + e] + as_f32(old[e]));
-                            } else {
-#pragma unroll
-                                for (int e = 0; e < EPV; ++e) o[e] = (E)v[h * EPV + e];
-                            }
-                            *(EV *)(c + h * EPV) = o;
-                        }
-                    }
-                }
-            }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int n = n0 + (wn * TN + j) * 32 + l32;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + (wm * TM + i) * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-                if (m >= m_own && n >= n_own) {
-                    E *c = Cg + (long)m * g.ldc + n;
-                    float v = acc[i][j][r];
-                    if (g.beta != 0.f) v += as_f32(*c);
-                    *c = (E)v;
-                }
-            }
-        }
+    // ---- epilogue: the result itself, or this piece's fp32 partial sums when the reduction is split
+    __syncthreads();  // every wave is past the last step: the A half of LDS is free
+    const Origin o = {m0, n0, m_own, n_own, (wm * TM) * 32, (wn * TN) * 32};
+    if (g.splits > 1)
+        store_tile<T, float>(acc, (float *)As0, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o);
+    else
+        store_tile<T, E>(acc, (float *)As0, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
+                         g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o);
 }
 
 template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC>
 static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
     typedef Tile<E, BM, BN, WGM, WGN, A_KC, B_KC> T;
     const int tilesM = ceil_div(g.M, BM), tilesN = ceil_div(g.N, BN);
-    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, g.batch), dim3(T::NT), 0, stream, g, tilesM, tilesN);
+    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, g.batch * g.splits), dim3(T::NT), 0, stream, g, tilesM, tilesN);
     D8_LAUNCH_CHECK();
     return 0;
 }
@@ -384,7 +413,7 @@ static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
 template <typename E, bool A_KC, bool B_KC>
 static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     static const char *force = getenv("D8_GEMM_TILE");  // tuning aid
-    const long big_tiles = (long)ceil_div(g.M, 256) * ceil_div(g.N, 256) * g.batch;
+    const long big_tiles = (long)ceil_div(g.M, 256) * ceil_div(g.N, 256) * g.batch * g.splits;
     bool big = g.M >= 256 && g.N >= 256 && big_tiles >= (long)cu_count() * 3 / 4;
     if (force && g.M >= 256 && g.N >= 256) big = atoi(force) != 128;
     // fp32 runs 64-cycle MFMAs on a quarter of the bytes per flop: the 128 x 128 tile already
@@ -396,30 +425,35 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
 }
 
 template <typename E>
-static bool gemm_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc) {
-    constexpr int ES = sizeof(E), EPV = 16 / ES, BK = 128 / ES;
-    if (g.red != 1 || g.splits != 1) return false;
-    // byte offsets inside one matrix are 32-bit
-    if ((long)(transA ? g.K : g.M) * g.lda * ES >= (1L << 31) || (long)(transB ? g.N : g.K) * g.ldb * ES >= (1L << 31))
-        return false;
+static bool eligible(const GemmArgs &g, int transA, int transB) {
+    constexpr long ES = sizeof(E), EPV = 16 / ES, BK = 128 / ES;
+    // byte offsets inside one operand (all summed products of it included) are 32-bit
+    if (((g.red - 1) * g.sA + (long)(transA ? g.K : g.M) * g.lda) * ES >= (1L << 31)) return false;
+    if (((g.red - 1) * g.sB + (long)(transB ? g.N : g.K) * g.ldb) * ES >= (1L << 31)) return false;
     if (g.M < 128 || g.N < 128 || g.K < BK || g.K % BK || g.lda % EPV || g.ldb % EPV || g.sA % EPV || g.sB % EPV)
         return false;
     if (((size_t)g.A | (size_t)g.B) & 15) return false;
     if (transA && g.M % EPV) return false;
     if (!transB && g.N % EPV) return false;
-    if ((long)ceil_div(g.M, 128) * ceil_div(g.N, 128) > 0x7fffffffL || g.batch > 65535) return false;
-    if (!transA && !transB) *rc = pick_tile<E, true, false>(g, stream);
-    else if (!transA && transB) *rc = pick_tile<E, true, true>(g, stream);
-    else *rc = pick_tile<E, false, false>(g, stream);
+    if ((long)ceil_div(g.M, 128) * ceil_div(g.N, 128) > 0x7fffffffL || (long)g.batch * 128 > 65535) return false;
     return true;
 }
 
-bool gemm_f16_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc) {
-    return gemm_tiled<f16>(g, transA, transB, stream, rc);
+template <typename E>
+static int launch_any(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
+    if (!transA && !transB) return pick_tile<E, true, false>(g, stream);
+    if (!transA && transB) return pick_tile<E, true, true>(g, stream);
+    return pick_tile<E, false, false>(g, stream);
 }
 
-bool gemm_f32_tiled(const GemmArgs &g, int transA, int transB, hipStream_t stream, int *rc) {
-    return gemm_tiled<float>(g, transA, transB, stream, rc);
+int gemm_tiled_k_step(int dtype) { return dtype == D8_FLOAT16 ? 64 : 32; }
+
+bool gemm_tiled_eligible(int dtype, const GemmArgs &g, int transA, int transB) {
+    return dtype == D8_FLOAT16 ? eligible<f16>(g, transA, transB) : eligible<float>(g, transA, transB);
+}
+
+int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipStream_t stream) {
+    return dtype == D8_FLOAT16 ? launch_any<f16>(g, transA, transB, stream) : launch_any<float>(g, transA, transB, stream);
 }
 
 }  // namespace d8

@@ -129,6 +129,33 @@ def test_gemm_long_reduction_split(oracle_port, use_ws):
     assert rel_fro(ops.gemm(1, 0, Ar, Br, C0, 1.0, use_workspace=use_ws), want) <= FP32_TOL
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("M,N,K,nb", [(256, 384, 8192, 1), (130, 264, 4096, 1), (256, 136, 192, 7), (512, 512, 64, 12),
+                                      (128, 128, 2048, 3)])
+def test_gemm_tiled_split_and_summed(oracle_port, ta, tb, dtype, M, N, K, nb):
+    """Shapes the tiled kernels take whose output has too few tiles for the chip: the reduction (all
+    nb summed products of it) is cut into pieces that meet again in the fp32 workspace."""
+    from deep8_amd import ops
+    r = rng(M + N + K + nb)
+    hi = 2 if dtype == np.float16 else 20
+    c = (lambda a: h(a)) if dtype == np.float16 else (lambda a: a)
+    lead = (nb,) if nb > 1 else ()
+    A = ints(r, lead + ((K, M) if ta else (M, K)), hi)
+    B = ints(r, lead + ((N, K) if tb else (K, N)), hi)
+    if dtype == np.float16:  # thin the operands so every sum stays an exact fp16 integer
+        A = A * (r.random(A.shape) < 0.15)
+        B = B * (r.random(B.shape) < 0.15)
+    C0 = ints(r, (M, N), 3)
+    want = C0.copy()
+    for b in range(nb):
+        want = oracle_port.gemm(ta, tb, A[b] if nb > 1 else A, B[b] if nb > 1 else B, want, 1.0)
+    assert dtype == np.float32 or np.abs(want).max() < 2048
+    for use_ws in (True, False):
+        got = ops.gemm(ta, tb, c(A), c(B), c(C0), 1.0, use_workspace=use_ws)
+        assert np.array_equal(f(got), want), (ta, tb, M, N, K, nb, use_ws)
+
+
 def test_gemm_argument_errors():
     from deep8_amd import capi
     lib = capi.init()
