@@ -118,6 +118,9 @@ struct Tile {
     static constexpr int A_ROWS = A_KC ? NT / 8 : NT / (BM / EPV);
     static constexpr int B_ROWS = B_KC ? NT / 8 : NT / (BN / EPV);
     static constexpr int A_RD = A_KC ? 1 : EL::TR_READS, B_RD = B_KC ? 1 : EL::TR_READS;
+    // the epilogue's transposing patches reuse the larger of the two operand areas
+    static constexpr bool PATCH_IN_A = A_SZ >= B_SZ;
+    static constexpr int PATCH_SZ = PATCH_IN_A ? A_SZ : B_SZ;
 };
 
 // Pieces [lo(q), lo(q+1)) are written to LDS during quarter q = 0, 1, 2 of a step and re-fetched
@@ -218,7 +221,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
                                            bool aligned, int N, const Origin &o) {
     constexpr int TM = T::TM, TN = T::TN, OPV = 16 / sizeof(O);
     typedef O OV __attribute__((ext_vector_type(OPV)));
-    static_assert((size_t)T::A_SZ * T::ES >= (size_t)T::NT / 64 * 32 * 36 * sizeof(float), "patch space");
+    static_assert((size_t)T::PATCH_SZ * T::ES >= (size_t)T::NT / 64 * 32 * 36 * sizeof(float), "patch space");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lhi = lane >> 5;
     if (aligned && N % 8 == 0) {
         float *patch = lds + wave * (32 * 36);
@@ -392,12 +395,13 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     }
 
     // ---- epilogue: the result itself, or this piece's fp32 partial sums when the reduction is split
-    __syncthreads();  // every wave is past the last step: the A half of LDS is free
+    __syncthreads();  // every wave is past the last step: the operand areas are free
     const Origin o = {m0, n0, m_own, n_own, (wm * TM) * 32, (wn * TN) * 32};
+    float *patches = (float *)(T::PATCH_IN_A ? As0 : Bs0);
     if (g.splits > 1)
-        store_tile<T, float>(acc, (float *)As0, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o);
+        store_tile<T, float>(acc, patches, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o);
     else
-        store_tile<T, E>(acc, (float *)As0, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
+        store_tile<T, E>(acc, patches, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
                          g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o);
 }
 
@@ -421,6 +425,9 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     if constexpr (sizeof(E) == 2) {
         if (big) return launch_tiled<E, 256, 256, 4, 2, A_KC, B_KC>(g, stream);
     }
+    // a 64-wide side gets a tile of that width (im2col products with 64 output channels)
+    if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC>(g, stream);
+    if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC>(g, stream);
     return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC>(g, stream);
 }
 
@@ -430,7 +437,7 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
     // byte offsets inside one operand (all summed products of it included) are 32-bit
     if (((g.red - 1) * g.sA + (long)(transA ? g.K : g.M) * g.lda) * ES >= (1L << 31)) return false;
     if (((g.red - 1) * g.sB + (long)(transB ? g.N : g.K) * g.ldb) * ES >= (1L << 31)) return false;
-    if (g.M < 128 || g.N < 128 || g.K < BK || g.K % BK || g.lda % EPV || g.ldb % EPV || g.sA % EPV || g.sB % EPV)
+    if (g.M < 64 || g.N < 64 || (g.M < 128 && g.N < 128) || g.K < BK || g.K % BK || g.lda % EPV || g.ldb % EPV || g.sA % EPV || g.sB % EPV)
         return false;
     if (((size_t)g.A | (size_t)g.B) & 15) return false;
     if (transA && g.M % EPV) return false;

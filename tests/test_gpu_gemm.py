@@ -50,7 +50,8 @@ def test_gemm_f16_integer_exact(oracle_port, ta, tb, M, N, K):
 
 @pytest.mark.parametrize("ta,tb", TRANS)
 @pytest.mark.parametrize("M,N,K", [(300, 264, 128), (136, 130, 64), (512, 520, 256), (1000, 392, 192), (304, 261, 128),
-                                   (256, 256, 64), (768, 1280, 448)])
+                                   (256, 256, 64), (768, 1280, 448), (1000, 64, 192), (64, 520, 256), (300, 72, 128),
+                                   (96, 264, 64), (128, 64, 64), (64, 128, 128), (2000, 120, 576)])
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 def test_gemm_tiled_kernels_edge_tiles(oracle_port, ta, tb, M, N, K, dtype):
     """Shapes that take the tiled kernels (K a multiple of 64, rows movable in 16-byte pieces) with
@@ -132,7 +133,7 @@ def test_gemm_long_reduction_split(oracle_port, use_ws):
 @pytest.mark.parametrize("ta,tb", TRANS)
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 @pytest.mark.parametrize("M,N,K,nb", [(256, 384, 8192, 1), (130, 264, 4096, 1), (256, 136, 192, 7), (512, 512, 64, 12),
-                                      (128, 128, 2048, 3)])
+                                      (128, 128, 2048, 3), (64, 576, 8192, 1), (264, 64, 4096, 1), (96, 192, 128, 9)])
 def test_gemm_tiled_split_and_summed(oracle_port, ta, tb, dtype, M, N, K, nb):
     """Shapes the tiled kernels take whose output has too few tiles for the chip: the reduction (all
     nb summed products of it) is cut into pieces that meet again in the fp32 workspace."""
