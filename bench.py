@@ -28,6 +28,12 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"f16": 2500.0, "f32": 157.3}   # dense MFMA TFLOP/s, MI355X
 HBM_PEAK = 8000.0                      # GB/s
+# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this file (each counter scaled by what it reads for a plain copy of known size; the
+# summaries are kept under profiles/).  None where no counter run has been made.
+MEASURED_TRAFFIC = {
+    "c3": int((192.1 + 224.1 + 224.1) / 3 * 2**20 + 33.6 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
+}
 
 
 def _dev(a):
@@ -82,6 +88,7 @@ class MatMulWorkload:
         self.ws = capi.DeviceArray((max(nb, 16),), np.uint8)
         m, k, n = xs[1], xs[2], ys[2]
         self.flops = 3 * 2.0 * zb * m * k * n
+        self.kernel = "gemm_tiled_kernel<%s> (one launch each for fwd, dX, dY)" % ("f16" if self.dtype == np.float16 else "f32")
         es = self.dtype.itemsize
         nx, ny, nz = np.prod(xs), np.prod(ys), np.prod(self.zs)
         # fwd reads x,y writes z; dX reads dz,y and read-modify-writes dx; dY likewise
@@ -183,6 +190,30 @@ class ConvWorkload:
         f = self.flops / 3
         return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
 
+    def map_roofline(self, reps):
+        """The gather map that builds the GEMM operand (im2col for Conv2d, the dz gather for
+        DeConv2d), launched alone through the C ABI and timed with HIP events: algorithmic bytes
+        (source read once + matrix written once) / launch duration against the HBM peak."""
+        from deep8_amd import capi, ops
+        B, IH, IW, IC = self.xd
+        OC, FH, FW, _ = self.wd
+        es = self.dtype.itemsize
+        mat = capi.DeviceArray((self.mat_bytes // es,), self.dtype)
+        if self.deconv:
+            OH, OW, pt, pl = ops.deconv2d_geometry(IH, IW, FH, FW, *self.geo)
+            fn = lambda: capi.check(self.lib.d8_deconv_im2col(self.dt, self.gz.ptr, mat.ptr, B, IH, IW, OH, OW, OC, FH, FW,
+                                                              self.geo[1], self.geo[2], pt, pl, None))
+            name, nbytes = "deconv_im2col_kernel", es * B * OH * OW * OC + self.mat_bytes
+        else:
+            OH, OW, pt, pl = ops.conv2d_geometry(IH, IW, FH, FW, *self.geo)
+            fn = lambda: capi.check(self.lib.d8_im2col(self.dt, self.x.ptr, mat.ptr, B, IH, IW, IC, OH, OW, FH, FW,
+                                                       self.geo[1], self.geo[2], self.geo[3], self.geo[4], pt, pl, None))
+            name, nbytes = "im2col_kernel", es * B * IH * IW * IC + self.mat_bytes
+        ms = _time_events(fn, reps)
+        ach = nbytes / (ms * 1e-3) / 1e9
+        return {"bound": "hbm", "kernel": name, "achieved": round(ach, 1), "peak": HBM_PEAK, "unit": "GB/s",
+                "frac": round(ach / HBM_PEAK, 4), "launch_us": round(ms * 1e3, 2), "traffic": None}
+
 
 def _uni(r, s):
     return r.uniform(-1, 1, s).astype(np.float32)
@@ -214,52 +245,78 @@ def make_workload(key):
     raise SystemExit("unknown workload %r" % key)
 
 
-def cpu_baseline(key):
-    """Deep8's CPU path on a bounded sample of the workload (forward + both gradients)."""
+def _repeat_for(fn, seconds):
+    """run fn (after one untimed call) until about `seconds` have passed; returns (calls, elapsed)"""
+    fn()
+    n, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds:
+            return n, dt
+
+
+def cpu_baseline(key, seconds=12.0):
+    """Deep8's CPU path on a bounded sample of the workload (forward + both gradients), repeated
+    for about `seconds` of CPU work."""
     import oracle
     src = oracle.ref if oracle.ref is not None else oracle.port
     kind = "reference" if oracle.ref is not None else "port"
     r = np.random.default_rng(9)
     if key in ("c4", "c5"):
         # the reference runs Conv2d/DeConv2d on Eigen's thread pool: all host cores
-        B = 2
+        B = 8
         if key == "c4":
             x, w = r.standard_normal((B, 56, 56, 64)).astype(np.float32), r.standard_normal((64, 3, 3, 64)).astype(np.float32)
             args, f3 = (True, 1, 1, 1, 1), (src.conv2d, src.conv2d_grad_x, src.conv2d_grad_y)
-            flops = 3 * 2.0 * B * 56 * 56 * 576 * 64
         else:
             x, w = r.standard_normal((B, 28, 28, 128)).astype(np.float32), r.standard_normal((64, 4, 4, 128)).astype(np.float32)
             args, f3 = (False, 2, 2), (src.deconv2d, src.deconv2d_grad_x, src.deconv2d_grad_y)
-            flops = 3 * 2.0 * B * 28 * 28 * 128 * 1024
-        z = f3[0](x, w, *args)
-        gz = r.standard_normal(z.shape).astype(np.float32)
-        t0 = time.perf_counter()
-        f3[0](x, w, *args)
-        f3[1](x, w, gz, *args)
-        f3[2](x, w, gz, *args)
-        dt = time.perf_counter() - t0
-        return {"value": B / dt, "unit": "images/s", "cores": src.threads(), "kind": kind,
-                "sample": "%s fwd+dX+dW on %d images (fp32 CPU path), %.2f s" % (key, B, dt),
-                "tflops": flops / dt / 1e12}
+        gz = r.standard_normal(f3[0](x, w, *args).shape).astype(np.float32)
+
+        def one():
+            f3[0](x, w, *args)
+            f3[1](x, w, gz, *args)
+            f3[2](x, w, gz, *args)
+        n, dt = _repeat_for(one, seconds)
+        return {"value": n * B / dt, "unit": "images/s", "cores": src.threads(), "kind": kind,
+                "sample": "%s fwd+dX+dW on %d images x %d repeats (fp32 CPU path), %.1f s" % (key, B, n, dt)}
     # MatrixMultiply: Eigen's dense product is single-threaded in the reference build
     if key == "c3":
-        m, k, n, b = 256, 4096, 4096, 1
+        m, k, n_, b = 256, 4096, 4096, 1
     elif key in ("c2a", "c2b"):
-        m, k, n, b = 512, 512, 512, 8
+        m, k, n_, b = 512, 512, 512, 8
     else:
-        m, k, n, b = 64, 128, 256, 1
-    x, y = r.uniform(-1, 1, (b, m, k)).astype(np.float32), r.uniform(-1, 1, (1 if key != "c2a" else b, k, n)).astype(np.float32)
-    dz = r.uniform(-1, 1, (b, m, n)).astype(np.float32)
-    src.matmul(x[:, :8], y)  # warm the library
-    t0 = time.perf_counter()
-    src.matmul(x, y)
-    src.matmul_grad_x(x, y, dz)
-    src.matmul_grad_y(x, y, dz)
-    dt = time.perf_counter() - t0
-    flops = 3 * 2.0 * b * m * k * n
+        m, k, n_, b = 64, 128, 256, 1
+    x, y = r.uniform(-1, 1, (b, m, k)).astype(np.float32), r.uniform(-1, 1, (1 if key != "c2a" else b, k, n_)).astype(np.float32)
+    dz = r.uniform(-1, 1, (b, m, n_)).astype(np.float32)
+
+    def one():
+        src.matmul(x, y)
+        src.matmul_grad_x(x, y, dz)
+        src.matmul_grad_y(x, y, dz)
+    n, dt = _repeat_for(one, seconds)
+    flops = n * 3 * 2.0 * b * m * k * n_
     return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1 if kind == "reference" else src.threads(),
             "kind": kind,
-            "sample": "fwd+dX+dY of %d x [%dx%d]x[%dx%d] fp32 (the reference has no CPU half), %.2f s" % (b, m, k, k, n, dt)}
+            "sample": "fwd+dX+dY of %d x [%dx%d]x[%dx%d] fp32 (the reference has no CPU half) x %d repeats, %.1f s"
+                      % (b, m, k, k, n_, n, dt)}
+
+
+def calibrate_copy(mib):
+    """A plain copy of known size (the im2col kernel with a 1x1 filter is exactly that), run under
+    `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` to find what those counters read per byte moved."""
+    from deep8_amd import capi
+    lib = capi.init()
+    n = mib * (1 << 20) // 4
+    rows = n // 64
+    src = capi.DeviceArray((rows, 64), np.float32, zero=True)
+    dst = capi.DeviceArray((rows, 64), np.float32, zero=True)
+    for _ in range(5):
+        capi.check(lib.d8_im2col(capi.FLOAT32, src.ptr, dst.ptr, 1, rows, 1, 64, rows, 1, 1, 1, 1, 1, 1, 1, 0, 0, None))
+    capi.sync()
+    print(json.dumps({"copy_kernel": "im2col_kernel (1x1 filter)", "bytes_read": rows * 256, "bytes_written": rows * 256}))
 
 
 def main():
@@ -270,6 +327,8 @@ def main():
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-others", action="store_true")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
@@ -277,6 +336,8 @@ def main():
 
     from deep8_amd import capi
     capi.init()
+    if a.calibrate_copy:
+        return calibrate_copy(a.calibrate_copy)
 
     wl = make_workload(a.workload)
     ms = _time_steps(wl.step, a.steps, a.warmup)
@@ -288,14 +349,16 @@ def main():
     for pname, (fn, fl) in wl.parts().items():
         pms = _time_events(fn, max(5, a.steps))
         parts[pname] = {"ms": round(pms, 4), "tflops": round(fl / (pms * 1e-3) / 1e12, 2)}
-    slow = max(parts, key=lambda p: parts[p]["ms"])
-    roof = {"bound": "mfma", "kernel": "%s GEMM launch (%s)" % (a.workload, slow),
-            "achieved": parts[slow]["tflops"], "peak": PEAK[dtype], "unit": "TFLOP/s",
-            "frac": round(parts[slow]["tflops"] / PEAK[dtype], 4), "traffic": None}
     if is_conv:
-        roof = {"bound": "hbm", "kernel": "%s whole step (gather maps + GEMMs)" % a.workload,
-                "achieved": round(wl.bytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK, "unit": "GB/s",
-                "frac": round(wl.bytes / (ms * 1e-3) / 1e9 / HBM_PEAK, 4), "traffic": None}
+        roof = wl.map_roofline(max(5, a.steps))
+    else:
+        # each of fwd / dX / dY is ONE launch of the same tiled GEMM kernel (its NN, NT and TN
+        # instances): flops per launch / average launch duration, HIP events on the launch stream
+        avg_ms = sum(p["ms"] for p in parts.values()) / len(parts)
+        ach = wl.flops / 3 / (avg_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "kernel": wl.kernel, "achieved": round(ach, 2), "peak": PEAK[dtype],
+                "unit": "TFLOP/s", "frac": round(ach / PEAK[dtype], 4), "launch_us": round(avg_ms * 1e3, 2),
+                "traffic": MEASURED_TRAFFIC.get(a.workload)}
 
     out = {
         "metric": "Conv2d fwd+bwd images/s" if is_conv else "MatrixMultiply fwd+bwd TFLOP/s",

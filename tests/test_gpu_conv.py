@@ -160,3 +160,77 @@ def test_deconv2d_real_tolerance(oracle_port, cfg):
                    oracle_port.deconv2d_grad_x(f(xh), f(wh), f(gzh), *a)) <= FP16_TOL
     assert rel_fro(f(ops.deconv2d_grad_y(xh, wh, gzh, *a)),
                    oracle_port.deconv2d_grad_y(f(xh), f(wh), f(gzh), *a)) <= FP16_TOL
+
+
+def test_config4_full_size_properties(oracle_port):
+    """BASELINE config 4 (Conv2d fp32, B32 56x56x64, 3x3x64 -> 64, same padding) at full size:
+    two sampled images against the oracle (forward and dX are independent per image), dW through
+    its additivity over the batch, and the adjoint identity <z, dz> == <x, dx> == <w, dw>."""
+    from deep8_amd import ops
+    r = rng(44)
+    B = 32
+    x, w = nrm(r, (B, 56, 56, 64)), nrm(r, (64, 3, 3, 64), np.sqrt(2.0 / 576))
+    gz = nrm(r, (B, 56, 56, 64))
+    a = (True, 1, 1, 1, 1)
+    z, gx, gw = ops.conv2d(x, w, *a), ops.conv2d_grad_x(x, w, gz, *a), ops.conv2d_grad_y(x, w, gz, *a)
+    assert z.shape == (B, 56, 56, 64)
+    pick = [3, 30]
+    assert rel_fro(z[pick], oracle_port.conv2d(x[pick], w, *a)) <= FP32_TOL
+    assert rel_fro(gx[pick], oracle_port.conv2d_grad_x(x[pick], w, gz[pick], *a)) <= FP32_TOL
+    halves = ops.conv2d_grad_y(x[:16], w, gz[:16], *a) + ops.conv2d_grad_y(x[16:], w, gz[16:], *a)
+    assert rel_fro(gw, halves) <= FP32_TOL
+    assert rel_fro(ops.conv2d_grad_y(x[pick], w, gz[pick], *a), oracle_port.conv2d_grad_y(x[pick], w, gz[pick], *a)) <= FP32_TOL
+    ip = lambda u, v: float(np.sum(u.astype(np.float64) * v.astype(np.float64)))
+    t = ip(z, gz)
+    assert abs(ip(x, gx) - t) <= 1e-5 * abs(t) + 1e-2 and abs(ip(w, gw) - t) <= 1e-5 * abs(t) + 1e-2
+
+
+@pytest.mark.parametrize("cov", [False, True])
+def test_config5_full_size_properties(oracle_port, cov):
+    """BASELINE config 5 (DeConv2d half, B16 28x28x128, 4x4 stride 2 -> 64 channels) at Deep8's two
+    legal output sizes (58 when not covered, 55 when covered)."""
+    from deep8_amd import ops
+    r = rng(55)
+    B = 16
+    x, w = h(nrm(r, (B, 28, 28, 128))), h(nrm(r, (64, 4, 4, 128), np.sqrt(2.0 / 2048)))
+    a = (cov, 2, 2)
+    z = ops.deconv2d(x, w, *a)
+    assert z.shape == (B, 58, 58, 64) if not cov else (B, 55, 55, 64)
+    gz = h(nrm(r, z.shape))
+    gx, gw = ops.deconv2d_grad_x(x, w, gz, *a), ops.deconv2d_grad_y(x, w, gz, *a)
+    pick = [0, 9]
+    xf, wf, gzf = f(x), f(w), f(gz)
+    assert rel_fro(f(z[pick]), oracle_port.deconv2d(xf[pick], wf, *a)) <= FP16_TOL
+    assert rel_fro(f(gx[pick]), oracle_port.deconv2d_grad_x(xf[pick], wf, gzf[pick], *a)) <= FP16_TOL
+    assert rel_fro(f(ops.deconv2d_grad_y(x[pick], w, gz[pick], *a)),
+                   oracle_port.deconv2d_grad_y(xf[pick], wf, gzf[pick], *a)) <= FP16_TOL
+    ip = lambda u, v: float(np.sum(f(u).astype(np.float64) * f(v).astype(np.float64)))
+    t = ip(z, gz)
+    assert abs(ip(x, gx) - t) <= 4e-3 * abs(t) + 1.0 and abs(ip(w, gw) - t) <= 4e-3 * abs(t) + 1.0
+
+
+def test_config5_literal_56x56_through_explicit_pads(oracle_port):
+    """The config's literal geometry (28 -> 56, PyTorch's ConvTranspose2d(k=4, s=2, p=1)) is not a
+    shape Deep8's DeConv2d admits, but the kernel-level entry points take explicit pads:
+    padTop = padLeft = 2 gives it.  GEMM + gather map here against torch's conv_transpose2d."""
+    torch = pytest.importorskip("torch")
+    from deep8_amd import ops
+    r = rng(56)
+    B, IH, IC, OC, FH, S, OH, P = 2, 28, 128, 64, 4, 2, 56, 2
+    x, w = h(nrm(r, (B, IH, IH, IC))), h(nrm(r, (OC, FH, FH, IC), np.sqrt(2.0 / 2048)))
+    zmat = ops.gemm(0, 1, x.reshape(B * IH * IH, IC), w.reshape(OC * FH * FH, IC))        # [B*IH*IW, OC*FH*FW]
+    z = ops.deconv_col2im(zmat, B, IH, IH, OH, OH, OC, FH, FH, S, S, P, P)
+    assert np.array_equal(f(z), oracle_port.deconv_col2im(f(zmat), B, IH, IH, OH, OH, OC, FH, FH, S, S, P, P).astype(np.float16).astype(np.float32))
+    tx = torch.tensor(f(x), dtype=torch.float64).permute(0, 3, 1, 2)
+    wt = torch.flip(torch.tensor(f(w), dtype=torch.float64), (1, 2)).permute(3, 0, 1, 2)
+    tz = torch.nn.functional.conv_transpose2d(tx, wt, stride=S, padding=FH - 1 - P)
+    assert tuple(tz.shape) == (B, OC, OH, OH)
+    assert rel_fro(f(z), tz.permute(0, 2, 3, 1).numpy()) <= FP16_TOL
+    # and the gradient-side gather with the same pads is the exact transpose of the forward one
+    dz = h(ints(r, (B, OH, OH, OC), 4))
+    dzmat = ops.deconv_im2col(dz, IH, IH, FH, FH, S, S, P, P)
+    assert np.array_equal(f(dzmat), oracle_port.deconv_im2col(f(dz), IH, IH, FH, FH, S, S, P, P))
+    zi = h(ints(r, zmat.shape, 4))
+    lhs = float(np.sum(f(dzmat).astype(np.float64) * f(zi)))
+    rhs = float(np.sum(f(dz).astype(np.float64) * f(ops.deconv_col2im(zi, B, IH, IH, OH, OH, OC, FH, FH, S, S, P, P))))
+    assert lhs == rhs
