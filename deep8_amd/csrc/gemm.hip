@@ -227,6 +227,20 @@ static int launch(GemmArgs &g, int transA, int transB, bool tiled, hipStream_t s
     return 0;
 }
 
+size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red) {
+    int tps = 0;
+    const int splits = plan_splits(gemm_tiled_k_step(dtype), M, N, K, 1, red, (size_t)-1, &tps);
+    return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
+int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
+                   hipStream_t stream) {
+    g.ws = (float *)workspace;
+    g.splits = plan_splits(gemm_tiled_k_step(dtype), g.M, g.N, g.K, g.batch, g.red, workspace ? workspace_bytes : 0,
+                           &g.tiles_per_split);
+    return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, true, stream) : launch<float>(g, transA, transB, true, stream);
+}
+
 }  // namespace d8
 
 using namespace d8;
@@ -285,6 +299,8 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     g.batch = g.red > 1 ? 1 : batch;
     g.splits = 1;
     g.tiles_per_split = 0;
+    g.virt = VIRT_NONE;
+    memset(&g.pg, 0, sizeof(g.pg));
     const bool tiled = K > 0 && gemm_tiled_eligible(dtype, g, transA, transB);
     if (K > 0) {  // K == 0 is the empty reduction: C = beta * C
         const int BK = tiled ? gemm_tiled_k_step(dtype) : (dtype == D8_FLOAT16 ? Tile<f16>::BK : Tile<float>::BK);

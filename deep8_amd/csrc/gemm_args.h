@@ -6,6 +6,22 @@
 
 namespace d8 {
 
+// A patch matrix that is never written out: row m = (b, oy, ox) enumerates an OH x OW grid per
+// image, column (t, c) is channel c of filter tap t = fy * FW + fx, and the element is
+//   image[b][oy * sy + fy * dy - pt][ox * sx + fx * dx - pl][c]      (0 outside the image).
+// dy, dx, pt, pl may be negative, which expresses the gradient-side gather of a stride-1
+// convolution (source row = iy + pt - fy * dy) with the same formula.
+struct PatchGeom {
+    int H, W, C;    // the image [B][H][W][C] the patches are cut from
+    int OH, OW;     // the grid the rows enumerate
+    int FW;         // taps per filter row
+    int sy, sx, dy, dx, pt, pl;
+    unsigned mg_plane, mg_ow;  // floor(2^32 / (OH * OW)), floor(2^32 / OW): division by multiplication
+    unsigned bytes;            // size of the image
+};
+
+enum { VIRT_NONE = 0, VIRT_A_ROWS = 1, VIRT_B_KROWS = 2 };
+
 struct GemmArgs {
     const void *A;
     const void *B;
@@ -19,6 +35,12 @@ struct GemmArgs {
     int splits;           // pieces the extended reduction (red x K tiles) is cut into
     int tiles_per_split;  // K tiles per piece
     float beta;
+    // Implicit convolution: one operand is a patch matrix read straight from the image.
+    //   VIRT_A_ROWS   A is the image; product r of the `red` summed products is filter tap r, its
+    //                 A[m][k] = channel k of tap r of patch row m (K = channels per tap)
+    //   VIRT_B_KROWS  B is the image; B[k][n] = column n of patch row k (N = taps x channels)
+    int virt;
+    PatchGeom pg;
 };
 
 // Tiled kernels (fp16 and fp32) for shapes whose operands can be moved in 16-byte pieces.
@@ -27,6 +49,12 @@ int gemm_tiled_k_step(int dtype);  // K elements per step: 64 (fp16) or 32 (fp32
 bool gemm_tiled_eligible(int dtype, const GemmArgs &g, int transA, int transB);
 // Launch; with g.splits > 1 the fp32 partial sums go to g.ws for the caller to reduce.
 int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipStream_t stream);
+
+// Plan the split of the reduction, launch the tiled kernel (which must be eligible) and reduce.
+int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
+                   hipStream_t stream);
+// Workspace gemm_tiled_run may use for this shape.
+size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red);
 
 }  // namespace d8
 

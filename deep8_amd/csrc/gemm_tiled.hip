@@ -94,12 +94,15 @@ struct Elem<float> {
     }
 };
 
-template <typename E_, int BM_, int BN_, int WGM_, int WGN_, bool A_KC_, bool B_KC_>
+template <typename E_, int BM_, int BN_, int WGM_, int WGN_, bool A_KC_, bool B_KC_, int VIRT_ = VIRT_NONE>
 struct Tile {
     typedef E_ E;
     typedef Elem<E> EL;
     static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
     static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
+    static constexpr int VIRT = VIRT_;  // which operand, if any, is a patch matrix read from its image
+    static_assert(VIRT != VIRT_A_ROWS || A_KC, "patch rows are K-contiguous");
+    static_assert(VIRT != VIRT_B_KROWS || !B_KC, "patch k-rows are N-contiguous");
     static constexpr int ES = sizeof(E), EPV = 16 / ES;  // element size, elements per 16-byte piece
     static constexpr int BK = 128 / ES;                  // K step: 128 bytes of a row
     static constexpr int QUARTERS = 4, KQ = BK / QUARTERS;
@@ -133,13 +136,13 @@ __device__ __host__ constexpr int slot_of(int t, int n, int MQ) { return t * MQ 
 // One K step.  Ar/Br: this lane's operand addresses in the LDS half being multiplied; An/Bn: the
 // same in the other half (next step); Aw/Bw: where this thread's pieces of the next step go;
 // ra/rb: buffer descriptors of the A and B matrices; ga/gb: wave-uniform byte offset (tile origin +
-// K step) of the pieces of the step after that, a_off/b_off: this thread's byte offset in a piece.
+// K step) of the pieces of the step after that, av/bv: this thread's byte offset for each piece.
 template <typename T>
 __device__ __forceinline__ void k_step(const typename T::E *Ar, const typename T::E *Br, const typename T::E *An,
                                        const typename T::E *Bn, typename T::E *Aw, typename T::E *Bw,
                                        __amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb, unsigned ga, unsigned gb,
-                                       unsigned a_pass, unsigned b_pass, unsigned a_off, unsigned b_off,
-                                       u32x4 (&R)[T::NP], typename T::EL::Frag (&fa)[2][T::TM],
+                                       unsigned a_pass, unsigned b_pass, const unsigned (&av)[T::A_IT],
+                                       const unsigned (&bv)[T::B_IT], u32x4 (&R)[T::NP], typename T::EL::Frag (&fa)[2][T::TM],
                                        typename T::EL::Frag (&fb)[2][T::TN], f32x16 (&acc)[T::TM][T::TN]) {
     typedef typename T::E E;
     typedef typename T::EL EL;
@@ -166,8 +169,8 @@ __device__ __forceinline__ void k_step(const typename T::E *Ar, const typename T
             for (int t = 0; t < g_n; ++t)
                 if (slot_of(t, g_n, MQ) == m) {
                     const int p = g_lo + t;
-                    R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, ga + p * a_pass, 0)
-                                    : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, gb + (p - A_IT) * b_pass, 0);
+                    R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, av[p < A_IT ? p : 0], ga + p * a_pass, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(rb, bv[p < A_IT ? 0 : p - A_IT], gb + (p - A_IT) * b_pass, 0);
                 }
             // operands of the next quarter (of the next step's first quarter when q == 3)
 #pragma unroll
@@ -315,21 +318,53 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // blockIdx.z = output batch index * splits + piece of the reduction.  The reduction runs over
     // `red` products (1 unless the whole batch is summed into one C) times K, cut into `splits`.
     const int b = blockIdx.z / g.splits, split = blockIdx.z - b * g.splits;
+    constexpr int VIRT = T::VIRT, B_IT = T::B_IT;
+    const PatchGeom &pg = g.pg;
     const long a_rows = A_KC ? g.M : g.K, b_rows = B_KC ? g.N : g.K;
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)((const E *)g.A + (long)b * g.sA), 0, (int)(ES * ((g.red - 1) * g.sA + a_rows * g.lda)), 0x00020000);
+        (void *)((const E *)g.A + (long)b * g.sA), 0,
+        VIRT == VIRT_A_ROWS ? (int)pg.bytes : (int)(ES * ((g.red - 1) * g.sA + a_rows * g.lda)), 0x00020000);
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)((const E *)g.B + (long)b * g.sB), 0, (int)(ES * ((g.red - 1) * g.sB + b_rows * g.ldb)), 0x00020000);
+        (void *)((const E *)g.B + (long)b * g.sB), 0,
+        VIRT == VIRT_B_KROWS ? (int)pg.bytes : (int)(ES * ((g.red - 1) * g.sB + b_rows * g.ldb)), 0x00020000);
     const unsigned Au = (unsigned)ES * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0);
     const unsigned Bu = (unsigned)ES * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
     const int a_r = A_KC ? tid >> 3 : tid / (BM / EPV), a_c = A_KC ? tid & 7 : tid % (BM / EPV);
     const int b_r = B_KC ? tid >> 3 : tid / (BN / EPV), b_c = B_KC ? tid & 7 : tid % (BN / EPV);
-    const unsigned a_off = (unsigned)ES * ((unsigned)a_r * (unsigned)g.lda + a_c * EPV);
-    const unsigned b_off = (unsigned)ES * ((unsigned)b_r * (unsigned)g.ldb + b_c * EPV);
     const int a_dst = a_r * A_LD + a_c * EPV, b_dst = b_r * B_LD + b_c * EPV;
-    const unsigned a_pass = (unsigned)ES * T::A_ROWS * g.lda, b_pass = (unsigned)ES * T::B_ROWS * g.ldb;  // bytes
+    const unsigned a_pass = VIRT == VIRT_A_ROWS ? 0u : (unsigned)ES * T::A_ROWS * g.lda;  // bytes
+    const unsigned b_pass = VIRT == VIRT_B_KROWS ? 0u : (unsigned)ES * T::B_ROWS * g.ldb;
     const unsigned a_step = A_KC ? 128u : (unsigned)ES * BK * g.lda;
     const unsigned b_step = B_KC ? 128u : (unsigned)ES * BK * g.ldb;
+    // per-thread byte offset of each piece: one value for a real matrix, recomputed every step
+    // for a patch matrix (an offset beyond the image makes the buffer load return zeros)
+    constexpr unsigned OUTSIDE = 0x80000000u;
+    unsigned av[A_IT], bv[B_IT];
+#pragma unroll
+    for (int p = 0; p < A_IT; ++p) av[p] = (unsigned)ES * ((unsigned)a_r * (unsigned)g.lda + a_c * EPV);
+#pragma unroll
+    for (int p = 0; p < B_IT; ++p) bv[p] = (unsigned)ES * ((unsigned)b_r * (unsigned)g.ldb + b_c * EPV);
+    // patch rows as A: this thread's rows never change; a step selects the tap
+    int va_base[A_IT], va_iy[A_IT], va_ix[A_IT];
+    if constexpr (VIRT == VIRT_A_ROWS) {
+        const int plane = pg.OH * pg.OW;
+#pragma unroll
+        for (int p = 0; p < A_IT; ++p) {
+            const int m = m0 + a_r + p * T::A_ROWS, img = m / plane, rem = m - img * plane;
+            const int oy = rem / pg.OW, ox = rem - oy * pg.OW;
+            va_iy[p] = oy * pg.sy - pg.pt;
+            va_ix[p] = ox * pg.sx - pg.pl;
+            va_base[p] = (((img * pg.H + va_iy[p]) * pg.W + va_ix[p]) * pg.C + a_c * EPV) * ES;
+        }
+    }
+    // patch k-rows as B: this thread's tap and channel never change; a step selects the rows
+    int vb_dy = 0, vb_dx = 0, vb_c = 0;
+    if constexpr (VIRT == VIRT_B_KROWS) {
+        const int n = n0 + b_c * EPV, t = n / pg.C, fy = t / pg.FW, fx = t - fy * pg.FW;
+        vb_c = n - t * pg.C;
+        vb_dy = fy * pg.dy - pg.pt;
+        vb_dx = fx * pg.dx - pg.pl;
+    }
 
     // ---- per-lane LDS offsets of its MFMA operands
     const int a_frag = A_KC ? EL::kc_offset(lane, A_LD, wm * TM * 32) : EL::tr_offset(lane, A_LD, wm * TM * 32);
@@ -350,13 +385,40 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const int ktiles = g.K / BK;
     const int x0 = split * g.tiles_per_split, nsteps = min(g.red * ktiles, x0 + g.tiles_per_split) - x0;
     const unsigned a_prod = (unsigned)ES * (unsigned)g.sA, b_prod = (unsigned)ES * (unsigned)g.sB;
-    auto step_a = [&](int i) {
+    auto step_a = [&](int i) -> unsigned {
         const int x = x0 + min(i, nsteps - 1), r = x / ktiles;  // past the end: refetch the last step, never used
-        return Au + (g.red > 1 ? r * a_prod : 0u) + (x - r * ktiles) * a_step;
+        if constexpr (VIRT == VIRT_A_ROWS) {
+            const int fy = r / pg.FW, fx = r - fy * pg.FW, tdy = fy * pg.dy, tdx = fx * pg.dx;
+            const int toff = ((tdy * pg.W + tdx) * pg.C + (x - r * ktiles) * BK) * ES;
+#pragma unroll
+            for (int p = 0; p < A_IT; ++p) {
+                const bool inside = (unsigned)(va_iy[p] + tdy) < (unsigned)pg.H && (unsigned)(va_ix[p] + tdx) < (unsigned)pg.W;
+                av[p] = inside ? (unsigned)(va_base[p] + toff) : OUTSIDE;
+            }
+            return 0u;
+        } else {
+            return Au + (g.red > 1 ? r * a_prod : 0u) + (x - r * ktiles) * a_step;
+        }
     };
-    auto step_b = [&](int i) {
+    auto step_b = [&](int i) -> unsigned {
         const int x = x0 + min(i, nsteps - 1), r = x / ktiles;
-        return Bu + (g.red > 1 ? r * b_prod : 0u) + (x - r * ktiles) * b_step;
+        if constexpr (VIRT == VIRT_B_KROWS) {
+            const unsigned plane = pg.OH * pg.OW;
+#pragma unroll
+            for (int p = 0; p < B_IT; ++p) {
+                const unsigned m = (unsigned)x * BK + b_r + p * T::B_ROWS;
+                unsigned img = __umulhi(m, pg.mg_plane), rem = m - img * plane;
+                if (rem >= plane) ++img, rem -= plane;
+                unsigned oy = __umulhi(rem, pg.mg_ow), ox = rem - oy * pg.OW;
+                if (ox >= (unsigned)pg.OW) ++oy, ox -= pg.OW;
+                const int iy = (int)oy * pg.sy + vb_dy, ix = (int)ox * pg.sx + vb_dx;
+                const bool inside = (unsigned)iy < (unsigned)pg.H && (unsigned)ix < (unsigned)pg.W;
+                bv[p] = inside ? (unsigned)(((((int)img * pg.H + iy) * pg.W + ix) * pg.C + vb_c) * ES) : OUTSIDE;
+            }
+            return 0u;
+        } else {
+            return Bu + (g.red > 1 ? r * b_prod : 0u) + (x - r * ktiles) * b_step;
+        }
     };
 
     // ---- prologue: step 0 into LDS half 0, step 1 into registers, first operands of step 0
@@ -364,8 +426,8 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         const unsigned pa = step_a(0), pb = step_b(0);
 #pragma unroll
         for (int p = 0; p < NP; ++p)
-            R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, pa + p * a_pass, 0)
-                            : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, pb + (p - A_IT) * b_pass, 0);
+            R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, av[p < A_IT ? p : 0], pa + p * a_pass, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(rb, bv[p < A_IT ? 0 : p - A_IT], pb + (p - A_IT) * b_pass, 0);
     }
 #pragma unroll
     for (int p = 0; p < NP; ++p)
@@ -374,8 +436,8 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         const unsigned pa = step_a(1), pb = step_b(1);
 #pragma unroll
         for (int p = 0; p < NP; ++p)
-            R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, a_off, pa + p * a_pass, 0)
-                            : __builtin_amdgcn_raw_buffer_load_b128(rb, b_off, pb + (p - A_IT) * b_pass, 0);
+            R[p] = p < A_IT ? __builtin_amdgcn_raw_buffer_load_b128(ra, av[p < A_IT ? p : 0], pa + p * a_pass, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(rb, bv[p < A_IT ? 0 : p - A_IT], pb + (p - A_IT) * b_pass, 0);
     }
     __syncthreads();
 #pragma unroll
@@ -387,11 +449,16 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
 
     // ---- main loop, two steps per trip so that the LDS half of every access is known statically;
     for (int i = 0; i < nsteps; i += 2) {
-        k_step<T>(As0 + a_frag, Bs0 + b_frag, As1 + a_frag, Bs1 + b_frag, As1 + a_dst, Bs1 + b_dst, ra, rb,
-                  step_a(i + 2), step_b(i + 2), a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
-        if (i + 1 < nsteps)
-            k_step<T>(As1 + a_frag, Bs1 + b_frag, As0 + a_frag, Bs0 + b_frag, As0 + a_dst, Bs0 + b_dst, ra, rb,
-                      step_a(i + 3), step_b(i + 3), a_pass, b_pass, a_off, b_off, R, fa, fb, acc);
+        {
+            const unsigned pa = step_a(i + 2), pb = step_b(i + 2);
+            k_step<T>(As0 + a_frag, Bs0 + b_frag, As1 + a_frag, Bs1 + b_frag, As1 + a_dst, Bs1 + b_dst, ra, rb, pa, pb,
+                      a_pass, b_pass, av, bv, R, fa, fb, acc);
+        }
+        if (i + 1 < nsteps) {
+            const unsigned pa = step_a(i + 3), pb = step_b(i + 3);
+            k_step<T>(As1 + a_frag, Bs1 + b_frag, As0 + a_frag, Bs0 + b_frag, As0 + a_dst, Bs0 + b_dst, ra, rb, pa, pb,
+                      a_pass, b_pass, av, bv, R, fa, fb, acc);
+        }
     }
 
     // ---- epilogue: the result itself, or this piece's fp32 partial sums when the reduction is split
@@ -405,16 +472,16 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
                          g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o);
 }
 
-template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC>
+template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int VIRT>
 static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
-    typedef Tile<E, BM, BN, WGM, WGN, A_KC, B_KC> T;
+    typedef Tile<E, BM, BN, WGM, WGN, A_KC, B_KC, VIRT> T;
     const int tilesM = ceil_div(g.M, BM), tilesN = ceil_div(g.N, BN);
     hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, g.batch * g.splits), dim3(T::NT), 0, stream, g, tilesM, tilesN);
     D8_LAUNCH_CHECK();
     return 0;
 }
 
-template <typename E, bool A_KC, bool B_KC>
+template <typename E, bool A_KC, bool B_KC, int VIRT = VIRT_NONE>
 static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     static const char *force = getenv("D8_GEMM_TILE");  // tuning aid
     const long big_tiles = (long)ceil_div(g.M, 256) * ceil_div(g.N, 256) * g.batch * g.splits;
@@ -423,22 +490,27 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     // fp32 runs 64-cycle MFMAs on a quarter of the bytes per flop: the 128 x 128 tile already
     // keeps the matrix pipe fed, and the compiler cannot hold the 256 x 256 variant in registers
     if constexpr (sizeof(E) == 2) {
-        if (big) return launch_tiled<E, 256, 256, 4, 2, A_KC, B_KC>(g, stream);
+        if (big) return launch_tiled<E, 256, 256, 4, 2, A_KC, B_KC, VIRT>(g, stream);
     }
     // a 64-wide side gets a tile of that width (im2col products with 64 output channels)
-    if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC>(g, stream);
-    if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC>(g, stream);
-    return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC>(g, stream);
+    if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+    if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+    return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
 }
 
 template <typename E>
 static bool eligible(const GemmArgs &g, int transA, int transB) {
     constexpr long ES = sizeof(E), EPV = 16 / ES, BK = 128 / ES;
+    const bool va = g.virt == VIRT_A_ROWS, vb = g.virt == VIRT_B_KROWS;
+    if (va && (transA || g.K != g.pg.C)) return false;                       // a K step stays inside one tap
+    if (vb && (!transA || transB || g.red != 1 || g.pg.C % EPV || g.N % g.pg.C)) return false;  // a piece stays inside one tap
+    if ((va || vb) && (g.pg.bytes >= (1u << 31) || g.batch != 1)) return false;
     // byte offsets inside one operand (all summed products of it included) are 32-bit
-    if (((g.red - 1) * g.sA + (long)(transA ? g.K : g.M) * g.lda) * ES >= (1L << 31)) return false;
-    if (((g.red - 1) * g.sB + (long)(transB ? g.N : g.K) * g.ldb) * ES >= (1L << 31)) return false;
-    if (g.M < 64 || g.N < 64 || (g.M < 128 && g.N < 128) || g.K < BK || g.K % BK || g.lda % EPV || g.ldb % EPV || g.sA % EPV || g.sB % EPV)
-        return false;
+    if (!va && ((g.red - 1) * g.sA + (long)(transA ? g.K : g.M) * g.lda) * ES >= (1L << 31)) return false;
+    if (!vb && ((g.red - 1) * g.sB + (long)(transB ? g.N : g.K) * g.ldb) * ES >= (1L << 31)) return false;
+    if (g.M < 64 || g.N < 64 || (g.M < 128 && g.N < 128) || g.K < BK || g.K % BK) return false;
+    if (!va && (g.lda % EPV || g.sA % EPV)) return false;
+    if (!vb && (g.ldb % EPV || g.sB % EPV)) return false;
     if (((size_t)g.A | (size_t)g.B) & 15) return false;
     if (transA && g.M % EPV) return false;
     if (!transB && g.N % EPV) return false;
@@ -448,6 +520,8 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
 
 template <typename E>
 static int launch_any(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
+    if (g.virt == VIRT_A_ROWS) return transB ? pick_tile<E, true, true, VIRT_A_ROWS>(g, stream) : pick_tile<E, true, false, VIRT_A_ROWS>(g, stream);
+    if (g.virt == VIRT_B_KROWS) return pick_tile<E, false, false, VIRT_B_KROWS>(g, stream);
     if (!transA && !transB) return pick_tile<E, true, false>(g, stream);
     if (!transA && transB) return pick_tile<E, true, true>(g, stream);
     return pick_tile<E, false, false>(g, stream);

@@ -5,7 +5,7 @@
 //   MatrixMultiply   deep8/src/math/MatrixMultiply.cu:21-57 (fwd), :193-232 (GradX), :381-420 (GradY)
 //   Conv2d           deep8/src/math/Conv2d.cu:145-196, :440-492, :750-802, pads :332-336
 //   DeConv2d         deep8/src/math/DeConv2d.cu:76-131, :371-429, :642-700, pads :99-100
-#include "common.h"
+#include "gemm_args.h"
 
 namespace d8 {
 
@@ -74,6 +74,59 @@ static int check_conv(const char *who, int dtype, int B, int IH, int IW, int IC,
     D8_REQUIRE(B > 0 && IH > 0 && IW > 0 && IC > 0 && OC > 0 && FH > 0 && FW > 0, "%s: sizes must be positive", who);
     D8_REQUIRE(sy >= 1 && sx >= 1 && dy >= 1 && dx >= 1, "%s: the stride and dilation must >= 1", who);
     return 0;
+}
+
+// ---- implicit convolution: the patch matrix is read straight from the image by the GEMM's tile
+// loader instead of being written out and read back.  which: 0 forward, 1 gradient of x (stride 1
+// only), 2 gradient of the filter.  Returns false when the shape does not qualify; the caller then
+// takes the im2col / col2im route.
+struct ConvShape {
+    int B, IH, IW, IC, OC, FH, FW, OH, OW, sy, sx, dy, dx, pt, pl;
+};
+
+static unsigned magic_of(unsigned d) { return d <= 1 ? 0xFFFFFFFFu : (unsigned)((1ull << 32) / d); }
+
+static bool conv_implicit_plan(int dtype, int which, const ConvShape &c, const void *x, const void *w, const void *z,
+                               GemmArgs &g, int &ta, int &tb) {
+    const bool off = getenv("D8_CONV_EXPLICIT") != nullptr;  // tuning and test aid: force the im2col route
+    if (off) return false;
+    const long es = (long)dtype_bytes(dtype);
+    const long taps = (long)c.FH * c.FW, M = (long)c.B * c.OH * c.OW, K = taps * c.IC;
+    if (M >= (1L << 31) || K >= (1L << 31) || (long)c.B * c.IH * c.IW * c.IC * es >= (1L << 31) || M * c.OC * es >= (1L << 31))
+        return false;
+    memset(&g, 0, sizeof(g));
+    g.batch = 1;
+    g.red = 1;
+    g.splits = 1;
+    PatchGeom &pg = g.pg;
+    if (which == 1) {  // dx[(b,iy,ix)][ic] += sum over taps of dz[b][iy + pt - fy*dy][ix + pl - fx*dx][:] . w[:][tap][ic]
+        if (c.sy != 1 || c.sx != 1) return false;
+        pg = {c.OH, c.OW, c.OC, c.IH, c.IW, c.FW, 1, 1, -c.dy, -c.dx, -c.pt, -c.pl, 0, 0, (unsigned)(M * c.OC * es)};
+        g.virt = VIRT_A_ROWS;
+        g.A = z, g.B = w, g.C = (void *)x;
+        g.M = c.B * c.IH * c.IW, g.N = c.IC, g.K = c.OC;
+        g.ldb = (int)K, g.sB = c.IC, g.ldc = c.IC, g.red = (int)taps, g.beta = 1.f;
+        ta = 0, tb = 0;
+    } else {
+        pg = {c.IH, c.IW, c.IC, c.OH, c.OW, c.FW, c.sy, c.sx, c.dy, c.dx, c.pt, c.pl, 0, 0,
+              (unsigned)((long)c.B * c.IH * c.IW * c.IC * es)};
+        if (which == 0) {  // z[(b,oy,ox)][oc] = sum over taps of patch_tap(x) . w[oc][tap][:]
+            g.virt = VIRT_A_ROWS;
+            g.A = x, g.B = w, g.C = (void *)z;
+            g.M = (int)M, g.N = c.OC, g.K = c.IC;
+            g.ldb = (int)K, g.sB = c.IC, g.ldc = c.OC, g.red = (int)taps, g.beta = 0.f;
+            ta = 0, tb = 1;
+        } else {  // dw[oc][(tap,ic)] += sum over patch rows of dz[row][oc] . patch(x)[row][(tap,ic)]
+            g.virt = VIRT_B_KROWS;
+            g.A = z, g.B = x, g.C = (void *)w;
+            g.M = c.OC, g.N = (int)K, g.K = (int)M;
+            g.lda = c.OC, g.ldc = (int)K, g.beta = 1.f;
+            ta = 1, tb = 0;
+        }
+    }
+    pg.mg_plane = magic_of((unsigned)pg.OH * pg.OW);
+    pg.mg_ow = magic_of((unsigned)pg.OW);
+    return gemm_tiled_eligible(dtype, g, ta, tb);
 }
 
 }  // namespace d8
@@ -164,6 +217,11 @@ size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int 
     if (check_conv("d8_conv2d_scratch_bytes", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return 0;
     if (d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return 0;
     const int M = B * g[0] * g[1], K = FH * FW * IC;
+    const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
+    GemmArgs ga;
+    int ta, tb;
+    if (conv_implicit_plan(dtype, which, cs, nullptr, nullptr, nullptr, ga, ta, tb))
+        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
     return col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
 }
@@ -177,7 +235,15 @@ int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
     if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
     const int M = B * g[0] * g[1], K = FH * FW * IC;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
-    D8_REQUIRE(x && w && z && scratch, "d8_conv2d: null tensor");
+    D8_REQUIRE(x && w && z, "d8_conv2d: null tensor");
+    {
+        const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
+        GemmArgs ga;
+        int ta, tb;
+        if (conv_implicit_plan(dtype, 0, cs, x, w, z, ga, ta, tb))
+            return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+    }
+    D8_REQUIRE(scratch, "d8_conv2d: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d: scratch too small");
     if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
         return rc;
@@ -194,7 +260,15 @@ int d8_conv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
     if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
     const int M = B * g[0] * g[1], K = FH * FW * IC;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
-    D8_REQUIRE(gx && w && gz && scratch, "d8_conv2d_grad_x: null tensor");
+    D8_REQUIRE(gx && w && gz, "d8_conv2d_grad_x: null tensor");
+    {
+        const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
+        GemmArgs ga;
+        int ta, tb;
+        if (conv_implicit_plan(dtype, 1, cs, gx, w, gz, ga, ta, tb))
+            return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+    }
+    D8_REQUIRE(scratch, "d8_conv2d_grad_x: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_x: scratch too small");
     const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
     if (int rc = run(dtype, conv_plan(1, M, K, OC, scratch, w, gz), ws ? (char *)scratch + col : nullptr, ws, stream))
@@ -211,7 +285,15 @@ int d8_conv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
     if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
     const int M = B * g[0] * g[1], K = FH * FW * IC;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
-    D8_REQUIRE(x && gw && gz && scratch, "d8_conv2d_grad_y: null tensor");
+    D8_REQUIRE(x && gw && gz, "d8_conv2d_grad_y: null tensor");
+    {
+        const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
+        GemmArgs ga;
+        int ta, tb;
+        if (conv_implicit_plan(dtype, 2, cs, x, gw, gz, ga, ta, tb))
+            return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+    }
+    D8_REQUIRE(scratch, "d8_conv2d_grad_y: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_y: scratch too small");
     if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
         return rc;

@@ -234,3 +234,59 @@ def test_config5_literal_56x56_through_explicit_pads(oracle_port):
     lhs = float(np.sum(f(dzmat).astype(np.float64) * f(zi)))
     rhs = float(np.sum(f(dz).astype(np.float64) * f(ops.deconv_col2im(zi, B, IH, IH, OH, OH, OC, FH, FH, S, S, P, P))))
     assert lhs == rhs
+
+
+# Shapes whose patch matrix is read by the GEMM's tile loader straight from the image (channel
+# counts that are multiples of the K step; 64-wide or wider outputs).  (cfg, passes expected implicit
+# for fp32, for half)
+IMPLICIT = [
+    ((2, 16, 16, 64, 64, 3, 3, True, 1, 1, 1, 1), (0, 1, 2), (0, 1, 2)),
+    ((2, 16, 16, 64, 128, 3, 3, False, 1, 1, 1, 1), (0, 1), (0, 1)),       # 392 patch rows: ragged tiles, explicit dW
+    ((4, 16, 16, 32, 64, 3, 3, True, 2, 2, 1, 1), (0, 2), (2,)),           # stride 2: dX stays explicit
+    ((2, 20, 12, 64, 96, 5, 3, True, 1, 1, 2, 2), (0, 1, 2), (0,)),       # dilation, 5x3 filter, non-square image
+    ((8, 8, 8, 64, 192, 2, 2, False, 1, 1, 1, 1), (0, 1), (0, 1)),
+    ((1, 16, 16, 128, 64, 3, 3, True, 1, 1, 1, 1), (0, 1, 2), (0, 1, 2)),
+]
+
+
+@pytest.mark.parametrize("cfg,imp32,imp16", IMPLICIT)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_conv2d_implicit_route(oracle_port, monkeypatch, cfg, imp32, imp16, dtype):
+    """The implicit route against the oracle (integers bit-exact, reals within tolerance) and
+    against the im2col route forced through the same entry points."""
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    a = (cov, sy, sx, dy, dx)
+    OH, OW, _, _ = ops.conv2d_geometry(IH, IW, FH, FW, *a)
+    for which in range(3):  # the implicit route asks for a different scratch size than the im2col route
+        q = lambda: lib.d8_conv2d_scratch_bytes(capi.dtype_id(np.dtype(dtype)), which, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx, dy, dx)
+        monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+        explicit = q()
+        assert explicit >= B * OH * OW * FH * FW * IC * np.dtype(dtype).itemsize
+        monkeypatch.delenv("D8_CONV_EXPLICIT")
+        assert (q() != explicit) == (which in (imp32 if dtype == np.float32 else imp16)), (which, q(), explicit)
+    r = rng(B + IH + OC + 77)
+    c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
+    hi = 3 if dtype == np.float16 else 20
+    tol = FP16_TOL if dtype == np.float16 else FP32_TOL
+    # integers, thinned for half so that every sum stays exact
+    x, w = ints(r, (B, IH, IW, IC), hi), ints(r, (OC, FH, FW, IC), hi)
+    gz = ints(r, (B, OH, OW, OC), hi)
+    if dtype == np.float16:
+        x, w, gz = x * (r.random(x.shape) < 0.3), w * (r.random(w.shape) < 0.3), gz * (r.random(gz.shape) < 0.1)
+    want = (oracle_port.conv2d(x, w, *a), oracle_port.conv2d_grad_x(x, w, gz, *a, x), oracle_port.conv2d_grad_y(x, w, gz, *a, w))
+    assert dtype == np.float32 or max(np.abs(t).max() for t in want) < 2048
+    got = (ops.conv2d(c(x), c(w), *a), ops.conv2d_grad_x(c(x), c(w), c(gz), *a, c(x)), ops.conv2d_grad_y(c(x), c(w), c(gz), *a, c(w)))
+    for g_, w_ in zip(got, want):
+        assert np.array_equal(f(g_), w_)
+    # reals: both routes within tolerance of the oracle
+    x, w = c(nrm(r, (B, IH, IW, IC))), c(nrm(r, (OC, FH, FW, IC), np.sqrt(2.0 / (FH * FW * IC))))
+    gz = c(nrm(r, (B, OH, OW, OC)))
+    want = (oracle_port.conv2d(f(x), f(w), *a), oracle_port.conv2d_grad_x(f(x), f(w), f(gz), *a), oracle_port.conv2d_grad_y(f(x), f(w), f(gz), *a))
+    for route in ("implicit", "explicit"):
+        if route == "explicit":
+            monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+        got = (ops.conv2d(x, w, *a), ops.conv2d_grad_x(x, w, gz, *a), ops.conv2d_grad_y(x, w, gz, *a))
+        for k, (g_, w_) in enumerate(zip(got, want)):
+            assert rel_fro(f(g_), w_) <= tol, (route, k)
