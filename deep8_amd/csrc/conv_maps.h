@@ -1,0 +1,24 @@
+// Geometry of the gather maps and their internal launchers (the exported entry points check their
+// arguments and call these; the DeConv2d operators call them with a mirrored geometry).
+#ifndef DEEP8_AMD_CONV_MAPS_H
+#define DEEP8_AMD_CONV_MAPS_H
+
+#include "common.h"
+
+namespace d8 {
+
+// Patch row (b, oy, ox) of an OH x OW grid, tap (fy, fx), reads image pixel
+// (oy * sy + fy * dy - pt, ox * sx + fx * dx - pl) of a [B][IH][IW][C] image.  dy, dx, pt, pl may
+// be negative (the DeConv2d maps are this map with dy = dx = -1 and negated pads).
+struct MapGeom {
+    int B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, pt, pl;
+};
+
+// col[(b,oy,ox)][(fy,fx,c)] = image pixel or 0
+int launch_im2col(int dtype, const void *im, void *col, const MapGeom &g, hipStream_t stream);
+// im (+)= the transpose of that map applied to col; taps added in (fy, fx) ascending order
+int launch_col2im(int dtype, const void *col, void *im, const MapGeom &g, bool accumulate, hipStream_t stream);
+
+}  // namespace d8
+
+#endif

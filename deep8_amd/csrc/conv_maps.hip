@@ -4,13 +4,9 @@
 //
 // Replaces Conv2dIm2ColKernel / Conv2dCol2ImKernel (deep8/src/math/Conv2d.cu:10-118) and
 // DeConv2dCol2ImKernel / DeConv2dIm2ColKernel (deep8/src/math/DeConv2d.cu:11-58,310-351).
-#include "common.h"
+#include "conv_maps.h"
 
 namespace d8 {
-
-struct MapGeom {
-    int B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, pt, pl;
-};
 
 static inline int grid_for(long work, int block) {
     long blocks = (work + block - 1) / block;
@@ -47,7 +43,7 @@ __global__ __launch_bounds__(256) void im2col_kernel(const V *__restrict__ im, V
 
 // ---- col2im: one thread owns VEC channels of one image pixel; taps are added in (fy, fx)
 // ascending order into registers, then the pixel is written once. -----------------------------
-template <typename T, int VEC>
+template <typename T, int VEC, bool ACC>
 __global__ __launch_bounds__(256) void col2im_kernel(const T *__restrict__ col, T *__restrict__ im,
                                                      MapGeom g, long total) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
@@ -62,7 +58,9 @@ __global__ __launch_bounds__(256) void col2im_kernel(const T *__restrict__ col, 
         const int iy = (int)(q % g.IH), b = (int)(q / g.IH);
         T *dst = im + p * g.C + (long)cv * VEC;
         float acc[VEC];
-        {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+        if (ACC) {
             VT v = *(const VT *)dst;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc[e] = (float)v[e];
@@ -90,7 +88,7 @@ __global__ __launch_bounds__(256) void col2im_kernel(const T *__restrict__ col, 
     }
 }
 
-template <typename T>
+template <typename T, bool ACC>
 __global__ __launch_bounds__(256) void col2im_scalar_kernel(const T *__restrict__ col, T *__restrict__ im,
                                                             MapGeom g, long total) {
     const long K = (long)g.FH * g.FW * g.C;
@@ -101,7 +99,7 @@ __global__ __launch_bounds__(256) void col2im_scalar_kernel(const T *__restrict_
         const int ix = (int)(p % g.IW);
         const long q = p / g.IW;
         const int iy = (int)(q % g.IH), b = (int)(q / g.IH);
-        float acc = (float)im[idx];
+        float acc = ACC ? (float)im[idx] : 0.f;
         for (int fy = 0; fy < g.FH; ++fy) {
             const int ty = iy + g.pt - fy * g.dy;
             if (ty < 0 || ty % g.sy) continue;
@@ -188,6 +186,52 @@ static int check_geom(const char *who, int dtype, const void *a, const void *b, 
 
 static inline bool aligned16(const void *p) { return ((size_t)p & 15) == 0; }
 
+int launch_im2col(int dtype, const void *im, void *col, const MapGeom &g, hipStream_t s) {
+    if (g.B == 0) return 0;
+    const size_t es = dtype_bytes(dtype);
+    const long elems = (long)g.B * g.OH * g.OW * g.FH * g.FW * g.C;
+    const size_t row_bytes = (size_t)g.C * es;
+    if (row_bytes % 16 == 0 && aligned16(im) && aligned16(col)) {
+        const int CV = (int)(row_bytes / 16);
+        const long total = elems / (16 / es);
+        hipLaunchKernelGGL((im2col_kernel<uint4>), dim3(grid_for(total, 256)), dim3(256), 0, s,
+                           (const uint4 *)im, (uint4 *)col, g, CV, total);
+    } else if (es == 4) {
+        hipLaunchKernelGGL((im2col_kernel<unsigned>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned *)im, (unsigned *)col, g, g.C, elems);
+    } else {
+        hipLaunchKernelGGL((im2col_kernel<unsigned short>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned short *)im, (unsigned short *)col, g, g.C, elems);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename T, int VEC, bool ACC>
+static void launch_col2im_t(const void *col, void *im, const MapGeom &g, bool vec, long elems, hipStream_t s) {
+    if (vec)
+        hipLaunchKernelGGL((col2im_kernel<T, VEC, ACC>), dim3(grid_for(elems / VEC, 256)), dim3(256), 0, s,
+                           (const T *)col, (T *)im, g, elems / VEC);
+    else
+        hipLaunchKernelGGL((col2im_scalar_kernel<T, ACC>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const T *)col, (T *)im, g, elems);
+}
+
+int launch_col2im(int dtype, const void *col, void *im, const MapGeom &g, bool accumulate, hipStream_t s) {
+    if (g.B == 0) return 0;
+    const long elems = (long)g.B * g.IH * g.IW * g.C;
+    const bool al = aligned16(im) && aligned16(col);
+    if (dtype == D8_FLOAT32) {
+        if (accumulate) launch_col2im_t<float, 4, true>(col, im, g, g.C % 4 == 0 && al, elems, s);
+        else launch_col2im_t<float, 4, false>(col, im, g, g.C % 4 == 0 && al, elems, s);
+    } else {
+        if (accumulate) launch_col2im_t<f16, 8, true>(col, im, g, g.C % 8 == 0 && al, elems, s);
+        else launch_col2im_t<f16, 8, false>(col, im, g, g.C % 8 == 0 && al, elems, s);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
 }  // namespace d8
 
 using namespace d8;
@@ -199,25 +243,7 @@ int d8_im2col(int dtype, const void *im, void *col,
               int sy, int sx, int dy, int dx, int padTop, int padLeft, void *stream) {
     MapGeom g = {B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft};
     if (int rc = check_geom("d8_im2col", dtype, im, col, g)) return rc;
-    if (B == 0) return 0;
-    const size_t es = dtype_bytes(dtype);
-    const long elems = (long)B * OH * OW * FH * FW * C;
-    const size_t row_bytes = (size_t)C * es;
-    hipStream_t s = as_stream(stream);
-    if (row_bytes % 16 == 0 && aligned16(im) && aligned16(col)) {
-        const int CV = (int)(row_bytes / 16);
-        const long total = elems / (16 / es);
-        hipLaunchKernelGGL((im2col_kernel<uint4>), dim3(grid_for(total, 256)), dim3(256), 0, s,
-                           (const uint4 *)im, (uint4 *)col, g, CV, total);
-    } else if (es == 4) {
-        hipLaunchKernelGGL((im2col_kernel<unsigned>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
-                           (const unsigned *)im, (unsigned *)col, g, C, elems);
-    } else {
-        hipLaunchKernelGGL((im2col_kernel<unsigned short>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
-                           (const unsigned short *)im, (unsigned short *)col, g, C, elems);
-    }
-    D8_LAUNCH_CHECK();
-    return 0;
+    return launch_im2col(dtype, im, col, g, as_stream(stream));
 }
 
 int d8_col2im(int dtype, const void *col, void *im,
@@ -225,27 +251,7 @@ int d8_col2im(int dtype, const void *col, void *im,
               int sy, int sx, int dy, int dx, int padTop, int padLeft, void *stream) {
     MapGeom g = {B, IH, IW, C, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft};
     if (int rc = check_geom("d8_col2im", dtype, col, im, g)) return rc;
-    if (B == 0) return 0;
-    const long elems = (long)B * IH * IW * C;
-    hipStream_t s = as_stream(stream);
-    const bool al = aligned16(im) && aligned16(col);
-    if (dtype == D8_FLOAT32) {
-        if (C % 4 == 0 && al)
-            hipLaunchKernelGGL((col2im_kernel<float, 4>), dim3(grid_for(elems / 4, 256)), dim3(256), 0, s,
-                               (const float *)col, (float *)im, g, elems / 4);
-        else
-            hipLaunchKernelGGL((col2im_scalar_kernel<float>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
-                               (const float *)col, (float *)im, g, elems);
-    } else {
-        if (C % 8 == 0 && al)
-            hipLaunchKernelGGL((col2im_kernel<f16, 8>), dim3(grid_for(elems / 8, 256)), dim3(256), 0, s,
-                               (const f16 *)col, (f16 *)im, g, elems / 8);
-        else
-            hipLaunchKernelGGL((col2im_scalar_kernel<f16>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
-                               (const f16 *)col, (f16 *)im, g, elems);
-    }
-    D8_LAUNCH_CHECK();
-    return 0;
+    return launch_col2im(dtype, col, im, g, true, as_stream(stream));
 }
 
 int d8_deconv_col2im(int dtype, const void *zmat, void *z,

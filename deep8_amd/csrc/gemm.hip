@@ -163,9 +163,42 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(GemmArgs g) {
         }
 }
 
-// C[b][m][n] = beta * C + sum_s ws[b][s][m][n]; partials are added in split order.
+// C[b][m][n] = beta * C + sum_s ws[b][s][m][n].  A workgroup covers 32 groups of 4 consecutive
+// outputs; its 8 thread rows each add every 8th partial (16-byte loads), and the 8 sums meet in
+// LDS in a fixed order, so the result does not depend on scheduling.
 template <typename T>
-__global__ void gemm_split_reduce_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(GemmArgs g) {
+    __shared__ f32x4 part[8][32];
+    const long mn = (long)g.M * g.N;
+    const int lane = threadIdx.x & 31, row = threadIdx.x >> 5;
+    const long e = ((long)blockIdx.x * 32 + lane) * 4;  // first of this thread's 4 outputs (N % 4 == 0)
+    const bool live = e < mn * g.batch;
+    const int b = live ? (int)(e / mn) : 0;
+    const long r = e - (long)b * mn;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        const float *p = g.ws + (long)b * g.splits * mn + r;
+        for (int s = row; s < g.splits; s += 8) v += *(const f32x4 *)(p + (long)s * mn);
+    }
+    part[row][lane] = v;
+    __syncthreads();
+    if (row == 0 && live) {
+#pragma unroll
+        for (int k = 1; k < 8; ++k) v += part[k][lane];
+        const int m = (int)(r / g.N), n = (int)(r - (long)m * g.N);
+        T *c = (T *)g.C + (long)b * g.sC + (long)m * g.ldc + n;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float o = v[k];
+            if (g.beta != 0.f) o += to_f32(c[k]);
+            c[k] = (T)o;
+        }
+    }
+}
+
+// The same for N not a multiple of 4: one output per thread, partials added in split order.
+template <typename T>
+__global__ void gemm_split_reduce_scalar_kernel(GemmArgs g) {
     const long mn = (long)g.M * g.N;
     const long total = mn * g.batch;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
@@ -219,9 +252,13 @@ static int launch(GemmArgs &g, int transA, int transB, bool tiled, hipStream_t s
     }
     if (g.splits > 1) {
         const long total = (long)g.M * g.N * g.batch;
-        int blocks = (int)((total + 255) / 256);
-        if (blocks > 4096) blocks = 4096;
-        hipLaunchKernelGGL((gemm_split_reduce_kernel<T>), dim3(blocks), dim3(256), 0, stream, g);
+        if (g.N % 4 == 0 && ((size_t)g.ws & 15) == 0) {
+            hipLaunchKernelGGL((gemm_split_reduce_kernel<T>), dim3((unsigned)((total / 4 + 31) / 32)), dim3(256), 0, stream, g);
+        } else {
+            int blocks = (int)((total + 255) / 256);
+            if (blocks > 4096) blocks = 4096;
+            hipLaunchKernelGGL((gemm_split_reduce_scalar_kernel<T>), dim3(blocks), dim3(256), 0, stream, g);
+        }
         D8_LAUNCH_CHECK();
     }
     return 0;
@@ -236,7 +273,7 @@ size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red) {
 int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
                    hipStream_t stream) {
     g.ws = (float *)workspace;
-    g.splits = plan_splits(gemm_tiled_k_step(dtype), g.M, g.N, g.K, g.batch, g.red, workspace ? workspace_bytes : 0,
+    g.splits = plan_splits(gemm_tiled_k_step(dtype), g.M, g.N, g.K, g.batch, g.red, (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0,
                            &g.tiles_per_split);
     return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, true, stream) : launch<float>(g, transA, transB, true, stream);
 }
@@ -304,7 +341,7 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     const bool tiled = K > 0 && gemm_tiled_eligible(dtype, g, transA, transB);
     if (K > 0) {  // K == 0 is the empty reduction: C = beta * C
         const int BK = tiled ? gemm_tiled_k_step(dtype) : (dtype == D8_FLOAT16 ? Tile<f16>::BK : Tile<float>::BK);
-        g.splits = plan_splits(BK, M, N, K, g.batch, g.red, workspace ? workspace_bytes : 0, &g.tiles_per_split);
+        g.splits = plan_splits(BK, M, N, K, g.batch, g.red, (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0, &g.tiles_per_split);
     }
     return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, tiled, as_stream(stream))
                                : launch<float>(g, transA, transB, tiled, as_stream(stream));

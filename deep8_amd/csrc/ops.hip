@@ -5,6 +5,7 @@
 //   MatrixMultiply   deep8/src/math/MatrixMultiply.cu:21-57 (fwd), :193-232 (GradX), :381-420 (GradY)
 //   Conv2d           deep8/src/math/Conv2d.cu:145-196, :440-492, :750-802, pads :332-336
 //   DeConv2d         deep8/src/math/DeConv2d.cu:76-131, :371-429, :642-700, pads :99-100
+#include "conv_maps.h"
 #include "gemm_args.h"
 
 namespace d8 {
@@ -302,20 +303,51 @@ int d8_conv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
 }
 
 // ---------------------------------------------------------------------------------------------
-// DeConv2d GEMMs on zmat / dzmat [M x NP], M = B*IH*IW, NP = OC*FH*FW, filter viewed [NP x IC].
-static Gemm deconv_plan(int which, int M, int NP, int IC, const void *mat, const void *w, const void *xx) {
-    if (which == 0) return {0, 1, M, NP, IC, xx, IC, 0, w, IC, 0, 0.f, (void *)mat, NP, 0, 1};  // zmat = x W^T
-    if (which == 1) return {0, 0, M, IC, NP, mat, NP, 0, w, IC, 0, 1.f, (void *)xx, IC, 0, 1};  // dx += dzmat W
-    return {1, 0, NP, IC, M, mat, NP, 0, xx, IC, 0, 1.f, (void *)w, IC, 0, 1};                  // dW += dzmat^T x
+// DeConv2d.  The interim matrix is kept tap-major, [B*IH*IW][FH*FW][OC] (the reference's kernels use
+// [.][OC][FH*FW]; the layout is private to the operator), so that both gather maps move whole
+// channel vectors: they are then exactly the Conv2d maps of a mirrored geometry -- image = the
+// DeConv2d output, patch grid = the DeConv2d input, dilation -1, negated pads -- and the GEMMs
+// become one product per tap against the filter slice w[:, tap, :] (row stride FH*FW*IC).
+static MapGeom deconv_mirror(int B, int IH, int IW, int OC, int FH, int FW, int sy, int sx, const int *g) {
+    return {B, g[0], g[1], OC, IH, IW, FH, FW, sy, sx, -1, -1, -g[2], -g[3]};
+}
+
+static Gemm deconv_plan(int which, int M, int T, int OC, int IC, const void *mat, const void *w, const void *xx) {
+    const int NP = T * OC, KW = T * IC;
+    if (which == 0) return {0, 1, M, OC, IC, xx, IC, 0, w, KW, IC, 0.f, (void *)mat, NP, OC, T};  // zmat[:, t, :] = x w_t^T
+    if (which == 1) return {0, 0, M, IC, OC, mat, NP, OC, w, KW, IC, 1.f, (void *)xx, IC, 0, T};  // dx += sum_t dzmat[:, t, :] w_t
+    return {1, 0, OC, IC, M, mat, NP, OC, xx, IC, 0, 1.f, (void *)w, KW, IC, T};                  // dw_t += dzmat[:, t, :]^T x
+}
+
+// dx += sum over taps of (rows of dz gathered for that tap) . w_t, the gather done by the GEMM's loader
+static bool deconv_implicit_grad_x(int dtype, int B, int IH, int IW, int IC, int OC, int FH, int FW, int sy, int sx,
+                                   const int *geo, const void *gx, const void *w, const void *gz, GemmArgs &g) {
+    if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
+    const long es = (long)dtype_bytes(dtype), T = (long)FH * FW;
+    const long zbytes = (long)B * geo[0] * geo[1] * OC * es;
+    if (zbytes >= (1L << 31) || (long)B * IH * IW >= (1L << 31) || T * IC >= (1L << 31)) return false;
+    memset(&g, 0, sizeof(g));
+    g.pg = {geo[0], geo[1], OC, IH, IW, FW, sy, sx, -1, -1, -geo[2], -geo[3],
+            magic_of((unsigned)IH * IW), magic_of((unsigned)IW), (unsigned)zbytes};
+    g.virt = VIRT_A_ROWS;
+    g.A = gz, g.B = w, g.C = (void *)gx;
+    g.M = B * IH * IW, g.N = IC, g.K = OC;
+    g.ldb = (int)(T * IC), g.sB = IC, g.ldc = IC;
+    g.batch = 1, g.red = (int)T, g.splits = 1, g.beta = 1.f;
+    return gemm_tiled_eligible(dtype, g, 0, 0);
 }
 
 size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                  int OC, int FH, int FW, int covered, int sy, int sx) {
-    (void)covered;
+    int geo[4];
     if (check_conv("d8_deconv2d_scratch_bytes", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return 0;
-    const int M = B * IH * IW, NP = OC * FH * FW;
-    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
-    return mat + gemm_ws(dtype, deconv_plan(which, M, NP, IC, nullptr, nullptr, nullptr));
+    if (d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, geo)) return 0;
+    const int M = B * IH * IW, T = FH * FW;
+    GemmArgs ga;
+    if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
+        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
+    const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
+    return mat + gemm_ws(dtype, deconv_plan(which, M, T, OC, IC, nullptr, nullptr, nullptr));
 }
 
 int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
@@ -325,14 +357,14 @@ int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
     int g[4];
     if (int rc = check_conv("d8_deconv2d", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
-    const int M = B * IH * IW, NP = OC * FH * FW;
-    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
+    const int M = B * IH * IW, T = FH * FW;
+    const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(x && w && z && scratch, "d8_deconv2d: null tensor");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * NP * dtype_bytes(dtype), "d8_deconv2d: scratch too small");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d: scratch too small");
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
-    if (int rc = run(dtype, deconv_plan(0, M, NP, IC, scratch, w, x), ws ? (char *)scratch + mat : nullptr, ws, stream))
+    if (int rc = run(dtype, deconv_plan(0, M, T, OC, IC, scratch, w, x), ws ? (char *)scratch + mat : nullptr, ws, stream))
         return rc;
-    return d8_deconv_col2im(dtype, scratch, z, B, IH, IW, g[0], g[1], OC, FH, FW, sy, sx, g[2], g[3], stream);
+    return launch_col2im(dtype, scratch, z, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), false, as_stream(stream));
 }
 
 int d8_deconv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
@@ -342,14 +374,20 @@ int d8_deconv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
     int g[4];
     if (int rc = check_conv("d8_deconv2d_grad_x", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
-    const int M = B * IH * IW, NP = OC * FH * FW;
-    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
-    D8_REQUIRE(gx && w && gz && scratch, "d8_deconv2d_grad_x: null tensor");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * NP * dtype_bytes(dtype), "d8_deconv2d_grad_x: scratch too small");
-    if (int rc = d8_deconv_im2col(dtype, gz, scratch, B, IH, IW, g[0], g[1], OC, FH, FW, sy, sx, g[2], g[3], stream))
+    const int M = B * IH * IW, T = FH * FW;
+    const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
+    D8_REQUIRE(gx && w && gz, "d8_deconv2d_grad_x: null tensor");
+    {
+        GemmArgs ga;
+        if (deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, gx, w, gz, ga))
+            return gemm_tiled_run(dtype, ga, 0, 0, scratch, scratch_bytes, as_stream(stream));
+    }
+    D8_REQUIRE(scratch, "d8_deconv2d_grad_x: null scratch");
+    D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d_grad_x: scratch too small");
+    if (int rc = launch_im2col(dtype, gz, scratch, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), as_stream(stream)))
         return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
-    return run(dtype, deconv_plan(1, M, NP, IC, scratch, w, gx), ws ? (char *)scratch + mat : nullptr, ws, stream);
+    return run(dtype, deconv_plan(1, M, T, OC, IC, scratch, w, gx), ws ? (char *)scratch + mat : nullptr, ws, stream);
 }
 
 int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
@@ -359,14 +397,14 @@ int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
     int g[4];
     if (int rc = check_conv("d8_deconv2d_grad_y", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
-    const int M = B * IH * IW, NP = OC * FH * FW;
-    const size_t mat = align256((size_t)M * NP * dtype_bytes(dtype));
+    const int M = B * IH * IW, T = FH * FW;
+    const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(x && gw && gz && scratch, "d8_deconv2d_grad_y: null tensor");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * NP * dtype_bytes(dtype), "d8_deconv2d_grad_y: scratch too small");
-    if (int rc = d8_deconv_im2col(dtype, gz, scratch, B, IH, IW, g[0], g[1], OC, FH, FW, sy, sx, g[2], g[3], stream))
+    D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d_grad_y: scratch too small");
+    if (int rc = launch_im2col(dtype, gz, scratch, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), as_stream(stream)))
         return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
-    return run(dtype, deconv_plan(2, M, NP, IC, scratch, gw, x), ws ? (char *)scratch + mat : nullptr, ws, stream);
+    return run(dtype, deconv_plan(2, M, T, OC, IC, scratch, gw, x), ws ? (char *)scratch + mat : nullptr, ws, stream);
 }
 
 }  // extern "C"

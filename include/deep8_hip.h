@@ -66,7 +66,8 @@ int d8_event_elapsed_ms(void *start, void *stop, float *ms);  /* synchronises on
  * fp16 operands accumulate in fp32 and are rounded once; beta = 1 adds the old C in fp32.
  *
  * `workspace` (may be NULL) lets the kernel split the reduction (long K / summed batch, small
- * M x N) over more workgroups; d8_gemm_workspace_bytes says how much it can use.
+ * M x N) over more workgroups; d8_gemm_workspace_bytes says how much it can use.  It must be
+ * 16-byte aligned (a misaligned workspace is ignored).
  *
  * Replaces the 27 cublas{S,H}gemm call sites in deep8/src/math/MatrixMultiply.cu:36-55,
  * 75-94,115-134 (forward), :211-230,253-272,296-315 (GradX), :399-418,441-460,484-503

@@ -33,6 +33,9 @@ DECONV = [
     (1, 5, 6, 3, 5, 3, 3, False, 1, 1),
     (2, 6, 5, 4, 3, 3, 2, True, 2, 2),
     (1, 4, 4, 2, 2, 2, 2, False, 3, 3),     # stride > filter
+    (2, 8, 8, 64, 64, 4, 4, False, 2, 2),   # wide enough for the tiled GEMMs and the implicit dX
+    (2, 7, 7, 128, 32, 3, 3, True, 2, 2),
+    (1, 12, 12, 72, 64, 4, 4, False, 3, 3),
 ]
 
 
