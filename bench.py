@@ -33,6 +33,8 @@ HBM_PEAK = 8000.0                      # GB/s
 # summaries are kept under profiles/).  None where no counter run has been made.
 MEASURED_TRAFFIC = {
     "c3": int((192.1 + 224.1 + 224.1) / 3 * 2**20 + 33.6 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
+    "c4": int((26.5 + 24.5) * 2**20),                                # Conv2d forward kernel: fetch + write
+    "c5": int((17.6 + 24.5) * 2**20),                                # DeConv2d forward GEMM: fetch + write
 }
 
 
@@ -127,6 +129,7 @@ class ConvWorkload:
     def __init__(self, name, dtype, deconv, B, IH, IW, IC, OC, FH, FW, covered, sy, sx, seed):
         from deep8_amd import capi, ops
         self.name, self.dtype, self.deconv = name, np.dtype(dtype), deconv
+        self.key = name.split(":")[0]
         self.lib = capi.init()
         self.dt = capi.dtype_id(self.dtype)
         self.B = B
@@ -156,11 +159,9 @@ class ConvWorkload:
         es = self.dtype.itemsize
         nx, nw, nz = B * IH * IW * IC, OC * FH * FW * IC, B * OH * OW * OC
         self.mat_bytes = mat * es
-        # per pass: gather map (read source, write matrix) + GEMM (read matrix, operand, write result)
-        self.bytes = es * ((nx + mat) + (mat + nw + nz)        # fwd
-                           + (nz + nw + mat) + (mat + 2 * nx)  # grad x
-                           + (nx + mat) + (mat + nz + 2 * nw)) if not deconv else \
-            es * ((nx + nw + mat) + (mat + nz) + (nz + mat) + (mat + nw + 2 * nx) + (nz + mat) + (mat + nx + 2 * nw))
+        # operator-level algorithmic bytes: each pass reads its two operands and writes (forward) or
+        # reads and writes (gradients) its result; the interim matrix is an implementation detail
+        self.bytes = es * ((nx + nw + nz) + (nz + nw + 2 * nx) + (nx + nz + 2 * nw))
 
     def _call(self, fn, a, b, c):
         from deep8_amd.capi import check
@@ -190,29 +191,30 @@ class ConvWorkload:
         f = self.flops / 3
         return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
 
-    def map_roofline(self, reps):
-        """The gather map that builds the GEMM operand (im2col for Conv2d, the dz gather for
-        DeConv2d), launched alone through the C ABI and timed with HIP events: algorithmic bytes
-        (source read once + matrix written once) / launch duration against the HBM peak."""
-        from deep8_amd import capi, ops
+    def gemm_roofline(self, reps):
+        """The pass-forward GEMM launch, timed alone with HIP events, against the MFMA peak of its
+        element type.  Conv2d forward is ONE launch of the tiled kernel (its tile loader reads the
+        patch matrix straight from the image); DeConv2d forward's GEMM (one product per filter tap,
+        a single batched launch) is issued here through d8_gemm with the operator's own arguments."""
+        from deep8_amd import capi
         B, IH, IW, IC = self.xd
         OC, FH, FW, _ = self.wd
         es = self.dtype.itemsize
-        mat = capi.DeviceArray((self.mat_bytes // es,), self.dtype)
+        dtype = "f16" if self.dtype == np.float16 else "f32"
+        flops = self.flops / 3
         if self.deconv:
-            OH, OW, pt, pl = ops.deconv2d_geometry(IH, IW, FH, FW, *self.geo)
-            fn = lambda: capi.check(self.lib.d8_deconv_im2col(self.dt, self.gz.ptr, mat.ptr, B, IH, IW, OH, OW, OC, FH, FW,
-                                                              self.geo[1], self.geo[2], pt, pl, None))
-            name, nbytes = "deconv_im2col_kernel", es * B * OH * OW * OC + self.mat_bytes
+            T, M = FH * FW, B * IH * IW
+            mat = capi.DeviceArray((M * T * OC,), self.dtype)
+            fn = lambda: capi.check(self.lib.d8_gemm(self.dt, 0, 1, M, OC, IC, self.x.ptr, IC, 0, self.w.ptr, T * IC, IC, 0.0,
+                                                     mat.ptr, T * OC, OC, T, None, 0, None))
+            name = "gemm_tiled_kernel<%s> (DeConv2d forward: %d per-tap products [%dx%d]x[%dx%d]^T, one launch)" % (dtype, T, M, IC, OC, IC)
         else:
-            OH, OW, pt, pl = ops.conv2d_geometry(IH, IW, FH, FW, *self.geo)
-            fn = lambda: capi.check(self.lib.d8_im2col(self.dt, self.x.ptr, mat.ptr, B, IH, IW, IC, OH, OW, FH, FW,
-                                                       self.geo[1], self.geo[2], self.geo[3], self.geo[4], pt, pl, None))
-            name, nbytes = "im2col_kernel", es * B * IH * IW * IC + self.mat_bytes
+            fn = self.fwd
+            name = "gemm_tiled_kernel<%s> (Conv2d forward, patch matrix read by the tile loader, one launch)" % dtype
         ms = _time_events(fn, reps)
-        ach = nbytes / (ms * 1e-3) / 1e9
-        return {"bound": "hbm", "kernel": name, "achieved": round(ach, 1), "peak": HBM_PEAK, "unit": "GB/s",
-                "frac": round(ach / HBM_PEAK, 4), "launch_us": round(ms * 1e3, 2), "traffic": None}
+        ach = flops / (ms * 1e-3) / 1e12
+        return {"bound": "mfma", "kernel": name, "achieved": round(ach, 2), "peak": PEAK[dtype], "unit": "TFLOP/s",
+                "frac": round(ach / PEAK[dtype], 4), "launch_us": round(ms * 1e3, 2), "traffic": MEASURED_TRAFFIC.get(self.key)}
 
 
 def _uni(r, s):
@@ -350,7 +352,7 @@ def main():
         pms = _time_events(fn, max(5, a.steps))
         parts[pname] = {"ms": round(pms, 4), "tflops": round(fl / (pms * 1e-3) / 1e12, 2)}
     if is_conv:
-        roof = wl.map_roofline(max(5, a.steps))
+        roof = wl.gemm_roofline(max(5, a.steps))
     else:
         # each of fwd / dX / dY is ONE launch of the same tiled GEMM kernel (its NN, NT and TN
         # instances): flops per launch / average launch duration, HIP events on the launch stream
