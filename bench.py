@@ -221,8 +221,14 @@ def _uni(r, s):
     return r.uniform(-1, 1, s).astype(np.float32)
 
 
+ZERO_OPERANDS = False   # --operands zeros: same launches on all-zero data (shows how much of the rate the data costs)
+
+
 def make_workload(key):
     U = {"x": _uni, "y": _uni, "dz": _uni}
+    if ZERO_OPERANDS:
+        zero = lambda r, s: np.zeros(s, np.float32)
+        U = {"x": zero, "y": zero, "dz": zero}
     if key == "c1":
         return MatMulWorkload("c1: MatrixMultiply fwd+dX+dY fp32 [64x128]x[128x256]", np.float32,
                               (1, 64, 128), (1, 128, 256), U, 1)
@@ -237,7 +243,7 @@ def make_workload(key):
              "y": lambda r, s: (r.standard_normal(s) / 64.0).astype(np.float32),
              "dz": lambda r, s: r.standard_normal(s).astype(np.float32)}
         return MatMulWorkload("c3: MatrixMultiply fwd+dX+dY half [4096x4096]x[4096x4096]", np.float16,
-                              (1, 4096, 4096), (1, 4096, 4096), g, 4)
+                              (1, 4096, 4096), (1, 4096, 4096), U if ZERO_OPERANDS else g, 4)
     if key == "c4":
         return ConvWorkload("c4: Conv2d fwd+dX+dW fp32 B32 56x56x64 3x3x64->64 s1 same", np.float32, False,
                             32, 56, 56, 64, 64, 3, 3, True, 1, 1, 5)
@@ -329,9 +335,14 @@ def main():
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-others", action="store_true")
+    ap.add_argument("--operands", choices=("config", "zeros"), default="config",
+                    help="zeros: run the MatrixMultiply workloads on all-zero operands (a diagnostic: the chip "
+                         "clocks higher when the data does not toggle; not a valid benchmark value)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
+    global ZERO_OPERANDS
+    ZERO_OPERANDS = a.operands == "zeros"
     if a.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
                          "no second device anywhere in the path)" % a.gpus)
@@ -368,7 +379,8 @@ def main():
         "unit": "images/s" if is_conv else "TFLOP/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dtype, "data": "synthetic (seeded numpy generators, resident in HBM before timing)",
+        "dtype": dtype, "data": "ALL-ZERO OPERANDS (diagnostic run, not a benchmark value)" if ZERO_OPERANDS else
+        "synthetic (seeded numpy generators, resident in HBM before timing)",
         "config": {"workload": wl.name},
         "pct_mfma_peak": round(100.0 * tflops / PEAK[dtype], 2),
         "tflops": round(tflops, 2),
