@@ -19,6 +19,8 @@ _I, _L, _Z, _F, _P = c_int, c_long, c_size_t, c_float, c_void_p
 _PP = ctypes.POINTER(c_void_p)
 
 # name -> (restype, argtypes); mirrors include/deep8_hip.h declaration by declaration
+_IP = ctypes.POINTER(ctypes.c_int)
+
 SIGNATURES = {
     "d8_last_error": (ctypes.c_char_p, []),
     "d8_device_init": (_I, [_I]),
@@ -60,6 +62,11 @@ SIGNATURES = {
     "d8_deconv2d": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
     "d8_deconv2d_grad_x": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
     "d8_deconv2d_grad_y": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
+    "d8_add": (_I, [_I, _P, _IP, _P, _IP, _P, _IP, _P]),
+    "d8_add_grad_scratch_bytes": (_Z, [_I, _IP, _IP]),
+    "d8_add_grad": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
+    "d8_relu": (_I, [_I, _P, _P, ctypes.c_long, _P]),
+    "d8_relu_grad": (_I, [_I, _P, _P, _P, ctypes.c_long, _P]),
 }
 
 

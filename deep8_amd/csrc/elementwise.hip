@@ -1,0 +1,410 @@
+// Add (numpy-style broadcasting over [batch, d0..d3]) and ReLu, forward and gradients: the steps
+// that follow every MatrixMultiply / Conv2d in a Deep8 network (bias, activation).  All are
+// HBM-bandwidth bound: 16-byte accesses along the contiguous axis, every output written once, and
+// the broadcast-gradient reductions are two deterministic passes (no atomics).
+//
+// Replaces AddGPU / AddGradXGPU / AddGradYGPU (deep8/src/math/Add.cu:21-133 over
+// deep8/include/math/GPUBinaryElementWise.h) and ReLuGPU / ReLuGradGPU (deep8/src/math/ReLu.cu:20-116).
+#include "common.h"
+
+namespace d8 {
+
+__device__ inline float ew_f32(float v) { return v; }
+__device__ inline float ew_f32(f16 v) { return (float)v; }
+
+static inline int ew_grid(long work, int block) {
+    long blocks = (work + block - 1) / block;
+    const long cap = (long)cu_count() * 32;
+    if (blocks > cap) blocks = cap;
+    return (int)(blocks < 1 ? 1 : blocks);
+}
+
+// Up to 5 merged axes, outermost first.  n[a] is the extent, xs / ys the element stride of the
+// operand along it (0 where the operand is broadcast).
+struct BroadcastGeom {
+    int nd;
+    int n[5];
+    long xs[5], ys[5];
+};
+
+// z = x + y.  A thread owns VEC consecutive elements of the innermost axis; an operand that is
+// broadcast along that axis contributes one scalar to all of them.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void add_kernel(const T *__restrict__ x, const T *__restrict__ y, T *__restrict__ z,
+                                                  BroadcastGeom g, long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    const int last = g.nd - 1;
+    const long inner = g.n[last] / VEC;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        long rem = idx / inner;
+        const long i0 = (idx - rem * inner) * VEC;
+        long xo = i0 * g.xs[last], yo = i0 * g.ys[last];
+        for (int a = last - 1; a >= 0; --a) {
+            const long q = rem / g.n[a], i = rem - q * g.n[a];
+            rem = q;
+            xo += i * g.xs[a];
+            yo += i * g.ys[a];
+        }
+        float xv[VEC], yv[VEC];
+        if (g.xs[last]) {
+            const VT v = *(const VT *)(x + xo);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xv[e] = ew_f32(v[e]);
+        } else {
+            const float s = ew_f32(x[xo]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) xv[e] = s;
+        }
+        if (g.ys[last]) {
+            const VT v = *(const VT *)(y + yo);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) yv[e] = ew_f32(v[e]);
+        } else {
+            const float s = ew_f32(y[yo]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) yv[e] = s;
+        }
+        VT o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = (T)(xv[e] + yv[e]);
+        *(VT *)(z + idx * VEC) = o;
+    }
+}
+
+// g += dz, same shape.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void accumulate_kernel(T *__restrict__ g, const T *__restrict__ dz, long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const VT a = *(const VT *)(g + idx * VEC), b = *(const VT *)(dz + idx * VEC);
+        VT o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(a[e]) + ew_f32(b[e]));
+        *(VT *)(g + idx * VEC) = o;
+    }
+}
+
+// dz viewed [K0][R][C]; sums over R.  Block (x: column group, y: chunk of R, z: k0); TX threads
+// across column vectors, 256 / TX rows in flight.  The row lanes meet in LDS in a fixed order.
+// With one chunk the sums go straight into g (+=); otherwise into partial[k0][chunk][C].
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ dz, T *__restrict__ g,
+                                                         float *__restrict__ partial, int R, int C, int TX,
+                                                         int rows_per_chunk, int chunks) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    __shared__ float part[256][VEC];
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX, lanes = 256 / TX;
+    const int cv = blockIdx.x * TX + tx;
+    const int k0 = blockIdx.z, chunk = blockIdx.y;
+    const bool live = (long)cv * VEC < C;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    if (live) {
+        const int r1 = min(R, (chunk + 1) * rows_per_chunk);
+        const T *p = dz + ((long)k0 * R) * C + (long)cv * VEC;
+        for (int r = chunk * rows_per_chunk + ty; r < r1; r += lanes) {
+            const VT v = *(const VT *)(p + (long)r * C);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += ew_f32(v[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) part[threadIdx.x][e] = acc[e];
+    __syncthreads();
+    if (ty == 0 && live) {
+        for (int k = 1; k < lanes; ++k)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += part[k * TX + tx][e];
+        if (chunks == 1) {
+            T *o = g + (long)k0 * C + (long)cv * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(o[e]) + acc[e]);
+        } else {
+            float *o = partial + ((long)k0 * chunks + chunk) * C + (long)cv * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = acc[e];
+        }
+    }
+}
+
+// g[k0][c] += sum over chunks of partial[k0][chunk][c], chunks added in order.
+template <typename T>
+__global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__restrict__ partial, T *__restrict__ g,
+                                                                int C, int chunks, long total) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long k0 = idx / C;
+        const int c = (int)(idx - k0 * C);
+        const float *p = partial + k0 * chunks * C + c;
+        float v = 0.f;
+        for (int k = 0; k < chunks; ++k) v += p[(long)k * C];
+        g[idx] = (T)(ew_f32(g[idx]) + v);
+    }
+}
+
+// Any other pattern of kept and summed axes: a thread per element of g walks the summed index
+// space in memory order (the order of the reference kernel, GPUBinaryElementWise.h:42-95).
+struct ReduceGeom {
+    int n[5];      // extents of dz
+    int kept[5];   // 1 where g has the same extent, 0 where it is summed (or the extent is 1)
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void broadcast_sum_kernel(const T *__restrict__ dz, T *__restrict__ g, ReduceGeom q,
+                                                            long total) {
+    long zs[5];
+    zs[4] = 1;
+    for (int a = 3; a >= 0; --a) zs[a] = zs[a + 1] * q.n[a + 1];
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        long rem = idx, base = 0;
+        for (int a = 4; a >= 0; --a)
+            if (q.kept[a]) {
+                const long t = rem / q.n[a];
+                base += (rem - t * q.n[a]) * zs[a];
+                rem = t;
+            }
+        float acc = 0.f;
+        int i[5] = {0, 0, 0, 0, 0};
+        while (true) {
+            long off = base;
+            for (int a = 0; a < 5; ++a) off += (long)i[a] * zs[a];
+            acc += ew_f32(dz[off]);
+            int a = 4;
+            for (; a >= 0; --a) {
+                if (q.kept[a]) continue;
+                if (++i[a] < q.n[a]) break;
+                i[a] = 0;
+            }
+            if (a < 0) break;
+        }
+        g[idx] = (T)(ew_f32(g[idx]) + acc);
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void relu_kernel(const T *__restrict__ x, T *__restrict__ y, long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const VT v = *(const VT *)(x + idx * VEC);
+        VT o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = v[e] > (T)0 ? v[e] : (T)0;
+        *(VT *)(y + idx * VEC) = o;
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void relu_grad_kernel(const T *__restrict__ x, T *__restrict__ dx,
+                                                        const T *__restrict__ dy, long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const VT v = *(const VT *)(x + idx * VEC), d = *(const VT *)(dy + idx * VEC), old = *(const VT *)(dx + idx * VEC);
+        VT o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(old[e]) + (v[e] > (T)0 ? ew_f32(d[e]) : 0.f));
+        *(VT *)(dx + idx * VEC) = o;
+    }
+}
+
+static inline bool al16(const void *p) { return ((size_t)p & 15) == 0; }
+
+static int check_dims(const char *who, const int *d, const int *zd) {
+    for (int a = 0; a < 5; ++a) {
+        D8_REQUIRE(d[a] >= 1 && zd[a] >= 1, "%s: extents must be positive", who);
+        D8_REQUIRE(d[a] == 1 || d[a] == zd[a], "%s: the shape is error (axis %d: %d against %d)", who, a, d[a], zd[a]);
+    }
+    return 0;
+}
+
+static long prod5(const int *d) {
+    long n = 1;
+    for (int a = 0; a < 5; ++a) n *= d[a];
+    return n;
+}
+
+// The gradient's reduction, with consecutive axes of the same kind merged:
+// kind 0: g += dz; kind 1: dz is [K0][R][C], summed over R; kind 2: anything else.
+struct ReducePlan {
+    int kind;
+    long K0, R, C;
+    int chunks, rows_per_chunk;
+};
+
+static ReducePlan plan_reduce(const int *d, const int *zd) {
+    int kinds[5], ext[5], n = 0;  // 1 kept, 0 summed; extent-1 axes dropped
+    for (int a = 0; a < 5; ++a) {
+        if (zd[a] == 1) continue;
+        const int k = d[a] == zd[a];
+        if (n && kinds[n - 1] == k) ext[n - 1] *= zd[a];
+        else kinds[n] = k, ext[n] = zd[a], ++n;
+    }
+    ReducePlan p = {2, 1, 1, 1, 1, 1};
+    if (n == 0 || (n == 1 && kinds[0] == 1)) {
+        p.kind = 0;
+        return p;
+    }
+    if (n == 1) p.kind = 1, p.R = ext[0];                                              // [R]
+    else if (n == 2 && kinds[0] == 0) p.kind = 1, p.R = ext[0], p.C = ext[1];          // [R][C]
+    else if (n == 2) p.kind = 1, p.K0 = ext[0], p.R = ext[1];                          // [K0][R]
+    else if (n == 3 && kinds[0] == 1) p.kind = 1, p.K0 = ext[0], p.R = ext[1], p.C = ext[2];  // [K0][R][C]
+    if (p.kind == 1) {
+        if (p.K0 > 65535 || p.R >= (1L << 31) || p.C >= (1L << 31)) {
+            p.kind = 2;
+            return p;
+        }
+        const long colblocks = (p.C + 255) / 256;  // upper bound on column groups
+        long chunks = (4L * cu_count()) / (colblocks * p.K0);
+        const long max_chunks = (p.R + 63) / 64;
+        if (chunks > max_chunks) chunks = max_chunks;
+        if (chunks > 1024) chunks = 1024;
+        if (chunks < 1) chunks = 1;
+        p.rows_per_chunk = (int)((p.R + chunks - 1) / chunks);
+        p.chunks = (int)((p.R + p.rows_per_chunk - 1) / p.rows_per_chunk);
+    }
+    return p;
+}
+
+template <typename T, int WIDE>
+static int add_grad_t(T *g, const int *d, const T *dz, const int *zd, void *scratch, size_t scratch_bytes, hipStream_t s) {
+    const ReducePlan p = plan_reduce(d, zd);
+    const long ng = prod5(d);
+    if (p.kind == 0) {
+        if (ng % WIDE == 0 && al16(g) && al16(dz))
+            hipLaunchKernelGGL((accumulate_kernel<T, WIDE>), dim3(ew_grid(ng / WIDE, 256)), dim3(256), 0, s, g, dz, ng / WIDE);
+        else
+            hipLaunchKernelGGL((accumulate_kernel<T, 1>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, g, dz, ng);
+    } else if (p.kind == 1) {
+        int chunks = p.chunks, rpc = p.rows_per_chunk;
+        const size_t need = (size_t)p.K0 * chunks * p.C * sizeof(float);
+        if (chunks > 1 && (!scratch || scratch_bytes < need || !al16(scratch))) chunks = 1, rpc = (int)p.R;  // one pass, still exact
+        const bool wide = p.C % WIDE == 0 && al16(g) && al16(dz);
+        const int vec = wide ? WIDE : 1;
+        const long cvs = p.C / vec;
+        int TX = 1;
+        while (TX < 32 && TX < cvs) TX *= 2;
+        dim3 grid((unsigned)((cvs + TX - 1) / TX), (unsigned)chunks, (unsigned)p.K0);
+        if (wide)
+            hipLaunchKernelGGL((column_sum_kernel<T, WIDE>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
+                               TX, rpc, chunks);
+        else
+            hipLaunchKernelGGL((column_sum_kernel<T, 1>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
+                               TX, rpc, chunks);
+        if (chunks > 1) {
+            D8_LAUNCH_CHECK();
+            hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, (const float *)scratch, g,
+                               (int)p.C, chunks, ng);
+        }
+    } else {
+        ReduceGeom q;
+        for (int a = 0; a < 5; ++a) q.n[a] = zd[a], q.kept[a] = (d[a] == zd[a] && zd[a] > 1) ? 1 : 0;
+        hipLaunchKernelGGL((broadcast_sum_kernel<T>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, dz, g, q, ng);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename T, int WIDE>
+static int add_t(const T *x, const int *xd, const T *y, const int *yd, T *z, const int *zd, hipStream_t s) {
+    // merge consecutive axes on which both operands behave the same way
+    BroadcastGeom g;
+    int kx[5], ky[5];
+    g.nd = 0;
+    for (int a = 0; a < 5; ++a) {
+        if (zd[a] == 1) continue;
+        const int fx = xd[a] != 1, fy = yd[a] != 1;
+        if (g.nd && kx[g.nd - 1] == fx && ky[g.nd - 1] == fy) g.n[g.nd - 1] *= zd[a];
+        else kx[g.nd] = fx, ky[g.nd] = fy, g.n[g.nd] = zd[a], ++g.nd;
+    }
+    if (g.nd == 0) g.nd = 1, g.n[0] = 1, kx[0] = ky[0] = 1;
+    long sx = 1, sy = 1;
+    for (int a = g.nd - 1; a >= 0; --a) {
+        g.xs[a] = kx[a] ? sx : 0;
+        g.ys[a] = ky[a] ? sy : 0;
+        if (kx[a]) sx *= g.n[a];
+        if (ky[a]) sy *= g.n[a];
+    }
+    const long n = prod5(zd);
+    if (g.n[g.nd - 1] % WIDE == 0 && al16(x) && al16(y) && al16(z))
+        hipLaunchKernelGGL((add_kernel<T, WIDE>), dim3(ew_grid(n / WIDE, 256)), dim3(256), 0, s, x, y, z, g, n / WIDE);
+    else
+        hipLaunchKernelGGL((add_kernel<T, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, x, y, z, g, n);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace d8
+
+using namespace d8;
+
+extern "C" {
+
+int d8_add(int dtype, const void *x, const int *xdims, const void *y, const int *ydims, void *z, const int *zdims,
+           void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32) return fail(D8_ERR_DTYPE, "d8_add: element type %d is not supported", dtype);
+    D8_REQUIRE(x && y && z && xdims && ydims && zdims, "d8_add: null argument");
+    if (int rc = check_dims("d8_add", xdims, zdims)) return rc;
+    if (int rc = check_dims("d8_add", ydims, zdims)) return rc;
+    for (int a = 0; a < 5; ++a)
+        D8_REQUIRE(zdims[a] == (xdims[a] > ydims[a] ? xdims[a] : ydims[a]), "d8_add: the shape is error (axis %d)", a);
+    return dtype == D8_FLOAT32 ? add_t<float, 4>((const float *)x, xdims, (const float *)y, ydims, (float *)z, zdims, as_stream(stream))
+                               : add_t<f16, 8>((const f16 *)x, xdims, (const f16 *)y, ydims, (f16 *)z, zdims, as_stream(stream));
+}
+
+size_t d8_add_grad_scratch_bytes(int dtype, const int *gdims, const int *zdims) {
+    (void)dtype;
+    if (!gdims || !zdims) return 0;
+    for (int a = 0; a < 5; ++a)
+        if (gdims[a] < 1 || zdims[a] < 1 || (gdims[a] != 1 && gdims[a] != zdims[a])) return 0;
+    const ReducePlan p = plan_reduce(gdims, zdims);
+    return p.kind == 1 && p.chunks > 1 ? (size_t)p.K0 * p.chunks * p.C * sizeof(float) : 0;
+}
+
+int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                void *scratch, size_t scratch_bytes, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_add_grad: element type %d is not supported", dtype);
+    D8_REQUIRE(g && dz && gdims && zdims, "d8_add_grad: null argument");
+    if (int rc = check_dims("d8_add_grad", gdims, zdims)) return rc;
+    return dtype == D8_FLOAT32
+               ? add_grad_t<float, 4>((float *)g, gdims, (const float *)dz, zdims, scratch, scratch_bytes, as_stream(stream))
+               : add_grad_t<f16, 8>((f16 *)g, gdims, (const f16 *)dz, zdims, scratch, scratch_bytes, as_stream(stream));
+}
+
+int d8_relu(int dtype, const void *x, void *y, long n, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32) return fail(D8_ERR_DTYPE, "d8_relu: element type %d is not supported", dtype);
+    D8_REQUIRE(n >= 0, "d8_relu: negative size");
+    if (n == 0) return 0;
+    D8_REQUIRE(x && y, "d8_relu: null tensor");
+    hipStream_t s = as_stream(stream);
+    const bool al = al16(x) && al16(y);
+    if (dtype == D8_FLOAT32) {
+        if (al && n % 4 == 0) hipLaunchKernelGGL((relu_kernel<float, 4>), dim3(ew_grid(n / 4, 256)), dim3(256), 0, s, (const float *)x, (float *)y, n / 4);
+        else hipLaunchKernelGGL((relu_kernel<float, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const float *)x, (float *)y, n);
+    } else {
+        if (al && n % 8 == 0) hipLaunchKernelGGL((relu_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)y, n / 8);
+        else hipLaunchKernelGGL((relu_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)y, n);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_relu_grad: element type %d is not supported", dtype);
+    D8_REQUIRE(n >= 0, "d8_relu_grad: negative size");
+    if (n == 0) return 0;
+    D8_REQUIRE(x && dx && dy, "d8_relu_grad: null tensor");
+    hipStream_t s = as_stream(stream);
+    const bool al = al16(x) && al16(dx) && al16(dy);
+    if (dtype == D8_FLOAT32) {
+        if (al && n % 4 == 0) hipLaunchKernelGGL((relu_grad_kernel<float, 4>), dim3(ew_grid(n / 4, 256)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, n / 4);
+        else hipLaunchKernelGGL((relu_grad_kernel<float, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, n);
+    } else {
+        if (al && n % 8 == 0) hipLaunchKernelGGL((relu_grad_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n / 8);
+        else hipLaunchKernelGGL((relu_grad_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -256,3 +256,61 @@ def deconv_im2col(dz, IH, IW, FH, FW, sy, sx, padTop, padLeft):
     check(lib.d8_deconv_im2col(capi.dtype_id(dz.dtype), ddz.ptr, m.ptr, B, IH, IW, OH, OW, OC, FH, FW,
                                sy, sx, padTop, padLeft, None))
     return m.numpy()
+
+
+# ---- Add (broadcasting) / ReLu ---------------------------------------------------------------------
+def _enlarged(shape):
+    """(batch, 1..4 dims) -> ctypes int[5] in Deep8's enlarged form [batch, 1.., dims]"""
+    shape = tuple(shape)
+    if not 2 <= len(shape) <= 5:
+        raise ValueError("a tensor is (batch, 1..4 dims)")
+    return (ctypes.c_int * 5)(*((shape[0],) + (1,) * (5 - len(shape)) + shape[1:]))
+
+
+def _broadcast(xs, ys):
+    nd = max(len(xs), len(ys)) - 1
+    ex = (xs[0],) + (1,) * (nd - len(xs) + 1) + tuple(xs[1:])
+    ey = (ys[0],) + (1,) * (nd - len(ys) + 1) + tuple(ys[1:])
+    return tuple(max(a, b) for a, b in zip(ex, ey))
+
+
+def add(x, y):
+    lib = capi.init()
+    x, y = np.ascontiguousarray(x), np.ascontiguousarray(y)
+    dt = _same_dtype(x, y)
+    zs = _broadcast(x.shape, y.shape)
+    dx_, dy_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray(zs, x.dtype)
+    check(lib.d8_add(dt, dx_.ptr, _enlarged(x.shape), dy_.ptr, _enlarged(y.shape), dz_.ptr, _enlarged(zs), None))
+    return dz_.numpy()
+
+
+def add_grad(g, dz, use_scratch=True):
+    """returns g + dz summed over the axes g is broadcast along (g: (batch, dims..), right-aligned to dz)"""
+    lib = capi.init()
+    g, dz = np.ascontiguousarray(g), np.ascontiguousarray(dz)
+    dt = _same_dtype(g, dz)
+    gs = (g.shape[0],) + (1,) * (dz.ndim - g.ndim) + tuple(g.shape[1:])
+    gd, zd = _enlarged(gs), _enlarged(dz.shape)
+    dg, ddz = DeviceArray.from_numpy(g), DeviceArray.from_numpy(dz)
+    nb = lib.d8_add_grad_scratch_bytes(dt, gd, zd) if use_scratch else 0
+    ws = _scratch(nb)
+    check(lib.d8_add_grad(dt, dg.ptr, gd, ddz.ptr, zd, ws.ptr if nb else None, nb, None))
+    return dg.numpy()
+
+
+def relu(x):
+    lib = capi.init()
+    x = np.ascontiguousarray(x)
+    dx_, dy_ = DeviceArray.from_numpy(x), DeviceArray(x.shape, x.dtype)
+    check(lib.d8_relu(capi.dtype_id(x.dtype), dx_.ptr, dy_.ptr, x.size, None))
+    return dy_.numpy()
+
+
+def relu_grad(x, dy, dx=None):
+    lib = capi.init()
+    x, dy = np.ascontiguousarray(x), np.ascontiguousarray(dy)
+    dt = _same_dtype(x, dy)
+    dx = np.zeros_like(x) if dx is None else np.ascontiguousarray(dx)
+    a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
+    check(lib.d8_relu_grad(dt, a.ptr, b.ptr, c.ptr, x.size, None))
+    return b.numpy()

@@ -168,6 +168,28 @@ int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
                        int covered, int sy, int sx,
                        void *scratch, size_t scratch_bytes, void *stream);
 
+/* ---- Add (broadcasting) and ReLu -----------------------------------------------------------
+ * The element-wise steps that follow MatrixMultiply / Conv2d in a network (bias, activation).
+ * Shapes are Deep8's 5-entry enlarged form [batch, d0, d1, d2, d3]: dims right-aligned, padded
+ * with 1 (deep8/include/utils/ShapeUtils.h:41-56); an operand axis equals z's or is 1.
+ *
+ * d8_add       z = x + y with broadcasting.  Replaces Math::AddGPU (deep8/include/math/Add.h:20,
+ *              deep8/src/math/Add.cu:21-52).
+ * d8_add_grad  g += dz summed over the axes where g has extent 1 and dz does not; this one map
+ *              is both Math::AddGradXGPU and Math::AddGradYGPU (Add.h:31,42; Add.cu:64-133:
+ *              the gradient op returns dz).  `scratch` (may be NULL; size from
+ *              d8_add_grad_scratch_bytes, 16-byte aligned) lets the reduction run in two passes.
+ * d8_relu      y = x > 0 ? x : 0.   Replaces Math::ReLuGPU (deep8/include/math/ReLu.h:19,
+ *              deep8/src/math/ReLu.cu:20-59).
+ * d8_relu_grad dx += x > 0 ? dy : 0.  Replaces Math::ReLuGradGPU (ReLu.h:30, ReLu.cu:61-116).     */
+int d8_add(int dtype, const void *x, const int *xdims, const void *y, const int *ydims,
+           void *z, const int *zdims, void *stream);
+size_t d8_add_grad_scratch_bytes(int dtype, const int *gdims, const int *zdims);
+int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                void *scratch, size_t scratch_bytes, void *stream);
+int d8_relu(int dtype, const void *x, void *y, long n, void *stream);
+int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

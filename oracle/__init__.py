@@ -62,6 +62,32 @@ def matmul_out_shape(x, y):
     return (max(xb, yb), xr) if yc == 1 else (max(xb, yb), xr, yc)
 
 
+def enlarged(shape):
+    """(batch, d0, ..) of an array -> the 5-entry form [batch, 1.., dims] (utils/ShapeUtils.h:41-56)"""
+    shape = tuple(shape)
+    assert 2 <= len(shape) <= 5, "a tensor is (batch, 1..4 dims)"
+    return (shape[0],) + (1,) * (5 - len(shape)) + shape[1:]
+
+
+def broadcast_shape(xs, ys):
+    """Deep8's broadcastShape (utils/ShapeUtils.h:19-36) on (batch, dims..) tuples"""
+    nd = max(len(xs), len(ys)) - 1
+    ex = (xs[0],) + (1,) * (nd - len(xs) + 1) + tuple(xs[1:])
+    ey = (ys[0],) + (1,) * (nd - len(ys) + 1) + tuple(ys[1:])
+    for a, b in zip(ex, ey):
+        if not (a == 1 or b == 1 or a == b):
+            raise ValueError("the Shape can not Broadcast")
+    return tuple(max(a, b) for a, b in zip(ex, ey))
+
+
+def _i5(shape):
+    return (ctypes.c_int * 5)(*enlarged(shape))
+
+
+def _nd(a):
+    return _i(a.shape[0]), _i(a.ndim - 1), (ctypes.c_int * 4)(*(list(a.shape[1:]) + [0] * (5 - a.ndim)))
+
+
 def _filt(w):
     w = _c(w)
     if w.ndim == 5:
@@ -206,6 +232,35 @@ class _Port:
         return m
 
 
+    # -- Add / ReLu (arrays are (batch, 1..4 dims)) ---------------------------------------------
+    def add(self, x, y):
+        x, y = _c(x), _c(y)
+        z = np.zeros(broadcast_shape(x.shape, y.shape), np.float32)
+        self.lib.orc_add(_p(x), _i5(x.shape), _p(y), _i5(y.shape), _p(z), _i5(z.shape))
+        return z
+
+    def add_grad(self, like, dz, g=None):
+        """g (shaped like `like`) += dz summed over the broadcast axes"""
+        dz = _c(dz)
+        g = np.zeros(np.shape(like), np.float32) if g is None else _c(g).copy()
+        nd = dz.ndim
+        gs = (g.shape[0],) + (1,) * (nd - g.ndim) + tuple(g.shape[1:])
+        self.lib.orc_add_grad(_p(g), _i5(gs), _p(dz), _i5(dz.shape))
+        return g
+
+    def relu(self, x):
+        x = _c(x)
+        y = np.zeros_like(x)
+        self.lib.orc_relu(_p(x), _p(y), ctypes.c_long(x.size))
+        return y
+
+    def relu_grad(self, x, dy, dx=None):
+        x, dy = _c(x), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        self.lib.orc_relu_grad(_p(x), _p(dx), _p(dy), ctypes.c_long(x.size))
+        return dx
+
+
 class _Ref:
     """Deep8's own CPU path (float only)."""
     name = "reference"
@@ -318,6 +373,34 @@ class _Ref:
         self._chk(self.lib.ref_image_patches(_p(im), B, H, W, C, FH, FW, sy, sx, dy, dx, iy, ix,
                                              pt, pb, pl, pr, OH, OW, _p(out)))
         return out
+
+    def add(self, x, y, z_shape=None):
+        x, y = _c(x), _c(y)
+        z = np.zeros(broadcast_shape(x.shape, y.shape) if z_shape is None else z_shape, np.float32)
+        self._chk(self.lib.ref_add(_p(x), *_nd(x), _p(y), *_nd(y), _p(z), *_nd(z)))
+        return z
+
+    def add_grad(self, which, x, y, dz, g=None):
+        """which 0: AddGradX, 1: AddGradY; returns g + gradient"""
+        x, y, dz = _c(x), _c(y), _c(dz)
+        like = x if which == 0 else y
+        g = np.zeros_like(like) if g is None else _c(g).copy()
+        z = np.zeros_like(dz)
+        self._chk(self.lib.ref_add_grad(_i(which), _p(x), *_nd(x), _p(y), *_nd(y), _p(g), _p(z), _p(dz), *_nd(dz)))
+        return g
+
+    def relu(self, x):
+        x = _c(x)
+        y = np.zeros_like(x)
+        self._chk(self.lib.ref_relu(_p(x), _p(y), *_nd(x)))
+        return y
+
+    def relu_grad(self, x, dy, dx=None):
+        x, dy = _c(x), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        y = np.maximum(x, 0)
+        self._chk(self.lib.ref_relu_grad(_p(x), _p(dx), _p(y), _p(dy), *_nd(x)))
+        return dx
 
 
 port = _Port(PORT_PATH) if os.path.exists(PORT_PATH) else None

@@ -30,10 +30,64 @@
 #include "deep8_oracle.h"
 
 #include <stddef.h>
+#include <stdlib.h>
 #include <string.h>
 #ifdef _OPENMP
 #include <omp.h>
 #endif
+
+/* ---- Add / ReLu -------------------------------------------------------------------------------
+ * orc_add       deep8/src/math/Add.cpp:110-142 (reshape to 5 axes, broadcast the size-1 axes, add)
+ * orc_add_grad  deep8/src/math/Add.cpp:163-184 (dxy += dz.sum(axes that differ)); the sum is carried
+ *               in double here
+ * orc_relu      deep8/src/math/ReLu.cpp:38-44 (cwiseMax(0));  orc_relu_grad  ReLu.cpp:62-77
+ * Pins: numpy broadcasting / np.sum over the same axes, the live reference build and the golden
+ * fixtures (tests/test_oracle_pins.py). */
+static long stride5(const int *d, int axis) {
+    long s = 1;
+    for (int i = 4; i > axis; --i) s *= d[i];
+    return s;
+}
+
+void orc_add(const float *x, const int *xd, const float *y, const int *yd, float *z, const int *zd) {
+    long n = 1;
+    for (int i = 0; i < 5; ++i) n *= zd[i];
+    for (long e = 0; e < n; ++e) {
+        long rem = e, xi = 0, yi = 0;
+        for (int a = 0; a < 5; ++a) {
+            const long zs = stride5(zd, a), idx = rem / zs;
+            rem -= idx * zs;
+            if (xd[a] != 1) xi += idx * stride5(xd, a);
+            if (yd[a] != 1) yi += idx * stride5(yd, a);
+        }
+        z[e] = x[xi] + y[yi];
+    }
+}
+
+void orc_add_grad(float *dxy, const int *d, const float *dz, const int *zd) {
+    long n = 1, nz = 1;
+    for (int i = 0; i < 5; ++i) n *= d[i], nz *= zd[i];
+    double *acc = (double *)calloc((size_t)n, sizeof(double));
+    for (long e = 0; e < nz; ++e) {
+        long rem = e, o = 0;
+        for (int a = 0; a < 5; ++a) {
+            const long zs = stride5(zd, a), idx = rem / zs;
+            rem -= idx * zs;
+            if (d[a] != 1) o += idx * stride5(d, a);
+        }
+        acc[o] += (double)dz[e];
+    }
+    for (long o = 0; o < n; ++o) dxy[o] += (float)acc[o];
+    free(acc);
+}
+
+void orc_relu(const float *x, float *y, long n) {
+    for (long i = 0; i < n; ++i) y[i] = x[i] > 0.f ? x[i] : 0.f;
+}
+
+void orc_relu_grad(const float *x, float *dx, const float *dy, long n) {
+    for (long i = 0; i < n; ++i) dx[i] += x[i] > 0.f ? dy[i] : 0.f;
+}
 
 int orc_threads(void) {
 #ifdef _OPENMP

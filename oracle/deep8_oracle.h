@@ -72,6 +72,16 @@ void orc_deconv_col2im(const float *zmat, float *z, int B, int IH, int IW, int O
 void orc_deconv_im2col(const float *dz, float *dzmat, int B, int IH, int IW, int OH, int OW, int OC,
                        int FH, int FW, int sy, int sx, int padTop, int padLeft);
 
+/* ---- Add (broadcasting) and ReLu ------------------------------------------------------------
+ * Shapes are the 5-entry enlarged form [batch, d0, d1, d2, d3], dims right-aligned and padded
+ * with 1 (deep8/include/utils/ShapeUtils.h:41-56); an operand axis is either equal to z's or 1. */
+void orc_add(const float *x, const int *xd, const float *y, const int *yd, float *z, const int *zd);
+/* dxy += dz summed over the axes where dxy has extent 1 and dz does not (AddGradX == AddGradY) */
+void orc_add_grad(float *dxy, const int *d, const float *dz, const int *zd);
+void orc_relu(const float *x, float *y, long n);
+/* dx += x > 0 ? dy : 0 */
+void orc_relu_grad(const float *x, float *dx, const float *dy, long n);
+
 int orc_threads(void);
 
 #ifdef __cplusplus

@@ -8,6 +8,8 @@
  *   Math::MatrixMultiply / GradX / GradY      deep8/src/math/MatrixMultiply.cpp:7-91
  *   Math::Conv2d / GradX / GradY              deep8/src/math/Conv2d.cpp:46-96,140-193,237-290
  *   Math::DeConv2d / GradX / GradY            deep8/src/math/DeConv2d.cpp:43-82,122-162,203-243
+ *   Math::Add / AddGradX / AddGradY           deep8/src/math/Add.cpp:7-107
+ *   Math::ReLu / ReLuGrad                     deep8/src/math/ReLu.cpp:6-36
  *
  * plus one materialisation of the patch expression the CPU Conv2d contracts over
  * (deep8/src/math/Conv2d.cpp:352-356), which is the "CPU Eigen im2col" the HIP im2col must
@@ -21,6 +23,8 @@
 #include "math/MatrixMultiply.h"
 #include "math/Conv2d.h"
 #include "math/DeConv2d.h"
+#include "math/Add.h"
+#include "math/ReLu.h"
 
 #include <chrono>
 #include <cstring>
@@ -234,6 +238,59 @@ int ref_image_patches(const float *im, int B, int H, int W, int C,
         o.device(*cpu()->eigenDevice) =
             t.extract_image_patches(FW, FH, sx, sy, dx, dy, ix, iy, padTop, padBottom, padLeft, padRight, 0.f)
                 .reshape(pre);
+    });
+}
+
+/* Add / ReLu.  A tensor is (batch, nd in 1..4, dims[nd]). */
+static std::vector<size_t> vdims(int nd, const int *d) { return std::vector<size_t>(d, d + nd); }
+
+int ref_add(const float *x, int xb, int xnd, const int *xd, const float *y, int yb, int ynd, const int *yd,
+            float *z, int zb, int znd, const int *zd) {
+    return guarded([&] {
+        Wrapped X, Y, Z;
+        wrap(X, x, xb, vdims(xnd, xd));
+        wrap(Y, y, yb, vdims(ynd, yd));
+        wrap(Z, z, zb, vdims(znd, zd));
+        Math::Add(*X.t, *Y.t, *Z.t);
+    });
+}
+
+/* which = 0: AddGradX (g plays dx), 1: AddGradY (g plays dy) */
+int ref_add_grad(int which, const float *x, int xb, int xnd, const int *xd, const float *y, int yb, int ynd,
+                 const int *yd, float *g, const float *z, const float *dz, int zb, int znd, const int *zd) {
+    return guarded([&] {
+        Wrapped X, Y, Z, G, DZ;
+        wrap(X, x, xb, vdims(xnd, xd));
+        wrap(Y, y, yb, vdims(ynd, yd));
+        wrap(Z, z, zb, vdims(znd, zd));
+        wrap(DZ, dz, zb, vdims(znd, zd));
+        if (0 == which) {
+            wrap(G, g, xb, vdims(xnd, xd));
+            Math::AddGradX(*X.t, *G.t, *Y.t, *Z.t, *DZ.t);
+        } else {
+            wrap(G, g, yb, vdims(ynd, yd));
+            Math::AddGradY(*X.t, *Y.t, *G.t, *Z.t, *DZ.t);
+        }
+    });
+}
+
+int ref_relu(const float *x, float *y, int b, int nd, const int *d) {
+    return guarded([&] {
+        Wrapped X, Y;
+        wrap(X, x, b, vdims(nd, d));
+        wrap(Y, y, b, vdims(nd, d));
+        Math::ReLu(*X.t, *Y.t);
+    });
+}
+
+int ref_relu_grad(const float *x, float *dx, const float *y, const float *dy, int b, int nd, const int *d) {
+    return guarded([&] {
+        Wrapped X, DX, Y, DY;
+        wrap(X, x, b, vdims(nd, d));
+        wrap(DX, dx, b, vdims(nd, d));
+        wrap(Y, y, b, vdims(nd, d));
+        wrap(DY, dy, b, vdims(nd, d));
+        Math::ReLuGrad(*X.t, *DX.t, *Y.t, *DY.t);
     });
 }
 

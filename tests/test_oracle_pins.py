@@ -288,3 +288,48 @@ def test_special_cases(oracle_port):
     assert oracle_port.conv2d_geometry(56, 56, 3, 3, True, 1, 1, 1, 1) == (56, 56, 1, 1)
     assert oracle_port.deconv2d_geometry(28, 28, 4, 4, False, 2, 2) == (58, 58, 3, 3)
     assert oracle_port.deconv2d_geometry(28, 28, 4, 4, True, 2, 2) == (55, 55, 1, 1)
+
+
+# ---- Add / ReLu ------------------------------------------------------------------------------------------------------
+ADD_PAIRS = [((2, 3, 4), (2, 3, 4)), ((10, 50, 20), (1, 20)), ((2, 5, 6, 8), (1, 8)), ((1, 4, 1), (3, 1, 5)),
+             ((3, 7), (1, 1)), ((2, 2, 3, 4, 5), (2, 1, 3, 1, 5)), ((2, 6, 6, 8), (2, 1, 1, 8))]
+
+
+def _ex(a, nd):
+    return a.reshape((a.shape[0],) + (1,) * (nd - a.ndim) + a.shape[1:])
+
+
+@pytest.mark.parametrize("xs,ys", ADD_PAIRS)
+def test_add_against_numpy_and_reference(oracle_port, oracle_ref, xs, ys):
+    """numpy broadcasting (batch axis first, dims right-aligned) fixes the index map; np.sum over the
+    broadcast axes fixes the gradient; the live reference build must agree wherever it is present."""
+    r = rng(sum(xs) + sum(ys))
+    x, y = ints(r, xs), ints(r, ys)
+    nd = max(x.ndim, y.ndim)
+    ex, ey = _ex(x, nd), _ex(y, nd)
+    z = oracle_port.add(x, y)
+    assert np.array_equal(z, ex + ey)
+    dz = ints(r, z.shape)
+    for which, a, ea in ((0, x, ex), (1, y, ey)):
+        axes = tuple(i for i in range(nd) if ea.shape[i] == 1 and z.shape[i] != 1)
+        want = dz.sum(axis=axes, keepdims=True).reshape(a.shape) + a
+        assert np.array_equal(oracle_port.add_grad(a, dz, a), want)
+        if oracle_ref is not None:
+            assert np.array_equal(oracle_ref.add_grad(which, x, y, dz, a), want)
+    if oracle_ref is not None:
+        assert np.array_equal(oracle_ref.add(x, y), z)
+        xr, yr, dzr = nrm(r, xs), nrm(r, ys), nrm(r, z.shape)
+        assert np.array_equal(oracle_ref.add(xr, yr), oracle_port.add(xr, yr))
+        assert rel_fro(oracle_ref.add_grad(1, xr, yr, dzr), oracle_port.add_grad(yr, dzr)) <= 1e-6
+
+
+def test_relu_against_numpy_and_reference(oracle_port, oracle_ref):
+    r = rng(12)
+    x, dy, dx0 = nrm(r, (3, 9, 11)), nrm(r, (3, 9, 11)), nrm(r, (3, 9, 11))
+    x[0, 0, :3] = (0.0, -0.0, 1e-30)
+    assert np.array_equal(oracle_port.relu(x), np.maximum(x, 0))
+    want = dx0 + np.where(x > 0, dy, 0).astype(np.float32)
+    assert np.array_equal(oracle_port.relu_grad(x, dy, dx0), want)
+    if oracle_ref is not None:
+        assert np.array_equal(oracle_ref.relu(x), np.maximum(x, 0))
+        assert np.array_equal(oracle_ref.relu_grad(x, dy, dx0), want)
