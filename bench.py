@@ -217,6 +217,44 @@ class ConvWorkload:
                 "frac": round(ach / PEAK[dtype], 4), "launch_us": round(ms * 1e3, 2), "traffic": MEASURED_TRAFFIC.get(self.key)}
 
 
+class BiasReluWorkload:
+    """The element-wise steps after a convolution: Add (per-channel bias, broadcast) -> ReLu, and back:
+    ReLuGrad -> AddGradY (bias gradient: a sum over batch, rows and columns).  HBM-bound."""
+
+    def __init__(self, name, dtype, B, H, W, C, seed):
+        import ctypes
+        from deep8_amd import capi
+        self.name, self.dtype, self.key = name, np.dtype(dtype), name.split(":")[0]
+        self.lib = capi.init()
+        self.dt = capi.dtype_id(self.dtype)
+        r = np.random.default_rng(seed)
+        self.n = B * H * W * C
+        self.B = B
+        self.z = _dev(r.standard_normal((B, H, W, C)).astype(np.float32).astype(dtype))
+        self.b = _dev(r.standard_normal((1, C)).astype(np.float32).astype(dtype))
+        self.gy = _dev(r.standard_normal((B, H, W, C)).astype(np.float32).astype(dtype))
+        self.pre, self.act, self.gpre = (capi.DeviceArray((B, H, W, C), dtype) for _ in range(3))
+        self.gb = capi.DeviceArray((1, C), dtype)
+        I5 = ctypes.c_int * 5
+        self.zd, self.bd = I5(B, 1, H, W, C), I5(1, 1, 1, 1, C)
+        self.ws_bytes = self.lib.d8_add_grad_scratch_bytes(self.dt, self.bd, self.zd)
+        self.ws = capi.DeviceArray((max(self.ws_bytes, 16),), np.uint8)
+        es = self.dtype.itemsize
+        self.flops = 4.0 * self.n
+        # add: r z, w pre | relu: r pre, w act | relu_grad: r pre, r gy, rw gpre | bias grad: r gpre
+        self.bytes = es * self.n * 9
+
+    def step(self):
+        from deep8_amd.capi import check
+        L = self.lib
+        check(L.d8_add(self.dt, self.z.ptr, self.zd, self.b.ptr, self.bd, self.pre.ptr, self.zd, None))
+        check(L.d8_relu(self.dt, self.pre.ptr, self.act.ptr, self.n, None))
+        self.gpre.zero_()
+        self.gb.zero_()
+        check(L.d8_relu_grad(self.dt, self.pre.ptr, self.gpre.ptr, self.gy.ptr, self.n, None))
+        check(L.d8_add_grad(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
+
+
 def _uni(r, s):
     return r.uniform(-1, 1, s).astype(np.float32)
 
@@ -250,6 +288,8 @@ def make_workload(key):
     if key == "c5":
         return ConvWorkload("c5: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 58x58x64 (Deep8 covered=false)",
                             np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
+    if key == "e4":
+        return BiasReluWorkload("e4: bias Add + ReLu fwd+bwd on config 4's output, fp32 B32 56x56x64", np.float32, 32, 56, 56, 64, 7)
     raise SystemExit("unknown workload %r" % key)
 
 
@@ -391,7 +431,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5"):
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5", "e4"):
             if key == a.workload:
                 continue
             del wl
@@ -399,7 +439,7 @@ def main():
             oms = _time_steps(wl.step, 5, 2)
             o = {"ms_per_step": round(oms, 4), "tflops": round(wl.flops / (oms * 1e-3) / 1e12, 2),
                  "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
-            if isinstance(wl, ConvWorkload):
+            if isinstance(wl, (ConvWorkload, BiasReluWorkload)):
                 o["images_per_s"] = round(wl.B / (oms * 1e-3), 1)
             others[key] = o
         out["others"] = others

@@ -86,6 +86,9 @@ Variable &operator*(Variable &x, Variable &y);  // MatrixMultiply
 Variable &matrixMultiply(Variable &x, Variable &y);
 Variable &conv2d(Variable &x, Variable &filter, bool covered = true, int strideY = 1, int strideX = 1, int dilationY = 1, int dilationX = 1);
 Variable &deConv2d(Variable &x, Variable &filter, bool covered = false, int strideY = 1, int strideX = 1);
+Variable &operator+(Variable &x, Variable &y);  // Add, with broadcasting
+Variable &add(Variable &x, Variable &y);
+Variable &relu(Variable &x);
 
 }  // namespace Deep8
 

@@ -54,6 +54,20 @@ size_t DeConv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, co
 void DeConv2dGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
 void DeConv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
 
+// Add (broadcasting) and ReLu: deep8/include/math/Add.h:15-42 (checks deep8/src/math/Add.cpp:7-107),
+// deep8/include/math/ReLu.h:14-30 (checks deep8/src/math/ReLu.cpp:6-36).  Unlike the reference, whose
+// shape loop tests only the batch axis (Add.cpp:16-19), every axis is checked.
+void Add(const Tensor &x, const Tensor &y, Tensor &z);
+void AddGPU(const Tensor &x, const Tensor &y, Tensor &z);
+void AddGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz);
+void AddGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz);
+void AddGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+void AddGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+void ReLu(const Tensor &x, Tensor &y);
+void ReLuGPU(const Tensor &x, Tensor &y);
+void ReLuGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
+void ReLuGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
+
 }  // namespace Math
 }  // namespace Deep8
 

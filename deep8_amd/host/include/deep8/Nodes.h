@@ -91,9 +91,12 @@ public:
     Variable &matrixMultiply(Variable &y);
     Variable &conv2d(Variable &filter, bool covered = true, int strideY = 1, int strideX = 1, int dilationY = 1, int dilationX = 1);
     Variable &deConv2d(Variable &filter, bool covered = false, int strideY = 1, int strideX = 1);
+    // the element-wise steps that follow them
+    Variable &add(Variable &y);
+    Variable &relu();
 };
 
-enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply };
+enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply, Add, ReLu };
 
 class Function : public Node {
 protected:
@@ -148,6 +151,31 @@ public:
     void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
                   size_t index, Tensor *iGradient) override;
 };
+
+// z = x + y under numpy's broadcasting rule (deep8/include/nodes/Add.h:8-27, deep8/src/nodes/Add.cpp:6-45)
+class Add : public Function {
+public:
+    explicit Add(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+// y = max(x, 0) (deep8/include/nodes/ReLu.h:8-26, deep8/src/nodes/ReLu.cpp:6-33)
+class ReLu : public Function {
+public:
+    explicit ReLu(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+// Shape of x + y (deep8/include/utils/ShapeUtils.h:19-36)
+Shape broadcastShape(const Shape &shape1, const Shape &shape2);
 
 }  // namespace Deep8
 

@@ -241,4 +241,8 @@ Variable &deConv2d(Variable &x, Variable &filter, bool covered, int strideY, int
     return x.deConv2d(filter, covered, strideY, strideX);
 }
 
+Variable &operator+(Variable &x, Variable &y) { return x.add(y); }
+Variable &add(Variable &x, Variable &y) { return x.add(y); }
+Variable &relu(Variable &x) { return x.relu(); }
+
 }  // namespace Deep8

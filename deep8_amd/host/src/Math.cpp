@@ -303,5 +303,108 @@ void DeConv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor
 
 #undef DECONV_ARGS
 
+// ---- Add / ReLu -------------------------------------------------------------------------------------------------
+namespace {
+
+// [batch, d0..d3] with the dims right-aligned and padded with 1 (deep8/include/utils/ShapeUtils.h:41-56)
+struct Dims5 {
+    int d[5];
+};
+
+Dims5 enlargeShapeToMaxDim(const Shape &shape) {
+    DEEP8_ARGUMENT_CHECK(MAX_TENSOR_DIMS >= shape.nDims && shape.nDims >= 1, "the dim is error");
+    Dims5 r;
+    r.d[0] = (int)shape.batch;
+    for (int i = MAX_TENSOR_DIMS, j = (int)shape.nDims - 1; i > 0; --i, --j) r.d[i] = j >= 0 ? (int)shape.dim(j) : 1;
+    return r;
+}
+
+void checkBroadcast(const Tensor &x, const Tensor &y, const Tensor &z) {
+    const Dims5 xa = enlargeShapeToMaxDim(x.shape), ya = enlargeShapeToMaxDim(y.shape), za = enlargeShapeToMaxDim(z.shape);
+    for (int i = 0; i <= MAX_TENSOR_DIMS; ++i) {
+        DEEP8_ARGUMENT_CHECK(1 == xa.d[i] || xa.d[i] == za.d[i], "the shape is error");
+        DEEP8_ARGUMENT_CHECK(1 == ya.d[i] || ya.d[i] == za.d[i], "the shape is error");
+        DEEP8_ARGUMENT_CHECK(za.d[i] == (xa.d[i] > ya.d[i] ? xa.d[i] : ya.d[i]), "the shape is error");
+    }
+}
+
+void addGradGPU(Tensor &g, const Tensor &dz) {
+    const Dims5 ga = enlargeShapeToMaxDim(g.shape), za = enlargeShapeToMaxDim(dz.shape);
+    const int dt = dtypeOf(g);
+    PoolScratch ws(g.device(), d8_add_grad_scratch_bytes(dt, ga.d, za.d));
+    D8_CHECK(d8_add_grad(dt, g.raw(), ga.d, dz.raw(), za.d, ws.ptr, ws.bytes, nullptr));
+}
+
+}  // namespace
+
+void Add(const Tensor &x, const Tensor &y, Tensor &z) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType() && x.deviceType() == z.deviceType(), "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the param data type must be same");
+    checkBroadcast(x, y, z);
+    requireGPU(x);
+    AddGPU(x, y, z);
+}
+
+void AddGPU(const Tensor &x, const Tensor &y, Tensor &z) {
+    const Dims5 xa = enlargeShapeToMaxDim(x.shape), ya = enlargeShapeToMaxDim(y.shape), za = enlargeShapeToMaxDim(z.shape);
+    D8_CHECK(d8_add(dtypeOf(x), x.raw(), xa.d, y.raw(), ya.d, z.raw(), za.d, nullptr));
+}
+
+void AddGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == dx.deviceType() && x.deviceType() == y.deviceType() &&
+                             x.deviceType() == z.deviceType() && x.deviceType() == dz.deviceType(),
+                         "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape, "the x shape is error");
+    DEEP8_ARGUMENT_CHECK(z.shape == dz.shape, "the z shape is error");
+    checkBroadcast(x, y, z);
+    requireGPU(x);
+    AddGradXGPU(x, dx, y, z, dz);
+}
+
+void AddGradXGPU(const Tensor &, Tensor &dx, const Tensor &, const Tensor &, const Tensor &dz) { addGradGPU(dx, dz); }
+
+void AddGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType() && x.deviceType() == dy.deviceType() &&
+                             x.deviceType() == z.deviceType() && x.deviceType() == dz.deviceType(),
+                         "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == dy.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape, "the y shape is error");
+    DEEP8_ARGUMENT_CHECK(z.shape == dz.shape, "the z shape is error");
+    checkBroadcast(x, y, z);
+    requireGPU(x);
+    AddGradYGPU(x, y, dy, z, dz);
+}
+
+void AddGradYGPU(const Tensor &, const Tensor &, Tensor &dy, const Tensor &, const Tensor &dz) { addGradGPU(dy, dz); }
+
+void ReLu(const Tensor &x, Tensor &y) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType(), "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType, "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == y.shape, "the param shape must be same");
+    requireGPU(x);
+    ReLuGPU(x, y);
+}
+
+void ReLuGPU(const Tensor &x, Tensor &y) { D8_CHECK(d8_relu(dtypeOf(x), x.raw(), y.raw(), (long)x.shape.size(), nullptr)); }
+
+void ReLuGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == dx.deviceType() && x.deviceType() == y.deviceType() && x.deviceType() == dy.deviceType(),
+                         "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == dy.elementType,
+                         "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && x.shape == y.shape && x.shape == dy.shape, "the param shape must be same");
+    requireGPU(x);
+    ReLuGradGPU(x, dx, y, dy);
+}
+
+void ReLuGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy) {
+    D8_CHECK(d8_relu_grad(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), (long)x.shape.size(), nullptr));
+}
+
 }  // namespace Math
 }  // namespace Deep8

@@ -154,6 +154,18 @@ Variable &Variable::matrixMultiply(Variable &y) {
     return *executor->addFunction(new MatrixMultiply(in));
 }
 
+Variable &Variable::add(Variable &y) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this, &y};
+    return *executor->addFunction(new Add(in));
+}
+
+Variable &Variable::relu() {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this};
+    return *executor->addFunction(new ReLu(in));
+}
+
 Variable &Variable::conv2d(Variable &filter, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
     DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
     std::vector<Node *> in = {this, &filter};
@@ -362,6 +374,63 @@ void DeConv2d::backward(const std::vector<const Tensor *> &in, const Tensor *out
     } else {
         DEEP8_RUNTIME_ERROR("the index of DeConv2d backward is error");
     }
+}
+
+// ---- Add / ReLu -------------------------------------------------------------------------------------------------
+Shape broadcastShape(const Shape &shape1, const Shape &shape2) {
+    DEEP8_ARGUMENT_CHECK(1 == shape1.batch || 1 == shape2.batch || shape1.batch == shape2.batch, "the batch must be 1 or equal");
+    const size_t nDims = std::max<size_t>(shape1.nDims, shape2.nDims);
+    std::vector<size_t> ret(nDims);
+    for (int i = (int)nDims - 1, i1 = (int)shape1.nDims - 1, i2 = (int)shape2.nDims - 1; i >= 0; --i, --i1, --i2) {
+        const size_t size1 = i1 >= 0 ? shape1.dim(i1) : 1, size2 = i2 >= 0 ? shape2.dim(i2) : 1;
+        DEEP8_ARGUMENT_CHECK(1 == size1 || 1 == size2 || size1 == size2, "the Shape can not Broadcast");
+        ret[i] = std::max<size_t>(size1, size2);
+    }
+    return Shape(std::max<size_t>(shape1.batch, shape2.batch), ret);
+}
+
+Add::Add(std::vector<Node *> &in) : Function(in) {
+    DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the Add Function needs 2 input");
+}
+
+Shape Add::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputShapes.size(), "the input count must be 2");
+    return broadcastShape(inputShapes[0], inputShapes[1]);
+}
+
+ElementType Add::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputTypes.size(), "the input count must be 2");
+    return Function::checkElementType(inputTypes);
+}
+
+void Add::forward(const std::vector<const Tensor *> &in, Tensor *output) { Math::Add(*in[0], *in[1], *output); }
+
+void Add::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t index,
+                   Tensor *iGradient) {
+    if (0 == index) Math::AddGradX(*in[0], *iGradient, *in[1], *output, *outputGradient);
+    else if (1 == index) Math::AddGradY(*in[0], *in[1], *iGradient, *output, *outputGradient);
+    else DEEP8_RUNTIME_ERROR("the index is error");
+}
+
+ReLu::ReLu(std::vector<Node *> &in) : Function(in) {
+    DEEP8_ARGUMENT_CHECK(1 == inputs.size(), "the ReLu Function needs 1 input");
+}
+
+Shape ReLu::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputShapes.size(), "the input count must be 1");
+    return inputShapes[0];
+}
+
+ElementType ReLu::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputTypes.size(), "the input count must be 1");
+    return Function::checkElementType(inputTypes);
+}
+
+void ReLu::forward(const std::vector<const Tensor *> &in, Tensor *output) { Math::ReLu(*in[0], *output); }
+
+void ReLu::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t,
+                    Tensor *iGradient) {
+    Math::ReLuGrad(*in[0], *iGradient, *output, *outputGradient);
 }
 
 }  // namespace Deep8

@@ -485,6 +485,136 @@ TEST_GPU(eager_executor_matmul_chain) {
     EXPECT(executor.nodeByName(interimName) == nullptr);  // interim nodes are gone after backward
 }
 
+// ---- Add / ReLu: the shapes of test/AddTest.h (a batch of matrices plus one row shared by all) --------------
+void addCase(ElementType type, size_t xb, std::vector<size_t> xd, size_t yb, std::vector<size_t> yd, int hi) {
+    HostTensor x = randomTensor(type, xb, xd, hi), y = randomTensor(type, yb, yd, hi);
+    Variable v0 = placeholder(type), v1 = placeholder(type);
+    std::vector<Node *> in = {&v0, &v1};
+    Add add(in);
+    std::vector<Shape> shapes = {x.t.shape, y.t.shape};
+    Shape zs = add.checkShape(shapes);
+    std::vector<size_t> zd(zs.dims, zs.dims + zs.nDims);
+    HostTensor z = randomTensor(type, zs.batch, zd, 0), dz = randomTensor(type, zs.batch, zd, hi);
+    HostTensor dx = randomTensor(type, xb, xd, hi), dy = randomTensor(type, yb, yd, hi);
+    std::vector<float> wdx = dx.host, wdy = dy.host;
+
+    std::vector<const Tensor *> tin = {&x.t, &y.t};
+    add.forward(tin, &z.t);
+    add.backward(tin, &z.t, &dz.t, 0, &dx.t);
+    add.backward(tin, &z.t, &dz.t, 1, &dy.t);
+    download(z);
+    download(dx);
+    download(dy);
+
+    // walk z with the five enlarged axes; an operand index ignores the axes it is broadcast along
+    auto enlarge = [](const Shape &s) {
+        std::vector<size_t> d(5, 1);
+        d[0] = s.batch;
+        for (int i = 4, j = (int)s.nDims - 1; j >= 0; --i, --j) d[i] = s.dim(j);
+        return d;
+    };
+    const std::vector<size_t> xe = enlarge(x.t.shape), ye = enlarge(y.t.shape), ze = enlarge(zs);
+    std::vector<float> wz(z.host.size());
+    for (size_t e = 0; e < wz.size(); ++e) {
+        size_t rem = e, xi = 0, yi = 0, idx[5];
+        for (int a = 4; a >= 0; --a) idx[a] = rem % ze[a], rem /= ze[a];
+        for (int a = 0; a < 5; ++a) {
+            xi = xi * xe[a] + (xe[a] == 1 ? 0 : idx[a]);
+            yi = yi * ye[a] + (ye[a] == 1 ? 0 : idx[a]);
+        }
+        wz[e] = x.host[xi] + y.host[yi];
+        wdx[xi] += dz.host[e];
+        wdy[yi] += dz.host[e];
+    }
+    EXPECT(z.host == wz);
+    EXPECT(dx.host == wdx);
+    EXPECT(dy.host == wdy);
+}
+
+TEST_GPU(add_float_shared_row) { addCase(ElementType::from<float>(), 10, {50, 20}, 1, {20}, 50); }
+TEST_GPU(add_float_same_shape) { addCase(ElementType::from<float>(), 3, {7, 5}, 3, {7, 5}, 50); }
+TEST_GPU(add_float_both_broadcast) { addCase(ElementType::from<float>(), 1, {6, 1}, 4, {1, 9}, 50); }
+TEST_GPU(add_float_channel_bias) { addCase(ElementType::from<float>(), 2, {6, 6, 8}, 1, {8}, 50); }
+TEST_GPU(add_half) { addCase(ElementType::from<half>(), 2, {6, 8}, 1, {8}, 4); }
+
+TEST_GPU(relu_float_and_errors) {
+    ElementType type = ElementType::from<float>();
+    HostTensor x = randomTensor(type, 2, {9, 7}, 21), y = randomTensor(type, 2, {9, 7}, 0);
+    for (float &f : x.host) f -= 10.f;  // integers in [-10, 10]
+    upload(x);
+    HostTensor dy = randomTensor(type, 2, {9, 7}, 20), dx = randomTensor(type, 2, {9, 7}, 20);
+    std::vector<float> wdx = dx.host;
+    Variable v0 = placeholder(type);
+    std::vector<Node *> in = {&v0};
+    ReLu relu(in);
+    std::vector<const Tensor *> tin = {&x.t};
+    relu.forward(tin, &y.t);
+    relu.backward(tin, &y.t, &dy.t, 0, &dx.t);
+    download(y);
+    download(dx);
+    for (size_t i = 0; i < x.host.size(); ++i) {
+        EXPECT(y.host[i] == (x.host[i] > 0 ? x.host[i] : 0.f));
+        EXPECT(dx.host[i] == wdx[i] + (x.host[i] > 0 ? dy.host[i] : 0.f));
+    }
+    HostTensor bad = randomTensor(type, 2, {9, 8}, 0), row = randomTensor(type, 1, {5}, 0);
+    EXPECT(throws<std::invalid_argument>([&] { Math::ReLu(x.t, bad.t); }));
+    EXPECT(throws<std::invalid_argument>([&] { Math::Add(x.t, row.t, y.t); }));  // 7 against 5 cannot broadcast
+    std::vector<Shape> shapes = {x.t.shape, row.t.shape};
+    Variable v1 = placeholder(type);
+    std::vector<Node *> two = {&v0, &v1};
+    Add add(two);
+    EXPECT(throws<std::invalid_argument>([&] { add.checkShape(shapes); }));
+}
+
+TEST_GPU(eager_executor_dense_layer_with_bias_and_relu) {
+    EagerExecutor executor(DeviceType::GPU);
+    const size_t B = 4, K = 24, N = 16;
+    Variable &x = inputParameter(&executor, {B, K});
+    Variable &W = parameter(&executor, {K, N});
+    Variable &b = parameter(&executor, {N});
+    Variable &v = parameter(&executor, {N});
+    Variable &u = inputParameter(&executor, {1, B});
+    std::vector<float> hx(B * K), hW(K * N), hb(N), hv(N), hu(B, 1.f);
+    u.feed(hu.data());
+    for (float &f : hx) f = randInt(7) - 3.f;
+    for (float &f : hW) f = randInt(7) - 3.f;
+    for (float &f : hb) f = randInt(7) - 3.f;
+    for (float &f : hv) f = randInt(5);
+    x.feed(hx.data());
+    W.feed(hW.data());
+    b.feed(hb.data());
+    v.feed(hv.data());
+
+    Variable &act = relu(x * W + b);  // [B x N], the bias row shared by all rows
+    Variable &out = act * v;          // [B]
+    Variable &loss = u * out;         // their sum: a scalar to start the backward pass from
+    EXPECT(act.shape() == Shape(1, {B, N}) && out.shape() == Shape(1, {B}) && loss.isScalar());
+    std::vector<float> got(B);
+    out.fetch(got.data());
+    std::vector<float> pre(B * N), gb(N, 0.f), gW(K * N, 0.f);
+    for (size_t i = 0; i < B; ++i) {
+        float want = 0;
+        for (size_t n = 0; n < N; ++n) {
+            float a = hb[n];
+            for (size_t k = 0; k < K; ++k) a += hx[i * K + k] * hW[k * N + n];
+            pre[i * N + n] = a;
+            want += (a > 0 ? a : 0.f) * hv[n];
+        }
+        EXPECT(got[i] == want);
+    }
+    backward(loss);  // d loss / d pre = v where pre > 0
+    for (size_t i = 0; i < B; ++i)
+        for (size_t n = 0; n < N; ++n) {
+            const float g = pre[i * N + n] > 0 ? hv[n] : 0.f;
+            gb[n] += g;
+            for (size_t k = 0; k < K; ++k) gW[k * N + n] += hx[i * K + k] * g;
+        }
+    std::vector<float> rb(N), rW(K * N);
+    gpu().copyFromGPUToCPU(b.gradient.raw(), rb.data(), rb.size() * 4);
+    gpu().copyFromGPUToCPU(W.gradient.raw(), rW.data(), rW.size() * 4);
+    EXPECT(rb == gb && rW == gW);
+}
+
 TEST_GPU(eager_executor_conv_to_scalar) {
     EagerExecutor executor(DeviceType::GPU);
     Variable &x = parameter(&executor, 1, {3, 3, 2});
