@@ -128,16 +128,26 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
     }
 }
 
-// g[k0][c] += sum over chunks of partial[k0][chunk][c], chunks added in order.
+// g[k0][c] += sum over chunks of partial[k0][chunk][c].  A block covers 32 outputs; 8 lanes per
+// output each add every 8th chunk and meet in LDS in a fixed order.
 template <typename T>
 __global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__restrict__ partial, T *__restrict__ g,
                                                                 int C, int chunks, long total) {
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    __shared__ float part[8][32];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const long idx = (long)blockIdx.x * 32 + tx;
+    float v = 0.f;
+    if (idx < total) {
         const long k0 = idx / C;
         const int c = (int)(idx - k0 * C);
         const float *p = partial + k0 * chunks * C + c;
-        float v = 0.f;
-        for (int k = 0; k < chunks; ++k) v += p[(long)k * C];
+        for (int k = ty; k < chunks; k += 8) v += p[(long)k * C];
+    }
+    part[ty][tx] = v;
+    __syncthreads();
+    if (ty == 0 && idx < total) {
+#pragma unroll
+        for (int k = 1; k < 8; ++k) v += part[k][tx];
         g[idx] = (T)(ew_f32(g[idx]) + v);
     }
 }
@@ -256,7 +266,7 @@ static ReducePlan plan_reduce(const int *d, const int *zd) {
         long chunks = (4L * cu_count()) / (colblocks * p.K0);
         const long max_chunks = (p.R + 63) / 64;
         if (chunks > max_chunks) chunks = max_chunks;
-        if (chunks > 1024) chunks = 1024;
+        if (chunks > 256) chunks = 256;
         if (chunks < 1) chunks = 1;
         p.rows_per_chunk = (int)((p.R + chunks - 1) / chunks);
         p.chunks = (int)((p.R + p.rows_per_chunk - 1) / p.rows_per_chunk);
@@ -291,8 +301,8 @@ static int add_grad_t(T *g, const int *d, const T *dz, const int *zd, void *scra
                                TX, rpc, chunks);
         if (chunks > 1) {
             D8_LAUNCH_CHECK();
-            hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, (const float *)scratch, g,
-                               (int)p.C, chunks, ng);
+            hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3((unsigned)((ng + 31) / 32)), dim3(256), 0, s,
+                               (const float *)scratch, g, (int)p.C, chunks, ng);
         }
     } else {
         ReduceGeom q;
