@@ -123,6 +123,27 @@ class MatMulWorkload:
         return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
 
 
+def mfma_stream_ceiling(wl, dtype_name):
+    """TFLOP/s of back-to-back MFMAs on this workload's own operand bits (registers only, no LDS or
+    global traffic): the matrix pipe's sustained rate under the power limit, which depends on the
+    data.  Timed with HIP events like the GEMM launches."""
+    import ctypes
+    from deep8_amd import capi
+    lib = wl.lib
+    out = capi.DeviceArray((lib.d8_mfma_stream_out_bytes(),), np.uint8)
+    flops = ctypes.c_double(0)
+    iters = 100 if wl.dtype == np.float16 else 400  # 100-200 us per launch, like the GEMMs
+
+    def run():
+        capi.check(lib.d8_mfma_stream(wl.dt, wl.x.ptr, wl.x.nbytes, out.ptr, iters, ctypes.byref(flops), None))
+    for _ in range(10):
+        run()
+    ms = _time_events(run, 30)
+    t = flops.value / (ms * 1e-3) / 1e12
+    return {"tflops": round(t, 1), "frac_of_peak": round(t / PEAK[dtype_name], 4), "launch_us": round(ms * 1e3, 1),
+            "operands": "x of this workload", "note": "MFMA instructions only, operands in registers"}
+
+
 class ConvWorkload:
     """Conv2d or DeConv2d forward + GradX + GradY through d8_conv2d* / d8_deconv2d*."""
 
@@ -412,6 +433,7 @@ def main():
         roof = {"bound": "mfma", "kernel": wl.kernel, "achieved": round(ach, 2), "peak": PEAK[dtype],
                 "unit": "TFLOP/s", "frac": round(ach / PEAK[dtype], 4), "launch_us": round(avg_ms * 1e3, 2),
                 "traffic": MEASURED_TRAFFIC.get(a.workload)}
+        roof["mfma_stream_ceiling"] = mfma_stream_ceiling(wl, dtype)
 
     out = {
         "metric": "Conv2d fwd+bwd images/s" if is_conv else "MatrixMultiply fwd+bwd TFLOP/s",

@@ -67,6 +67,8 @@ SIGNATURES = {
     "d8_add_grad": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
     "d8_relu": (_I, [_I, _P, _P, ctypes.c_long, _P]),
     "d8_relu_grad": (_I, [_I, _P, _P, _P, ctypes.c_long, _P]),
+    "d8_mfma_stream_out_bytes": (_Z, []),
+    "d8_mfma_stream": (_I, [_I, _P, _Z, _P, _I, ctypes.POINTER(ctypes.c_double), _P]),
 }
 
 

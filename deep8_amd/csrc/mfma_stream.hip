@@ -1,0 +1,96 @@
+// Measurement aid: the rate the matrix pipe sustains on given operand bits when nothing else
+// runs -- no LDS, no global loads in the loop.  The tiled GEMM's MFMA instruction is issued back
+// to back on operands held in registers, two waves per SIMD, on every CU.  The achievable clock
+// under matrix load depends on how many operand bits toggle, so this gives the ceiling any GEMM
+// kernel has on that data (it is well below the nominal peak for real-valued operands).
+#include "common.h"
+
+namespace d8 {
+
+// A wave keeps 2 A and 4 B fragments per set and cycles through SETS sets, so that the operand
+// registers differ from one MFMA to the next as they do in a GEMM.
+template <typename E>
+struct StreamOp;
+template <>
+struct StreamOp<f16> {
+    typedef f16x8 Frag;
+    static constexpr double FLOPS = 2.0 * 32 * 32 * 16;
+    __device__ static f32x16 mfma(Frag a, Frag b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <>
+struct StreamOp<float> {
+    typedef float Frag;
+    static constexpr double FLOPS = 2.0 * 32 * 32 * 2;
+    __device__ static f32x16 mfma(Frag a, Frag b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+};
+
+template <typename E, int SETS>
+__global__ __launch_bounds__(256) void mfma_stream_kernel(const typename StreamOp<E>::Frag *data, unsigned nfrag,
+                                                          float *out, int iters) {
+    typedef StreamOp<E> Op;
+    const unsigned t = blockIdx.x * 256 + threadIdx.x;
+    typename Op::Frag a[SETS][2], b[SETS][4];
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a[s][i] = data[(t * 6 * SETS + s * 6 + i) % nfrag];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[s][j] = data[(t * 6 * SETS + s * 6 + 2 + j) % nfrag];
+    }
+    f32x16 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int s = 0; s < SETS; ++s)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = Op::mfma(a[s][i], b[s][j], acc[i][j]);
+    }
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) v += acc[i][j][r];
+    out[t] = v;
+}
+
+}  // namespace d8
+
+using namespace d8;
+
+extern "C" {
+
+size_t d8_mfma_stream_out_bytes(void) { return (size_t)cu_count() * 2 * 256 * sizeof(float); }
+
+int d8_mfma_stream(int dtype, const void *operands, size_t operand_bytes, void *out, int iters, double *flops, void *stream) {
+    D8_REQUIRE(dtype == D8_FLOAT16 || dtype == D8_FLOAT32, "dtype %d not supported", dtype);
+    D8_REQUIRE(operands && out && flops, "null argument");
+    D8_REQUIRE(((size_t)operands & 15) == 0 && operand_bytes >= 16, "operands must be 16-byte aligned and hold 16 bytes or more");
+    D8_REQUIRE(iters > 0, "iters must be positive");
+    constexpr int SETS = 4;
+    const int blocks = cu_count() * 2;
+    const size_t frag = dtype == D8_FLOAT16 ? 16 : 4;
+    const size_t nfrag = operand_bytes / frag;
+    D8_REQUIRE(nfrag < (1ull << 32), "at most 2^32 fragments");
+    if (dtype == D8_FLOAT16) {
+        hipLaunchKernelGGL((mfma_stream_kernel<f16, SETS>), dim3(blocks), dim3(256), 0, as_stream(stream), (const f16x8 *)operands,
+                           (unsigned)nfrag, (float *)out, iters);
+        *flops = StreamOp<f16>::FLOPS * 8 * SETS * iters * 4.0 * blocks;
+    } else {
+        hipLaunchKernelGGL((mfma_stream_kernel<float, SETS>), dim3(blocks), dim3(256), 0, as_stream(stream), (const float *)operands,
+                           (unsigned)nfrag, (float *)out, iters);
+        *flops = StreamOp<float>::FLOPS * 8 * SETS * iters * 4.0 * blocks;
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -190,6 +190,16 @@ int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int 
 int d8_relu(int dtype, const void *x, void *y, long n, void *stream);
 int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, void *stream);
 
+/* ---- measurement aid (no counterpart in the reference) ---------------------------------------
+ * d8_mfma_stream issues the tiled GEMM's MFMA instruction back to back on operands taken from
+ * `operands` (any device buffer; 16-byte aligned) and held in registers: two waves per SIMD on
+ * every CU, no LDS or global traffic in the loop.  Timing one launch gives the rate the matrix
+ * pipe sustains on those operand bits, i.e. the ceiling a GEMM has on that data.  `out` takes
+ * d8_mfma_stream_out_bytes() bytes; *flops receives the flops one launch performs.             */
+size_t d8_mfma_stream_out_bytes(void);
+int d8_mfma_stream(int dtype, const void *operands, size_t operand_bytes, void *out, int iters,
+                   double *flops, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
