@@ -90,7 +90,10 @@ class MatMulWorkload:
         self.ws = capi.DeviceArray((max(nb, 16),), np.uint8)
         m, k, n = xs[1], xs[2], ys[2]
         self.flops = 3 * 2.0 * zb * m * k * n
-        self.kernel = "gemm_tiled_kernel<%s> (one launch each for fwd, dX, dY)" % ("f16" if self.dtype == np.float16 else "f32")
+        wide = self.dtype == np.float16 and m >= 256 and n >= 256 and k % 64 == 0 and zb * (-(-m // 256)) * (-(-n // 256)) >= 192
+        self.kernel = "%s (one launch each for fwd, dX, dY)" % (
+            "gemm_wide_kernel (fp16, 256x256 tiles)" if wide else
+            "gemm_tiled_kernel<%s>" % ("f16" if self.dtype == np.float16 else "f32"))
         es = self.dtype.itemsize
         nx, ny, nz = np.prod(xs), np.prod(ys), np.prod(self.zs)
         # fwd reads x,y writes z; dX reads dz,y and read-modify-writes dx; dY likewise
@@ -132,7 +135,7 @@ def mfma_stream_ceiling(wl, dtype_name):
     lib = wl.lib
     out = capi.DeviceArray((lib.d8_mfma_stream_out_bytes(),), np.uint8)
     flops = ctypes.c_double(0)
-    iters = 100 if wl.dtype == np.float16 else 400  # 100-200 us per launch, like the GEMMs
+    iters = 200 if wl.dtype == np.float16 else 100  # 100-200 us per launch, like the GEMMs
 
     def run():
         capi.check(lib.d8_mfma_stream(wl.dt, wl.x.ptr, wl.x.nbytes, out.ptr, iters, ctypes.byref(flops), None))

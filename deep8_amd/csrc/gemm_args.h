@@ -50,6 +50,11 @@ bool gemm_tiled_eligible(int dtype, const GemmArgs &g, int transA, int transB);
 // Launch; with g.splits > 1 the fp32 partial sums go to g.ws for the caller to reduce.
 int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipStream_t stream);
 
+// fp16 kernel for large outputs (256 x 256 tiles, v_mfma_f32_16x16x32_f16, loads straight into
+// LDS): unsplit, unsummed products of real matrices with M, N >= 256 and K a multiple of 64.
+bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB);
+int gemm_wide_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);
+
 // Plan the split of the reduction, launch the tiled kernel (which must be eligible) and reduce.
 int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
                    hipStream_t stream);

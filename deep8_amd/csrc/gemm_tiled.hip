@@ -490,6 +490,9 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     // fp32 runs 64-cycle MFMAs on a quarter of the bytes per flop: the 128 x 128 tile already
     // keeps the matrix pipe fed, and the compiler cannot hold the 256 x 256 variant in registers
     if constexpr (sizeof(E) == 2) {
+        static const char *wide = getenv("D8_GEMM_WIDE");  // tuning aid: 0 keeps the 32x32x16 kernel
+        if (big && VIRT == VIRT_NONE && !(wide && atoi(wide) == 0) && gemm_wide_eligible(g, !A_KC, B_KC))
+            return gemm_wide_launch(g, !A_KC, B_KC, stream);
         if (big) return launch_tiled<E, 256, 256, 4, 2, A_KC, B_KC, VIRT>(g, stream);
     }
     // a 64-wide side gets a tile of that width (im2col products with 64 output channels)

@@ -1,6 +1,8 @@
 // Measurement aid: the rate the matrix pipe sustains on given operand bits when nothing else
-// runs -- no LDS, no global loads in the loop.  The tiled GEMM's MFMA instruction is issued back
-// to back on operands held in registers, two waves per SIMD, on every CU.  The achievable clock
+// runs -- no LDS, no global loads in the loop.  The GEMM kernels' MFMA instruction
+// (v_mfma_f32_16x16x32_f16 as an 8 x 8 block per wave, one wave per SIMD, accumulators in AGPRs,
+// like the fp16 kernel for large outputs; v_mfma_f32_32x32x2_f32 as 2 x 4, two waves per SIMD,
+// like the fp32 tiles) is issued back to back on operands held in registers, on every CU.  The achievable clock
 // under matrix load depends on how many operand bits toggle, so this gives the ceiling any GEMM
 // kernel has on that data (it is well below the nominal peak for real-valued operands).
 #include "common.h"
@@ -11,12 +13,6 @@ namespace d8 {
 // registers differ from one MFMA to the next as they do in a GEMM.
 template <typename E>
 struct StreamOp;
-template <>
-struct StreamOp<f16> {
-    typedef f16x8 Frag;
-    static constexpr double FLOPS = 2.0 * 32 * 32 * 16;
-    __device__ static f32x16 mfma(Frag a, Frag b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-};
 template <>
 struct StreamOp<float> {
     typedef float Frag;
@@ -62,6 +58,40 @@ __global__ __launch_bounds__(256) void mfma_stream_kernel(const typename StreamO
     out[t] = v;
 }
 
+// fp16: 8 A and 8 B fragments, 64 accumulator blocks pinned to AGPRs and updated in place.
+__global__ __launch_bounds__(256) void mfma_stream_f16_kernel(const f16x8 *data, unsigned nfrag, float *out, int iters) {
+    const unsigned t = blockIdx.x * 256 + threadIdx.x;
+    f16x8 a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        a[i] = data[(t * 16 + i) % nfrag];
+        b[i] = data[(t * 16 + 8 + i) % nfrag];
+    }
+    f32x4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+            asm volatile("" : "+a"(acc[i][j]));
+        }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(a[i]), "v"(b[j]));
+    }
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v += acc[i][j][r];
+    out[t] = v;
+}
+
 }  // namespace d8
 
 using namespace d8;
@@ -81,9 +111,9 @@ int d8_mfma_stream(int dtype, const void *operands, size_t operand_bytes, void *
     const size_t nfrag = operand_bytes / frag;
     D8_REQUIRE(nfrag < (1ull << 32), "at most 2^32 fragments");
     if (dtype == D8_FLOAT16) {
-        hipLaunchKernelGGL((mfma_stream_kernel<f16, SETS>), dim3(blocks), dim3(256), 0, as_stream(stream), (const f16x8 *)operands,
+        hipLaunchKernelGGL(mfma_stream_f16_kernel, dim3(blocks / 2), dim3(256), 0, as_stream(stream), (const f16x8 *)operands,
                            (unsigned)nfrag, (float *)out, iters);
-        *flops = StreamOp<f16>::FLOPS * 8 * SETS * iters * 4.0 * blocks;
+        *flops = 2.0 * 16 * 16 * 32 * 64 * iters * 4.0 * (blocks / 2);
     } else {
         hipLaunchKernelGGL((mfma_stream_kernel<float, SETS>), dim3(blocks), dim3(256), 0, as_stream(stream), (const float *)operands,
                            (unsigned)nfrag, (float *)out, iters);

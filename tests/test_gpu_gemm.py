@@ -157,6 +157,36 @@ def test_gemm_tiled_split_and_summed(oracle_port, ta, tb, dtype, M, N, K, nb):
         assert np.array_equal(f(got), want), (ta, tb, M, N, K, nb, use_ws)
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("M,N,K,nb,shared_b", [(4096, 4096, 64, 1, False), (3600, 3848, 128, 1, False),
+                                               (2048, 2056, 192, 4, False), (1024, 1280, 448, 16, True)])
+def test_gemm_wide_f16_kernel(oracle_port, ta, tb, M, N, K, nb, shared_b):
+    """fp16 outputs large enough for the 256 x 256-tile kernel (16x16x32 MFMA, loads straight into
+    LDS with an exclusive-or swizzle): ragged edge tiles, beta 0 and 1, strided and shared-operand
+    batches.  Integer operands, so the result is exact; numpy gives the full expected matrix and the
+    oracle's GEMM confirms a band of its rows."""
+    from deep8_amd import ops
+    r = rng(M + 5 * N + 11 * K + nb)
+    lead = (nb,) if nb > 1 else ()
+    A = ints(r, lead + ((K, M) if ta else (M, K)), 3) * (r.random(lead + ((K, M) if ta else (M, K))) < 0.5)
+    B = ints(r, (() if shared_b else lead) + ((N, K) if tb else (K, N)), 3)
+    C0 = ints(r, lead + (M, N), 3)
+    A3, B3 = (A if nb > 1 else A[None]), (B if (nb > 1 and not shared_b) else B[None])
+    opA = np.swapaxes(A3, 1, 2) if ta else A3
+    opB = np.swapaxes(B3, 1, 2) if tb else B3
+    prod = np.matmul(opA.astype(np.float32), opB.astype(np.float32))
+    assert np.abs(prod).max() + 3 < 2048
+    band = slice(M - 300, M - 236)  # crosses the last, shifted tile row
+    for beta in (0.0, 1.0):
+        want = prod + beta * (C0 if nb > 1 else C0[None])
+        got = ops.gemm(ta, tb, h(A), h(B3 if shared_b else B), h(C0), beta)
+        got3 = f(got) if nb > 1 else f(got)[None]
+        assert np.array_equal(got3, want), (ta, tb, M, N, K, nb, beta)
+        a_band = (A3[-1][:, band] if ta else A3[-1][band]).copy()
+        chk = oracle_port.gemm(ta, tb, a_band, B3[-1], (C0 if nb > 1 else C0[None])[-1][band].copy(), beta)
+        assert np.array_equal(got3[-1][band], chk)
+
+
 def test_gemm_argument_errors():
     from deep8_amd import capi
     lib = capi.init()
