@@ -55,15 +55,16 @@ __device__ __forceinline__ wu32x4 make_desc(const void *p, unsigned bytes) {
 }
 
 // One 16-byte piece per lane from global memory straight into LDS: lane i's piece lands at LDS
-// byte address `lds` + 16 * i (`lds`, `soffset` and the descriptor are wave-uniform).  Written
-// as asm so that the compiler does not know LDS is written behind its back by loads that are
-// still in flight: it would otherwise hold every later LDS read until all of them have landed.
-// The barrier of each step (with its vmcnt(0)) is what orders these writes against the reads.
-__device__ __forceinline__ void load_to_lds(const wu32x4 &desc, unsigned lds, unsigned voffset, unsigned soffset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "s"(lds), "v"(voffset), "s"(desc), "s"(soffset)
-                 : "memory");  // m0: a reserved register the compiler sets right before each of its own uses
+// byte address m0 + 16 * i (m0, `soffset` and the descriptor are wave-uniform).  Written as asm so
+// that the compiler does not know LDS is written behind its back by loads that are still in
+// flight: it would otherwise hold every later LDS read until all of them have landed.  The barrier
+// of each step (with its vmcnt(0)) is what orders these writes against the reads.  m0 must be
+// written at least one instruction before the load that uses it (the hardware does not interlock
+// that), so the two are separate statements with an MFMA between them; m0 is a reserved register
+// that the compiler only ever sets right before a use of its own.
+__device__ __forceinline__ void set_lds_target(unsigned lds) { asm volatile("s_mov_b32 m0, %0" : : "s"(lds) : "memory"); }
+__device__ __forceinline__ void load_to_lds(const wu32x4 &desc, unsigned voffset, unsigned soffset) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voffset), "s"(desc), "s"(soffset) : "memory");
 }
 
 // Per-thread constants of one operand: how it fetches its pieces and where its fragments lie.
@@ -101,8 +102,11 @@ struct Operand {
     }
 
     // fetch this operand's tile of one step: 8 rounds of 4 KB, this wave's KB of each
-    __device__ __forceinline__ void fetch_round(const wu32x4 &rsrc, const char *stage, int wave, unsigned sbase, int t) const {
-        load_to_lds(rsrc, (unsigned)(size_t)WIDE_LDS(const char, stage) + (t * 4 + wave) * 1024, voff[t & 1], sbase + t * round_bytes);
+    __device__ __forceinline__ void aim_round(const char *stage, int wave, int t) const {
+        set_lds_target((unsigned)(size_t)WIDE_LDS(const char, stage) + (t * 4 + wave) * 1024);
+    }
+    __device__ __forceinline__ void fetch_round(const wu32x4 &rsrc, unsigned sbase, int t) const {
+        load_to_lds(rsrc, voff[t & 1], sbase + t * round_bytes);
     }
 
     // fragment n (16 rows or columns) of k group kg
@@ -178,8 +182,12 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
         const int step = min(s, nsteps - 1);
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            oa.fetch_round(ra, lds + s * STAGE_BYTES, wave, a_org + step * a_step, t);
-            ob.fetch_round(rb, lds + s * STAGE_BYTES + OPERAND_BYTES, wave, b_org + step * b_step, t);
+            oa.aim_round(lds + s * STAGE_BYTES, wave, t);
+            asm volatile("s_nop 0");
+            oa.fetch_round(ra, a_org + step * a_step, t);
+            ob.aim_round(lds + s * STAGE_BYTES + OPERAND_BYTES, wave, t);
+            asm volatile("s_nop 0");
+            ob.fetch_round(rb, b_org + step * b_step, t);
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces are in LDS
@@ -211,6 +219,10 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
         __syncthreads();
 #pragma unroll
         for (int m = 0; m < 64; ++m) {
+            if ((m & 3) == 0) {
+                if ((m >> 2) < 8) oa.aim_round(As, wave, m >> 2);
+                else ob.aim_round(Bs, wave, (m >> 2) - 8);
+            }
             mfma(acc[m >> 3][m & 7], fa[1][m >> 3], fb[1][m & 7]);
             if ((m & 3) == 0) {
                 // 16 loads into the stage every wave has finished with, one per 4 MFMAs: a load
@@ -218,8 +230,8 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
                 // four waves issue theirs in the same window; issued closer together they hold up
                 // instruction issue (2600 cycles per step at one per 2 MFMAs, 2330 at one per 4)
                 const int d = m >> 2;
-                if (d < 8) oa.fetch_round(ra, As, wave, a_src, d);
-                else ob.fetch_round(rb, Bs, wave, b_src, d - 8);
+                if (d < 8) oa.fetch_round(ra, a_src, d);
+                else ob.fetch_round(rb, b_src, d - 8);
             }
             if (m % 3 == 1 && m < 48) {
                 const int e = m / 3;  // fragments of the next step's k group 0
