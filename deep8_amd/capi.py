@@ -67,6 +67,15 @@ SIGNATURES = {
     "d8_add_grad": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
     "d8_relu": (_I, [_I, _P, _P, ctypes.c_long, _P]),
     "d8_relu_grad": (_I, [_I, _P, _P, _P, ctypes.c_long, _P]),
+    "d8_minus": (_I, [_I, _P, _IP, _P, _IP, _P, _IP, _P]),
+    "d8_minus_grad_y": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
+    "d8_l1norm": (_I, [_I, _P, _P, _I, ctypes.c_long, _P, _Z, _P]),
+    "d8_l1norm_grad": (_I, [_I, _P, _P, _P, _I, ctypes.c_long, _P]),
+    "d8_l2norm": (_I, [_I, _P, _P, _I, ctypes.c_long, _P, _Z, _P]),
+    "d8_l2norm_grad": (_I, [_I, _P, _P, _P, _P, _I, ctypes.c_long, _P]),
+    "d8_reduce_mean": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
+    "d8_reduce_mean_grad": (_I, [_I, _P, _IP, _P, _IP, _P]),
+    "d8_axpby": (_I, [_I, _P, _F, _P, _F, _P, ctypes.c_long, _P]),
     "d8_mfma_stream_out_bytes": (_Z, []),
     "d8_mfma_stream": (_I, [_I, _P, _Z, _P, _I, ctypes.POINTER(ctypes.c_double), _P]),
 }

@@ -3,8 +3,16 @@
 // HBM-bandwidth bound: 16-byte accesses along the contiguous axis, every output written once, and
 // the broadcast-gradient reductions are two deterministic passes (no atomics).
 //
+// The same kernels, with a scale on the second operand or on the reduced sum and an optional
+// transform of the loaded value, also serve Minus, L1Norm / L2Norm (row reductions of |x| and
+// x^2), ReduceMean and its gradient; AXPBY is the trainers' update step.
+//
 // Replaces AddGPU / AddGradXGPU / AddGradYGPU (deep8/src/math/Add.cu:21-133 over
-// deep8/include/math/GPUBinaryElementWise.h) and ReLuGPU / ReLuGradGPU (deep8/src/math/ReLu.cu:20-116).
+// deep8/include/math/GPUBinaryElementWise.h), ReLuGPU / ReLuGradGPU (deep8/src/math/ReLu.cu:20-116),
+// MinusGPU / MinusGradXGPU / MinusGradYGPU (deep8/src/math/Minus.cu:21-147), L1NormGPU / L1NormGradGPU
+// (deep8/src/math/L1Norm.cu:27-136), L2NormGPU / L2NormGradGPU (deep8/src/math/L2Norm.cu),
+// ReduceMeanGPU / ReduceMeanGradGPU (deep8/src/math/ReduceMean.cu:30-203 over GPUReduce.h) and AXPBYGPU
+// (deep8/src/math/AXPBY.cu:9-47).
 #include "common.h"
 
 namespace d8 {
@@ -27,11 +35,12 @@ struct BroadcastGeom {
     long xs[5], ys[5];
 };
 
-// z = x + y.  A thread owns VEC consecutive elements of the innermost axis; an operand that is
-// broadcast along that axis contributes one scalar to all of them.
+// z = x + ys * y.  A thread owns VEC consecutive elements of the innermost axis; an operand that
+// is broadcast along that axis contributes one scalar to all of them.  z may be x itself when x
+// is not broadcast (each thread then reads exactly the elements it writes).
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void add_kernel(const T *__restrict__ x, const T *__restrict__ y, T *__restrict__ z,
-                                                  BroadcastGeom g, long total) {
+__global__ __launch_bounds__(256) void add_kernel(const T *x, const T *__restrict__ y, T *z, BroadcastGeom g, long total,
+                                                  float ys) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
     const int last = g.nd - 1;
     const long inner = g.n[last] / VEC;
@@ -66,31 +75,37 @@ __global__ __launch_bounds__(256) void add_kernel(const T *__restrict__ x, const
         }
         VT o;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) o[e] = (T)(xv[e] + yv[e]);
+        for (int e = 0; e < VEC; ++e) o[e] = (T)(xv[e] + ys * yv[e]);
         *(VT *)(z + idx * VEC) = o;
     }
 }
 
-// g += dz, same shape.
-template <typename T, int VEC>
-__global__ __launch_bounds__(256) void accumulate_kernel(T *__restrict__ g, const T *__restrict__ dz, long total) {
+// What a reduction does to each value it loads.
+enum { LOAD_ID = 0, LOAD_ABS = 1, LOAD_SQUARE = 2 };
+template <int OP>
+__device__ inline float ew_load(float v) { return OP == LOAD_ABS ? fabsf(v) : (OP == LOAD_SQUARE ? v * v : v); }
+
+// g += scale * op(dz), same shape.
+template <typename T, int VEC, int OP>
+__global__ __launch_bounds__(256) void accumulate_kernel(T *__restrict__ g, const T *__restrict__ dz, long total, float scale) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const VT a = *(const VT *)(g + idx * VEC), b = *(const VT *)(dz + idx * VEC);
         VT o;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(a[e]) + ew_f32(b[e]));
+        for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(a[e]) + scale * ew_load<OP>(ew_f32(b[e])));
         *(VT *)(g + idx * VEC) = o;
     }
 }
 
 // dz viewed [K0][R][C]; sums over R.  Block (x: column group, y: chunk of R, z: k0); TX threads
 // across column vectors, 256 / TX rows in flight.  The row lanes meet in LDS in a fixed order.
-// With one chunk the sums go straight into g (+=); otherwise into partial[k0][chunk][C].
-template <typename T, int VEC>
+// With one chunk the sums go straight into g (g += scale * sum); otherwise into
+// partial[k0][chunk][C].
+template <typename T, int VEC, int OP>
 __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ dz, T *__restrict__ g,
                                                          float *__restrict__ partial, int R, int C, int TX,
-                                                         int rows_per_chunk, int chunks) {
+                                                         int rows_per_chunk, int chunks, float scale) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
     __shared__ float part[256][VEC];
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX, lanes = 256 / TX;
@@ -106,7 +121,7 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
         for (int r = chunk * rows_per_chunk + ty; r < r1; r += lanes) {
             const VT v = *(const VT *)(p + (long)r * C);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) acc[e] += ew_f32(v[e]);
+            for (int e = 0; e < VEC; ++e) acc[e] += ew_load<OP>(ew_f32(v[e]));
         }
     }
 #pragma unroll
@@ -119,7 +134,7 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
         if (chunks == 1) {
             T *o = g + (long)k0 * C + (long)cv * VEC;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(o[e]) + acc[e]);
+            for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(o[e]) + scale * acc[e]);
         } else {
             float *o = partial + ((long)k0 * chunks + chunk) * C + (long)cv * VEC;
 #pragma unroll
@@ -132,7 +147,7 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
 // output each add every 8th chunk and meet in LDS in a fixed order.
 template <typename T>
 __global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__restrict__ partial, T *__restrict__ g,
-                                                                int C, int chunks, long total) {
+                                                                int C, int chunks, long total, float scale) {
     __shared__ float part[8][32];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const long idx = (long)blockIdx.x * 32 + tx;
@@ -148,7 +163,7 @@ __global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__r
     if (ty == 0 && idx < total) {
 #pragma unroll
         for (int k = 1; k < 8; ++k) v += part[k][tx];
-        g[idx] = (T)(ew_f32(g[idx]) + v);
+        g[idx] = (T)(ew_f32(g[idx]) + scale * v);
     }
 }
 
@@ -159,9 +174,9 @@ struct ReduceGeom {
     int kept[5];   // 1 where g has the same extent, 0 where it is summed (or the extent is 1)
 };
 
-template <typename T>
+template <typename T, int OP>
 __global__ __launch_bounds__(256) void broadcast_sum_kernel(const T *__restrict__ dz, T *__restrict__ g, ReduceGeom q,
-                                                            long total) {
+                                                            long total, float scale) {
     long zs[5];
     zs[4] = 1;
     for (int a = 3; a >= 0; --a) zs[a] = zs[a + 1] * q.n[a + 1];
@@ -178,7 +193,7 @@ __global__ __launch_bounds__(256) void broadcast_sum_kernel(const T *__restrict_
         while (true) {
             long off = base;
             for (int a = 0; a < 5; ++a) off += (long)i[a] * zs[a];
-            acc += ew_f32(dz[off]);
+            acc += ew_load<OP>(ew_f32(dz[off]));
             int a = 4;
             for (; a >= 0; --a) {
                 if (q.kept[a]) continue;
@@ -187,7 +202,7 @@ __global__ __launch_bounds__(256) void broadcast_sum_kernel(const T *__restrict_
             }
             if (a < 0) break;
         }
-        g[idx] = (T)(ew_f32(g[idx]) + acc);
+        g[idx] = (T)(ew_f32(g[idx]) + scale * acc);
     }
 }
 
@@ -213,6 +228,50 @@ __global__ __launch_bounds__(256) void relu_grad_kernel(const T *__restrict__ x,
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(old[e]) + (v[e] > (T)0 ? ew_f32(d[e]) : 0.f));
         *(VT *)(dx + idx * VEC) = o;
+    }
+}
+
+// dx[b][i] += dy[b] * sign(x[b][i])        (L1, deep8/src/math/L1Norm.cu:77-95)
+// dx[b][i] += dy[b] / y[b] * x[b][i]       (L2)
+template <typename T, int VEC, bool L2>
+__global__ __launch_bounds__(256) void norm_grad_kernel(const T *__restrict__ x, T *__restrict__ dx, const T *__restrict__ y,
+                                                        const T *__restrict__ dy, long row_vecs, long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long b = idx / row_vecs;
+        const float s = L2 ? ew_f32(dy[b]) / ew_f32(y[b]) : ew_f32(dy[b]);
+        const VT v = *(const VT *)(x + idx * VEC), old = *(const VT *)(dx + idx * VEC);
+        VT o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float xv = ew_f32(v[e]);
+            const float gx = L2 ? s * xv : (xv > 0.f ? s : (xv == 0.f ? 0.f : -s));
+            o[e] = (T)(ew_f32(old[e]) + gx);
+        }
+        *(VT *)(dx + idx * VEC) = o;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void sqrt_kernel(T *p, long n) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) p[i] = (T)sqrtf(ew_f32(p[i]));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void ew_zero_kernel(T *p, long n) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) p[i] = (T)0;
+}
+
+// z = alpha * x + beta * y (z may be x or y)
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void axpby_kernel(const T *x, float alpha, const T *y, float beta, T *z, long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const VT a = *(const VT *)(x + idx * VEC), b = *(const VT *)(y + idx * VEC);
+        VT o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = (T)(alpha * ew_f32(a[e]) + beta * ew_f32(b[e]));
+        *(VT *)(z + idx * VEC) = o;
     }
 }
 
@@ -274,15 +333,17 @@ static ReducePlan plan_reduce(const int *d, const int *zd) {
     return p;
 }
 
-template <typename T, int WIDE>
-static int add_grad_t(T *g, const int *d, const T *dz, const int *zd, void *scratch, size_t scratch_bytes, hipStream_t s) {
+// g += scale * (op(dz) summed over the axes where g has extent 1 and dz does not)
+template <typename T, int WIDE, int OP = LOAD_ID>
+static int reduce_t(T *g, const int *d, const T *dz, const int *zd, void *scratch, size_t scratch_bytes, hipStream_t s,
+                    float scale = 1.f) {
     const ReducePlan p = plan_reduce(d, zd);
     const long ng = prod5(d);
     if (p.kind == 0) {
         if (ng % WIDE == 0 && al16(g) && al16(dz))
-            hipLaunchKernelGGL((accumulate_kernel<T, WIDE>), dim3(ew_grid(ng / WIDE, 256)), dim3(256), 0, s, g, dz, ng / WIDE);
+            hipLaunchKernelGGL((accumulate_kernel<T, WIDE, OP>), dim3(ew_grid(ng / WIDE, 256)), dim3(256), 0, s, g, dz, ng / WIDE, scale);
         else
-            hipLaunchKernelGGL((accumulate_kernel<T, 1>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, g, dz, ng);
+            hipLaunchKernelGGL((accumulate_kernel<T, 1, OP>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, g, dz, ng, scale);
     } else if (p.kind == 1) {
         int chunks = p.chunks, rpc = p.rows_per_chunk;
         const size_t need = (size_t)p.K0 * chunks * p.C * sizeof(float);
@@ -294,27 +355,27 @@ static int add_grad_t(T *g, const int *d, const T *dz, const int *zd, void *scra
         while (TX < 32 && TX < cvs) TX *= 2;
         dim3 grid((unsigned)((cvs + TX - 1) / TX), (unsigned)chunks, (unsigned)p.K0);
         if (wide)
-            hipLaunchKernelGGL((column_sum_kernel<T, WIDE>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
-                               TX, rpc, chunks);
+            hipLaunchKernelGGL((column_sum_kernel<T, WIDE, OP>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
+                               TX, rpc, chunks, scale);
         else
-            hipLaunchKernelGGL((column_sum_kernel<T, 1>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
-                               TX, rpc, chunks);
+            hipLaunchKernelGGL((column_sum_kernel<T, 1, OP>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
+                               TX, rpc, chunks, scale);
         if (chunks > 1) {
             D8_LAUNCH_CHECK();
             hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3((unsigned)((ng + 31) / 32)), dim3(256), 0, s,
-                               (const float *)scratch, g, (int)p.C, chunks, ng);
+                               (const float *)scratch, g, (int)p.C, chunks, ng, scale);
         }
     } else {
         ReduceGeom q;
         for (int a = 0; a < 5; ++a) q.n[a] = zd[a], q.kept[a] = (d[a] == zd[a] && zd[a] > 1) ? 1 : 0;
-        hipLaunchKernelGGL((broadcast_sum_kernel<T>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, dz, g, q, ng);
+        hipLaunchKernelGGL((broadcast_sum_kernel<T, OP>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, dz, g, q, ng, scale);
     }
     D8_LAUNCH_CHECK();
     return 0;
 }
 
 template <typename T, int WIDE>
-static int add_t(const T *x, const int *xd, const T *y, const int *yd, T *z, const int *zd, hipStream_t s) {
+static int add_t(const T *x, const int *xd, const T *y, const int *yd, T *z, const int *zd, hipStream_t s, float ys = 1.f) {
     // merge consecutive axes on which both operands behave the same way
     BroadcastGeom g;
     int kx[5], ky[5];
@@ -335,10 +396,42 @@ static int add_t(const T *x, const int *xd, const T *y, const int *yd, T *z, con
     }
     const long n = prod5(zd);
     if (g.n[g.nd - 1] % WIDE == 0 && al16(x) && al16(y) && al16(z))
-        hipLaunchKernelGGL((add_kernel<T, WIDE>), dim3(ew_grid(n / WIDE, 256)), dim3(256), 0, s, x, y, z, g, n / WIDE);
+        hipLaunchKernelGGL((add_kernel<T, WIDE>), dim3(ew_grid(n / WIDE, 256)), dim3(256), 0, s, x, y, z, g, n / WIDE, ys);
     else
-        hipLaunchKernelGGL((add_kernel<T, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, x, y, z, g, n);
+        hipLaunchKernelGGL((add_kernel<T, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, x, y, z, g, n, ys);
     D8_LAUNCH_CHECK();
+    return 0;
+}
+
+// y[b] = sum over i of op(x[b][i]) (then the square root for L2): zero, reduce, finish.
+template <typename T, int WIDE, int OP>
+static int norm_t(const T *x, T *y, int batch, long size, void *scratch, size_t scratch_bytes, hipStream_t s) {
+    const int yd[5] = {batch, 1, 1, 1, 1}, xd[5] = {batch, 1, 1, 1, (int)size};
+    hipLaunchKernelGGL((ew_zero_kernel<T>), dim3(ew_grid(batch, 256)), dim3(256), 0, s, y, (long)batch);
+    D8_LAUNCH_CHECK();
+    if (int rc = reduce_t<T, WIDE, OP>(y, yd, x, xd, scratch, scratch_bytes, s)) return rc;
+    if (OP == LOAD_SQUARE) {
+        hipLaunchKernelGGL((sqrt_kernel<T>), dim3(ew_grid(batch, 256)), dim3(256), 0, s, y, (long)batch);
+        D8_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+template <typename T, int WIDE, bool L2>
+static int norm_grad_t(const T *x, T *dx, const T *y, const T *dy, int batch, long size, hipStream_t s) {
+    const long n = (long)batch * size;
+    if (size % WIDE == 0 && al16(x) && al16(dx))
+        hipLaunchKernelGGL((norm_grad_kernel<T, WIDE, L2>), dim3(ew_grid(n / WIDE, 256)), dim3(256), 0, s, x, dx, y, dy, size / WIDE, n / WIDE);
+    else
+        hipLaunchKernelGGL((norm_grad_kernel<T, 1, L2>), dim3(ew_grid(n, 256)), dim3(256), 0, s, x, dx, y, dy, size, n);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+static int check_norm(const char *who, int dtype, const void *x, const void *y, int batch, long size) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32) return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
+    D8_REQUIRE(x && y, "%s: null tensor", who);
+    D8_REQUIRE(batch >= 1 && size >= 1 && size < (1L << 31), "%s: the shape is error", who);
     return 0;
 }
 
@@ -376,8 +469,8 @@ int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int 
     D8_REQUIRE(g && dz && gdims && zdims, "d8_add_grad: null argument");
     if (int rc = check_dims("d8_add_grad", gdims, zdims)) return rc;
     return dtype == D8_FLOAT32
-               ? add_grad_t<float, 4>((float *)g, gdims, (const float *)dz, zdims, scratch, scratch_bytes, as_stream(stream))
-               : add_grad_t<f16, 8>((f16 *)g, gdims, (const f16 *)dz, zdims, scratch, scratch_bytes, as_stream(stream));
+               ? reduce_t<float, 4>((float *)g, gdims, (const float *)dz, zdims, scratch, scratch_bytes, as_stream(stream))
+               : reduce_t<f16, 8>((f16 *)g, gdims, (const f16 *)dz, zdims, scratch, scratch_bytes, as_stream(stream));
 }
 
 int d8_relu(int dtype, const void *x, void *y, long n, void *stream) {
@@ -412,6 +505,116 @@ int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, voi
     } else {
         if (al && n % 8 == 0) hipLaunchKernelGGL((relu_grad_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n / 8);
         else hipLaunchKernelGGL((relu_grad_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int d8_minus(int dtype, const void *x, const int *xdims, const void *y, const int *ydims, void *z, const int *zdims,
+             void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32) return fail(D8_ERR_DTYPE, "d8_minus: element type %d is not supported", dtype);
+    D8_REQUIRE(x && y && z && xdims && ydims && zdims, "d8_minus: null argument");
+    if (int rc = check_dims("d8_minus", xdims, zdims)) return rc;
+    if (int rc = check_dims("d8_minus", ydims, zdims)) return rc;
+    for (int a = 0; a < 5; ++a)
+        D8_REQUIRE(zdims[a] == (xdims[a] > ydims[a] ? xdims[a] : ydims[a]), "d8_minus: the shape is error (axis %d)", a);
+    return dtype == D8_FLOAT32
+               ? add_t<float, 4>((const float *)x, xdims, (const float *)y, ydims, (float *)z, zdims, as_stream(stream), -1.f)
+               : add_t<f16, 8>((const f16 *)x, xdims, (const f16 *)y, ydims, (f16 *)z, zdims, as_stream(stream), -1.f);
+}
+
+int d8_minus_grad_y(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                    void *scratch, size_t scratch_bytes, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_minus_grad_y: element type %d is not supported", dtype);
+    D8_REQUIRE(g && dz && gdims && zdims, "d8_minus_grad_y: null argument");
+    if (int rc = check_dims("d8_minus_grad_y", gdims, zdims)) return rc;
+    return dtype == D8_FLOAT32
+               ? reduce_t<float, 4>((float *)g, gdims, (const float *)dz, zdims, scratch, scratch_bytes, as_stream(stream), -1.f)
+               : reduce_t<f16, 8>((f16 *)g, gdims, (const f16 *)dz, zdims, scratch, scratch_bytes, as_stream(stream), -1.f);
+}
+
+int d8_l1norm(int dtype, const void *x, void *y, int batch, long size, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_norm("d8_l1norm", dtype, x, y, batch, size)) return rc;
+    return dtype == D8_FLOAT32
+               ? norm_t<float, 4, LOAD_ABS>((const float *)x, (float *)y, batch, size, scratch, scratch_bytes, as_stream(stream))
+               : norm_t<f16, 8, LOAD_ABS>((const f16 *)x, (f16 *)y, batch, size, scratch, scratch_bytes, as_stream(stream));
+}
+
+int d8_l1norm_grad(int dtype, const void *x, void *dx, const void *dy, int batch, long size, void *stream) {
+    if (int rc = check_norm("d8_l1norm_grad", dtype, x, dx, batch, size)) return rc;
+    D8_REQUIRE(dy, "d8_l1norm_grad: null tensor");
+    return dtype == D8_FLOAT32
+               ? norm_grad_t<float, 4, false>((const float *)x, (float *)dx, (const float *)dy, (const float *)dy, batch, size, as_stream(stream))
+               : norm_grad_t<f16, 8, false>((const f16 *)x, (f16 *)dx, (const f16 *)dy, (const f16 *)dy, batch, size, as_stream(stream));
+}
+
+int d8_l2norm(int dtype, const void *x, void *y, int batch, long size, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_norm("d8_l2norm", dtype, x, y, batch, size)) return rc;
+    return dtype == D8_FLOAT32
+               ? norm_t<float, 4, LOAD_SQUARE>((const float *)x, (float *)y, batch, size, scratch, scratch_bytes, as_stream(stream))
+               : norm_t<f16, 8, LOAD_SQUARE>((const f16 *)x, (f16 *)y, batch, size, scratch, scratch_bytes, as_stream(stream));
+}
+
+int d8_l2norm_grad(int dtype, const void *x, void *dx, const void *y, const void *dy, int batch, long size, void *stream) {
+    if (int rc = check_norm("d8_l2norm_grad", dtype, x, dx, batch, size)) return rc;
+    D8_REQUIRE(y && dy, "d8_l2norm_grad: null tensor");
+    return dtype == D8_FLOAT32
+               ? norm_grad_t<float, 4, true>((const float *)x, (float *)dx, (const float *)y, (const float *)dy, batch, size, as_stream(stream))
+               : norm_grad_t<f16, 8, true>((const f16 *)x, (f16 *)dx, (const f16 *)y, (const f16 *)dy, batch, size, as_stream(stream));
+}
+
+static int mean_count(const char *who, const int *xdims, const int *ydims, double *count) {
+    if (int rc = check_dims(who, ydims, xdims)) return rc;
+    *count = (double)prod5(xdims) / (double)prod5(ydims);
+    return 0;
+}
+
+int d8_reduce_mean(int dtype, const void *x, const int *xdims, void *y, const int *ydims,
+                   void *scratch, size_t scratch_bytes, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_reduce_mean: element type %d is not supported", dtype);
+    D8_REQUIRE(x && y && xdims && ydims, "d8_reduce_mean: null argument");
+    double count = 1;
+    if (int rc = mean_count("d8_reduce_mean", xdims, ydims, &count)) return rc;
+    hipStream_t s = as_stream(stream);
+    const long ny = prod5(ydims);
+    const float scale = (float)(1.0 / count);
+    if (dtype == D8_FLOAT32) {
+        hipLaunchKernelGGL((ew_zero_kernel<float>), dim3(ew_grid(ny, 256)), dim3(256), 0, s, (float *)y, ny);
+        D8_LAUNCH_CHECK();
+        return reduce_t<float, 4>((float *)y, ydims, (const float *)x, xdims, scratch, scratch_bytes, s, scale);
+    }
+    hipLaunchKernelGGL((ew_zero_kernel<f16>), dim3(ew_grid(ny, 256)), dim3(256), 0, s, (f16 *)y, ny);
+    D8_LAUNCH_CHECK();
+    return reduce_t<f16, 8>((f16 *)y, ydims, (const f16 *)x, xdims, scratch, scratch_bytes, s, scale);
+}
+
+int d8_reduce_mean_grad(int dtype, void *dx, const int *xdims, const void *dy, const int *ydims, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_reduce_mean_grad: element type %d is not supported", dtype);
+    D8_REQUIRE(dx && dy && xdims && ydims, "d8_reduce_mean_grad: null argument");
+    double count = 1;
+    if (int rc = mean_count("d8_reduce_mean_grad", xdims, ydims, &count)) return rc;
+    const float ys = (float)(1.0 / count);
+    return dtype == D8_FLOAT32
+               ? add_t<float, 4>((const float *)dx, xdims, (const float *)dy, ydims, (float *)dx, xdims, as_stream(stream), ys)
+               : add_t<f16, 8>((const f16 *)dx, xdims, (const f16 *)dy, ydims, (f16 *)dx, xdims, as_stream(stream), ys);
+}
+
+int d8_axpby(int dtype, const void *x, float alpha, const void *y, float beta, void *z, long n, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32) return fail(D8_ERR_DTYPE, "d8_axpby: element type %d is not supported", dtype);
+    D8_REQUIRE(n >= 0, "d8_axpby: negative size");
+    if (n == 0) return 0;
+    D8_REQUIRE(x && y && z, "d8_axpby: null tensor");
+    hipStream_t s = as_stream(stream);
+    const bool al = al16(x) && al16(y) && al16(z);
+    if (dtype == D8_FLOAT32) {
+        if (al && n % 4 == 0) hipLaunchKernelGGL((axpby_kernel<float, 4>), dim3(ew_grid(n / 4, 256)), dim3(256), 0, s, (const float *)x, alpha, (const float *)y, beta, (float *)z, n / 4);
+        else hipLaunchKernelGGL((axpby_kernel<float, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const float *)x, alpha, (const float *)y, beta, (float *)z, n);
+    } else {
+        if (al && n % 8 == 0) hipLaunchKernelGGL((axpby_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (const f16 *)x, alpha, (const f16 *)y, beta, (f16 *)z, n / 8);
+        else hipLaunchKernelGGL((axpby_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const f16 *)x, alpha, (const f16 *)y, beta, (f16 *)z, n);
     }
     D8_LAUNCH_CHECK();
     return 0;

@@ -314,3 +314,109 @@ def relu_grad(x, dy, dx=None):
     a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
     check(lib.d8_relu_grad(dt, a.ptr, b.ptr, c.ptr, x.size, None))
     return b.numpy()
+
+
+# ---- Minus, L1Norm / L2Norm, ReduceMean, AXPBY ----------------------------------------------------
+def minus(x, y):
+    lib = capi.init()
+    x, y = np.ascontiguousarray(x), np.ascontiguousarray(y)
+    dt = _same_dtype(x, y)
+    zs = _broadcast(x.shape, y.shape)
+    dx_, dy_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray(zs, x.dtype)
+    check(lib.d8_minus(dt, dx_.ptr, _enlarged(x.shape), dy_.ptr, _enlarged(y.shape), dz_.ptr, _enlarged(zs), None))
+    return dz_.numpy()
+
+
+def minus_grad_y(g, dz, use_scratch=True):
+    """returns g - dz summed over the axes g is broadcast along"""
+    lib = capi.init()
+    g, dz = np.ascontiguousarray(g), np.ascontiguousarray(dz)
+    dt = _same_dtype(g, dz)
+    gs = (g.shape[0],) + (1,) * (dz.ndim - g.ndim) + tuple(g.shape[1:])
+    gd, zd = _enlarged(gs), _enlarged(dz.shape)
+    dg, ddz = DeviceArray.from_numpy(g), DeviceArray.from_numpy(dz)
+    nb = lib.d8_add_grad_scratch_bytes(dt, gd, zd) if use_scratch else 0
+    ws = _scratch(nb)
+    check(lib.d8_minus_grad_y(dt, dg.ptr, gd, ddz.ptr, zd, ws.ptr if nb else None, nb, None))
+    return dg.numpy()
+
+
+def _norm(fn_name, x, use_scratch):
+    lib = capi.init()
+    x = np.ascontiguousarray(x)
+    dt = capi.dtype_id(x.dtype)
+    batch, size = x.shape[0], int(np.prod(x.shape[1:]))
+    dx_, dy_ = DeviceArray.from_numpy(x), DeviceArray((batch, 1), x.dtype)
+    nb = lib.d8_add_grad_scratch_bytes(dt, _enlarged((batch, 1)), _enlarged((batch, size))) if use_scratch else 0
+    ws = _scratch(nb)
+    check(getattr(lib, fn_name)(dt, dx_.ptr, dy_.ptr, batch, size, ws.ptr if nb else None, nb, None))
+    return dy_.numpy()
+
+
+def l1norm(x, use_scratch=True):
+    """x: (batch, dims..) -> (batch, 1)"""
+    return _norm("d8_l1norm", x, use_scratch)
+
+
+def l2norm(x, use_scratch=True):
+    return _norm("d8_l2norm", x, use_scratch)
+
+
+def l1norm_grad(x, dy, dx=None):
+    lib = capi.init()
+    x, dy = np.ascontiguousarray(x), np.ascontiguousarray(dy)
+    dt = _same_dtype(x, dy)
+    dx = np.zeros_like(x) if dx is None else np.ascontiguousarray(dx)
+    a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
+    check(lib.d8_l1norm_grad(dt, a.ptr, b.ptr, c.ptr, x.shape[0], int(np.prod(x.shape[1:])), None))
+    return b.numpy()
+
+
+def l2norm_grad(x, y, dy, dx=None):
+    lib = capi.init()
+    x, y, dy = np.ascontiguousarray(x), np.ascontiguousarray(y), np.ascontiguousarray(dy)
+    dt = _same_dtype(x, dy)
+    dx = np.zeros_like(x) if dx is None else np.ascontiguousarray(dx)
+    a, b, c, d = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dx), DeviceArray.from_numpy(y), DeviceArray.from_numpy(dy)
+    check(lib.d8_l2norm_grad(dt, a.ptr, b.ptr, c.ptr, d.ptr, x.shape[0], int(np.prod(x.shape[1:])), None))
+    return b.numpy()
+
+
+def _kept_shape(shape, axes):
+    """keepDims form of the output shape of a reduction of `shape` (batch first) over `axes` (empty: all)"""
+    rank = len(shape)
+    red = set(range(rank)) if not axes else {(a + rank) % rank for a in axes}
+    return tuple(1 if i in red else shape[i] for i in range(rank))
+
+
+def reduce_mean(x, axes=(), use_scratch=True):
+    """mean over `axes` of x (batch is axis 0; empty = every axis); returns the keepDims form"""
+    lib = capi.init()
+    x = np.ascontiguousarray(x)
+    dt = capi.dtype_id(x.dtype)
+    ys = _kept_shape(x.shape, axes)
+    xd, yd = _enlarged(x.shape), _enlarged(ys)
+    dx_, dy_ = DeviceArray.from_numpy(x), DeviceArray(ys, x.dtype)
+    nb = lib.d8_add_grad_scratch_bytes(dt, yd, xd) if use_scratch else 0
+    ws = _scratch(nb)
+    check(lib.d8_reduce_mean(dt, dx_.ptr, xd, dy_.ptr, yd, ws.ptr if nb else None, nb, None))
+    return dy_.numpy()
+
+
+def reduce_mean_grad(dx, dy):
+    """returns dx + dy / count with dy (keepDims form) broadcast over the reduced axes"""
+    lib = capi.init()
+    dx, dy = np.ascontiguousarray(dx), np.ascontiguousarray(dy)
+    dt = _same_dtype(dx, dy)
+    a, b = DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
+    check(lib.d8_reduce_mean_grad(dt, a.ptr, _enlarged(dx.shape), b.ptr, _enlarged(dy.shape), None))
+    return a.numpy()
+
+
+def axpby(x, alpha, y, beta):
+    lib = capi.init()
+    x, y = np.ascontiguousarray(x), np.ascontiguousarray(y)
+    dt = _same_dtype(x, y)
+    a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray(x.shape, x.dtype)
+    check(lib.d8_axpby(dt, a.ptr, alpha, b.ptr, beta, c.ptr, x.size, None))
+    return c.numpy()

@@ -190,6 +190,44 @@ int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int 
 int d8_relu(int dtype, const void *x, void *y, long n, void *stream);
 int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, void *stream);
 
+/* ---- Minus, L1Norm / L2Norm, ReduceMean, AXPBY ------------------------------------------------
+ * What a loss and a trainer step need on top of the operators above.  Shapes as for d8_add.
+ * Reductions take an optional two-pass `scratch` (16-byte aligned; size from
+ * d8_add_grad_scratch_bytes(dtype, shape of the reduced tensor, shape of the full tensor)).
+ *
+ * d8_minus            z = x - y with broadcasting.  Math::MinusGPU (deep8/include/math/Minus.h:16,
+ *                     deep8/src/math/Minus.cu:21-52).  Math::MinusGradXGPU (Minus.h:27) is d8_add_grad.
+ * d8_minus_grad_y     g -= dz summed over the axes where g has extent 1.  Math::MinusGradYGPU
+ *                     (Minus.h:38, Minus.cu:103-147).
+ * d8_l1norm           y[b] = sum_i |x[b][i]|.  Math::L1NormGPU (deep8/include/math/L1Norm.h,
+ *                     deep8/src/math/L1Norm.cu:27-75).
+ * d8_l1norm_grad      dx[b][i] += dy[b] * sign(x[b][i]) (sign(0) = 0).  Math::L1NormGradGPU
+ *                     (L1Norm.cu:77-136).
+ * d8_l2norm           y[b] = sqrt(sum_i x[b][i]^2).  Math::L2NormGPU (deep8/src/math/L2Norm.cu).
+ * d8_l2norm_grad      dx[b][i] += dy[b] / y[b] * x[b][i].  Math::L2NormGradGPU.
+ * d8_reduce_mean      y = mean of x over the axes where ydims is 1 and xdims is not (ydims is the
+ *                     keepDims form of the output shape; dropping the axes does not move data).
+ *                     Math::ReduceMeanGPU (deep8/include/math/ReduceMean.h, deep8/src/math/ReduceMean.cu:30-110).
+ * d8_reduce_mean_grad dx += dy / count, dy broadcast over the reduced axes.  Math::ReduceMeanGradGPU
+ *                     (ReduceMean.cu:112-203).
+ * d8_axpby            z = alpha * x + beta * y (z may be x or y).  Math::AXPBYGPU
+ *                     (deep8/include/math/AXPBY.h, deep8/src/math/AXPBY.cu:9-47): the SGD update.       */
+int d8_minus(int dtype, const void *x, const int *xdims, const void *y, const int *ydims,
+             void *z, const int *zdims, void *stream);
+int d8_minus_grad_y(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                    void *scratch, size_t scratch_bytes, void *stream);
+int d8_l1norm(int dtype, const void *x, void *y, int batch, long size,
+              void *scratch, size_t scratch_bytes, void *stream);
+int d8_l1norm_grad(int dtype, const void *x, void *dx, const void *dy, int batch, long size, void *stream);
+int d8_l2norm(int dtype, const void *x, void *y, int batch, long size,
+              void *scratch, size_t scratch_bytes, void *stream);
+int d8_l2norm_grad(int dtype, const void *x, void *dx, const void *y, const void *dy, int batch, long size,
+                   void *stream);
+int d8_reduce_mean(int dtype, const void *x, const int *xdims, void *y, const int *ydims,
+                   void *scratch, size_t scratch_bytes, void *stream);
+int d8_reduce_mean_grad(int dtype, void *dx, const int *xdims, const void *dy, const int *ydims, void *stream);
+int d8_axpby(int dtype, const void *x, float alpha, const void *y, float beta, void *z, long n, void *stream);
+
 /* ---- measurement aid (no counterpart in the reference) ---------------------------------------
  * d8_mfma_stream issues the tiled GEMM's MFMA instruction back to back on operands taken from
  * `operands` (any device buffer; 16-byte aligned) and held in registers: two waves per SIMD on

@@ -80,6 +80,13 @@ def broadcast_shape(xs, ys):
     return tuple(max(a, b) for a, b in zip(ex, ey))
 
 
+def kept_shape(shape, axes):
+    """keepDims form of the output shape of a reduction of `shape` (batch first) over `axes` (empty: all)"""
+    rank = len(shape)
+    red = set(range(rank)) if not axes else {(a + rank) % rank for a in axes}
+    return tuple(1 if i in red else shape[i] for i in range(rank))
+
+
 def _i5(shape):
     return (ctypes.c_int * 5)(*enlarged(shape))
 
@@ -260,6 +267,64 @@ class _Port:
         self.lib.orc_relu_grad(_p(x), _p(dx), _p(dy), ctypes.c_long(x.size))
         return dx
 
+    # -- Minus, L1Norm / L2Norm, ReduceMean, AXPBY ---------------------------------------------
+    def minus(self, x, y):
+        x, y = _c(x), _c(y)
+        z = np.zeros(broadcast_shape(x.shape, y.shape), np.float32)
+        self.lib.orc_minus(_p(x), _i5(x.shape), _p(y), _i5(y.shape), _p(z), _i5(z.shape))
+        return z
+
+    def minus_grad_y(self, like, dz, g=None):
+        """g (shaped like `like`) -= dz summed over the broadcast axes"""
+        dz = _c(dz)
+        g = np.zeros(np.shape(like), np.float32) if g is None else _c(g).copy()
+        gs = (g.shape[0],) + (1,) * (dz.ndim - g.ndim) + tuple(g.shape[1:])
+        self.lib.orc_minus_grad_y(_p(g), _i5(gs), _p(dz), _i5(dz.shape))
+        return g
+
+    def l1norm(self, x):
+        x = _c(x)
+        y = np.zeros((x.shape[0], 1), np.float32)
+        self.lib.orc_l1norm(_p(x), _p(y), _i(x.shape[0]), ctypes.c_long(x.size // x.shape[0]))
+        return y
+
+    def l1norm_grad(self, x, dy, dx=None):
+        x, dy = _c(x), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        self.lib.orc_l1norm_grad(_p(x), _p(dx), _p(dy), _i(x.shape[0]), ctypes.c_long(x.size // x.shape[0]))
+        return dx
+
+    def l2norm(self, x):
+        x = _c(x)
+        y = np.zeros((x.shape[0], 1), np.float32)
+        self.lib.orc_l2norm(_p(x), _p(y), _i(x.shape[0]), ctypes.c_long(x.size // x.shape[0]))
+        return y
+
+    def l2norm_grad(self, x, y, dy, dx=None):
+        x, y, dy = _c(x), _c(y), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        self.lib.orc_l2norm_grad(_p(x), _p(dx), _p(y), _p(dy), _i(x.shape[0]), ctypes.c_long(x.size // x.shape[0]))
+        return dx
+
+    def reduce_mean(self, x, axes=()):
+        """mean over `axes` (batch is axis 0; empty = all); returns the keepDims form"""
+        x = _c(x)
+        ys = kept_shape(x.shape, axes)
+        y = np.zeros(ys, np.float32)
+        self.lib.orc_reduce_mean(_p(x), _i5(x.shape), _p(y), _i5(ys))
+        return y
+
+    def reduce_mean_grad(self, dx, dy):
+        dx, dy = _c(dx).copy(), _c(dy)
+        self.lib.orc_reduce_mean_grad(_p(dx), _i5(dx.shape), _p(dy), _i5(dy.shape))
+        return dx
+
+    def axpby(self, x, alpha, y, beta):
+        x, y = _c(x), _c(y)
+        z = np.zeros_like(x)
+        self.lib.orc_axpby(_p(x), ctypes.c_float(alpha), _p(y), ctypes.c_float(beta), _p(z), ctypes.c_long(x.size))
+        return z
+
 
 class _Ref:
     """Deep8's own CPU path (float only)."""
@@ -401,6 +466,56 @@ class _Ref:
         y = np.maximum(x, 0)
         self._chk(self.lib.ref_relu_grad(_p(x), _p(dx), _p(y), _p(dy), *_nd(x)))
         return dx
+
+    # -- Minus, L1Norm / L2Norm, ReduceMean, AXPBY through the reference's Math:: functions -------
+    def minus(self, x, y):
+        x, y = _c(x), _c(y)
+        z = np.zeros(broadcast_shape(x.shape, y.shape), np.float32)
+        self._chk(self.lib.ref_minus(_p(x), *_nd(x), _p(y), *_nd(y), _p(z), *_nd(z)))
+        return z
+
+    def minus_grad(self, which, x, y, dz, g=None):
+        """which 0: MinusGradX, 1: MinusGradY; returns g + gradient"""
+        x, y, dz = _c(x), _c(y), _c(dz)
+        like = x if which == 0 else y
+        g = np.zeros_like(like) if g is None else _c(g).copy()
+        z = np.zeros_like(dz)
+        self._chk(self.lib.ref_minus_grad(_i(which), _p(x), *_nd(x), _p(y), *_nd(y), _p(g), _p(z), _p(dz), *_nd(dz)))
+        return g
+
+    def norm(self, which, x):
+        """which 1: L1Norm, 2: L2Norm; x (batch, dims..) -> (batch, 1)"""
+        x = _c(x)
+        y = np.zeros((x.shape[0], 1), np.float32)
+        self._chk(self.lib.ref_norm(_i(which), _p(x), *_nd(x), _p(y)))
+        return y
+
+    def norm_grad(self, which, x, y, dy, dx=None):
+        x, y, dy = _c(x), _c(y), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        self._chk(self.lib.ref_norm_grad(_i(which), _p(x), _p(dx), *_nd(x), _p(y), _p(dy)))
+        return dx
+
+    def reduce_mean(self, x, axes=(), keep=True):
+        x = _c(x)
+        ys = kept_shape(x.shape, axes)
+        y = np.zeros(ys, np.float32)
+        ax = (ctypes.c_int * max(1, len(axes)))(*axes)
+        self._chk(self.lib.ref_reduce_mean(_p(x), *_nd(x), _p(y), ax, _i(len(axes)), _i(int(keep))))
+        return y
+
+    def reduce_mean_grad(self, x, y, dy, axes=(), keep=True, dx=None):
+        x, y, dy = _c(x), _c(y), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        ax = (ctypes.c_int * max(1, len(axes)))(*axes)
+        self._chk(self.lib.ref_reduce_mean_grad(_p(x), _p(dx), *_nd(x), _p(y), _p(dy), ax, _i(len(axes)), _i(int(keep))))
+        return dx
+
+    def axpby(self, x, alpha, y, beta):
+        x, y = _c(x), _c(y)
+        z = np.zeros_like(x)
+        self._chk(self.lib.ref_axpby(_p(x), ctypes.c_float(alpha), _p(y), ctypes.c_float(beta), _p(z), *_nd(x)))
+        return z
 
 
 port = _Port(PORT_PATH) if os.path.exists(PORT_PATH) else None

@@ -29,6 +29,7 @@
  */
 #include "deep8_oracle.h"
 
+#include <math.h>
 #include <stddef.h>
 #include <stdlib.h>
 #include <string.h>
@@ -87,6 +88,116 @@ void orc_relu(const float *x, float *y, long n) {
 
 void orc_relu_grad(const float *x, float *dx, const float *dy, long n) {
     for (long i = 0; i < n; ++i) dx[i] += x[i] > 0.f ? dy[i] : 0.f;
+}
+
+/* ---- Minus, L1Norm / L2Norm, ReduceMean, AXPBY ------------------------------------------------
+ * orc_minus            deep8/src/math/Minus.cpp:109-143 (z = x - y, size-1 axes broadcast)
+ * orc_minus_grad_y     deep8/src/math/Minus.cpp:268-294 (dy -= dz.sum(axes that differ)); MinusGradX
+ *                      (Minus.cpp:163-189) is orc_add_grad
+ * orc_l1norm           deep8/src/math/L1Norm.cpp:42-54   (y[b] = sum |x[b][:]|)
+ * orc_l1norm_grad      deep8/src/math/L1Norm.cpp:72-99   (dx += dy[b] * sign(x), sign(0) = 0)
+ * orc_l2norm           deep8/src/math/L2Norm.cpp:45-57   (y[b] = sqrt(sum x^2))
+ * orc_l2norm_grad      deep8/src/math/L2Norm.cpp:77-90   (dx += dy[b] / y[b] * x)
+ * orc_reduce_mean      deep8/src/math/ReduceMean.cpp:124-157 (mean over the axes where yd is 1)
+ * orc_reduce_mean_grad deep8/src/math/ReduceMean.cpp:285-320 (dx += dy broadcast / ratio)
+ * orc_axpby            deep8/src/math/AXPBY.cpp:23-31    (z = x * alpha + y * beta)
+ * Sums are carried in double.  Pins: numpy expressions of the same formulas, the live reference
+ * build and the golden fixtures (tests/test_oracle_pins.py). */
+void orc_minus(const float *x, const int *xd, const float *y, const int *yd, float *z, const int *zd) {
+    long n = 1;
+    for (int i = 0; i < 5; ++i) n *= zd[i];
+    for (long e = 0; e < n; ++e) {
+        long rem = e, xi = 0, yi = 0;
+        for (int a = 0; a < 5; ++a) {
+            const long zs = stride5(zd, a), idx = rem / zs;
+            rem -= idx * zs;
+            if (xd[a] != 1) xi += idx * stride5(xd, a);
+            if (yd[a] != 1) yi += idx * stride5(yd, a);
+        }
+        z[e] = x[xi] - y[yi];
+    }
+}
+
+/* out[o] = sum of scale-free dz over the axes where d is 1 and zd is not, in double */
+static double *sum_to(const int *d, const float *dz, const int *zd, long *n_out) {
+    long n = 1, nz = 1;
+    for (int i = 0; i < 5; ++i) n *= d[i], nz *= zd[i];
+    double *acc = (double *)calloc((size_t)n, sizeof(double));
+    for (long e = 0; e < nz; ++e) {
+        long rem = e, o = 0;
+        for (int a = 0; a < 5; ++a) {
+            const long zs = stride5(zd, a), idx = rem / zs;
+            rem -= idx * zs;
+            if (d[a] != 1) o += idx * stride5(d, a);
+        }
+        acc[o] += (double)dz[e];
+    }
+    *n_out = n;
+    return acc;
+}
+
+void orc_minus_grad_y(float *dy, const int *d, const float *dz, const int *zd) {
+    long n;
+    double *acc = sum_to(d, dz, zd, &n);
+    for (long o = 0; o < n; ++o) dy[o] -= (float)acc[o];
+    free(acc);
+}
+
+void orc_l1norm(const float *x, float *y, int batch, long size) {
+    for (int b = 0; b < batch; ++b) {
+        double acc = 0;
+        for (long i = 0; i < size; ++i) acc += fabs((double)x[b * size + i]);
+        y[b] = (float)acc;
+    }
+}
+
+void orc_l1norm_grad(const float *x, float *dx, const float *dy, int batch, long size) {
+    for (int b = 0; b < batch; ++b)
+        for (long i = 0; i < size; ++i) {
+            const float v = x[b * size + i];
+            dx[b * size + i] += v > 0.f ? dy[b] : (v == 0.f ? 0.f : -dy[b]);
+        }
+}
+
+void orc_l2norm(const float *x, float *y, int batch, long size) {
+    for (int b = 0; b < batch; ++b) {
+        double acc = 0;
+        for (long i = 0; i < size; ++i) acc += (double)x[b * size + i] * (double)x[b * size + i];
+        y[b] = (float)sqrt(acc);
+    }
+}
+
+void orc_l2norm_grad(const float *x, float *dx, const float *y, const float *dy, int batch, long size) {
+    for (int b = 0; b < batch; ++b)
+        for (long i = 0; i < size; ++i) dx[b * size + i] += dy[b] / y[b] * x[b * size + i];
+}
+
+void orc_reduce_mean(const float *x, const int *xd, float *y, const int *yd) {
+    long n, nx = 1;
+    for (int i = 0; i < 5; ++i) nx *= xd[i];
+    double *acc = sum_to(yd, x, xd, &n);
+    const double count = (double)nx / (double)n;
+    for (long o = 0; o < n; ++o) y[o] = (float)(acc[o] / count);
+    free(acc);
+}
+
+void orc_reduce_mean_grad(float *dx, const int *xd, const float *dy, const int *yd) {
+    long nx = 1, ny = 1;
+    for (int i = 0; i < 5; ++i) nx *= xd[i], ny *= yd[i];
+    const float ratio = (float)(nx / ny);
+    for (long e = 0; e < nx; ++e) {
+        long rem = e, o = 0;
+        for (int a = 0; a < 5; ++a) {
+            const long zs = stride5(xd, a), idx = rem / zs;
+            rem -= idx * zs;
+            if (yd[a] != 1) o += idx * stride5(yd, a);
+        }
+        dx[e] += dy[o] / ratio;
+    }
+}
+
+void orc_axpby(const float *x, float alpha, const float *y, float beta, float *z, long n) {
+    for (long i = 0; i < n; ++i) z[i] = x[i] * alpha + y[i] * beta;
 }
 
 int orc_threads(void) {

@@ -82,6 +82,18 @@ void orc_relu(const float *x, float *y, long n);
 /* dx += x > 0 ? dy : 0 */
 void orc_relu_grad(const float *x, float *dx, const float *dy, long n);
 
+/* ---- Minus, L1Norm / L2Norm, ReduceMean, AXPBY (shapes as above; yd of the mean is the keepDims
+ * form of its output shape) */
+void orc_minus(const float *x, const int *xd, const float *y, const int *yd, float *z, const int *zd);
+void orc_minus_grad_y(float *dy, const int *d, const float *dz, const int *zd);
+void orc_l1norm(const float *x, float *y, int batch, long size);
+void orc_l1norm_grad(const float *x, float *dx, const float *dy, int batch, long size);
+void orc_l2norm(const float *x, float *y, int batch, long size);
+void orc_l2norm_grad(const float *x, float *dx, const float *y, const float *dy, int batch, long size);
+void orc_reduce_mean(const float *x, const int *xd, float *y, const int *yd);
+void orc_reduce_mean_grad(float *dx, const int *xd, const float *dy, const int *yd);
+void orc_axpby(const float *x, float alpha, const float *y, float beta, float *z, long n);
+
 int orc_threads(void);
 
 #ifdef __cplusplus

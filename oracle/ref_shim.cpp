@@ -10,6 +10,11 @@
  *   Math::DeConv2d / GradX / GradY            deep8/src/math/DeConv2d.cpp:43-82,122-162,203-243
  *   Math::Add / AddGradX / AddGradY           deep8/src/math/Add.cpp:7-107
  *   Math::ReLu / ReLuGrad                     deep8/src/math/ReLu.cpp:6-36
+ *   Math::Minus / MinusGradX / MinusGradY     deep8/src/math/Minus.cpp:7-107
+ *   Math::L1Norm / L1NormGrad                 deep8/src/math/L1Norm.cpp:6-39
+ *   Math::L2Norm / L2NormGrad                 deep8/src/math/L2Norm.cpp:6-42
+ *   Math::ReduceMean / ReduceMeanGrad         deep8/src/math/ReduceMean.cpp:7-121
+ *   Math::AXPBY                               deep8/src/math/AXPBY.cpp:6-20
  *
  * plus one materialisation of the patch expression the CPU Conv2d contracts over
  * (deep8/src/math/Conv2d.cpp:352-356), which is the "CPU Eigen im2col" the HIP im2col must
@@ -25,6 +30,11 @@
 #include "math/DeConv2d.h"
 #include "math/Add.h"
 #include "math/ReLu.h"
+#include "math/Minus.h"
+#include "math/L1Norm.h"
+#include "math/L2Norm.h"
+#include "math/ReduceMean.h"
+#include "math/AXPBY.h"
 
 #include <chrono>
 #include <cstring>
@@ -291,6 +301,114 @@ int ref_relu_grad(const float *x, float *dx, const float *y, const float *dy, in
         wrap(Y, y, b, vdims(nd, d));
         wrap(DY, dy, b, vdims(nd, d));
         Math::ReLuGrad(*X.t, *DX.t, *Y.t, *DY.t);
+    });
+}
+
+int ref_minus(const float *x, int xb, int xnd, const int *xd, const float *y, int yb, int ynd, const int *yd,
+              float *z, int zb, int znd, const int *zd) {
+    return guarded([&] {
+        Wrapped X, Y, Z;
+        wrap(X, x, xb, vdims(xnd, xd));
+        wrap(Y, y, yb, vdims(ynd, yd));
+        wrap(Z, z, zb, vdims(znd, zd));
+        Math::Minus(*X.t, *Y.t, *Z.t);
+    });
+}
+
+/* which = 0: MinusGradX (g plays dx), 1: MinusGradY (g plays dy) */
+int ref_minus_grad(int which, const float *x, int xb, int xnd, const int *xd, const float *y, int yb, int ynd,
+                   const int *yd, float *g, const float *z, const float *dz, int zb, int znd, const int *zd) {
+    return guarded([&] {
+        Wrapped X, Y, Z, G, DZ;
+        wrap(X, x, xb, vdims(xnd, xd));
+        wrap(Y, y, yb, vdims(ynd, yd));
+        wrap(Z, z, zb, vdims(znd, zd));
+        wrap(DZ, dz, zb, vdims(znd, zd));
+        if (0 == which) {
+            wrap(G, g, xb, vdims(xnd, xd));
+            Math::MinusGradX(*X.t, *G.t, *Y.t, *Z.t, *DZ.t);
+        } else {
+            wrap(G, g, yb, vdims(ynd, yd));
+            Math::MinusGradY(*X.t, *Y.t, *G.t, *Z.t, *DZ.t);
+        }
+    });
+}
+
+/* which = 1: L1Norm, 2: L2Norm; y is (batch, {1}) */
+int ref_norm(int which, const float *x, int b, int nd, const int *d, float *y) {
+    return guarded([&] {
+        Wrapped X, Y;
+        wrap(X, x, b, vdims(nd, d));
+        wrap(Y, y, b, std::vector<size_t>{1});
+        if (1 == which) Math::L1Norm(*X.t, *Y.t);
+        else Math::L2Norm(*X.t, *Y.t);
+    });
+}
+
+int ref_norm_grad(int which, const float *x, float *dx, int b, int nd, const int *d, const float *y, const float *dy) {
+    return guarded([&] {
+        Wrapped X, DX, Y, DY;
+        wrap(X, x, b, vdims(nd, d));
+        wrap(DX, dx, b, vdims(nd, d));
+        wrap(Y, y, b, std::vector<size_t>{1});
+        wrap(DY, dy, b, std::vector<size_t>{1});
+        if (1 == which) Math::L1NormGrad(*X.t, *DX.t, *Y.t, *DY.t);
+        else Math::L2NormGrad(*X.t, *DX.t, *Y.t, *DY.t);
+    });
+}
+
+/* the output shape is derived as the reference's ReduceMean::checkShape does (deep8/src/nodes/ReduceMean.cpp:11-57) */
+static void mean_shape(int b, int nd, const int *d, const std::vector<int> &axis, bool keep, size_t &yb, std::vector<size_t> &yl) {
+    const int rank = nd + 1;
+    std::vector<bool> red(rank, axis.empty());
+    for (int a : axis) red[(a + rank) % rank] = true;
+    yb = red[0] ? 1 : (size_t)b;
+    for (int i = 1; i < rank; ++i) {
+        if (red[i]) {
+            if (keep) yl.push_back(1);
+        } else {
+            yl.push_back((size_t)d[i - 1]);
+        }
+    }
+    if (yl.empty()) yl.push_back(1);
+}
+
+int ref_reduce_mean(const float *x, int b, int nd, const int *d, float *y, const int *axis, int naxis, int keep) {
+    return guarded([&] {
+        std::vector<int> ax(axis, axis + naxis);
+        size_t yb;
+        std::vector<size_t> yl;
+        mean_shape(b, nd, d, ax, keep != 0, yb, yl);
+        Wrapped X, Y;
+        wrap(X, x, b, vdims(nd, d));
+        wrap(Y, y, (int)yb, yl);
+        Math::ReduceMean(*X.t, *Y.t, ax, keep != 0);
+    });
+}
+
+int ref_reduce_mean_grad(const float *x, float *dx, int b, int nd, const int *d, const float *y, const float *dy,
+                         const int *axis, int naxis, int keep) {
+    return guarded([&] {
+        std::vector<int> ax(axis, axis + naxis);
+        size_t yb;
+        std::vector<size_t> yl;
+        mean_shape(b, nd, d, ax, keep != 0, yb, yl);
+        Wrapped X, DX, Y, DY;
+        wrap(X, x, b, vdims(nd, d));
+        wrap(DX, dx, b, vdims(nd, d));
+        wrap(Y, y, (int)yb, yl);
+        wrap(DY, dy, (int)yb, yl);
+        Math::ReduceMeanGrad(*X.t, *DX.t, *Y.t, *DY.t, ax, keep != 0);
+    });
+}
+
+int ref_axpby(const float *x, float alpha, const float *y, float beta, float *z, int b, int nd, const int *d) {
+    return guarded([&] {
+        Wrapped X, Y, Z;
+        wrap(X, x, b, vdims(nd, d));
+        wrap(Y, y, b, vdims(nd, d));
+        wrap(Z, z, b, vdims(nd, d));
+        Math::AXPBY(*X.t, alpha, *Y.t, beta, *Z.t);
     });
 }
 

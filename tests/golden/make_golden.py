@@ -3,8 +3,8 @@
 
 Run in the build container, where oracle/_ref/libdeep8_ref.so has been compiled from the reference
 sources (`make -C oracle ref`):   python tests/golden/make_golden.py
-Every array is float32.  Case names: mm<i>_*, conv<i>_*, deconv<i>_*, patch<i>_*; the geometry of
-case i is stored in <kind><i>_cfg.
+Every array is float32.  Case names: mm<i>_*, conv<i>_*, deconv<i>_*, patch<i>_*, loss<i>_* (Minus,
+L1Norm, L2Norm, ReduceMean, AXPBY); the geometry of case i is stored in <kind><i>_cfg.
 """
 import os
 import sys
@@ -24,6 +24,8 @@ CONV = [(2, 9, 9, 3, 4, 3, 3, 1, 1, 1, 1, 1), (1, 12, 12, 2, 3, 4, 4, 1, 2, 2, 2
 # B, IH, IW, IC, OC, FH, FW, covered, sy, sx
 DECONV = [(2, 4, 4, 3, 2, 4, 4, 0, 3, 3), (2, 4, 4, 3, 2, 4, 4, 1, 3, 3), (1, 5, 5, 2, 3, 4, 4, 0, 2, 2),
           (1, 5, 5, 2, 3, 4, 4, 1, 2, 2), (1, 4, 5, 2, 2, 3, 3, 0, 1, 1)]
+LOSS = [((3, 7), (3, 7), ()), ((2, 5, 6), (1, 6), (0,)), ((4, 3, 2, 5), (4, 1, 1, 5), (1, 3)), ((1, 33), (1, 1), (-1,)),
+        ((2, 3, 4, 5, 6), (1, 3, 1, 5, 1), (0, 2, 4)), ((5, 64), (5, 64), (0,))]
 
 
 def main():
@@ -70,6 +72,22 @@ def main():
                     "deconv%d_z" % i: z, "deconv%d_gz" % i: gz, "deconv%d_gx0" % i: gx0, "deconv%d_gw0" % i: gw0,
                     "deconv%d_gx" % i: ref.deconv2d_grad_x(x, w, gz, *a, gx=gx0),
                     "deconv%d_gw" % i: ref.deconv2d_grad_y(x, w, gz, *a, gw=gw0), "deconv%d_gpatches" % i: gpatches})
+    # Minus / L1Norm / L2Norm / ReduceMean / AXPBY: x shape, y shape (Minus operand), mean axes
+    for i, (xs, ys, axes) in enumerate(LOSS):
+        x, y = u(xs), u(ys)
+        z = ref.minus(x, y)
+        dz = u(z.shape)
+        n1, n2 = ref.norm(1, x), ref.norm(2, x)
+        dn, dx0, dy0 = u(n1.shape), u(xs), u(ys)
+        m = ref.reduce_mean(x, axes)
+        dm = u(m.shape)
+        out.update({"loss%d_x" % i: x, "loss%d_y" % i: y, "loss%d_axes" % i: np.array(axes, np.int32), "loss%d_z" % i: z,
+                    "loss%d_dz" % i: dz, "loss%d_dx0" % i: dx0, "loss%d_dy0" % i: dy0, "loss%d_dn" % i: dn, "loss%d_dm" % i: dm,
+                    "loss%d_minus_gx" % i: ref.minus_grad(0, x, y, dz, dx0), "loss%d_minus_gy" % i: ref.minus_grad(1, x, y, dz, dy0),
+                    "loss%d_l1" % i: n1, "loss%d_l2" % i: n2,
+                    "loss%d_l1_gx" % i: ref.norm_grad(1, x, n1, dn, dx0), "loss%d_l2_gx" % i: ref.norm_grad(2, x, n2, dn, dx0),
+                    "loss%d_mean" % i: m, "loss%d_mean_gx" % i: ref.reduce_mean_grad(x, m, dm, axes, dx=dx0),
+                    "loss%d_axpby" % i: ref.axpby(x, -0.01, dx0, 0.999)})
     path = os.path.join(HERE, "deep8_cpu_reference.npz")
     np.savez_compressed(path, **out)
     print("wrote %s (%d arrays, %d bytes)" % (path, len(out), os.path.getsize(path)))

@@ -333,3 +333,94 @@ def test_relu_against_numpy_and_reference(oracle_port, oracle_ref):
     if oracle_ref is not None:
         assert np.array_equal(oracle_ref.relu(x), np.maximum(x, 0))
         assert np.array_equal(oracle_ref.relu_grad(x, dy, dx0), want)
+
+
+# ---- Minus / L1Norm / L2Norm / ReduceMean / AXPBY ------------------------------------------------------------
+@pytest.mark.parametrize("i", _n("loss"))
+def test_loss_ops_against_golden(oracle_port, i):
+    """Outputs of the reference's own CPU build for Minus, the two norms, ReduceMean and AXPBY."""
+    g = lambda k: GOLD["loss%d_%s" % (i, k)]
+    x, y, axes = g("x"), g("y"), tuple(int(a) for a in g("axes"))
+    assert np.array_equal(oracle_port.minus(x, y), g("z"))
+    assert rel_fro(oracle_port.add_grad(x, g("dz"), g("dx0")), g("minus_gx")) <= TOL
+    assert rel_fro(oracle_port.minus_grad_y(y, g("dz"), g("dy0")), g("minus_gy")) <= TOL
+    assert rel_fro(oracle_port.l1norm(x), g("l1")) <= TOL
+    assert rel_fro(oracle_port.l2norm(x), g("l2")) <= TOL
+    assert rel_fro(oracle_port.l1norm_grad(x, g("dn"), g("dx0")), g("l1_gx")) <= TOL
+    assert rel_fro(oracle_port.l2norm_grad(x, g("l2"), g("dn"), g("dx0")), g("l2_gx")) <= TOL
+    m = oracle_port.reduce_mean(x, axes)
+    assert m.size == g("mean").size and rel_fro(m.ravel(), g("mean").ravel()) <= TOL
+    assert rel_fro(oracle_port.reduce_mean_grad(g("dx0"), g("dm").reshape(m.shape)), g("mean_gx")) <= TOL
+    assert rel_fro(oracle_port.axpby(x, -0.01, g("dx0"), 0.999), g("axpby")) <= 1e-7
+
+
+@pytest.mark.parametrize("xs,ys", ADD_PAIRS)
+def test_minus_against_numpy_and_reference(oracle_port, oracle_ref, xs, ys):
+    r = rng(sum(xs) * 3 + sum(ys))
+    x, y = ints(r, xs), ints(r, ys)
+    nd = max(x.ndim, y.ndim)
+    ex, ey = _ex(x, nd), _ex(y, nd)
+    z = oracle_port.minus(x, y)
+    assert np.array_equal(z, ex - ey)
+    dz = ints(r, z.shape)
+    axes = tuple(i for i in range(nd) if ey.shape[i] == 1 and z.shape[i] != 1)
+    want = y - dz.sum(axis=axes, keepdims=True).reshape(y.shape)
+    assert np.array_equal(oracle_port.minus_grad_y(y, dz, y), want)
+    if oracle_ref is not None:
+        assert np.array_equal(oracle_ref.minus(x, y), z)
+        assert np.array_equal(oracle_ref.minus_grad(1, x, y, dz, y), want)
+        assert np.array_equal(oracle_ref.minus_grad(0, x, y, dz, x), oracle_port.add_grad(x, dz, x))
+
+
+@pytest.mark.parametrize("shape", [(3, 17), (1, 1000), (4, 5, 6, 7), (7, 1)])
+def test_norms_against_numpy_and_reference(oracle_port, oracle_ref, shape):
+    """np.abs().sum / np.sqrt((x*x).sum) per batch row; gradients by their closed forms, including
+    sign(0) = 0 for L1 and the accumulate-twice identity."""
+    r = rng(sum(shape))
+    x = ints(r, shape, 7) - 3  # integers -3..3, zeros included
+    flat = x.reshape(shape[0], -1).astype(np.float64)
+    assert np.array_equal(oracle_port.l1norm(x), np.abs(flat).sum(1, keepdims=True).astype(np.float32))
+    l2 = oracle_port.l2norm(x)
+    assert rel_fro(l2, np.sqrt((flat * flat).sum(1, keepdims=True))) <= 1e-7
+    dy = ints(r, (shape[0], 1), 5) + 1
+    bshape = (shape[0],) + (1,) * (len(shape) - 1)
+    g1 = oracle_port.l1norm_grad(x, dy)
+    assert np.array_equal(g1, (np.sign(x) * dy.reshape(bshape)).astype(np.float32))
+    assert np.array_equal(oracle_port.l1norm_grad(x, dy, g1), 2 * g1)
+    xr = nrm(r, shape) + 0.1
+    l2r = oracle_port.l2norm(xr)
+    g2 = oracle_port.l2norm_grad(xr, l2r, dy)
+    assert rel_fro(g2, xr * (dy / l2r).reshape(bshape)) <= 1e-6
+    if oracle_ref is not None:
+        assert np.array_equal(oracle_ref.norm(1, x), oracle_port.l1norm(x))
+        assert np.array_equal(oracle_ref.norm_grad(1, x, oracle_port.l1norm(x), dy), g1)
+        assert rel_fro(oracle_ref.norm(2, xr), l2r) <= 1e-6
+        assert rel_fro(oracle_ref.norm_grad(2, xr, l2r, dy), g2) <= 1e-6
+
+
+@pytest.mark.parametrize("shape,axes", [((3, 8), ()), ((3, 8), (0,)), ((3, 8), (1,)), ((2, 4, 5, 6), (1, 3)), ((2, 4, 5, 6), (-1,)),
+                                        ((2, 3, 4, 5, 6), (0, 2, 4)), ((1, 12), (0, 1))])
+def test_reduce_mean_against_numpy_and_reference(oracle_port, oracle_ref, shape, axes):
+    r = rng(sum(shape) + len(axes))
+    x = ints(r, shape, 9)
+    ax = tuple(range(len(shape))) if not axes else tuple((a + len(shape)) % len(shape) for a in axes)
+    want = x.astype(np.float64).mean(axis=ax, keepdims=True)
+    m = oracle_port.reduce_mean(x, axes)
+    assert m.shape == want.shape and rel_fro(m, want) <= 1e-7
+    dm, dx0 = ints(r, m.shape, 9), ints(r, shape, 9)
+    count = x.size // m.size
+    g = oracle_port.reduce_mean_grad(dx0, dm)
+    assert rel_fro(g, dx0 + np.broadcast_to(dm, shape) / count) <= 1e-7
+    if oracle_ref is not None:
+        for keep in (True, False):
+            assert rel_fro(oracle_ref.reduce_mean(x, axes, keep).ravel(), m.ravel()) <= 1e-6
+            assert rel_fro(oracle_ref.reduce_mean_grad(x, m, dm, axes, keep, dx0), g) <= 1e-6
+
+
+def test_axpby_against_numpy_and_reference(oracle_port, oracle_ref):
+    r = rng(5)
+    x, y = nrm(r, (3, 50)), nrm(r, (3, 50))
+    z = oracle_port.axpby(x, -0.01, y, 0.999)
+    assert np.array_equal(z, x * np.float32(-0.01) + y * np.float32(0.999))
+    if oracle_ref is not None:
+        assert rel_fro(oracle_ref.axpby(x, -0.01, y, 0.999), z) <= 1e-7
