@@ -6,4 +6,5 @@
 #include "deep8/Math.h"
 #include "deep8/Nodes.h"
 #include "deep8/Executor.h"
+#include "deep8/Trainer.h"
 #endif

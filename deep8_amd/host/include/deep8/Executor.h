@@ -3,7 +3,8 @@
 //   Executor        deep8/include/model/Executor.h:27-137, deep8/src/model/Executor.cpp:9-324
 //   EagerExecutor   deep8/src/model/EagerExecutor.cpp:8-93
 //   Net sugar       deep8/include/model/Net.h:41-167 (parameter, inputParameter, feed, fetch,
-//                   operator*, matrixMultiply, conv2d, deConv2d, backward)
+//                   operator*, operator+, operator-, matrixMultiply, conv2d, deConv2d, l1Norm, l2Norm,
+//                   reduceMean, l1NormLoss, l2NormLoss, backward)
 // Only DeviceType::GPU can be constructed in this build.
 #ifndef DEEP8_HOST_EXECUTOR_H
 #define DEEP8_HOST_EXECUTOR_H
@@ -89,6 +90,13 @@ Variable &deConv2d(Variable &x, Variable &filter, bool covered = false, int stri
 Variable &operator+(Variable &x, Variable &y);  // Add, with broadcasting
 Variable &add(Variable &x, Variable &y);
 Variable &relu(Variable &x);
+Variable &operator-(Variable &x, Variable &y);  // Minus, with broadcasting
+Variable &minus(Variable &x, Variable &y);
+Variable &l1Norm(Variable &x);
+Variable &l2Norm(Variable &x);
+Variable &reduceMean(Variable &x, std::vector<int> axis = {-1}, bool keepDims = true);
+Variable &l1NormLoss(Variable &x);
+Variable &l2NormLoss(Variable &x);
 
 }  // namespace Deep8
 

@@ -68,6 +68,37 @@ void ReLuGPU(const Tensor &x, Tensor &y);
 void ReLuGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
 void ReLuGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
 
+// Minus (broadcasting), L1Norm, L2Norm, ReduceMean and AXPBY: a loss and a trainer step on top of the
+// operators above.  deep8/include/math/Minus.h:14-42 (checks deep8/src/math/Minus.cpp:7-107),
+// L1Norm.h / L2Norm.h (checks deep8/src/math/L1Norm.cpp:6-39, L2Norm.cpp:6-42), ReduceMean.h (checks
+// and output shape deep8/src/math/ReduceMean.cpp:7-121), AXPBY.h (deep8/src/math/AXPBY.cpp:6-20).
+void Minus(const Tensor &x, const Tensor &y, Tensor &z);
+void MinusGPU(const Tensor &x, const Tensor &y, Tensor &z);
+void MinusGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz);
+void MinusGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz);
+void MinusGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+void MinusGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+/** y[b] = sum |x[b]|,  y is [batch, {1}] */
+void L1Norm(const Tensor &x, Tensor &y);
+void L1NormGPU(const Tensor &x, Tensor &y);
+void L1NormGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
+void L1NormGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
+/** y[b] = sqrt(sum x[b]^2) */
+void L2Norm(const Tensor &x, Tensor &y);
+void L2NormGPU(const Tensor &x, Tensor &y);
+void L2NormGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
+void L2NormGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy);
+/** mean over `axis` (0 is the batch; empty = every axis) */
+void ReduceMean(const Tensor &x, Tensor &y, const std::vector<int> &axis = {-1}, bool keepDims = true);
+void ReduceMeanGPU(const Tensor &x, Tensor &y, const std::vector<int> &axis, bool keepDims);
+void ReduceMeanGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, const std::vector<int> &axis = {-1}, bool keepDims = true);
+void ReduceMeanGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, const std::vector<int> &axis, bool keepDims);
+/** the output shape of ReduceMean (shared with the node's checkShape) */
+Shape ReduceMeanShape(const Shape &x, const std::vector<int> &axis, bool keepDims);
+/** z = alpha * x + beta * y */
+void AXPBY(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z);
+void AXPBYGPU(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z);
+
 }  // namespace Math
 }  // namespace Deep8
 

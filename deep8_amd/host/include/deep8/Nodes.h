@@ -94,9 +94,19 @@ public:
     // the element-wise steps that follow them
     Variable &add(Variable &y);
     Variable &relu();
+    // what a loss needs (deep8/src/nodes/Variable.cpp:342-346,461-465,521-535)
+    Variable &minus(Variable &y);
+    Variable &l1Norm();
+    Variable &l2Norm();
+    Variable &reduceMean(std::vector<int> axis = {-1}, bool keepDims = true);
+    Variable &l1NormLoss();  // l1Norm().reduceMean({}, false)
+    Variable &l2NormLoss();  // l2Norm().reduceMean({}, false)
+    // value ~ N(mean, stddev) drawn on the host and copied over (deep8/src/nodes/Variable.cpp:201-205; the
+    // reference draws on the device from an unseeded generator, so only the distribution is comparable)
+    Variable &gaussian(float mean = 0.0, float stddev = 0.01);
 };
 
-enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply, Add, ReLu };
+enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply, Add, ReLu, Minus, L1Norm, L2Norm, ReduceMean };
 
 class Function : public Node {
 protected:
@@ -167,6 +177,53 @@ public:
 class ReLu : public Function {
 public:
     explicit ReLu(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+// z = x - y under the same broadcasting rule (deep8/include/nodes/Minus.h, deep8/src/nodes/Minus.cpp:6-39)
+class Minus : public Function {
+public:
+    explicit Minus(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+// y[b] = sum |x[b]| and y[b] = sqrt(sum x[b]^2), output Shape(batch, {1})
+// (deep8/src/nodes/L1Norm.cpp:6-38, deep8/src/nodes/L2Norm.cpp:6-36)
+class L1Norm : public Function {
+public:
+    explicit L1Norm(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+class L2Norm : public Function {
+public:
+    explicit L2Norm(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+// mean over `axis` (0 is the batch axis, empty = all) (deep8/src/nodes/ReduceMean.cpp:7-75)
+class ReduceMean : public Function {
+public:
+    std::vector<int> axis;
+    bool keepDims;
+
+    explicit ReduceMean(std::vector<Node *> &inputs, std::vector<int> reduceAxis = {-1}, bool keep = true);
     Shape checkShape(std::vector<Shape> &inputShapes) override;
     ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;

@@ -243,6 +243,13 @@ Variable &deConv2d(Variable &x, Variable &filter, bool covered, int strideY, int
 
 Variable &operator+(Variable &x, Variable &y) { return x.add(y); }
 Variable &add(Variable &x, Variable &y) { return x.add(y); }
+Variable &operator-(Variable &x, Variable &y) { return x.minus(y); }
+Variable &minus(Variable &x, Variable &y) { return x.minus(y); }
+Variable &l1Norm(Variable &x) { return x.l1Norm(); }
+Variable &l2Norm(Variable &x) { return x.l2Norm(); }
+Variable &reduceMean(Variable &x, std::vector<int> axis, bool keepDims) { return x.reduceMean(axis, keepDims); }
+Variable &l1NormLoss(Variable &x) { return x.l1NormLoss(); }
+Variable &l2NormLoss(Variable &x) { return x.l2NormLoss(); }
 Variable &relu(Variable &x) { return x.relu(); }
 
 }  // namespace Deep8

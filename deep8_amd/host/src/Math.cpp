@@ -406,5 +406,196 @@ void ReLuGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy) 
     D8_CHECK(d8_relu_grad(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), (long)x.shape.size(), nullptr));
 }
 
+// ---- Minus / L1Norm / L2Norm / ReduceMean / AXPBY ---------------------------------------------------------------
+namespace {
+
+void checkBinaryGrad(const Tensor &x, const Tensor &y, const Tensor &z, const Tensor &g, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == g.deviceType() && x.deviceType() == y.deviceType() &&
+                             x.deviceType() == z.deviceType() && x.deviceType() == dz.deviceType(),
+                         "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == g.elementType && x.elementType == y.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(z.shape == dz.shape, "the z shape is error");
+    checkBroadcast(x, y, z);
+    requireGPU(x);
+}
+
+void checkNorm(const Tensor &x, const Tensor &y) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType(), "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType, "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.batch() == y.batch(), "the shape is error");
+    DEEP8_ARGUMENT_CHECK(1 == y.batchSize(), "the shape is error");
+    requireGPU(x);
+}
+
+void checkNormGrad(const Tensor &x, const Tensor &dx, const Tensor &y, const Tensor &dy) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == dx.deviceType() && x.deviceType() == y.deviceType() && x.deviceType() == dy.deviceType(),
+                         "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == dy.elementType,
+                         "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && y.shape == dy.shape, "the param shape error");
+    DEEP8_ARGUMENT_CHECK(x.batch() == y.batch(), "the shape is error");
+    DEEP8_ARGUMENT_CHECK(1 == y.batchSize(), "the shape is error");
+    requireGPU(x);
+}
+
+// [batch, dims..] of x and the same with 1 at every reduced axis, both in the enlarged 5-entry form
+void meanDims(const Shape &x, const std::vector<int> &axis, Dims5 &xa, Dims5 &ya) {
+    const int rank = (int)x.nDims + 1;
+    std::vector<bool> reduce(rank, axis.empty());
+    for (size_t i = 0; i < axis.size(); ++i) {
+        DEEP8_ARGUMENT_CHECK(-rank <= axis[i] && axis[i] < rank, "the reduce dim is error");
+        reduce[(axis[i] + rank) % rank] = true;
+    }
+    xa = enlargeShapeToMaxDim(x);
+    ya = xa;
+    if (reduce[0]) ya.d[0] = 1;
+    // dim i (1-based over [batch, dims..]) sits at enlarged position MAX_TENSOR_DIMS - nDims + i
+    for (int i = 1; i < rank; ++i)
+        if (reduce[i]) ya.d[MAX_TENSOR_DIMS - (int)x.nDims + i] = 1;
+}
+
+}  // namespace
+
+void Minus(const Tensor &x, const Tensor &y, Tensor &z) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType() && x.deviceType() == z.deviceType(), "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the param data type must be same");
+    checkBroadcast(x, y, z);
+    requireGPU(x);
+    MinusGPU(x, y, z);
+}
+
+void MinusGPU(const Tensor &x, const Tensor &y, Tensor &z) {
+    const Dims5 xa = enlargeShapeToMaxDim(x.shape), ya = enlargeShapeToMaxDim(y.shape), za = enlargeShapeToMaxDim(z.shape);
+    D8_CHECK(d8_minus(dtypeOf(x), x.raw(), xa.d, y.raw(), ya.d, z.raw(), za.d, nullptr));
+}
+
+void MinusGradX(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &z, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape, "the x shape is error");
+    checkBinaryGrad(x, y, z, dx, dz);
+    MinusGradXGPU(x, dx, y, z, dz);
+}
+
+void MinusGradXGPU(const Tensor &, Tensor &dx, const Tensor &, const Tensor &, const Tensor &dz) { addGradGPU(dx, dz); }
+
+void MinusGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape, "the y shape is error");
+    checkBinaryGrad(x, y, z, dy, dz);
+    MinusGradYGPU(x, y, dy, z, dz);
+}
+
+void MinusGradYGPU(const Tensor &, const Tensor &, Tensor &dy, const Tensor &, const Tensor &dz) {
+    const Dims5 ga = enlargeShapeToMaxDim(dy.shape), za = enlargeShapeToMaxDim(dz.shape);
+    const int dt = dtypeOf(dy);
+    PoolScratch ws(dy.device(), d8_add_grad_scratch_bytes(dt, ga.d, za.d));
+    D8_CHECK(d8_minus_grad_y(dt, dy.raw(), ga.d, dz.raw(), za.d, ws.ptr, ws.bytes, nullptr));
+}
+
+namespace {
+typedef int (*NormFn)(int, const void *, void *, int, long, void *, size_t, void *);
+void normGPU(NormFn fn, const Tensor &x, Tensor &y) {
+    const int dt = dtypeOf(x), batch = (int)x.batch();
+    const long size = (long)x.batchSize();
+    const int yd[5] = {batch, 1, 1, 1, 1}, xd[5] = {batch, 1, 1, 1, (int)size};
+    PoolScratch ws(x.device(), d8_add_grad_scratch_bytes(dt, yd, xd));
+    D8_CHECK(fn(dt, x.raw(), y.raw(), batch, size, ws.ptr, ws.bytes, nullptr));
+}
+}  // namespace
+
+void L1Norm(const Tensor &x, Tensor &y) {
+    checkNorm(x, y);
+    L1NormGPU(x, y);
+}
+void L1NormGPU(const Tensor &x, Tensor &y) { normGPU(d8_l1norm, x, y); }
+
+void L1NormGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy) {
+    checkNormGrad(x, dx, y, dy);
+    L1NormGradGPU(x, dx, y, dy);
+}
+void L1NormGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy) {
+    D8_CHECK(d8_l1norm_grad(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), (int)x.batch(), (long)x.batchSize(), nullptr));
+}
+
+void L2Norm(const Tensor &x, Tensor &y) {
+    checkNorm(x, y);
+    L2NormGPU(x, y);
+}
+void L2NormGPU(const Tensor &x, Tensor &y) { normGPU(d8_l2norm, x, y); }
+
+void L2NormGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy) {
+    checkNormGrad(x, dx, y, dy);
+    L2NormGradGPU(x, dx, y, dy);
+}
+void L2NormGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy) {
+    D8_CHECK(d8_l2norm_grad(dtypeOf(x), x.raw(), dx.raw(), y.raw(), dy.raw(), (int)x.batch(), (long)x.batchSize(), nullptr));
+}
+
+Shape ReduceMeanShape(const Shape &x, const std::vector<int> &axis, bool keepDims) {
+    const int rank = (int)x.nDims + 1;
+    std::vector<bool> reduce(rank, axis.empty());
+    for (size_t i = 0; i < axis.size(); ++i) {
+        DEEP8_ARGUMENT_CHECK(-rank <= axis[i] && axis[i] < rank, "the reduce dim is error");
+        reduce[(axis[i] + rank) % rank] = true;
+    }
+    DEEP8_ARGUMENT_CHECK(rank >= 2, "the shape is error");
+    const size_t batch = reduce[0] ? 1 : x.batch;
+    std::vector<size_t> list;
+    for (int i = 1; i < rank; ++i) {
+        if (reduce[i]) {
+            if (keepDims) list.emplace_back(1);
+        } else {
+            list.emplace_back(x.dim(i - 1));
+        }
+    }
+    if (list.empty()) list.emplace_back(1);
+    return Shape(batch, list);
+}
+
+void ReduceMean(const Tensor &x, Tensor &y, const std::vector<int> &axis, bool keepDims) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType(), "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType, "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(ReduceMeanShape(x.shape, axis, keepDims) == y.shape, "the y shape is error");
+    requireGPU(x);
+    ReduceMeanGPU(x, y, axis, keepDims);
+}
+
+void ReduceMeanGPU(const Tensor &x, Tensor &y, const std::vector<int> &axis, bool) {
+    Dims5 xa, ya;
+    meanDims(x.shape, axis, xa, ya);
+    const int dt = dtypeOf(x);
+    PoolScratch ws(x.device(), d8_add_grad_scratch_bytes(dt, ya.d, xa.d));
+    D8_CHECK(d8_reduce_mean(dt, x.raw(), xa.d, y.raw(), ya.d, ws.ptr, ws.bytes, nullptr));
+}
+
+void ReduceMeanGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, const std::vector<int> &axis, bool keepDims) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == dx.deviceType() && x.deviceType() == y.deviceType() && x.deviceType() == dy.deviceType(),
+                         "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == dy.elementType,
+                         "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && y.shape == dy.shape, "the x/dx or y/dy shape must be same");
+    DEEP8_ARGUMENT_CHECK(ReduceMeanShape(x.shape, axis, keepDims) == y.shape, "the y shape is error");
+    requireGPU(x);
+    ReduceMeanGradGPU(x, dx, y, dy, axis, keepDims);
+}
+
+void ReduceMeanGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy, const std::vector<int> &axis, bool) {
+    Dims5 xa, ya;
+    meanDims(x.shape, axis, xa, ya);
+    D8_CHECK(d8_reduce_mean_grad(dtypeOf(x), dx.raw(), xa.d, dy.raw(), ya.d, nullptr));
+}
+
+void AXPBY(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType() && x.deviceType() == z.deviceType(), "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape.size() == y.shape.size() && x.shape.size() == z.shape.size(), "the param shape size must be same");
+    requireGPU(x);
+    AXPBYGPU(x, alpha, y, beta, z);
+}
+
+void AXPBYGPU(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z) {
+    D8_CHECK(d8_axpby(dtypeOf(x), x.raw(), alpha, y.raw(), beta, z.raw(), (long)x.shape.size(), nullptr));
+}
+
 }  // namespace Math
 }  // namespace Deep8

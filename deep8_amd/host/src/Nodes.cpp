@@ -2,6 +2,7 @@
 #include "deep8/Nodes.h"
 
 #include <algorithm>
+#include <random>
 
 #include "deep8/Executor.h"
 #include "deep8/Math.h"
@@ -164,6 +165,42 @@ Variable &Variable::relu() {
     DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
     std::vector<Node *> in = {this};
     return *executor->addFunction(new ReLu(in));
+}
+
+Variable &Variable::minus(Variable &y) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this, &y};
+    return *executor->addFunction(new Minus(in));
+}
+
+Variable &Variable::l1Norm() {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this};
+    return *executor->addFunction(new L1Norm(in));
+}
+
+Variable &Variable::l2Norm() {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this};
+    return *executor->addFunction(new L2Norm(in));
+}
+
+Variable &Variable::reduceMean(std::vector<int> axis, bool keepDims) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this};
+    return *executor->addFunction(new ReduceMean(in, axis, keepDims));
+}
+
+Variable &Variable::l1NormLoss() { return l1Norm().reduceMean({}, false); }
+Variable &Variable::l2NormLoss() { return l2Norm().reduceMean({}, false); }
+
+Variable &Variable::gaussian(float mean, float stddev) {
+    DEEP8_ARGUMENT_CHECK(DType::Float32 == value.elementType.id, "gaussian() fills Float32 variables");
+    static std::mt19937 engine{std::random_device{}()};
+    std::normal_distribution<float> dist(mean, stddev);
+    std::vector<float> host(value.shape.size());
+    for (auto &v : host) v = dist(engine);
+    return feed(host.data());
 }
 
 Variable &Variable::conv2d(Variable &filter, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
@@ -431,6 +468,95 @@ void ReLu::forward(const std::vector<const Tensor *> &in, Tensor *output) { Math
 void ReLu::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t,
                     Tensor *iGradient) {
     Math::ReLuGrad(*in[0], *iGradient, *output, *outputGradient);
+}
+
+Minus::Minus(std::vector<Node *> &in) : Function(in) {
+    DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the Minus Function needs 2 input");
+}
+
+Shape Minus::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputShapes.size(), "the input count must be 2");
+    return broadcastShape(inputShapes[0], inputShapes[1]);
+}
+
+ElementType Minus::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(2 == inputTypes.size(), "the input count must be 2");
+    return Function::checkElementType(inputTypes);
+}
+
+void Minus::forward(const std::vector<const Tensor *> &in, Tensor *output) { Math::Minus(*in[0], *in[1], *output); }
+
+void Minus::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t index,
+                     Tensor *iGradient) {
+    if (0 == index) Math::MinusGradX(*in[0], *iGradient, *in[1], *output, *outputGradient);
+    else if (1 == index) Math::MinusGradY(*in[0], *in[1], *iGradient, *output, *outputGradient);
+    else DEEP8_RUNTIME_ERROR("the index is error");
+}
+
+L1Norm::L1Norm(std::vector<Node *> &in) : Function(in) {
+    DEEP8_ARGUMENT_CHECK(1 == inputs.size(), "the L1Norm Function needs 1 input");
+}
+
+Shape L1Norm::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputShapes.size(), "the input count must be 1");
+    return Shape(inputShapes[0].batch, {1});
+}
+
+ElementType L1Norm::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputTypes.size(), "the input count must be 1");
+    return Function::checkElementType(inputTypes);
+}
+
+void L1Norm::forward(const std::vector<const Tensor *> &in, Tensor *output) { Math::L1Norm(*in[0], *output); }
+
+void L1Norm::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t index,
+                      Tensor *iGradient) {
+    DEEP8_ARGUMENT_CHECK(0 == index, "the index of L1Norm backward is error");
+    Math::L1NormGrad(*in[0], *iGradient, *output, *outputGradient);
+}
+
+L2Norm::L2Norm(std::vector<Node *> &in) : Function(in) {
+    DEEP8_ARGUMENT_CHECK(1 == inputs.size(), "the L2Norm Function needs 1 input");
+}
+
+Shape L2Norm::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputShapes.size(), "the input count must be 1");
+    return Shape(inputShapes[0].batch, {1});
+}
+
+ElementType L2Norm::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputTypes.size(), "the input count must be 1");
+    return Function::checkElementType(inputTypes);
+}
+
+void L2Norm::forward(const std::vector<const Tensor *> &in, Tensor *output) { Math::L2Norm(*in[0], *output); }
+
+void L2Norm::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t index,
+                      Tensor *iGradient) {
+    DEEP8_ARGUMENT_CHECK(0 == index, "the index of L2Norm backward is error");
+    Math::L2NormGrad(*in[0], *iGradient, *output, *outputGradient);
+}
+
+ReduceMean::ReduceMean(std::vector<Node *> &in, std::vector<int> reduceAxis, bool keep)
+    : Function(in), axis(reduceAxis), keepDims(keep) {
+    DEEP8_ARGUMENT_CHECK(1 == inputs.size(), "the ReduceMean Function needs 1 input");
+}
+
+Shape ReduceMean::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputShapes.size(), "only have 1 input");
+    return Math::ReduceMeanShape(inputShapes[0], axis, keepDims);
+}
+
+ElementType ReduceMean::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputTypes.size(), "the input count must be 1");
+    return Function::checkElementType(inputTypes);
+}
+
+void ReduceMean::forward(const std::vector<const Tensor *> &in, Tensor *output) { Math::ReduceMean(*in[0], *output, axis, keepDims); }
+
+void ReduceMean::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t,
+                          Tensor *iGradient) {
+    Math::ReduceMeanGrad(*in[0], *iGradient, *output, *outputGradient, axis, keepDims);
 }
 
 }  // namespace Deep8

@@ -639,6 +639,141 @@ TEST_GPU(eager_executor_conv_to_scalar) {
     EXPECT(throws<std::runtime_error>([] { EagerExecutor cpu(DeviceType::CPU); }));
 }
 
+// ---- Minus / L1Norm / L2Norm / ReduceMean nodes, AXPBY, trainers ---------------------------------------------------
+TEST_GPU(loss_nodes_against_host_loops) {
+    EagerExecutor executor(DeviceType::GPU);
+    const size_t B = 3, R = 4, C = 5;
+    Variable &x = parameter(&executor, B, {R, C});
+    Variable &y = parameter(&executor, 1, {C});
+    std::vector<float> hx(B * R * C), hy(C);
+    for (float &f : hx) f = randInt(9) - 4.f;
+    for (float &f : hy) f = randInt(9) - 4.f;
+    x.feed(hx.data());
+    y.feed(hy.data());
+
+    Variable &d = x - y;  // y shared by every batch and row
+    EXPECT(d.shape() == Shape(B, {R, C}));
+    std::vector<float> hd(B * R * C), got(B * R * C);
+    for (size_t i = 0; i < hd.size(); ++i) hd[i] = hx[i] - hy[i % C];
+    d.fetch(got.data());
+    EXPECT(got == hd);
+
+    Variable &n1 = d.l1Norm();
+    EXPECT(n1.shape() == Shape(B, {1}));
+    std::vector<float> hn(B, 0.f), gn(B);
+    for (size_t b = 0; b < B; ++b)
+        for (size_t i = 0; i < R * C; ++i) hn[b] += std::fabs(hd[b * R * C + i]);
+    n1.fetch(gn.data());
+    EXPECT(gn == hn);
+
+    Variable &loss = n1.reduceMean({}, false);
+    EXPECT(loss.isScalar());
+    float gl = 0, hl = 0;
+    for (size_t b = 0; b < B; ++b) hl += hn[b];
+    hl /= (float)B;
+    loss.fetch(&gl);
+    EXPECT(std::fabs(gl - hl) <= 1e-6f * std::fabs(hl));
+
+    backward(loss);  // d loss / d x = sign(d) / B, d loss / d y = -sum over batch and rows of it
+    std::vector<float> gx(B * R * C), gy(C), wy(C, 0.f);
+    gpu().copyFromGPUToCPU(x.gradient.raw(), gx.data(), gx.size() * 4);
+    gpu().copyFromGPUToCPU(y.gradient.raw(), gy.data(), gy.size() * 4);
+    const float inv = 1.0f / (float)B;
+    for (size_t i = 0; i < hd.size(); ++i) {
+        const float g = hd[i] > 0 ? inv : (hd[i] == 0 ? 0.f : -inv);
+        EXPECT(gx[i] == g);
+        wy[i % C] -= g;
+    }
+    for (size_t c = 0; c < C; ++c) EXPECT(std::fabs(gy[c] - wy[c]) <= 1e-5f);
+
+    // L2Norm and ReduceMean over chosen axes, explicit-tensor form
+    HostTensor a = randomTensor(ElementType::from<float>(), 2, {3, 4}, 5);
+    HostTensor n2 = randomTensor(ElementType::from<float>(), 2, {1}, 0);
+    Math::L2Norm(a.t, n2.t);
+    download(n2);
+    std::vector<float> &r2 = n2.host;
+    for (size_t b = 0; b < 2; ++b) {
+        float sq = 0;
+        for (size_t i = 0; i < 12; ++i) sq += a.host[b * 12 + i] * a.host[b * 12 + i];
+        EXPECT(std::fabs(r2[b] - std::sqrt(sq)) <= 1e-6f * std::sqrt(sq) + 1e-12f);
+    }
+    HostTensor mean = randomTensor(ElementType::from<float>(), 1, {3, 1}, 0);
+    Tensor &m = mean.t;
+    Math::ReduceMean(a.t, m, {0, 2}, true);  // over the batch and the last axis
+    download(mean);
+    std::vector<float> &rm = mean.host;
+    for (size_t r = 0; r < 3; ++r) {
+        float sum = 0;
+        for (size_t b = 0; b < 2; ++b)
+            for (size_t c = 0; c < 4; ++c) sum += a.host[(b * 3 + r) * 4 + c];
+        EXPECT(std::fabs(rm[r] - sum / 8.f) <= 1e-6f);
+    }
+    EXPECT(Math::ReduceMeanShape(a.t.shape, {0, 2}, false) == Shape(1, {3}));
+    EXPECT(Math::ReduceMeanShape(a.t.shape, {}, false) == Shape(1, {1}));
+    EXPECT(throws<std::invalid_argument>([&] { Math::ReduceMean(a.t, m, {1}, true); }));
+    EXPECT(throws<std::invalid_argument>([&] { Math::L1Norm(a.t, m); }));
+}
+
+TEST_GPU(readme_regression_with_sgd_trainer) {
+    // The reference README's demo: find w with [[4,-1],[2,1]] w = [10,8], i.e. w = [3,2], by
+    // minimising l1NormLoss(input * w - output) with SGD.
+    float hx[4] = {4, -1, 2, 1}, hy[2] = {10, 8};
+    EagerExecutor executor;
+    LinearDecayLearningRateIterator learningRate(2000, 0.02f, 0.f);
+    SGDTrainer trainer(&learningRate);
+    Variable &w = parameter(&executor, {2});
+    w.gaussian();
+    Variable &input = parameter(&executor, {2, 2}, false);
+    Variable &output = parameter(&executor, {2}, false);
+    input.feed(hx);
+    output.feed(hy);
+    for (int i = 0; i < 2000; ++i) {
+        backward((input * w - output).l1NormLoss());
+        trainer.train(&executor);
+    }
+    float hw[2];
+    w.fetch(hw);
+    printf("     w = [%f, %f]\n", hw[0], hw[1]);
+    EXPECT(std::fabs(hw[0] - 3.f) < 0.05f && std::fabs(hw[1] - 2.f) < 0.05f);
+    EXPECT(executor.trainableParameters().size() == 1);
+}
+
+TEST_GPU(two_layer_convnet_trains_with_sgd) {
+    // conv 3x3 (4 -> 8) + bias + relu, conv 3x3 (8 -> 4), l2NormLoss against the output of a teacher
+    // network of the same shape: the loss must fall steadily under plain SGD.
+    EagerExecutor executor;
+    ConstantLearningRateIterator learningRate(0.02f);
+    SGDTrainer trainer(&learningRate);
+    const size_t B = 8, H = 8, W = 8;
+    std::mt19937 gen(7);
+    std::normal_distribution<float> nd(0.f, 1.f);
+    auto fill = [&](Variable &v, float scale) {
+        std::vector<float> h(v.shape().size());
+        for (float &f : h) f = nd(gen) * scale;
+        v.feed(h.data());
+    };
+    Variable &x = parameter(&executor, B, {H, W, 4}, false);  // retained across steps, no gradient
+    Variable &w1 = parameter(&executor, {8, 3, 3, 4}), &b1 = parameter(&executor, {8}), &w2 = parameter(&executor, {4, 3, 3, 8});
+    Variable &t1 = parameter(&executor, {8, 3, 3, 4}, false), &tb = parameter(&executor, {8}, false), &t2 = parameter(&executor, {4, 3, 3, 8}, false);
+    fill(x, 1.f);
+    fill(w1, 0.2f), fill(b1, 0.1f), fill(w2, 0.2f);
+    fill(t1, 0.2f), fill(tb, 0.1f), fill(t2, 0.2f);
+    auto net = [&](Variable &f1, Variable &bias, Variable &f2) -> Variable & { return relu(conv2d(x, f1) + bias).conv2d(f2); };
+    float first = 0, last = 0;
+    for (int i = 0; i < 300; ++i) {
+        Variable &loss = (net(w1, b1, w2) - net(t1, tb, t2)).l2NormLoss();
+        float v = 0;
+        loss.fetch(&v);
+        if (0 == i) first = v;
+        last = v;
+        backward(loss);
+        trainer.train(&executor);
+    }
+    printf("     loss %f -> %f\n", first, last);
+    EXPECT(std::isfinite(last) && last < 0.5f * first);
+    EXPECT(executor.trainableParameters().size() == 3);
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
