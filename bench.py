@@ -32,7 +32,7 @@ HBM_PEAK = 8000.0                      # GB/s
 # runs of this file (each counter scaled by what it reads for a plain copy of known size; the
 # summaries are kept under profiles/).  None where no counter run has been made.
 MEASURED_TRAFFIC = {
-    "c3": int((192.1 + 224.1 + 224.1) / 3 * 2**20 + 33.6 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
+    "c3": int((192.2 + 224.2 + 224.2) / 3 * 2**20 + 32.0 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
     "c4": int((26.5 + 24.5) * 2**20),                                # Conv2d forward kernel: fetch + write
     "c5": int((17.6 + 24.5) * 2**20),                                # DeConv2d forward GEMM: fetch + write
 }
