@@ -31,6 +31,9 @@ HBM_PEAK = 8000.0                      # GB/s
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this file (each counter scaled by what it reads for a plain copy of known size; the
 # summaries are kept under profiles/).  None where no counter run has been made.
+# --eager-zero: fill both gradients and accumulate into them (the reference executor's literal sequence)
+EAGER_ZERO = False
+
 MEASURED_TRAFFIC = {
     "c3": int((192.2 + 224.2 + 224.2) / 3 * 2**20 + 32.0 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
     "c4": int((26.5 + 24.5) * 2**20),                                # Conv2d forward kernel: fetch + write
@@ -114,16 +117,36 @@ class MatMulWorkload:
         check(self.lib.d8_matmul_grad_y(self.dt, self.x.ptr, *self.xs, self.dy.ptr, *self.ys, self.dz.ptr,
                                         self.ws.ptr, self.ws_bytes, None))
 
+    def grad_x_first(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_matmul_grad_x_overwrite(self.dt, self.dx.ptr, *self.xs, self.y.ptr, *self.ys, self.dz.ptr,
+                                                  self.ws.ptr, self.ws_bytes, None))
+
+    def grad_y_first(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_matmul_grad_y_overwrite(self.dt, self.x.ptr, *self.xs, self.dy.ptr, *self.ys, self.dz.ptr,
+                                                  self.ws.ptr, self.ws_bytes, None))
+
     def step(self):
+        """One forward + backward of a MatrixMultiply node as the executor issues it: forward, then the
+        two gradient products.  The executor's zeroGradient() before a backward pass is deferred
+        (Device::zeroLater), so the first product into each gradient is the overwrite form: same
+        result as fill + accumulate, without the fill and without reading the zeros back."""
         self.fwd()
-        self.dx.zero_()
-        self.dy.zero_()
-        self.grad_x()
-        self.grad_y()
+        if EAGER_ZERO:
+            self.dx.zero_()
+            self.dy.zero_()
+            self.grad_x()
+            self.grad_y()
+        else:
+            self.grad_x_first()
+            self.grad_y_first()
 
     def parts(self):
         f = self.flops / 3
-        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
+        if EAGER_ZERO:
+            return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
+        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x_first, f), "grad_y": (self.grad_y_first, f)}
 
 
 def mfma_stream_ceiling(wl, dtype_name):
@@ -402,11 +425,15 @@ def main():
     ap.add_argument("--operands", choices=("config", "zeros"), default="config",
                     help="zeros: run the MatrixMultiply workloads on all-zero operands (a diagnostic: the chip "
                          "clocks higher when the data does not toggle; not a valid benchmark value)")
+    ap.add_argument("--eager-zero", action="store_true",
+                    help="MatrixMultiply workloads: zero-fill the gradients and accumulate (the reference's literal "
+                         "sequence) instead of the executor's deferred zeroing + overwrite")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
-    global ZERO_OPERANDS
+    global ZERO_OPERANDS, EAGER_ZERO
     ZERO_OPERANDS = a.operands == "zeros"
+    EAGER_ZERO = a.eager_zero
     if a.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
                          "no second device anywhere in the path)" % a.gpus)

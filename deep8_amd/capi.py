@@ -52,6 +52,8 @@ SIGNATURES = {
     "d8_matmul": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_x": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_y": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "d8_matmul_grad_x_overwrite": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "d8_matmul_grad_y_overwrite": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_conv2d_geometry": (_I, [_I] * 9 + [ctypes.POINTER(_I)]),
     "d8_deconv2d_geometry": (_I, [_I] * 7 + [ctypes.POINTER(_I)]),
     "d8_conv2d_scratch_bytes": (_Z, [_I] * 14),

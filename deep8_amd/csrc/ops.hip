@@ -48,7 +48,7 @@ static int check_mm(const char *who, int dtype, int xb, int xr, int xc, int yb, 
 // which: 0 forward, 1 gradient of x, 2 gradient of y.  Pointers may be null when only the
 // shape is wanted (workspace query).
 static Gemm mm_plan(int which, const void *x, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
-                    const void *z) {
+                    const void *z, float grad_beta = 1.f) {
     const int zb = xb > yb ? xb : yb;
     const long xs = (long)xr * xc, ys = (long)yr * yc, zs = (long)xr * yc;
     Gemm g;
@@ -57,13 +57,13 @@ static Gemm mm_plan(int which, const void *x, int xb, int xr, int xc, const void
         else if (xb == 1 && yc == 1) g = {0, 1, yb, xr, xc, y, xc, 0, x, xc, 0, 0.f, (void *)z, xr, 0, 1};
         else g = {0, 0, xr, yc, xc, x, xc, xb == 1 ? 0 : xs, y, yc, ys, 0.f, (void *)z, yc, zs, zb};
     } else if (which == 1) {  // x plays dx (output), z plays dz
-        if (yb == 1) g = {0, 1, xb * xr, xc, yc, z, yc, 0, y, yc, 0, 1.f, (void *)x, xc, 0, 1};
-        else if (xb == 1 && yc == 1) g = {1, 0, xr, xc, yb, z, xr, 0, y, xc, 0, 1.f, (void *)x, xc, 0, 1};
-        else g = {0, 1, xr, xc, yc, z, yc, zs, y, yc, ys, 1.f, (void *)x, xc, xb == 1 ? 0 : xs, zb};
+        if (yb == 1) g = {0, 1, xb * xr, xc, yc, z, yc, 0, y, yc, 0, grad_beta, (void *)x, xc, 0, 1};
+        else if (xb == 1 && yc == 1) g = {1, 0, xr, xc, yb, z, xr, 0, y, xc, 0, grad_beta, (void *)x, xc, 0, 1};
+        else g = {0, 1, xr, xc, yc, z, yc, zs, y, yc, ys, grad_beta, (void *)x, xc, xb == 1 ? 0 : xs, zb};
     } else {  // y plays dy (output), z plays dz
-        if (yb == 1) g = {1, 0, yr, yc, xb * xr, x, xc, 0, z, yc, 0, 1.f, (void *)y, yc, 0, 1};
-        else if (xb == 1 && yc == 1) g = {0, 0, yb, xc, xr, z, xr, 0, x, xc, 0, 1.f, (void *)y, xc, 0, 1};
-        else g = {1, 0, yr, yc, xr, x, xc, xb == 1 ? 0 : xs, z, yc, zs, 1.f, (void *)y, yc, ys, zb};
+        if (yb == 1) g = {1, 0, yr, yc, xb * xr, x, xc, 0, z, yc, 0, grad_beta, (void *)y, yc, 0, 1};
+        else if (xb == 1 && yc == 1) g = {0, 0, yb, xc, xr, z, xr, 0, x, xc, 0, grad_beta, (void *)y, xc, 0, 1};
+        else g = {1, 0, yr, yc, xr, x, xc, xb == 1 ? 0 : xs, z, yc, zs, grad_beta, (void *)y, yc, ys, zb};
     }
     return g;
 }
@@ -161,6 +161,20 @@ int d8_matmul_grad_y(int dtype, const void *x, int xb, int xr, int xc, void *dy,
     if (int rc = check_mm("d8_matmul_grad_y", dtype, xb, xr, xc, yb, yr, yc)) return rc;
     D8_REQUIRE(x && dy && dz, "d8_matmul_grad_y: null tensor");
     return run(dtype, mm_plan(2, x, xb, xr, xc, dy, yb, yr, yc, dz), scratch, scratch_bytes, stream);
+}
+
+int d8_matmul_grad_x_overwrite(int dtype, void *dx, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
+                               const void *dz, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_mm("d8_matmul_grad_x_overwrite", dtype, xb, xr, xc, yb, yr, yc)) return rc;
+    D8_REQUIRE(dx && y && dz, "d8_matmul_grad_x_overwrite: null tensor");
+    return run(dtype, mm_plan(1, dx, xb, xr, xc, y, yb, yr, yc, dz, 0.f), scratch, scratch_bytes, stream);
+}
+
+int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc, void *dy, int yb, int yr, int yc,
+                               const void *dz, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_mm("d8_matmul_grad_y_overwrite", dtype, xb, xr, xc, yb, yr, yc)) return rc;
+    D8_REQUIRE(x && dy && dz, "d8_matmul_grad_y_overwrite: null tensor");
+    return run(dtype, mm_plan(2, x, xb, xr, xc, dy, yb, yr, yc, dz, 0.f), scratch, scratch_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -126,6 +126,17 @@ public:
     virtual void *gpuOneHalf() = 0;
     virtual void *gpuOneFloat() = 0;
     virtual void *gpuOneDouble() = 0;
+
+    // Deferred zeroing of whole allocations.  The executor zeroes every gradient before a backward
+    // pass (deep8/src/model/EagerExecutor.cpp:51-65) and most of them are then written exactly once,
+    // by a routine that can just as well overwrite.  zeroLater(ptr, size) records that the
+    // allocation starting at ptr reads as zeros from now on; settle(ptr) performs a recorded fill
+    // (Tensor::raw() calls it, so every ordinary reader and writer sees real zeros); takeZero(ptr)
+    // forgets the record and returns true when there was one -- the caller then owes a full
+    // overwrite of the allocation.  free() forgets the record too.
+    virtual void zeroLater(void *ptr, size_t size) { zero(ptr, size); }
+    virtual void settle(void *) {}
+    virtual bool takeZero(void *) { return false; }
 };
 
 // Buddy allocator over large hipMalloc'ed blocks.  Requests are rounded up to a power of two and
@@ -203,6 +214,13 @@ public:
     void *gpuOneDouble() override;
 
     void synchronize();  // wait for the default stream (fetch() does this implicitly)
+
+    void zeroLater(void *ptr, size_t size) override;
+    void settle(void *ptr) override;
+    bool takeZero(void *ptr) override;
+
+private:
+    std::unordered_map<void *, size_t> pendingZero;  // allocation -> bytes still to be zeroed
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -241,7 +259,20 @@ public:
     Device *device() const { return storage.device; }
     size_t *refPtr() const { return storage.refPtr; }
     size_t refCount() const { return storage.refPtr[0]; }
-    void *raw() const { return (byte *)storage.ptr + offset; }
+    // Device address of the first element; performs a deferred zero fill of the allocation first.
+    void *raw() const {
+        if (storage.device) storage.device->settle(storage.ptr);
+        return (byte *)storage.ptr + offset;
+    }
+    // For a routine that is about to write every element: true when the tensor is a whole
+    // allocation whose zero fill was still deferred (the fill is dropped: write, do not add);
+    // otherwise false, with any deferred fill performed.
+    bool takeZero() const {
+        if (!storage.device) return false;
+        if (0 == offset && byteCount() == storage.size) return storage.device->takeZero(storage.ptr);
+        storage.device->settle(storage.ptr);
+        return false;
+    }
 
     bool isScalar() const { return 1 == shape.size(); }
     void zero();

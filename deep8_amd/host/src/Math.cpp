@@ -101,7 +101,10 @@ void Constant(Tensor &x, float scalar) {
     ConstantGPU(x, scalar);
 }
 
-void ConstantGPU(Tensor &x, float scalar) { D8_CHECK(d8_fill(dtypeOf(x), x.raw(), x.size(), scalar, nullptr)); }
+void ConstantGPU(Tensor &x, float scalar) {
+    x.takeZero();  // every element is written: a deferred zero fill is moot
+    D8_CHECK(d8_fill(dtypeOf(x), x.raw(), x.size(), scalar, nullptr));
+}
 
 // ---- MatrixMultiply -------------------------------------------------------------------------------------------
 void MatrixMultiply(const Tensor &x, const Tensor &y, Tensor &z) {
@@ -136,7 +139,10 @@ void MatrixMultiplyGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const 
     const MM d = mmDims(x, y);
     const int dt = dtypeOf(x);
     PoolScratch ws(x.device(), d8_matmul_scratch_bytes(dt, 1, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
-    D8_CHECK(d8_matmul_grad_x(dt, dx.raw(), d.xb, d.xr, d.xc, y.raw(), d.yb, d.yr, d.yc, dz.raw(), ws.ptr, ws.bytes, nullptr));
+    // a gradient whose zero fill is still deferred is written, not added to
+    const bool fresh = dx.takeZero();
+    D8_CHECK((fresh ? d8_matmul_grad_x_overwrite : d8_matmul_grad_x)(dt, dx.raw(), d.xb, d.xr, d.xc, y.raw(), d.yb, d.yr, d.yc,
+                                                                    dz.raw(), ws.ptr, ws.bytes, nullptr));
 }
 
 void MatrixMultiplyGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz) {
@@ -156,7 +162,9 @@ void MatrixMultiplyGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const 
     const MM d = mmDims(x, y);
     const int dt = dtypeOf(x);
     PoolScratch ws(x.device(), d8_matmul_scratch_bytes(dt, 2, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
-    D8_CHECK(d8_matmul_grad_y(dt, x.raw(), d.xb, d.xr, d.xc, dy.raw(), d.yb, d.yr, d.yc, dz.raw(), ws.ptr, ws.bytes, nullptr));
+    const bool fresh = dy.takeZero();
+    D8_CHECK((fresh ? d8_matmul_grad_y_overwrite : d8_matmul_grad_y)(dt, x.raw(), d.xb, d.xr, d.xc, dy.raw(), d.yb, d.yr, d.yc,
+                                                                    dz.raw(), ws.ptr, ws.bytes, nullptr));
 }
 
 // ---- Conv2d -------------------------------------------------------------------------------------------------------

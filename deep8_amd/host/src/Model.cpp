@@ -284,7 +284,10 @@ GPUDevice::~GPUDevice() {
 }
 
 void *GPUDevice::malloc(size_t size) { return memoryPool->malloc(size); }
-void GPUDevice::free(void *ptr) { memoryPool->free(ptr); }
+void GPUDevice::free(void *ptr) {
+    pendingZero.erase(ptr);
+    memoryPool->free(ptr);
+}
 void *GPUDevice::mallocCPU(size_t size) { return memoryPool->mallocCPU(size); }
 void GPUDevice::freeCPU(void *ptr) { memoryPool->freeCPU(ptr); }
 void GPUDevice::zero(void *ptr, size_t size) { memoryPool->zero(ptr, size); }
@@ -296,6 +299,19 @@ void *GPUDevice::gpuOneHalf() { return oneHalf; }
 void *GPUDevice::gpuOneFloat() { return oneFloat; }
 void *GPUDevice::gpuOneDouble() { DEEP8_RUNTIME_ERROR("type float64 is not support"); }
 void GPUDevice::synchronize() { D8_CHECK(d8_stream_sync(nullptr)); }
+
+void GPUDevice::zeroLater(void *ptr, size_t size) { pendingZero[ptr] = size; }
+
+void GPUDevice::settle(void *ptr) {
+    if (pendingZero.empty()) return;
+    auto it = pendingZero.find(ptr);
+    if (it == pendingZero.end()) return;
+    const size_t size = it->second;
+    pendingZero.erase(it);
+    zero(ptr, size);
+}
+
+bool GPUDevice::takeZero(void *ptr) { return !pendingZero.empty() && pendingZero.erase(ptr) > 0; }
 
 // ---- TensorStorage ---------------------------------------------------------------------------------------------------
 TensorStorage::TensorStorage() : device(nullptr), ptr(nullptr), refPtr(nullptr), size(0) {}

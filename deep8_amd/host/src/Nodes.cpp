@@ -111,7 +111,12 @@ bool Variable::isScalar() { return updateGradient ? value.isScalar() && gradient
 
 void Variable::zeroGradient() {
     DEEP8_ARGUMENT_CHECK(updateGradient, "this variable does not have gradient");
-    Math::Constant(gradient, 0);
+    // a gradient that owns its whole allocation is zeroed lazily: the first routine that would add
+    // into it overwrites instead, any other access fills it first (Device::zeroLater)
+    if (0 == gradient.offset && gradient.byteCount() == gradient.storage.size)
+        gradient.device()->zeroLater(gradient.storage.ptr, gradient.storage.size);
+    else
+        Math::Constant(gradient, 0);
 }
 
 void Variable::oneGradient() {

@@ -714,6 +714,45 @@ TEST_GPU(loss_nodes_against_host_loops) {
     EXPECT(throws<std::invalid_argument>([&] { Math::L1Norm(a.t, m); }));
 }
 
+TEST_GPU(deferred_gradient_zeroing) {
+    // zeroGradient() on a gradient that owns its allocation only records the fill; a reader must
+    // see zeros, the first MatrixMultiply gradient overwrites, a second one adds.
+    EagerExecutor executor;
+    const size_t M = 6, K = 5, N = 4;
+    Variable &x = parameter(&executor, {M, K});
+    Variable &y = parameter(&executor, {K, N});
+    std::vector<float> hx(M * K), hy(K * N), garbage(M * K, 77.f), got(M * K);
+    for (float &f : hx) f = randInt(5);
+    for (float &f : hy) f = randInt(5);
+    x.feed(hx.data());
+    y.feed(hy.data());
+    gpu().copyFromCPUToGPU(garbage.data(), x.gradient.raw(), garbage.size() * 4);
+    x.zeroGradient();
+    gpu().copyFromGPUToCPU(x.gradient.raw(), got.data(), got.size() * 4);  // raw() performs the fill
+    for (float f : got) EXPECT(f == 0.f);
+
+    HostTensor dz = randomTensor(ElementType::from<float>(), 1, {M, N}, 5);
+    Tensor z = makeTensor(gpu(), ElementType::from<float>(), 1, {M, N});
+    std::vector<float> want(M * K, 0.f);
+    for (size_t m = 0; m < M; ++m)
+        for (size_t k = 0; k < K; ++k)
+            for (size_t n = 0; n < N; ++n) want[m * K + k] += dz.host[m * N + n] * hy[k * N + n];
+    gpu().copyFromCPUToGPU(garbage.data(), x.gradient.storage.ptr, garbage.size() * 4);  // behind raw()'s back
+    x.zeroGradient();
+    Math::MatrixMultiplyGradX(x.value, x.gradient, y.value, z, dz.t);  // overwrites the garbage
+    gpu().copyFromGPUToCPU(x.gradient.raw(), got.data(), got.size() * 4);
+    EXPECT(got == want);
+    Math::MatrixMultiplyGradX(x.value, x.gradient, y.value, z, dz.t);  // adds
+    gpu().copyFromGPUToCPU(x.gradient.raw(), got.data(), got.size() * 4);
+    for (size_t i = 0; i < got.size(); ++i) EXPECT(got[i] == 2 * want[i]);
+    // an element-wise gradient after a deferred zero: the fill happens first
+    x.zeroGradient();
+    HostTensor g = randomTensor(ElementType::from<float>(), 1, {M, K}, 9);
+    Math::AddGradX(x.value, x.gradient, x.value, x.value, g.t);
+    gpu().copyFromGPUToCPU(x.gradient.raw(), got.data(), got.size() * 4);
+    EXPECT(got == g.host);
+}
+
 TEST_GPU(readme_regression_with_sgd_trainer) {
     // The reference README's demo: find w with [[4,-1],[2,1]] w = [10,8], i.e. w = [3,2], by
     // minimising l1NormLoss(input * w - output) with SGD.

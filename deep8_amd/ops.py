@@ -70,7 +70,7 @@ def gemm(ta, tb, A, B, C=None, beta=0.0, use_workspace=True):
 
 
 # ---- MatrixMultiply ----------------------------------------------------------------------------
-def _mm(which, x, y, z):
+def _mm(which, x, y, z, overwrite=False):
     lib = capi.init()
     dt = _same_dtype(x, y, z)
     xb, xr, xc = _mat(x)
@@ -78,7 +78,8 @@ def _mm(which, x, y, z):
     dx_, dy_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray.from_numpy(z)
     nb = lib.d8_matmul_scratch_bytes(dt, which, xb, xr, xc, yb, yr, yc)
     ws = _scratch(nb) if nb else None
-    fn = (lib.d8_matmul, lib.d8_matmul_grad_x, lib.d8_matmul_grad_y)[which]
+    fn = (lib.d8_matmul, lib.d8_matmul_grad_x_overwrite if overwrite else lib.d8_matmul_grad_x,
+          lib.d8_matmul_grad_y_overwrite if overwrite else lib.d8_matmul_grad_y)[which]
     check(fn(dt, dx_.ptr, xb, xr, xc, dy_.ptr, yb, yr, yc, dz_.ptr, ws.ptr if ws else None, nb, None))
     return (dz_, dx_, dy_)[which].numpy()
 
@@ -89,17 +90,18 @@ def matmul(x, y):
     return _mm(0, x, y, z)
 
 
-def matmul_grad_x(x, y, dz, dx=None):
-    """returns dx + dz * y^T (dx defaults to zeros of x's shape; x only supplies the shape)"""
+def matmul_grad_x(x, y, dz, dx=None, overwrite=False):
+    """returns dx + dz * y^T (dx defaults to zeros of x's shape; x only supplies the shape); with
+    overwrite the destination's old contents are ignored: dz * y^T"""
     y, dz = np.ascontiguousarray(y), np.ascontiguousarray(dz)
     dx = np.zeros(np.shape(x), y.dtype) if dx is None else np.ascontiguousarray(dx)
-    return _mm(1, dx, y, dz)
+    return _mm(1, dx, y, dz, overwrite)
 
 
-def matmul_grad_y(x, y, dz, dy=None):
+def matmul_grad_y(x, y, dz, dy=None, overwrite=False):
     x, dz = np.ascontiguousarray(x), np.ascontiguousarray(dz)
     dy = np.zeros(np.shape(y), x.dtype) if dy is None else np.ascontiguousarray(dy)
-    return _mm(2, x, dy, dz)
+    return _mm(2, x, dy, dz, overwrite)
 
 
 # ---- geometry -------------------------------------------------------------------------------------

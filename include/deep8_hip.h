@@ -131,6 +131,16 @@ int d8_matmul_grad_x(int dtype, void *dx, int xb, int xr, int xc,
 int d8_matmul_grad_y(int dtype, const void *x, int xb, int xr, int xc,
                      void *dy, int yb, int yr, int yc, const void *dz,
                      void *scratch, size_t scratch_bytes, void *stream);
+/* The same two products written over their destination instead of added to it: what the pair
+ * "zero the gradient, then accumulate" (deep8/src/model/EagerExecutor.cpp:51-65 followed by
+ * Math::MatrixMultiplyGradX/YGPU) leaves behind, without the fill and without reading the zeros
+ * back.  For callers that know the destination holds zeros (or nothing yet).                    */
+int d8_matmul_grad_x_overwrite(int dtype, void *dx, int xb, int xr, int xc,
+                               const void *y, int yb, int yr, int yc, const void *dz,
+                               void *scratch, size_t scratch_bytes, void *stream);
+int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc,
+                               void *dy, int yb, int yr, int yc, const void *dz,
+                               void *scratch, size_t scratch_bytes, void *stream);
 
 /* out[0..3] = OH, OW, padTop, padLeft (deep8/src/math/Conv2d.cpp:20-32, Conv2d.cu:332-336;
  * deep8/src/math/DeConv2d.cpp:23-29, DeConv2d.cu:99-100) */

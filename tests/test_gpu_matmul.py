@@ -34,6 +34,26 @@ def test_matmul_integer_exact(oracle_port, xs, ys):
     assert np.array_equal(ops.matmul_grad_y(x, y, dz, dy0), oracle_port.matmul_grad_y(x, y, dz, dy0))
 
 
+@pytest.mark.parametrize("xs,ys", CASES + [((1, 512, 512), (1, 512, 512)), ((32, 128, 64), (1, 64, 128)), ((1, 4096, 64), (1, 64, 512))])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_matmul_gradients_overwrite_form(oracle_port, xs, ys, dtype):
+    """d8_matmul_grad_{x,y}_overwrite leave what "zero, then accumulate" leaves, whatever the
+    destination held before (split and summed reductions included)."""
+    from deep8_amd import ops
+    r = rng(sum(xs) + 2 * sum(ys))
+    c = (lambda a: h(a)) if dtype == np.float16 else (lambda a: a)
+    hi = 2 if dtype == np.float16 else 20
+    x, y = ints(r, xs, hi), ints(r, ys, hi)
+    if dtype == np.float16:
+        x, y = x * (r.random(xs) < 0.3), y * (r.random(ys) < 0.3)
+    dz = ints(r, oracle_port.matmul(x, y).shape, hi)
+    junk_x, junk_y = ints(r, xs, 1000) - 500, ints(r, ys, 1000) - 500
+    want_dx, want_dy = oracle_port.matmul_grad_x(x, y, dz), oracle_port.matmul_grad_y(x, y, dz)
+    assert dtype == np.float32 or max(np.abs(want_dx).max(), np.abs(want_dy).max()) < 2048
+    assert np.array_equal(f(ops.matmul_grad_x(c(x), c(y), c(dz), c(junk_x), overwrite=True)), want_dx)
+    assert np.array_equal(f(ops.matmul_grad_y(c(x), c(y), c(dz), c(junk_y), overwrite=True)), want_dy)
+
+
 @pytest.mark.parametrize("xs,ys", CASES)
 def test_matmul_half_integer_exact(oracle_port, xs, ys):
     from deep8_amd import ops
