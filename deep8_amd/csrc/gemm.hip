@@ -264,18 +264,55 @@ static int launch(GemmArgs &g, int transA, int transB, bool tiled, hipStream_t s
     return 0;
 }
 
-size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red) {
-    int tps = 0;
-    const int splits = plan_splits(gemm_tiled_k_step(dtype), M, N, K, 1, red, (size_t)-1, &tps);
-    return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+// A tall product whose output is one column of 128-row tiles (a convolution with up to 127 output
+// channels: M = images x pixels) rarely gives every CU the same number of tiles: 784 tiles on 256
+// CUs run as long as 1024 would.  Such a product is cut in two along M: the rows that fill whole
+// rounds of the chip run unsplit, the remaining band of rows runs as a second product whose
+// reduction is split so that it, too, occupies the whole chip for a fraction of a tile's time.
+// Returns the rows of the first part (0: do not cut).
+static int balanced_rows(const GemmArgs &g) {
+    if (g.batch != 1 || g.N >= 128 || g.M < 128 || g.virt == VIRT_B_KROWS) return 0;
+    const long tiles = ceil_div(g.M, 128), cus = cu_count();
+    const long rest = tiles % cus;
+    if (tiles < cus || rest == 0 || rest * 2 > cus) return 0;
+    return (int)((tiles - rest) * 128);
 }
 
-int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
-                   hipStream_t stream) {
+size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red) {
+    int tps = 0;
+    GemmArgs probe;
+    memset(&probe, 0, sizeof(probe));
+    probe.M = M, probe.N = N, probe.K = K, probe.batch = 1, probe.red = red;
+    const int head = balanced_rows(probe);
+    const int rows = head ? M - head : M;  // with a cut, only the second part is split
+    const int splits = plan_splits(gemm_tiled_k_step(dtype), rows, N, K, 1, red, (size_t)-1, &tps);
+    return splits > 1 ? (size_t)splits * rows * N * sizeof(float) : 0;
+}
+
+static int gemm_tiled_run_whole(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
+                                hipStream_t stream) {
     g.ws = (float *)workspace;
     g.splits = plan_splits(gemm_tiled_k_step(dtype), g.M, g.N, g.K, g.batch, g.red, (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0,
                            &g.tiles_per_split);
     return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, true, stream) : launch<float>(g, transA, transB, true, stream);
+}
+
+int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
+                   hipStream_t stream) {
+    static const bool no_cut = getenv("D8_GEMM_NO_ROW_CUT") != nullptr;  // tuning and test aid
+    const int head = (no_cut || transA) ? 0 : balanced_rows(g);
+    if (!head) return gemm_tiled_run_whole(dtype, g, transA, transB, workspace, workspace_bytes, stream);
+    const size_t es = dtype_bytes(dtype);
+    GemmArgs first = g, second = g;
+    first.M = head;
+    second.M = g.M - head;
+    second.C = (char *)g.C + (size_t)head * g.ldc * es;
+    if (g.virt == VIRT_A_ROWS) second.m_base = g.m_base + head;
+    else second.A = (const char *)g.A + (size_t)head * g.lda * es;
+    if (!gemm_tiled_eligible(dtype, second, transA, transB))
+        return gemm_tiled_run_whole(dtype, g, transA, transB, workspace, workspace_bytes, stream);
+    if (int rc = gemm_tiled_run_whole(dtype, first, transA, transB, nullptr, 0, stream)) return rc;
+    return gemm_tiled_run_whole(dtype, second, transA, transB, workspace, workspace_bytes, stream);
 }
 
 }  // namespace d8
@@ -337,6 +374,7 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     g.splits = 1;
     g.tiles_per_split = 0;
     g.virt = VIRT_NONE;
+    g.m_base = 0;
     memset(&g.pg, 0, sizeof(g.pg));
     const bool tiled = K > 0 && gemm_tiled_eligible(dtype, g, transA, transB);
     if (K > 0) {  // K == 0 is the empty reduction: C = beta * C

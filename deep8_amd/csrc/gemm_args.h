@@ -41,6 +41,7 @@ struct GemmArgs {
     //   VIRT_B_KROWS  B is the image; B[k][n] = column n of patch row k (N = taps x channels)
     int virt;
     PatchGeom pg;
+    int m_base;  // VIRT_A_ROWS: row 0 of this product is patch row m_base (a product over a band of rows)
 };
 
 // Tiled kernels (fp16 and fp32) for shapes whose operands can be moved in 16-byte pieces.

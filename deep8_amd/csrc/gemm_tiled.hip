@@ -350,7 +350,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         const int plane = pg.OH * pg.OW;
 #pragma unroll
         for (int p = 0; p < A_IT; ++p) {
-            const int m = m0 + a_r + p * T::A_ROWS, img = m / plane, rem = m - img * plane;
+            const int m = g.m_base + m0 + a_r + p * T::A_ROWS, img = m / plane, rem = m - img * plane;
             const int oy = rem / pg.OW, ox = rem - oy * pg.OW;
             va_iy[p] = oy * pg.sy - pg.pt;
             va_ix[p] = ox * pg.sx - pg.pl;
