@@ -220,17 +220,23 @@ class ConvWorkload:
         self._call(self.lib.d8_deconv2d if self.deconv else self.lib.d8_conv2d, self.x.ptr, self.w.ptr, self.z.ptr)
 
     def grad_x(self):
-        self._call(self.lib.d8_deconv2d_grad_x if self.deconv else self.lib.d8_conv2d_grad_x,
+        first = "" if EAGER_ZERO else "_overwrite"
+        self._call(getattr(self.lib, ("d8_deconv2d_grad_x" if self.deconv else "d8_conv2d_grad_x") + first),
                    self.gx.ptr, self.w.ptr, self.gz.ptr)
 
     def grad_y(self):
-        self._call(self.lib.d8_deconv2d_grad_y if self.deconv else self.lib.d8_conv2d_grad_y,
+        first = "" if EAGER_ZERO else "_overwrite"
+        self._call(getattr(self.lib, ("d8_deconv2d_grad_y" if self.deconv else "d8_conv2d_grad_y") + first),
                    self.x.ptr, self.gw.ptr, self.gz.ptr)
 
     def step(self):
+        """forward + both gradients as the executor issues them: its zeroGradient() is deferred, so the
+        first (here: only) product into each gradient is the overwrite form; --eager-zero fills and
+        accumulates instead"""
         self.fwd()
-        self.gx.zero_()
-        self.gw.zero_()
+        if EAGER_ZERO:
+            self.gx.zero_()
+            self.gw.zero_()
         self.grad_x()
         self.grad_y()
 
@@ -426,7 +432,7 @@ def main():
                     help="zeros: run the MatrixMultiply workloads on all-zero operands (a diagnostic: the chip "
                          "clocks higher when the data does not toggle; not a valid benchmark value)")
     ap.add_argument("--eager-zero", action="store_true",
-                    help="MatrixMultiply workloads: zero-fill the gradients and accumulate (the reference's literal "
+                    help="zero-fill the gradients and accumulate (the reference's literal "
                          "sequence) instead of the executor's deferred zeroing + overwrite")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")

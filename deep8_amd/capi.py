@@ -60,10 +60,14 @@ SIGNATURES = {
     "d8_conv2d": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "d8_conv2d_grad_x": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "d8_conv2d_grad_y": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
+    "d8_conv2d_grad_x_overwrite": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
+    "d8_conv2d_grad_y_overwrite": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "d8_deconv2d_scratch_bytes": (_Z, [_I] * 12),
     "d8_deconv2d": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
     "d8_deconv2d_grad_x": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
     "d8_deconv2d_grad_y": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
+    "d8_deconv2d_grad_x_overwrite": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
+    "d8_deconv2d_grad_y_overwrite": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _Z, _P]),
     "d8_add": (_I, [_I, _P, _IP, _P, _IP, _P, _IP, _P]),
     "d8_add_grad_scratch_bytes": (_Z, [_I, _IP, _IP]),
     "d8_add_grad": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),

@@ -266,10 +266,10 @@ int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
     return run(dtype, conv_plan(0, M, K, OC, scratch, w, z), ws ? (char *)scratch + col : nullptr, ws, stream);
 }
 
-int d8_conv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
+static int d8_conv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int IC,
                      const void *w, int OC, int FH, int FW, const void *gz,
                      int covered, int sy, int sx, int dy, int dx,
-                     void *scratch, size_t scratch_bytes, void *stream) {
+                     void *scratch, size_t scratch_bytes, void *stream, float beta) {
     int g[4];
     if (int rc = check_conv("d8_conv2d_grad_x", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return rc;
     if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
@@ -280,21 +280,25 @@ int d8_conv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
         const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
         GemmArgs ga;
         int ta, tb;
-        if (conv_implicit_plan(dtype, 1, cs, gx, w, gz, ga, ta, tb))
+        if (conv_implicit_plan(dtype, 1, cs, gx, w, gz, ga, ta, tb)) {
+            ga.beta = beta;
             return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+        }
     }
     D8_REQUIRE(scratch, "d8_conv2d_grad_x: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_x: scratch too small");
     const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
     if (int rc = run(dtype, conv_plan(1, M, K, OC, scratch, w, gz), ws ? (char *)scratch + col : nullptr, ws, stream))
         return rc;
+    if (beta == 0.f)  // col2im adds into its destination
+        if (int rc = d8_fill(dtype, gx, (size_t)B * IH * IW * IC, 0.f, stream)) return rc;
     return d8_col2im(dtype, scratch, gx, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream);
 }
 
-int d8_conv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
+static int d8_conv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
                      void *gw, int OC, int FH, int FW, const void *gz,
                      int covered, int sy, int sx, int dy, int dx,
-                     void *scratch, size_t scratch_bytes, void *stream) {
+                     void *scratch, size_t scratch_bytes, void *stream, float beta) {
     int g[4];
     if (int rc = check_conv("d8_conv2d_grad_y", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return rc;
     if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
@@ -305,15 +309,19 @@ int d8_conv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
         const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
         GemmArgs ga;
         int ta, tb;
-        if (conv_implicit_plan(dtype, 2, cs, x, gw, gz, ga, ta, tb))
+        if (conv_implicit_plan(dtype, 2, cs, x, gw, gz, ga, ta, tb)) {
+            ga.beta = beta;
             return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+        }
     }
     D8_REQUIRE(scratch, "d8_conv2d_grad_y: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_y: scratch too small");
     if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
         return rc;
     const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
-    return run(dtype, conv_plan(2, M, K, OC, scratch, gw, gz), ws ? (char *)scratch + col : nullptr, ws, stream);
+    Gemm plan = conv_plan(2, M, K, OC, scratch, gw, gz);
+    plan.beta = beta;
+    return run(dtype, plan, ws ? (char *)scratch + col : nullptr, ws, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -381,10 +389,10 @@ int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
     return launch_col2im(dtype, scratch, z, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), false, as_stream(stream));
 }
 
-int d8_deconv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
+static int d8_deconv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int IC,
                        const void *w, int OC, int FH, int FW, const void *gz,
                        int covered, int sy, int sx,
-                       void *scratch, size_t scratch_bytes, void *stream) {
+                       void *scratch, size_t scratch_bytes, void *stream, float beta) {
     int g[4];
     if (int rc = check_conv("d8_deconv2d_grad_x", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
@@ -393,21 +401,25 @@ int d8_deconv2d_grad_x(int dtype, void *gx, int B, int IH, int IW, int IC,
     D8_REQUIRE(gx && w && gz, "d8_deconv2d_grad_x: null tensor");
     {
         GemmArgs ga;
-        if (deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, gx, w, gz, ga))
+        if (deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, gx, w, gz, ga)) {
+            ga.beta = beta;
             return gemm_tiled_run(dtype, ga, 0, 0, scratch, scratch_bytes, as_stream(stream));
+        }
     }
     D8_REQUIRE(scratch, "d8_deconv2d_grad_x: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d_grad_x: scratch too small");
     if (int rc = launch_im2col(dtype, gz, scratch, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), as_stream(stream)))
         return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
-    return run(dtype, deconv_plan(1, M, T, OC, IC, scratch, w, gx), ws ? (char *)scratch + mat : nullptr, ws, stream);
+    Gemm plan = deconv_plan(1, M, T, OC, IC, scratch, w, gx);
+    plan.beta = beta;
+    return run(dtype, plan, ws ? (char *)scratch + mat : nullptr, ws, stream);
 }
 
-int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
+static int d8_deconv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
                        void *gw, int OC, int FH, int FW, const void *gz,
                        int covered, int sy, int sx,
-                       void *scratch, size_t scratch_bytes, void *stream) {
+                       void *scratch, size_t scratch_bytes, void *stream, float beta) {
     int g[4];
     if (int rc = check_conv("d8_deconv2d_grad_y", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
@@ -418,7 +430,40 @@ int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
     if (int rc = launch_im2col(dtype, gz, scratch, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), as_stream(stream)))
         return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
-    return run(dtype, deconv_plan(2, M, T, OC, IC, scratch, gw, x), ws ? (char *)scratch + mat : nullptr, ws, stream);
+    Gemm plan = deconv_plan(2, M, T, OC, IC, scratch, gw, x);
+    plan.beta = beta;
+    return run(dtype, plan, ws ? (char *)scratch + mat : nullptr, ws, stream);
 }
+
+#define D8_CONV_GRAD_PAIR(name, first, grad)                                                                      \
+    int name(int dtype, first, int B, int IH, int IW, int IC, grad, int OC, int FH, int FW, const void *gz,        \
+             int covered, int sy, int sx, int dy, int dx, void *scratch, size_t scratch_bytes, void *stream) {       \
+        return name##_impl(dtype, a0, B, IH, IW, IC, a1, OC, FH, FW, gz, covered, sy, sx, dy, dx, scratch,           \
+                           scratch_bytes, stream, 1.f);                                                              \
+    }                                                                                                                \
+    int name##_overwrite(int dtype, first, int B, int IH, int IW, int IC, grad, int OC, int FH, int FW,             \
+                         const void *gz, int covered, int sy, int sx, int dy, int dx, void *scratch,                 \
+                         size_t scratch_bytes, void *stream) {                                                       \
+        return name##_impl(dtype, a0, B, IH, IW, IC, a1, OC, FH, FW, gz, covered, sy, sx, dy, dx, scratch,           \
+                           scratch_bytes, stream, 0.f);                                                              \
+    }
+#define D8_DECONV_GRAD_PAIR(name, first, grad)                                                                    \
+    int name(int dtype, first, int B, int IH, int IW, int IC, grad, int OC, int FH, int FW, const void *gz,        \
+             int covered, int sy, int sx, void *scratch, size_t scratch_bytes, void *stream) {                       \
+        return name##_impl(dtype, a0, B, IH, IW, IC, a1, OC, FH, FW, gz, covered, sy, sx, scratch, scratch_bytes,    \
+                           stream, 1.f);                                                                             \
+    }                                                                                                                \
+    int name##_overwrite(int dtype, first, int B, int IH, int IW, int IC, grad, int OC, int FH, int FW,             \
+                         const void *gz, int covered, int sy, int sx, void *scratch, size_t scratch_bytes,           \
+                         void *stream) {                                                                             \
+        return name##_impl(dtype, a0, B, IH, IW, IC, a1, OC, FH, FW, gz, covered, sy, sx, scratch, scratch_bytes,    \
+                           stream, 0.f);                                                                             \
+    }
+
+// the accumulating entry points and their overwrite forms (the destination's old contents ignored)
+D8_CONV_GRAD_PAIR(d8_conv2d_grad_x, void *a0, const void *a1)
+D8_CONV_GRAD_PAIR(d8_conv2d_grad_y, const void *a0, void *a1)
+D8_DECONV_GRAD_PAIR(d8_deconv2d_grad_x, void *a0, const void *a1)
+D8_DECONV_GRAD_PAIR(d8_deconv2d_grad_y, const void *a0, void *a1)
 
 }  // extern "C"

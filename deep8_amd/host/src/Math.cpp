@@ -211,7 +211,8 @@ void Conv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &
     const ConvDims d = convDims(x, y, z);
     const int dt = dtypeOf(x);
     const size_t bytes = d8_conv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
-    D8_CHECK(d8_conv2d_grad_x(dt, dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS, dxcol, bytes, nullptr));
+    const bool fresh = dx.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_conv2d_grad_x_overwrite : d8_conv2d_grad_x)(dt, dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS, dxcol, bytes, nullptr));
 }
 
 size_t Conv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
@@ -234,7 +235,8 @@ void Conv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &
     const ConvDims d = convDims(x, y, z);
     const int dt = dtypeOf(x);
     const size_t bytes = d8_conv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);
-    D8_CHECK(d8_conv2d_grad_y(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS, xcol, bytes, nullptr));
+    const bool fresh = dy.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_conv2d_grad_y_overwrite : d8_conv2d_grad_y)(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS, xcol, bytes, nullptr));
 }
 
 #undef CONV_ARGS
@@ -283,7 +285,8 @@ void DeConv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor
     const ConvDims d = convDims(x, y, z);
     const int dt = dtypeOf(x);
     const size_t bytes = d8_deconv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
-    D8_CHECK(d8_deconv2d_grad_x(dt, dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
+    const bool fresh = dx.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_deconv2d_grad_x_overwrite : d8_deconv2d_grad_x)(dt, dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
 }
 
 size_t DeConv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX) {
@@ -306,7 +309,8 @@ void DeConv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor
     const ConvDims d = convDims(x, y, z);
     const int dt = dtypeOf(x);
     const size_t bytes = d8_deconv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
-    D8_CHECK(d8_deconv2d_grad_y(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
+    const bool fresh = dy.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_deconv2d_grad_y_overwrite : d8_deconv2d_grad_y)(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
 }
 
 #undef DECONV_ARGS

@@ -139,7 +139,7 @@ def conv2d(x, w, covered=True, sy=1, sx=1, dy=1, dx=1):
     return dz_.numpy()
 
 
-def conv2d_grad_x(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None):
+def conv2d_grad_x(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None, overwrite=False):
     lib = capi.init()
     w, gz = _filt(w), np.ascontiguousarray(gz)
     dt = _same_dtype(w, gz)
@@ -149,12 +149,12 @@ def conv2d_grad_x(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None):
     dgx, dw_, dgz = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
     nb = lib.d8_conv2d_scratch_bytes(dt, 1, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx)
     ws = _scratch(nb)
-    check(lib.d8_conv2d_grad_x(dt, dgx.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dgz.ptr, int(covered),
+    check((lib.d8_conv2d_grad_x_overwrite if overwrite else lib.d8_conv2d_grad_x)(dt, dgx.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dgz.ptr, int(covered),
                                sy, sx, dy, dx, ws.ptr, nb, None))
     return dgx.numpy()
 
 
-def conv2d_grad_y(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None):
+def conv2d_grad_y(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None, overwrite=False):
     lib = capi.init()
     x, gz = np.ascontiguousarray(x), np.ascontiguousarray(gz)
     dt = _same_dtype(x, gz)
@@ -164,7 +164,7 @@ def conv2d_grad_y(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None):
     dx_, dgw, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(gw), DeviceArray.from_numpy(gz)
     nb = lib.d8_conv2d_scratch_bytes(dt, 2, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx)
     ws = _scratch(nb)
-    check(lib.d8_conv2d_grad_y(dt, dx_.ptr, B, IH, IW, IC, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
+    check((lib.d8_conv2d_grad_y_overwrite if overwrite else lib.d8_conv2d_grad_y)(dt, dx_.ptr, B, IH, IW, IC, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
                                sy, sx, dy, dx, ws.ptr, nb, None))
     return dgw.numpy()
 
@@ -186,7 +186,7 @@ def deconv2d(x, w, covered=False, sy=1, sx=1):
     return dz_.numpy()
 
 
-def deconv2d_grad_x(x, w, gz, covered=False, sy=1, sx=1, gx=None):
+def deconv2d_grad_x(x, w, gz, covered=False, sy=1, sx=1, gx=None, overwrite=False):
     lib = capi.init()
     w, gz = _filt(w), np.ascontiguousarray(gz)
     dt = _same_dtype(w, gz)
@@ -196,12 +196,12 @@ def deconv2d_grad_x(x, w, gz, covered=False, sy=1, sx=1, gx=None):
     dgx, dw_, dgz = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
     nb = lib.d8_deconv2d_scratch_bytes(dt, 1, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx)
     ws = _scratch(nb)
-    check(lib.d8_deconv2d_grad_x(dt, dgx.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dgz.ptr, int(covered),
+    check((lib.d8_deconv2d_grad_x_overwrite if overwrite else lib.d8_deconv2d_grad_x)(dt, dgx.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dgz.ptr, int(covered),
                                  sy, sx, ws.ptr, nb, None))
     return dgx.numpy()
 
 
-def deconv2d_grad_y(x, w, gz, covered=False, sy=1, sx=1, gw=None):
+def deconv2d_grad_y(x, w, gz, covered=False, sy=1, sx=1, gw=None, overwrite=False):
     lib = capi.init()
     x, gz = np.ascontiguousarray(x), np.ascontiguousarray(gz)
     dt = _same_dtype(x, gz)
@@ -211,7 +211,7 @@ def deconv2d_grad_y(x, w, gz, covered=False, sy=1, sx=1, gw=None):
     dx_, dgw, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(gw), DeviceArray.from_numpy(gz)
     nb = lib.d8_deconv2d_scratch_bytes(dt, 2, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx)
     ws = _scratch(nb)
-    check(lib.d8_deconv2d_grad_y(dt, dx_.ptr, B, IH, IW, IC, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
+    check((lib.d8_deconv2d_grad_y_overwrite if overwrite else lib.d8_deconv2d_grad_y)(dt, dx_.ptr, B, IH, IW, IC, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
                                  sy, sx, ws.ptr, nb, None))
     return dgw.numpy()
 

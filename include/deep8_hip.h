@@ -178,6 +178,25 @@ int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
                        int covered, int sy, int sx,
                        void *scratch, size_t scratch_bytes, void *stream);
 
+/* Overwrite forms of the four convolution gradients: the destination's old contents are ignored
+ * (what "zero the gradient, then accumulate" leaves, without the fill and the read-back).      */
+int d8_conv2d_grad_x_overwrite(int dtype, void *gx, int B, int IH, int IW, int IC,
+                               const void *w, int OC, int FH, int FW, const void *gz,
+                               int covered, int sy, int sx, int dy, int dx,
+                               void *scratch, size_t scratch_bytes, void *stream);
+int d8_conv2d_grad_y_overwrite(int dtype, const void *x, int B, int IH, int IW, int IC,
+                               void *gw, int OC, int FH, int FW, const void *gz,
+                               int covered, int sy, int sx, int dy, int dx,
+                               void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_x_overwrite(int dtype, void *gx, int B, int IH, int IW, int IC,
+                                 const void *w, int OC, int FH, int FW, const void *gz,
+                                 int covered, int sy, int sx,
+                                 void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_y_overwrite(int dtype, const void *x, int B, int IH, int IW, int IC,
+                                 void *gw, int OC, int FH, int FW, const void *gz,
+                                 int covered, int sy, int sx,
+                                 void *scratch, size_t scratch_bytes, void *stream);
+
 /* ---- Add (broadcasting) and ReLu -----------------------------------------------------------
  * The element-wise steps that follow MatrixMultiply / Conv2d in a network (bias, activation).
  * Shapes are Deep8's 5-entry enlarged form [batch, d0, d1, d2, d3]: dims right-aligned, padded

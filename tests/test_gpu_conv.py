@@ -106,6 +106,11 @@ def test_conv2d_integer_exact(oracle_port, cfg):
                           oracle_port.conv2d_grad_x(x, w, gz, cov, sy, sx, dy, dx, gx0))
     assert np.array_equal(ops.conv2d_grad_y(x, w, gz, cov, sy, sx, dy, dx, gw0),
                           oracle_port.conv2d_grad_y(x, w, gz, cov, sy, sx, dy, dx, gw0))
+    # the overwrite forms ignore what the destination held
+    assert np.array_equal(ops.conv2d_grad_x(x, w, gz, cov, sy, sx, dy, dx, gx0 - 500, overwrite=True),
+                          oracle_port.conv2d_grad_x(x, w, gz, cov, sy, sx, dy, dx))
+    assert np.array_equal(ops.conv2d_grad_y(x, w, gz, cov, sy, sx, dy, dx, gw0 - 500, overwrite=True),
+                          oracle_port.conv2d_grad_y(x, w, gz, cov, sy, sx, dy, dx))
 
 
 @pytest.mark.parametrize("cfg", CONV)
@@ -143,6 +148,10 @@ def test_deconv2d_integer_exact(oracle_port, cfg):
                           oracle_port.deconv2d_grad_x(x, w, gz, cov, sy, sx, gx0))
     assert np.array_equal(ops.deconv2d_grad_y(x, w, gz, cov, sy, sx, gw0),
                           oracle_port.deconv2d_grad_y(x, w, gz, cov, sy, sx, gw0))
+    assert np.array_equal(ops.deconv2d_grad_x(x, w, gz, cov, sy, sx, gx0 - 500, overwrite=True),
+                          oracle_port.deconv2d_grad_x(x, w, gz, cov, sy, sx))
+    assert np.array_equal(ops.deconv2d_grad_y(x, w, gz, cov, sy, sx, gw0 - 500, overwrite=True),
+                          oracle_port.deconv2d_grad_y(x, w, gz, cov, sy, sx))
 
 
 @pytest.mark.parametrize("cfg", DECONV)
@@ -283,6 +292,8 @@ def test_conv2d_implicit_route(oracle_port, monkeypatch, cfg, imp32, imp16, dtyp
     got = (ops.conv2d(c(x), c(w), *a), ops.conv2d_grad_x(c(x), c(w), c(gz), *a, c(x)), ops.conv2d_grad_y(c(x), c(w), c(gz), *a, c(w)))
     for g_, w_ in zip(got, want):
         assert np.array_equal(f(g_), w_)
+    assert np.array_equal(f(ops.conv2d_grad_x(c(x), c(w), c(gz), *a, c(x), overwrite=True)), want[1] - x)
+    assert np.array_equal(f(ops.conv2d_grad_y(c(x), c(w), c(gz), *a, c(w), overwrite=True)), want[2] - w)
     # reals: both routes within tolerance of the oracle
     x, w = c(nrm(r, (B, IH, IW, IC))), c(nrm(r, (OC, FH, FW, IC), np.sqrt(2.0 / (FH * FW * IC))))
     gz = c(nrm(r, (B, OH, OW, OC)))
