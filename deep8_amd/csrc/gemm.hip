@@ -214,6 +214,12 @@ __global__ void gemm_split_reduce_scalar_kernel(GemmArgs g) {
     }
 }
 
+bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps) {
+    if (M < 128 || N < 128) return false;
+    const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch, cus = cu_count();
+    return tiles < cus && 4 * tiles >= cus && k_steps <= 32;
+}
+
 // How many pieces to cut the reduction into, for a kernel whose K step is BK.  Splitting is only
 // worth a second pass when the output alone gives the 256 CUs too few tiles; the long reductions
 // this catches are also the ones whose single fp32 accumulation chain would be longest.
@@ -223,6 +229,10 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     const int cus = cu_count();
     long splits = 1;
     if (tiles < cus) splits = (2L * cus + tiles - 1) / tiles;
+    // A short reduction over an output that half-height tiles spread over most of the chip is better
+    // left whole: the tiled kernel then takes 64 x 128 tiles (gemm_tiled_half_tiles) and the fp32
+    // partial sums, their round trip through memory and the second launch are saved.
+    if (gemm_tiled_half_tiles(M, N, batch, total)) splits = 1;
     const long max_by_len = total / 4 > 0 ? total / 4 : 1;  // at least 4 K steps per piece
     if (splits > max_by_len) splits = max_by_len;
     if (splits > 128) splits = 128;

@@ -56,6 +56,11 @@ int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipS
 bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB);
 int gemm_wide_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);
 
+// Whether an unsplit product of this shape should run on 64 x 128 tiles: too few 128 x 128 tiles
+// for the chip, enough half-height ones, and a reduction (k_steps K steps in all) too short to
+// be worth splitting.
+bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps);
+
 // Plan the split of the reduction, launch the tiled kernel (which must be eligible) and reduce.
 int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
                    hipStream_t stream);

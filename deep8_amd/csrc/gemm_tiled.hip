@@ -498,6 +498,8 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     // a 64-wide side gets a tile of that width (im2col products with 64 output channels)
     if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
     if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+    if (g.splits == 1 && gemm_tiled_half_tiles(g.M, g.N, g.batch, (long)g.red * (g.K / (128 / (int)sizeof(E)))))
+        return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
     return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
 }
 
