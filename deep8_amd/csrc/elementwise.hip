@@ -12,7 +12,7 @@
 // MinusGPU / MinusGradXGPU / MinusGradYGPU (deep8/src/math/Minus.cu:21-147), L1NormGPU / L1NormGradGPU
 // (deep8/src/math/L1Norm.cu:27-136), L2NormGPU / L2NormGradGPU (deep8/src/math/L2Norm.cu),
 // ReduceMeanGPU / ReduceMeanGradGPU (deep8/src/math/ReduceMean.cu:30-203 over GPUReduce.h) and AXPBYGPU
-// (deep8/src/math/AXPBY.cu:9-47).
+// (deep8/src/math/AXPBY.cu:9-47) and AdamUpdateGPU (deep8/src/math/AdamUpdate.cu:9-47).
 #include "common.h"
 
 namespace d8 {
@@ -272,6 +272,33 @@ __global__ __launch_bounds__(256) void axpby_kernel(const T *x, float alpha, con
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o[e] = (T)(alpha * ew_f32(a[e]) + beta * ew_f32(b[e]));
         *(VT *)(z + idx * VEC) = o;
+    }
+}
+
+// One Adam step (deep8/src/math/AdamUpdate.cu:9-20): g += wd * value; m = b1 m + (1 - b1) g;
+// v = b2 v + (1 - b2) g^2; value -= ratio * m / (sqrt(v) + eps).  All four tensors are read and
+// written once.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void adam_kernel(T *__restrict__ value, T *__restrict__ grad, T *__restrict__ m,
+                                                   T *__restrict__ v, float b1, float b2, float eps, float wd, float ratio,
+                                                   long total) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        VT x = *(const VT *)(value + idx * VEC), g = *(const VT *)(grad + idx * VEC);
+        VT mt = *(const VT *)(m + idx * VEC), vt = *(const VT *)(v + idx * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float xe = ew_f32(x[e]);
+            const float ge = ew_f32(g[e]) + xe * wd;
+            const float me = ew_f32(mt[e]) * b1 + (1.f - b1) * ge;
+            const float ve = ew_f32(vt[e]) * b2 + ge * ge * (1.f - b2);
+            g[e] = (T)ge, mt[e] = (T)me, vt[e] = (T)ve;
+            x[e] = (T)(xe - me / (sqrtf(ve) + eps) * ratio);
+        }
+        *(VT *)(value + idx * VEC) = x;
+        *(VT *)(grad + idx * VEC) = g;
+        *(VT *)(m + idx * VEC) = mt;
+        *(VT *)(v + idx * VEC) = vt;
     }
 }
 
@@ -615,6 +642,28 @@ int d8_axpby(int dtype, const void *x, float alpha, const void *y, float beta, v
     } else {
         if (al && n % 8 == 0) hipLaunchKernelGGL((axpby_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (const f16 *)x, alpha, (const f16 *)y, beta, (f16 *)z, n / 8);
         else hipLaunchKernelGGL((axpby_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const f16 *)x, alpha, (const f16 *)y, beta, (f16 *)z, n);
+    }
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int d8_adam_update(int dtype, void *value, void *gradient, void *m, void *v, float beta1, float beta2, float epsilon,
+                   float learning_rate, float weight_decay, long steps, long n, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_adam_update: element type %d is not supported", dtype);
+    D8_REQUIRE(n >= 0, "d8_adam_update: negative size");
+    if (n == 0) return 0;
+    D8_REQUIRE(value && gradient && m && v, "d8_adam_update: null tensor");
+    if (steps <= 0) steps = 1;  // avoid a division by zero (deep8/src/math/AdamUpdate.cpp:11-14)
+    const float ratio = learning_rate * sqrtf(1.0f - powf(beta2, (float)steps)) / (1.0f - powf(beta1, (float)steps));
+    hipStream_t s = as_stream(stream);
+    const bool al = al16(value) && al16(gradient) && al16(m) && al16(v);
+    if (dtype == D8_FLOAT32) {
+        if (al && n % 4 == 0) hipLaunchKernelGGL((adam_kernel<float, 4>), dim3(ew_grid(n / 4, 256)), dim3(256), 0, s, (float *)value, (float *)gradient, (float *)m, (float *)v, beta1, beta2, epsilon, weight_decay, ratio, n / 4);
+        else hipLaunchKernelGGL((adam_kernel<float, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (float *)value, (float *)gradient, (float *)m, (float *)v, beta1, beta2, epsilon, weight_decay, ratio, n);
+    } else {
+        if (al && n % 8 == 0) hipLaunchKernelGGL((adam_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (f16 *)value, (f16 *)gradient, (f16 *)m, (f16 *)v, beta1, beta2, epsilon, weight_decay, ratio, n / 8);
+        else hipLaunchKernelGGL((adam_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (f16 *)value, (f16 *)gradient, (f16 *)m, (f16 *)v, beta1, beta2, epsilon, weight_decay, ratio, n);
     }
     D8_LAUNCH_CHECK();
     return 0;

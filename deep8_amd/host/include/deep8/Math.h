@@ -98,6 +98,9 @@ Shape ReduceMeanShape(const Shape &x, const std::vector<int> &axis, bool keepDim
 /** z = alpha * x + beta * y */
 void AXPBY(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z);
 void AXPBYGPU(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z);
+/** one Adam step on value / gradient / m / v (deep8/include/math/AdamUpdate.h, checks deep8/src/math/AdamUpdate.cpp:6-23) */
+void AdamUpdate(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps);
+void AdamUpdateGPU(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps);
 
 }  // namespace Math
 }  // namespace Deep8

@@ -4,6 +4,7 @@
 //   Trainer       deep8/include/trainer/Trainer.h, deep8/src/trainer/Trainer.cpp:5-39
 //   SGDTrainer    deep8/include/trainer/SGDTrainer.h, deep8/src/trainer/SGDTrainer.cpp:6-17
 //                 value = (1 - lr * decay) * value - lr * gradient, one Math::AXPBY per parameter
+//   AdamTrainer   deep8/include/trainer/AdamTrainer.h, deep8/src/trainer/AdamTrainer.cpp:6-33
 #ifndef DEEP8_HOST_TRAINER_H
 #define DEEP8_HOST_TRAINER_H
 
@@ -50,6 +51,20 @@ public:
 class SGDTrainer : public Trainer {
 public:
     explicit SGDTrainer(LearningRateIterator *lr, float decay = 0);
+    void update(Executor *executor, Variable *parameter, float learningRate, float weightDecay, int64_t steps) override;
+};
+
+// Adam with bias-corrected step size; the moment estimates are Variables the executor keeps
+// (deep8/include/trainer/AdamTrainer.h, deep8/src/trainer/AdamTrainer.cpp:6-33).
+class AdamTrainer : public Trainer {
+public:
+    float beta1;
+    float beta2;
+    float epsilon;
+    std::unordered_map<Variable *, Variable *> m;
+    std::unordered_map<Variable *, Variable *> v;
+
+    explicit AdamTrainer(LearningRateIterator *lr, float beta1 = 0.9, float beta2 = 0.999, float epsilon = 1e-7, float decay = 0);
     void update(Executor *executor, Variable *parameter, float learningRate, float weightDecay, int64_t steps) override;
 };
 

@@ -609,5 +609,22 @@ void AXPBYGPU(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor 
     D8_CHECK(d8_axpby(dtypeOf(x), x.raw(), alpha, y.raw(), beta, z.raw(), (long)x.shape.size(), nullptr));
 }
 
+void AdamUpdate(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps) {
+    DEEP8_ARGUMENT_CHECK(value.deviceType() == gradient.deviceType() && value.deviceType() == m.deviceType() && value.deviceType() == v.deviceType(),
+                         "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(value.elementType == gradient.elementType && value.elementType == m.elementType && value.elementType == v.elementType,
+                         "the param data type must be same");
+    DEEP8_ARGUMENT_CHECK(value.shape.size() == gradient.shape.size() && value.shape.size() == m.shape.size() && value.shape.size() == v.shape.size(),
+                         "the param shape size must be same");
+    if (steps <= 0) steps = 1;  // avoid divide by 0
+    requireGPU(value);
+    AdamUpdateGPU(value, gradient, m, v, beta1, beta2, epsilon, learningRate, weightDecay, steps);
+}
+
+void AdamUpdateGPU(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps) {
+    D8_CHECK(d8_adam_update(dtypeOf(value), value.raw(), gradient.raw(), m.raw(), v.raw(), beta1, beta2, epsilon, learningRate, weightDecay,
+                            (long)steps, (long)value.shape.size(), nullptr));
+}
+
 }  // namespace Math
 }  // namespace Deep8

@@ -42,4 +42,23 @@ void SGDTrainer::update(Executor *, Variable *parameter, float learningRate, flo
     Math::AXPBY(gradient, alpha, value, beta, value);
 }
 
+AdamTrainer::AdamTrainer(LearningRateIterator *lr, float b1, float b2, float e, float decay)
+    : Trainer(lr, decay), beta1(b1), beta2(b2), epsilon(e) {}
+
+void AdamTrainer::update(Executor *executor, Variable *parameter, float learningRate, float weightDecay, int64_t steps) {
+    Tensor value = parameter->value, gradient = parameter->gradient;
+    if (m.find(parameter) == m.end()) {
+        Variable *mt = executor->addVariable(value.shape, value.elementType, false);
+        mt->value.zero();
+        m[parameter] = mt;
+    }
+    if (v.find(parameter) == v.end()) {
+        Variable *vt = executor->addVariable(value.shape, value.elementType, false);
+        vt->value.zero();
+        v[parameter] = vt;
+    }
+    Tensor mt = m[parameter]->value, vt = v[parameter]->value;
+    Math::AdamUpdate(value, gradient, mt, vt, beta1, beta2, epsilon, learningRate, weightDecay, steps);
+}
+
 }  // namespace Deep8

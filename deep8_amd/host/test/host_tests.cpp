@@ -777,6 +777,35 @@ TEST_GPU(readme_regression_with_sgd_trainer) {
     EXPECT(executor.trainableParameters().size() == 1);
 }
 
+TEST_GPU(readme_cpp_demo_with_adam_trainer) {
+    // The C++ demo of the reference's README, statement for statement (printing dropped).
+    float x[4] = {4, -1, 2, 1};
+    float y[2] = {10, 8};
+    EagerExecutor executor;
+    LinearDecayLearningRateIterator learningRate(1000);
+    AdamTrainer trainer(&learningRate);
+    auto &w = parameter(&executor, {2});
+    w.gaussian();
+    auto &input = parameter(&executor, {2, 2}, false);
+    auto &output = parameter(&executor, {2}, false);
+    input.feed(x);
+    output.feed(y);
+    float first = 0, last = 0;
+    for (int i = 0; i < 1000; ++i) {
+        auto &loss = (input * w - output).l1NormLoss();
+        loss.fetch(&last);
+        if (0 == i) first = last;
+        backward(loss);  // the README writes loss.backward(), which is Node's no-op in the reference too (Net.h:41 is the real one)
+        trainer.train(&executor, executor.trainableParameters());
+    }
+    float hw[2];
+    w.fetch(hw);
+    printf("     w = [%f, %f], loss %f -> %f\n", hw[0], hw[1], first, last);
+    // lr decays from 0.01 to 0 over 1000 steps: Adam moves each weight by at most about lr per step
+    // (sum = 5), enough to get from N(0, 0.01) to [3, 2]
+    EXPECT(std::fabs(hw[0] - 3.f) < 0.1f && std::fabs(hw[1] - 2.f) < 0.1f && last < 0.05f * first);
+}
+
 TEST_GPU(two_layer_convnet_trains_with_sgd) {
     // conv 3x3 (4 -> 8) + bias + relu, conv 3x3 (8 -> 4), l2NormLoss against the output of a teacher
     // network of the same shape: the loss must fall steadily under plain SGD.

@@ -422,3 +422,14 @@ def axpby(x, alpha, y, beta):
     a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray(x.shape, x.dtype)
     check(lib.d8_axpby(dt, a.ptr, alpha, b.ptr, beta, c.ptr, x.size, None))
     return c.numpy()
+
+
+def adam_update(value, gradient, m, v, beta1, beta2, epsilon, learning_rate, weight_decay, steps):
+    """one Adam step; returns the updated (value, gradient, m, v)"""
+    lib = capi.init()
+    arrs = [np.ascontiguousarray(a) for a in (value, gradient, m, v)]
+    dt = _same_dtype(*arrs)
+    dev = [DeviceArray.from_numpy(a) for a in arrs]
+    check(lib.d8_adam_update(dt, dev[0].ptr, dev[1].ptr, dev[2].ptr, dev[3].ptr, beta1, beta2, epsilon, learning_rate,
+                             weight_decay, steps, arrs[0].size, None))
+    return tuple(d.numpy() for d in dev)

@@ -256,6 +256,12 @@ int d8_reduce_mean(int dtype, const void *x, const int *xdims, void *y, const in
                    void *scratch, size_t scratch_bytes, void *stream);
 int d8_reduce_mean_grad(int dtype, void *dx, const int *xdims, const void *dy, const int *ydims, void *stream);
 int d8_axpby(int dtype, const void *x, float alpha, const void *y, float beta, void *z, long n, void *stream);
+/* d8_adam_update: gradient += weight_decay * value; m = beta1 m + (1 - beta1) gradient;
+ * v = beta2 v + (1 - beta2) gradient^2; value -= ratio * m / (sqrt(v) + epsilon) with
+ * ratio = learning_rate * sqrt(1 - beta2^steps) / (1 - beta1^steps), steps < 1 taken as 1.
+ * Math::AdamUpdateGPU (deep8/include/math/AdamUpdate.h, deep8/src/math/AdamUpdate.cu:9-47).      */
+int d8_adam_update(int dtype, void *value, void *gradient, void *m, void *v, float beta1, float beta2,
+                   float epsilon, float learning_rate, float weight_decay, long steps, long n, void *stream);
 
 /* ---- measurement aid (no counterpart in the reference) ---------------------------------------
  * d8_mfma_stream issues the tiled GEMM's MFMA instruction back to back on operands taken from

@@ -325,6 +325,13 @@ class _Port:
         self.lib.orc_axpby(_p(x), ctypes.c_float(alpha), _p(y), ctypes.c_float(beta), _p(z), ctypes.c_long(x.size))
         return z
 
+    def adam_update(self, value, gradient, m, v, beta1, beta2, epsilon, learning_rate, weight_decay, steps):
+        a = [_c(t).copy() for t in (value, gradient, m, v)]
+        cf = ctypes.c_float
+        self.lib.orc_adam_update(_p(a[0]), _p(a[1]), _p(a[2]), _p(a[3]), cf(beta1), cf(beta2), cf(epsilon), cf(learning_rate),
+                                 cf(weight_decay), ctypes.c_long(steps), ctypes.c_long(a[0].size))
+        return tuple(a)
+
 
 class _Ref:
     """Deep8's own CPU path (float only)."""
@@ -516,6 +523,13 @@ class _Ref:
         z = np.zeros_like(x)
         self._chk(self.lib.ref_axpby(_p(x), ctypes.c_float(alpha), _p(y), ctypes.c_float(beta), _p(z), *_nd(x)))
         return z
+
+    def adam_update(self, value, gradient, m, v, beta1, beta2, epsilon, learning_rate, weight_decay, steps):
+        a = [_c(t).copy() for t in (value, gradient, m, v)]
+        cf = ctypes.c_float
+        self._chk(self.lib.ref_adam_update(_p(a[0]), _p(a[1]), _p(a[2]), _p(a[3]), cf(beta1), cf(beta2), cf(epsilon),
+                                           cf(learning_rate), cf(weight_decay), ctypes.c_long(steps), *_nd(a[0])))
+        return tuple(a)
 
 
 port = _Port(PORT_PATH) if os.path.exists(PORT_PATH) else None

@@ -200,6 +200,21 @@ void orc_axpby(const float *x, float alpha, const float *y, float beta, float *z
     for (long i = 0; i < n; ++i) z[i] = x[i] * alpha + y[i] * beta;
 }
 
+/* deep8/src/math/AdamUpdate.cpp:25-41: the four Eigen statements in their order, float arithmetic
+ * as there (T = float); ratio computed in float from float pow / sqrt.  Pins: the live reference
+ * build, the golden fixtures and a textbook bias-corrected Adam step in numpy. */
+void orc_adam_update(float *value, float *gradient, float *m, float *v, float beta1, float beta2, float epsilon,
+                     float learning_rate, float weight_decay, long steps, long n) {
+    if (steps <= 0) steps = 1;
+    const float ratio = learning_rate * sqrtf(1.0f - powf(beta2, (float)steps)) / (1.0f - powf(beta1, (float)steps));
+    for (long i = 0; i < n; ++i) {
+        gradient[i] += value[i] * weight_decay;
+        m[i] = m[i] * beta1 + gradient[i] * (1.0f - beta1);
+        v[i] = v[i] * beta2 + gradient[i] * gradient[i] * (1.0f - beta2);
+        value[i] -= m[i] / (sqrtf(v[i]) + epsilon) * ratio;
+    }
+}
+
 int orc_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

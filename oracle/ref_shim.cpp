@@ -15,6 +15,7 @@
  *   Math::L2Norm / L2NormGrad                 deep8/src/math/L2Norm.cpp:6-42
  *   Math::ReduceMean / ReduceMeanGrad         deep8/src/math/ReduceMean.cpp:7-121
  *   Math::AXPBY                               deep8/src/math/AXPBY.cpp:6-20
+ *   Math::AdamUpdate                          deep8/src/math/AdamUpdate.cpp:6-23
  *
  * plus one materialisation of the patch expression the CPU Conv2d contracts over
  * (deep8/src/math/Conv2d.cpp:352-356), which is the "CPU Eigen im2col" the HIP im2col must
@@ -35,6 +36,7 @@
 #include "math/L2Norm.h"
 #include "math/ReduceMean.h"
 #include "math/AXPBY.h"
+#include "math/AdamUpdate.h"
 
 #include <chrono>
 #include <cstring>
@@ -409,6 +411,18 @@ int ref_axpby(const float *x, float alpha, const float *y, float beta, float *z,
         wrap(Y, y, b, vdims(nd, d));
         wrap(Z, z, b, vdims(nd, d));
         Math::AXPBY(*X.t, alpha, *Y.t, beta, *Z.t);
+    });
+}
+
+int ref_adam_update(float *value, float *gradient, float *m, float *v, float beta1, float beta2, float epsilon,
+                    float learningRate, float weightDecay, long steps, int b, int nd, const int *d) {
+    return guarded([&] {
+        Wrapped X, G, M, V;
+        wrap(X, value, b, vdims(nd, d));
+        wrap(G, gradient, b, vdims(nd, d));
+        wrap(M, m, b, vdims(nd, d));
+        wrap(V, v, b, vdims(nd, d));
+        Math::AdamUpdate(*X.t, *G.t, *M.t, *V.t, beta1, beta2, epsilon, learningRate, weightDecay, (int64_t)steps);
     });
 }
 

@@ -4,7 +4,7 @@
 Run in the build container, where oracle/_ref/libdeep8_ref.so has been compiled from the reference
 sources (`make -C oracle ref`):   python tests/golden/make_golden.py
 Every array is float32.  Case names: mm<i>_*, conv<i>_*, deconv<i>_*, patch<i>_*, loss<i>_* (Minus,
-L1Norm, L2Norm, ReduceMean, AXPBY); the geometry of case i is stored in <kind><i>_cfg.
+L1Norm, L2Norm, ReduceMean, AXPBY), adam<i>_* (AdamUpdate); the geometry of case i is stored in <kind><i>_cfg.
 """
 import os
 import sys
@@ -88,6 +88,15 @@ def main():
                     "loss%d_l1_gx" % i: ref.norm_grad(1, x, n1, dn, dx0), "loss%d_l2_gx" % i: ref.norm_grad(2, x, n2, dn, dx0),
                     "loss%d_mean" % i: m, "loss%d_mean_gx" % i: ref.reduce_mean_grad(x, m, dm, axes, dx=dx0),
                     "loss%d_axpby" % i: ref.axpby(x, -0.01, dx0, 0.999)})
+    # AdamUpdate: three consecutive steps from the same state, with weight decay
+    for i, n in enumerate((7, 64)):
+        st = [u((1, n)), None, np.zeros((1, n), np.float32), np.zeros((1, n), np.float32)]
+        out["adam%d_value0" % i] = st[0]
+        for step in (1, 2, 3):
+            g = u((1, n))
+            out["adam%d_grad%d" % (i, step)] = g
+            st = list(ref.adam_update(st[0], g, st[2], st[3], 0.9, 0.999, 1e-7, 0.01, 0.001, step))
+            out["adam%d_step%d" % (i, step)] = np.stack(st)  # value, gradient (with the decay term), m, v
     path = os.path.join(HERE, "deep8_cpu_reference.npz")
     np.savez_compressed(path, **out)
     print("wrote %s (%d arrays, %d bytes)" % (path, len(out), os.path.getsize(path)))

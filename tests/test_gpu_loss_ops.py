@@ -118,3 +118,23 @@ def test_loss_op_argument_errors():
     assert lib.d8_l1norm(12, a.ptr, a.ptr, 1, 4, None, 0, None) == 10002
     assert lib.d8_l2norm(capi.FLOAT32, a.ptr, a.ptr, 0, 4, None, 0, None) == 10001
     assert lib.d8_axpby(capi.FLOAT32, None, 1.0, None, 1.0, None, 0, None) == 0
+
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_adam_update(oracle_port, n, dtype):
+    """d8_adam_update against the oracle over three steps (the state of one step feeds the next)."""
+    from deep8_amd import ops
+    r = rng(n + 3)
+    c = _c(dtype)
+    st = [c(nrm(r, (1, n))), None, c(np.zeros((1, n))), c(np.zeros((1, n)))]
+    ref = [f(st[0]), None, f(st[2]), f(st[3])]
+    tol = 1e-5 if dtype == np.float32 else 4e-3
+    for step in (1, 2, 3):
+        g = c(nrm(r, (1, n)))
+        st = list(ops.adam_update(st[0], g, st[2], st[3], 0.9, 0.999, 1e-7, 0.01, 0.001, step))
+        ref = list(oracle_port.adam_update(ref[0], f(g), ref[2], ref[3], 0.9, 0.999, 1e-7, 0.01, 0.001, step))
+        for k in range(4):
+            assert rel_fro(f(st[k]), ref[k]) <= tol, (step, k)
+        if dtype == np.float16:
+            ref = [f(t) for t in st]  # follow the half-rounded state

@@ -424,3 +424,44 @@ def test_axpby_against_numpy_and_reference(oracle_port, oracle_ref):
     assert np.array_equal(z, x * np.float32(-0.01) + y * np.float32(0.999))
     if oracle_ref is not None:
         assert rel_fro(oracle_ref.axpby(x, -0.01, y, 0.999), z) <= 1e-7
+
+
+# ---- AdamUpdate -------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("i", _n("adam"))
+def test_adam_update_against_golden(oracle_port, i):
+    """Three consecutive steps of the reference's CPU AdamUpdate (weight decay 0.001)."""
+    g = lambda k: GOLD["adam%d_%s" % (i, k)]
+    st = [g("value0"), None, np.zeros_like(g("value0")), np.zeros_like(g("value0"))]
+    for step in (1, 2, 3):
+        st = list(oracle_port.adam_update(st[0], g("grad%d" % step), st[2], st[3], 0.9, 0.999, 1e-7, 0.01, 0.001, step))
+        want = g("step%d" % step)
+        for k in range(4):
+            assert rel_fro(st[k], want[k]) <= 1e-6, (step, k)
+
+
+def test_adam_update_against_textbook_and_reference(oracle_port, oracle_ref):
+    """Bias-corrected Adam in float64 numpy: m_hat = m / (1 - b1^t), v_hat = v / (1 - b2^t),
+    x -= lr * m_hat / (sqrt(v_hat) + eps'), which equals the reference's ratio form when epsilon is
+    scaled by sqrt(1 - b2^t); with epsilon = 0 the two coincide exactly."""
+    r = rng(77)
+    x, g = nrm(r, (2, 33)), nrm(r, (2, 33))
+    m, v = np.zeros_like(x), np.zeros_like(x)
+    b1, b2, lr = float(np.float32(0.9)), float(np.float32(0.999)), 0.01  # the betas as the float code sees them
+    X, M, V = x.astype(np.float64), m.astype(np.float64), v.astype(np.float64)
+    st = [x, None, m, v]
+    for t in (1, 2, 3, 4):
+        gt = nrm(r, x.shape)
+        st = list(oracle_port.adam_update(st[0], gt, st[2], st[3], b1, b2, 0.0, lr, 0.0, t))
+        M = b1 * M + (1 - b1) * gt
+        V = b2 * V + (1 - b2) * gt.astype(np.float64) ** 2
+        X = X - lr * (M / (1 - b1 ** t)) / np.sqrt(V / (1 - b2 ** t))
+        assert rel_fro(st[0], X) <= 1e-5 and rel_fro(st[2], M) <= 1e-6 and rel_fro(st[3], V) <= 1e-6
+    # steps <= 0 count as 1; weight decay adds wd * value to the gradient first
+    a = oracle_port.adam_update(x, g, m, v, b1, b2, 1e-7, lr, 0.5, 0)
+    b = oracle_port.adam_update(x, g + 0.5 * x, m, v, b1, b2, 1e-7, lr, 0.0, 1)
+    assert rel_fro(a[0], b[0]) <= 1e-6 and rel_fro(a[1], b[1]) <= 1e-7
+    if oracle_ref is not None:
+        want = oracle_ref.adam_update(x, g, m, v, b1, b2, 1e-7, lr, 0.001, 3)
+        got = oracle_port.adam_update(x, g, m, v, b1, b2, 1e-7, lr, 0.001, 3)
+        for k in range(4):
+            assert rel_fro(got[k], want[k]) <= 1e-6
