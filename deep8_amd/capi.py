@@ -82,6 +82,10 @@ SIGNATURES = {
     "d8_reduce_mean": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
     "d8_reduce_mean_grad": (_I, [_I, _P, _IP, _P, _IP, _P]),
     "d8_axpby": (_I, [_I, _P, _F, _P, _F, _P, ctypes.c_long, _P]),
+    "d8_maxpool2d": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
+    "d8_maxpool2d_grad": (_I, [_I, _P, _P, _P] + [_I] * 9 + [_P]),
+    "d8_avgpool2d": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
+    "d8_avgpool2d_grad": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
     "d8_adam_update": (_I, [_I, _P, _P, _P, _P, _F, _F, _F, _F, _F, ctypes.c_long, ctypes.c_long, _P]),
     "d8_mfma_stream_out_bytes": (_Z, []),
     "d8_mfma_stream": (_I, [_I, _P, _Z, _P, _I, ctypes.POINTER(ctypes.c_double), _P]),

@@ -98,6 +98,17 @@ Shape ReduceMeanShape(const Shape &x, const std::vector<int> &axis, bool keepDim
 /** z = alpha * x + beta * y */
 void AXPBY(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z);
 void AXPBYGPU(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor &z);
+/** x [B,IH,IW,C] -> y [B,OH,OW,C]; checks and output size deep8/src/math/MaxPooling2d.cpp:6-96, AvgPooling2d.cpp */
+void MaxPooling2d(const Tensor &x, Tensor &y, bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1);
+void MaxPooling2dGPU(const Tensor &x, Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX);
+void MaxPooling2dGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1);
+void MaxPooling2dGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX);
+void AvgPooling2d(const Tensor &x, Tensor &y, bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1);
+void AvgPooling2dGPU(const Tensor &x, Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX);
+void AvgPooling2dGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1);
+void AvgPooling2dGradGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX);
+/** [B, OH, OW, C] of a pooling over x (shared with the nodes' checkShape) */
+Shape Pooling2dShape(const Shape &x, bool covered, int filterHeight, int filterWidth, int strideY, int strideX);
 /** one Adam step on value / gradient / m / v (deep8/include/math/AdamUpdate.h, checks deep8/src/math/AdamUpdate.cpp:6-23) */
 void AdamUpdate(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps);
 void AdamUpdateGPU(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps);

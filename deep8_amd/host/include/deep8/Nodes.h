@@ -104,9 +104,12 @@ public:
     // value ~ N(mean, stddev) drawn on the host and copied over (deep8/src/nodes/Variable.cpp:201-205; the
     // reference draws on the device from an unseeded generator, so only the distribution is comparable)
     Variable &gaussian(float mean = 0.0, float stddev = 0.01);
+    // pooling (deep8/src/nodes/Variable.cpp: maxPooling2d / avgPooling2d)
+    Variable &maxPooling2d(bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1);
+    Variable &avgPooling2d(bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1);
 };
 
-enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply, Add, ReLu, Minus, L1Norm, L2Norm, ReduceMean };
+enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply, Add, ReLu, Minus, L1Norm, L2Norm, ReduceMean, MaxPooling2d, AvgPooling2d };
 
 class Function : public Node {
 protected:
@@ -229,6 +232,33 @@ public:
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
     void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
                   size_t index, Tensor *iGradient) override;
+};
+
+// Pooling over [B, H, W, C] (deep8/src/nodes/MaxPooling2d.cpp, deep8/src/nodes/AvgPooling2d.cpp)
+class Pooling2d : public Function {
+public:
+    bool isMax;
+    bool covered;
+    int filterHeight, filterWidth, strideY, strideX;
+
+    Pooling2d(std::vector<Node *> &inputs, bool isMax, bool covered, int filterHeight, int filterWidth, int strideY, int strideX);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+};
+
+class MaxPooling2d : public Pooling2d {
+public:
+    explicit MaxPooling2d(std::vector<Node *> &inputs, bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1)
+        : Pooling2d(inputs, true, covered, filterHeight, filterWidth, strideY, strideX) {}
+};
+
+class AvgPooling2d : public Pooling2d {
+public:
+    explicit AvgPooling2d(std::vector<Node *> &inputs, bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1)
+        : Pooling2d(inputs, false, covered, filterHeight, filterWidth, strideY, strideX) {}
 };
 
 // Shape of x + y (deep8/include/utils/ShapeUtils.h:19-36)

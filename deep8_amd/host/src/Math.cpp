@@ -609,6 +609,76 @@ void AXPBYGPU(const Tensor &x, float alpha, const Tensor &y, float beta, Tensor 
     D8_CHECK(d8_axpby(dtypeOf(x), x.raw(), alpha, y.raw(), beta, z.raw(), (long)x.shape.size(), nullptr));
 }
 
+// ---- MaxPooling2d / AvgPooling2d --------------------------------------------------------------------------------
+#define POOL_ARGS covered, filterHeight, filterWidth, strideY, strideX
+
+Shape Pooling2dShape(const Shape &x, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(3 == x.nDims, "the tensor dim must be 3");
+    DEEP8_ARGUMENT_CHECK(filterHeight >= 1 && filterWidth >= 1 && strideY >= 1 && strideX >= 1, "the params is error");
+    const int IH = (int)x.dim(0), IW = (int)x.dim(1);
+    int OH, OW;
+    if (!covered) {
+        OH = (IH - filterHeight) / strideY + 1;
+        OW = (IW - filterWidth) / strideX + 1;
+    } else {
+        OH = (IH - 1) / strideY + 1;
+        OW = (IW - 1) / strideX + 1;
+    }
+    DEEP8_ARGUMENT_CHECK(OH >= 1 && OW >= 1 && IH >= (covered ? 1 : filterHeight) && IW >= (covered ? 1 : filterWidth), "the shape is error");
+    return Shape(x.batch, {(size_t)OH, (size_t)OW, x.dim(2)});
+}
+
+namespace {
+void checkPool(const Tensor &x, const Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType(), "the param device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(3 == x.nDims() && 3 == y.nDims(), "the tensor dim must be 3");
+    DEEP8_ARGUMENT_CHECK(Pooling2dShape(x.shape, POOL_ARGS) == y.shape, "the shape is error");
+    requireGPU(x);
+}
+void checkPoolGrad(const Tensor &x, const Tensor &dx, const Tensor &y, const Tensor &dy, bool covered, int filterHeight, int filterWidth,
+                   int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape, "the x and dx shape must be same");
+    DEEP8_ARGUMENT_CHECK(y.shape == dy.shape, "the y and dy shape must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == dy.elementType, "the type must be same");
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == dx.deviceType() && x.deviceType() == y.deviceType() && x.deviceType() == dy.deviceType(),
+                         "the device type must be same");
+    checkPool(x, y, POOL_ARGS);
+}
+#define POOL_DIMS(t) (int)(t).batch(), (int)(t).dim(0), (int)(t).dim(1), (int)(t).dim(2)
+}  // namespace
+
+void MaxPooling2d(const Tensor &x, Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    checkPool(x, y, POOL_ARGS);
+    MaxPooling2dGPU(x, y, POOL_ARGS);
+}
+void MaxPooling2dGPU(const Tensor &x, Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    D8_CHECK(d8_maxpool2d(dtypeOf(x), x.raw(), y.raw(), POOL_DIMS(x), filterHeight, filterWidth, covered, strideY, strideX, nullptr));
+}
+void MaxPooling2dGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    checkPoolGrad(x, dx, y, dy, POOL_ARGS);
+    MaxPooling2dGradGPU(x, dx, y, dy, POOL_ARGS);
+}
+void MaxPooling2dGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    D8_CHECK(d8_maxpool2d_grad(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), POOL_DIMS(x), filterHeight, filterWidth, covered, strideY, strideX, nullptr));
+}
+void AvgPooling2d(const Tensor &x, Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    checkPool(x, y, POOL_ARGS);
+    AvgPooling2dGPU(x, y, POOL_ARGS);
+}
+void AvgPooling2dGPU(const Tensor &x, Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    D8_CHECK(d8_avgpool2d(dtypeOf(x), x.raw(), y.raw(), POOL_DIMS(x), filterHeight, filterWidth, covered, strideY, strideX, nullptr));
+}
+void AvgPooling2dGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    checkPoolGrad(x, dx, y, dy, POOL_ARGS);
+    AvgPooling2dGradGPU(x, dx, y, dy, POOL_ARGS);
+}
+void AvgPooling2dGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    D8_CHECK(d8_avgpool2d_grad(dtypeOf(x), dx.raw(), dy.raw(), POOL_DIMS(x), filterHeight, filterWidth, covered, strideY, strideX, nullptr));
+}
+#undef POOL_ARGS
+#undef POOL_DIMS
+
 void AdamUpdate(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps) {
     DEEP8_ARGUMENT_CHECK(value.deviceType() == gradient.deviceType() && value.deviceType() == m.deviceType() && value.deviceType() == v.deviceType(),
                          "the param device type must be same");

@@ -208,6 +208,18 @@ Variable &Variable::gaussian(float mean, float stddev) {
     return feed(host.data());
 }
 
+Variable &Variable::maxPooling2d(bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this};
+    return *executor->addFunction(new MaxPooling2d(in, covered, filterHeight, filterWidth, strideY, strideX));
+}
+
+Variable &Variable::avgPooling2d(bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this};
+    return *executor->addFunction(new AvgPooling2d(in, covered, filterHeight, filterWidth, strideY, strideX));
+}
+
 Variable &Variable::conv2d(Variable &filter, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
     DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
     std::vector<Node *> in = {this, &filter};
@@ -562,6 +574,34 @@ void ReduceMean::forward(const std::vector<const Tensor *> &in, Tensor *output) 
 void ReduceMean::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t,
                           Tensor *iGradient) {
     Math::ReduceMeanGrad(*in[0], *iGradient, *output, *outputGradient, axis, keepDims);
+}
+
+Pooling2d::Pooling2d(std::vector<Node *> &in, bool mx, bool cov, int fh, int fw, int sy, int sx)
+    : Function(in), isMax(mx), covered(cov), filterHeight(fh), filterWidth(fw), strideY(sy), strideX(sx) {
+    DEEP8_ARGUMENT_CHECK(1 == inputs.size(), "the pooling Function needs 1 input");
+    DEEP8_ARGUMENT_CHECK(fh >= 1 && fw >= 1 && sy >= 1 && sx >= 1, "the filter size or stride is error");
+}
+
+Shape Pooling2d::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputShapes.size(), "the input count must be 1");
+    return Math::Pooling2dShape(inputShapes[0], covered, filterHeight, filterWidth, strideY, strideX);
+}
+
+ElementType Pooling2d::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(1 == inputTypes.size(), "the input count must be 1");
+    return Function::checkElementType(inputTypes);
+}
+
+void Pooling2d::forward(const std::vector<const Tensor *> &in, Tensor *output) {
+    if (isMax) Math::MaxPooling2d(*in[0], *output, covered, filterHeight, filterWidth, strideY, strideX);
+    else Math::AvgPooling2d(*in[0], *output, covered, filterHeight, filterWidth, strideY, strideX);
+}
+
+void Pooling2d::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient, size_t index,
+                         Tensor *iGradient) {
+    DEEP8_ARGUMENT_CHECK(0 == index, "the index is error");
+    if (isMax) Math::MaxPooling2dGrad(*in[0], *iGradient, *output, *outputGradient, covered, filterHeight, filterWidth, strideY, strideX);
+    else Math::AvgPooling2dGrad(*in[0], *iGradient, *output, *outputGradient, covered, filterHeight, filterWidth, strideY, strideX);
 }
 
 }  // namespace Deep8

@@ -777,6 +777,44 @@ TEST_GPU(readme_regression_with_sgd_trainer) {
     EXPECT(executor.trainableParameters().size() == 1);
 }
 
+TEST_GPU(pooling_nodes_against_host_loops) {
+    EagerExecutor executor;
+    const size_t B = 2, H = 6, W = 6, C = 3;
+    Variable &x = parameter(&executor, B, {H, W, C});
+    std::vector<float> hx(B * H * W * C);
+    for (size_t i = 0; i < hx.size(); ++i) hx[i] = (float)((i * 37 + 11) % 101) - 50.f;  // distinct within any window
+    x.feed(hx.data());
+    Variable &mx = x.maxPooling2d(false, 2, 2, 2, 2);
+    Variable &av = x.avgPooling2d(false, 2, 2, 2, 2);
+    EXPECT(mx.shape() == Shape(B, {3, 3, C}) && av.shape() == Shape(B, {3, 3, C}));
+    std::vector<float> gm(B * 9 * C), ga(B * 9 * C);
+    mx.fetch(gm.data());
+    av.fetch(ga.data());
+    auto at = [&](size_t b, size_t h, size_t w, size_t c) { return hx[((b * H + h) * W + w) * C + c]; };
+    for (size_t b = 0; b < B; ++b)
+        for (size_t oh = 0; oh < 3; ++oh)
+            for (size_t ow = 0; ow < 3; ++ow)
+                for (size_t c = 0; c < C; ++c) {
+                    const float v[4] = {at(b, 2 * oh, 2 * ow, c), at(b, 2 * oh, 2 * ow + 1, c), at(b, 2 * oh + 1, 2 * ow, c), at(b, 2 * oh + 1, 2 * ow + 1, c)};
+                    const float m = std::max(std::max(v[0], v[1]), std::max(v[2], v[3]));
+                    const size_t o = ((b * 3 + oh) * 3 + ow) * C + c;
+                    EXPECT(gm[o] == m);
+                    EXPECT(std::fabs(ga[o] - (v[0] + v[1] + v[2] + v[3]) * 0.25f) <= 1e-5f);
+                }
+    Variable &loss = (mx + av).l1NormLoss();  // both pooling gradients flow into x
+    backward(loss);
+    std::vector<float> gx(hx.size());
+    gpu().copyFromGPUToCPU(x.gradient.raw(), gx.data(), gx.size() * 4);
+    float total = 0;
+    for (float g : gx) total += g;
+    EXPECT(std::isfinite(total) && total != 0.f);
+    std::vector<Shape> bad = {Shape(1, {3, 3})};
+    std::vector<Node *> in = {&x};
+    MaxPooling2d node(in, false, 2, 2, 2, 2);
+    EXPECT(throws<std::invalid_argument>([&] { node.checkShape(bad); }));
+    EXPECT(Math::Pooling2dShape(Shape(1, {7, 7, 4}), true, 3, 3, 2, 2) == Shape(1, {4, 4, 4}));
+}
+
 TEST_GPU(readme_cpp_demo_with_adam_trainer) {
     // The C++ demo of the reference's README, statement for statement (printing dropped).
     float x[4] = {4, -1, 2, 1};

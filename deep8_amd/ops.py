@@ -433,3 +433,46 @@ def adam_update(value, gradient, m, v, beta1, beta2, epsilon, learning_rate, wei
     check(lib.d8_adam_update(dt, dev[0].ptr, dev[1].ptr, dev[2].ptr, dev[3].ptr, beta1, beta2, epsilon, learning_rate,
                              weight_decay, steps, arrs[0].size, None))
     return tuple(d.numpy() for d in dev)
+
+
+# ---- MaxPooling2d / AvgPooling2d ------------------------------------------------------------------
+def _pool(kind, x, FH, FW, covered, sy, sx):
+    lib = capi.init()
+    x = np.ascontiguousarray(x)
+    B, IH, IW, C = x.shape
+    OH, OW, _, _ = conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, 1, 1)
+    dx_, dy_ = DeviceArray.from_numpy(x), DeviceArray((B, OH, OW, C), x.dtype)
+    fn = lib.d8_maxpool2d if kind == "max" else lib.d8_avgpool2d
+    check(fn(capi.dtype_id(x.dtype), dx_.ptr, dy_.ptr, B, IH, IW, C, FH, FW, int(covered), sy, sx, None))
+    return dy_.numpy()
+
+
+def maxpool2d(x, FH, FW, covered=False, sy=1, sx=1):
+    return _pool("max", x, FH, FW, covered, sy, sx)
+
+
+def avgpool2d(x, FH, FW, covered=False, sy=1, sx=1):
+    return _pool("avg", x, FH, FW, covered, sy, sx)
+
+
+def maxpool2d_grad(x, dy, FH, FW, covered=False, sy=1, sx=1, dx=None):
+    """returns dx + the gradient of maxpool2d at x"""
+    lib = capi.init()
+    x, dy = np.ascontiguousarray(x), np.ascontiguousarray(dy)
+    dt = _same_dtype(x, dy)
+    dx = np.zeros_like(x) if dx is None else np.ascontiguousarray(dx)
+    B, IH, IW, C = x.shape
+    a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
+    check(lib.d8_maxpool2d_grad(dt, a.ptr, b.ptr, c.ptr, B, IH, IW, C, FH, FW, int(covered), sy, sx, None))
+    return b.numpy()
+
+
+def avgpool2d_grad(xshape, dy, FH, FW, covered=False, sy=1, sx=1, dx=None):
+    lib = capi.init()
+    dy = np.ascontiguousarray(dy)
+    dx = np.zeros(xshape, dy.dtype) if dx is None else np.ascontiguousarray(dx)
+    dt = _same_dtype(dx, dy)
+    B, IH, IW, C = dx.shape
+    b, c = DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
+    check(lib.d8_avgpool2d_grad(dt, b.ptr, c.ptr, B, IH, IW, C, FH, FW, int(covered), sy, sx, None))
+    return b.numpy()

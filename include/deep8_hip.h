@@ -263,6 +263,26 @@ int d8_axpby(int dtype, const void *x, float alpha, const void *y, float beta, v
 int d8_adam_update(int dtype, void *value, void *gradient, void *m, void *v, float beta1, float beta2,
                    float epsilon, float learning_rate, float weight_decay, long steps, long n, void *stream);
 
+/* ---- MaxPooling2d / AvgPooling2d --------------------------------------------------------------
+ * x [B][IH][IW][C], y [B][OH][OW][C]; (OH, OW, padTop, padLeft) = d8_conv2d_geometry(IH, IW, FH, FW,
+ * covered, sy, sx, 1, 1).  Semantics are those of Deep8's CPU path: the forward window is cut from
+ * the zero-padded image (zeros take part in the maximum and in the mean, which divides by FH * FW);
+ * the max gradient goes to the first maximum of the window clipped to the image; gradients are
+ * added into dx.
+ * d8_maxpool2d / _grad  Math::MaxPooling2dGPU / MaxPooling2dGradGPU (deep8/include/math/MaxPooling2d.h,
+ *                       deep8/src/math/MaxPooling2d.cu:41-147 -- a cuDNN call there; checks and CPU
+ *                       semantics deep8/src/math/MaxPooling2d.cpp:6-251)
+ * d8_avgpool2d / _grad  Math::AvgPooling2dGPU / AvgPooling2dGradGPU (deep8/include/math/AvgPooling2d.h,
+ *                       deep8/src/math/AvgPooling2d.cu; CPU semantics AvgPooling2d.cpp:99-245)          */
+int d8_maxpool2d(int dtype, const void *x, void *y, int B, int IH, int IW, int C,
+                 int FH, int FW, int covered, int sy, int sx, void *stream);
+int d8_maxpool2d_grad(int dtype, const void *x, void *dx, const void *dy, int B, int IH, int IW, int C,
+                      int FH, int FW, int covered, int sy, int sx, void *stream);
+int d8_avgpool2d(int dtype, const void *x, void *y, int B, int IH, int IW, int C,
+                 int FH, int FW, int covered, int sy, int sx, void *stream);
+int d8_avgpool2d_grad(int dtype, void *dx, const void *dy, int B, int IH, int IW, int C,
+                      int FH, int FW, int covered, int sy, int sx, void *stream);
+
 /* ---- measurement aid (no counterpart in the reference) ---------------------------------------
  * d8_mfma_stream issues the tiled GEMM's MFMA instruction back to back on operands taken from
  * `operands` (any device buffer; 16-byte aligned) and held in registers: two waves per SIMD on

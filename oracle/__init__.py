@@ -325,6 +325,21 @@ class _Port:
         self.lib.orc_axpby(_p(x), ctypes.c_float(alpha), _p(y), ctypes.c_float(beta), _p(z), ctypes.c_long(x.size))
         return z
 
+    def pool2d(self, is_max, x, FH, FW, covered=False, sy=1, sx=1):
+        x = _c(x)
+        B, IH, IW, C = x.shape
+        OH, OW, _, _ = self.conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, 1, 1)
+        y = np.zeros((B, OH, OW, C), np.float32)
+        self.lib.orc_pool2d(_i(int(is_max)), _p(x), _p(y), B, IH, IW, C, FH, FW, int(covered), sy, sx)
+        return y
+
+    def pool2d_grad(self, is_max, x, dy, FH, FW, covered=False, sy=1, sx=1, dx=None):
+        x, dy = _c(x), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        B, IH, IW, C = x.shape
+        self.lib.orc_pool2d_grad(_i(int(is_max)), _p(x), _p(dx), _p(dy), B, IH, IW, C, FH, FW, int(covered), sy, sx)
+        return dx
+
     def adam_update(self, value, gradient, m, v, beta1, beta2, epsilon, learning_rate, weight_decay, steps):
         a = [_c(t).copy() for t in (value, gradient, m, v)]
         cf = ctypes.c_float
@@ -523,6 +538,24 @@ class _Ref:
         z = np.zeros_like(x)
         self._chk(self.lib.ref_axpby(_p(x), ctypes.c_float(alpha), _p(y), ctypes.c_float(beta), _p(z), *_nd(x)))
         return z
+
+    def pool2d(self, is_max, x, FH, FW, covered=False, sy=1, sx=1):
+        x = _c(x)
+        B, IH, IW, C = x.shape
+        OH, OW, _, _ = port.conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, 1, 1)
+        y = np.zeros((B, OH, OW, C), np.float32)
+        self._chk(self.lib.ref_pool2d(_i(int(is_max)), _p(x), _p(y), B, IH, IW, C, OH, OW, FH, FW, int(covered), sy, sx))
+        return y
+
+    def pool2d_grad(self, is_max, x, dy, FH, FW, covered=False, sy=1, sx=1, dx=None):
+        x, dy = _c(x), _c(dy)
+        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        B, IH, IW, C = x.shape
+        _, OH, OW, _ = dy.shape
+        y = np.zeros_like(dy)
+        self._chk(self.lib.ref_pool2d_grad(_i(int(is_max)), _p(x), _p(dx), _p(y), _p(dy), B, IH, IW, C, OH, OW, FH, FW,
+                                           int(covered), sy, sx))
+        return dx
 
     def adam_update(self, value, gradient, m, v, beta1, beta2, epsilon, learning_rate, weight_decay, steps):
         a = [_c(t).copy() for t in (value, gradient, m, v)]

@@ -215,6 +215,80 @@ void orc_adam_update(float *value, float *gradient, float *m, float *v, float be
     }
 }
 
+/* ---- MaxPooling2d / AvgPooling2d ----------------------------------------------------------------
+ * Forward: deep8/src/math/MaxPooling2d.cpp:99-142 and AvgPooling2d.cpp:99-142 -- patches of the image
+ * padded with zeros (pad = max(0, (O-1)s + F - I), top = pad / 2), reduced with maximum / mean over
+ * the FH x FW positions.  Gradients: MaxPooling2d.cpp:199-251 (first maximum of the window clipped
+ * to the image, strict >) and AvgPooling2d.cpp:199-245 (ratio = 1 / (FH FW) to every in-image
+ * element).  Pins: torch max_pool2d / avg_pool2d (+ autograd) for windows inside the image, a
+ * zero-padded copy for the others, the live reference build and the golden fixtures. */
+static void pool_geo(int IH, int IW, int FH, int FW, int covered, int sy, int sx, int *OH, int *OW, int *pt, int *pl) {
+    if (!covered) {
+        *OH = (IH - FH) / sy + 1;
+        *OW = (IW - FW) / sx + 1;
+    } else {
+        *OH = (IH - 1) / sy + 1;
+        *OW = (IW - 1) / sx + 1;
+    }
+    int py = (*OH - 1) * sy + FH - IH, px = (*OW - 1) * sx + FW - IW;
+    *pt = (py > 0 ? py : 0) / 2;
+    *pl = (px > 0 ? px : 0) / 2;
+}
+
+void orc_pool2d(int is_max, const float *x, float *y, int B, int IH, int IW, int C, int FH, int FW, int covered, int sy, int sx) {
+    int OH, OW, pt, pl;
+    pool_geo(IH, IW, FH, FW, covered, sy, sx, &OH, &OW, &pt, &pl);
+    for (int b = 0; b < B; ++b)
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow)
+                for (int c = 0; c < C; ++c) {
+                    double acc = 0;
+                    float mx = 0;
+                    int first = 1;
+                    for (int fh = 0; fh < FH; ++fh)
+                        for (int fw = 0; fw < FW; ++fw) {
+                            const int ih = oh * sy + fh - pt, iw = ow * sx + fw - pl;
+                            const float v = (ih >= 0 && ih < IH && iw >= 0 && iw < IW) ? x[(((size_t)b * IH + ih) * IW + iw) * C + c] : 0.f;
+                            acc += v;
+                            if (first || v > mx) mx = v;
+                            first = 0;
+                        }
+                    y[(((size_t)b * OH + oh) * OW + ow) * C + c] = is_max ? mx : (float)(acc / ((double)FH * FW));
+                }
+}
+
+void orc_pool2d_grad(int is_max, const float *x, float *dx, const float *dy, int B, int IH, int IW, int C, int FH, int FW,
+                     int covered, int sy, int sx) {
+    int OH, OW, pt, pl;
+    pool_geo(IH, IW, FH, FW, covered, sy, sx, &OH, &OW, &pt, &pl);
+    const float ratio = 1.0f / ((float)FH * (float)FW);
+    for (int b = 0; b < B; ++b)
+        for (int c = 0; c < C; ++c)
+            for (int oh = 0; oh < OH; ++oh)
+                for (int ow = 0; ow < OW; ++ow) {
+                    int h0 = oh * sy - pt, h1 = h0 + FH, w0 = ow * sx - pl, w1 = w0 + FW;
+                    if (h0 < 0) h0 = 0;
+                    if (h1 > IH) h1 = IH;
+                    if (w0 < 0) w0 = 0;
+                    if (w1 > IW) w1 = IW;
+                    if (h0 >= h1 || w0 >= w1) continue;
+                    const float g = dy[(((size_t)b * OH + oh) * OW + ow) * C + c];
+                    if (!is_max) {
+                        for (int h = h0; h < h1; ++h)
+                            for (int w = w0; w < w1; ++w) dx[(((size_t)b * IH + h) * IW + w) * C + c] += ratio * g;
+                        continue;
+                    }
+                    int mh = h0, mw = w0;
+                    float mv = x[(((size_t)b * IH + h0) * IW + w0) * C + c];
+                    for (int h = h0; h < h1; ++h)
+                        for (int w = w0; w < w1; ++w) {
+                            const float v = x[(((size_t)b * IH + h) * IW + w) * C + c];
+                            if (v > mv) mv = v, mh = h, mw = w;
+                        }
+                    dx[(((size_t)b * IH + mh) * IW + mw) * C + c] += g;
+                }
+}
+
 int orc_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

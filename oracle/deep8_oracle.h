@@ -93,6 +93,10 @@ void orc_l2norm_grad(const float *x, float *dx, const float *y, const float *dy,
 void orc_reduce_mean(const float *x, const int *xd, float *y, const int *yd);
 void orc_reduce_mean_grad(float *dx, const int *xd, const float *dy, const int *yd);
 void orc_axpby(const float *x, float alpha, const float *y, float beta, float *z, long n);
+/* MaxPooling2d (is_max) / AvgPooling2d on NHWC images; gradients are added into dx */
+void orc_pool2d(int is_max, const float *x, float *y, int B, int IH, int IW, int C, int FH, int FW, int covered, int sy, int sx);
+void orc_pool2d_grad(int is_max, const float *x, float *dx, const float *dy, int B, int IH, int IW, int C, int FH, int FW,
+                     int covered, int sy, int sx);
 void orc_adam_update(float *value, float *gradient, float *m, float *v, float beta1, float beta2, float epsilon,
                      float learning_rate, float weight_decay, long steps, long n);
 

@@ -16,6 +16,8 @@
  *   Math::ReduceMean / ReduceMeanGrad         deep8/src/math/ReduceMean.cpp:7-121
  *   Math::AXPBY                               deep8/src/math/AXPBY.cpp:6-20
  *   Math::AdamUpdate                          deep8/src/math/AdamUpdate.cpp:6-23
+ *   Math::MaxPooling2d / MaxPooling2dGrad     deep8/src/math/MaxPooling2d.cpp:6-96
+ *   Math::AvgPooling2d / AvgPooling2dGrad     deep8/src/math/AvgPooling2d.cpp
  *
  * plus one materialisation of the patch expression the CPU Conv2d contracts over
  * (deep8/src/math/Conv2d.cpp:352-356), which is the "CPU Eigen im2col" the HIP im2col must
@@ -37,6 +39,8 @@
 #include "math/ReduceMean.h"
 #include "math/AXPBY.h"
 #include "math/AdamUpdate.h"
+#include "math/MaxPooling2d.h"
+#include "math/AvgPooling2d.h"
 
 #include <chrono>
 #include <cstring>
@@ -423,6 +427,30 @@ int ref_adam_update(float *value, float *gradient, float *m, float *v, float bet
         wrap(M, m, b, vdims(nd, d));
         wrap(V, v, b, vdims(nd, d));
         Math::AdamUpdate(*X.t, *G.t, *M.t, *V.t, beta1, beta2, epsilon, learningRate, weightDecay, (int64_t)steps);
+    });
+}
+
+int ref_pool2d(int is_max, const float *x, float *y, int B, int IH, int IW, int C, int OH, int OW, int FH, int FW,
+               int covered, int sy, int sx) {
+    return guarded([&] {
+        Wrapped X, Y;
+        wrap(X, x, B, {(size_t)IH, (size_t)IW, (size_t)C});
+        wrap(Y, y, B, {(size_t)OH, (size_t)OW, (size_t)C});
+        if (is_max) Math::MaxPooling2d(*X.t, *Y.t, covered != 0, FH, FW, sy, sx);
+        else Math::AvgPooling2d(*X.t, *Y.t, covered != 0, FH, FW, sy, sx);
+    });
+}
+
+int ref_pool2d_grad(int is_max, const float *x, float *dx, const float *y, const float *dy, int B, int IH, int IW, int C,
+                    int OH, int OW, int FH, int FW, int covered, int sy, int sx) {
+    return guarded([&] {
+        Wrapped X, DX, Y, DY;
+        wrap(X, x, B, {(size_t)IH, (size_t)IW, (size_t)C});
+        wrap(DX, dx, B, {(size_t)IH, (size_t)IW, (size_t)C});
+        wrap(Y, y, B, {(size_t)OH, (size_t)OW, (size_t)C});
+        wrap(DY, dy, B, {(size_t)OH, (size_t)OW, (size_t)C});
+        if (is_max) Math::MaxPooling2dGrad(*X.t, *DX.t, *Y.t, *DY.t, covered != 0, FH, FW, sy, sx);
+        else Math::AvgPooling2dGrad(*X.t, *DX.t, *Y.t, *DY.t, covered != 0, FH, FW, sy, sx);
     });
 }
 

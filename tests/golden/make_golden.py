@@ -4,7 +4,7 @@
 Run in the build container, where oracle/_ref/libdeep8_ref.so has been compiled from the reference
 sources (`make -C oracle ref`):   python tests/golden/make_golden.py
 Every array is float32.  Case names: mm<i>_*, conv<i>_*, deconv<i>_*, patch<i>_*, loss<i>_* (Minus,
-L1Norm, L2Norm, ReduceMean, AXPBY), adam<i>_* (AdamUpdate); the geometry of case i is stored in <kind><i>_cfg.
+L1Norm, L2Norm, ReduceMean, AXPBY), adam<i>_* (AdamUpdate), pool<i>_* (MaxPooling2d / AvgPooling2d); the geometry of case i is stored in <kind><i>_cfg.
 """
 import os
 import sys
@@ -26,6 +26,8 @@ DECONV = [(2, 4, 4, 3, 2, 4, 4, 0, 3, 3), (2, 4, 4, 3, 2, 4, 4, 1, 3, 3), (1, 5,
           (1, 5, 5, 2, 3, 4, 4, 1, 2, 2), (1, 4, 5, 2, 2, 3, 3, 0, 1, 1)]
 LOSS = [((3, 7), (3, 7), ()), ((2, 5, 6), (1, 6), (0,)), ((4, 3, 2, 5), (4, 1, 1, 5), (1, 3)), ((1, 33), (1, 1), (-1,)),
         ((2, 3, 4, 5, 6), (1, 3, 1, 5, 1), (0, 2, 4)), ((5, 64), (5, 64), (0,))]
+POOL = [(2, 8, 8, 3, 2, 2, 0, 2, 2), (1, 9, 9, 4, 3, 3, 0, 2, 2), (2, 7, 7, 2, 3, 3, 1, 2, 2), (1, 6, 6, 5, 3, 3, 1, 1, 1),
+        (1, 10, 10, 2, 4, 4, 1, 3, 3)]
 
 
 def main():
@@ -97,6 +99,17 @@ def main():
             out["adam%d_grad%d" % (i, step)] = g
             st = list(ref.adam_update(st[0], g, st[2], st[3], 0.9, 0.999, 1e-7, 0.01, 0.001, step))
             out["adam%d_step%d" % (i, step)] = np.stack(st)  # value, gradient (with the decay term), m, v
+    # MaxPooling2d / AvgPooling2d: B, IH, IW, C, FH, FW, covered, sy, sx
+    for i, c in enumerate(POOL):
+        B, IH, IW, C, FH, FW, cov, sy, sx = c
+        x = u((B, IH, IW, C))
+        a = (FH, FW, bool(cov), sy, sx)
+        ymax, yavg = ref.pool2d(True, x, *a), ref.pool2d(False, x, *a)
+        dy, dx0 = u(ymax.shape), u(x.shape)
+        out.update({"pool%d_cfg" % i: np.array(c, np.int32), "pool%d_x" % i: x, "pool%d_max" % i: ymax, "pool%d_avg" % i: yavg,
+                    "pool%d_dy" % i: dy, "pool%d_dx0" % i: dx0,
+                    "pool%d_max_gx" % i: ref.pool2d_grad(True, x, dy, *a, dx=dx0),
+                    "pool%d_avg_gx" % i: ref.pool2d_grad(False, x, dy, *a, dx=dx0)})
     path = os.path.join(HERE, "deep8_cpu_reference.npz")
     np.savez_compressed(path, **out)
     print("wrote %s (%d arrays, %d bytes)" % (path, len(out), os.path.getsize(path)))

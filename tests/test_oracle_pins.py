@@ -465,3 +465,79 @@ def test_adam_update_against_textbook_and_reference(oracle_port, oracle_ref):
         got = oracle_port.adam_update(x, g, m, v, b1, b2, 1e-7, lr, 0.001, 3)
         for k in range(4):
             assert rel_fro(got[k], want[k]) <= 1e-6
+
+
+# ---- MaxPooling2d / AvgPooling2d ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("i", _n("pool"))
+def test_pooling_against_golden(oracle_port, i):
+    g = lambda k: GOLD["pool%d_%s" % (i, k)]
+    B, IH, IW, C, FH, FW, cov, sy, sx = (int(v) for v in g("cfg"))
+    a = (FH, FW, bool(cov), sy, sx)
+    assert np.array_equal(oracle_port.pool2d(True, g("x"), *a), g("max"))
+    assert rel_fro(oracle_port.pool2d(False, g("x"), *a), g("avg")) <= TOL
+    assert np.array_equal(oracle_port.pool2d_grad(True, g("x"), g("dy"), *a, dx=g("dx0")), g("max_gx"))
+    assert rel_fro(oracle_port.pool2d_grad(False, g("x"), g("dy"), *a, dx=g("dx0")), g("avg_gx")) <= TOL
+
+
+@pytest.mark.parametrize("cfg", [(2, 8, 8, 3, 2, 2, 2, 2), (1, 9, 9, 4, 3, 3, 2, 2), (2, 12, 10, 5, 3, 2, 1, 2), (1, 7, 7, 2, 7, 7, 1, 1)])
+def test_pooling_inside_the_image_against_torch(oracle_port, cfg):
+    """Windows that stay inside the image (covered = false): torch's max_pool2d / avg_pool2d and their
+    autograd gradients (distinct values, so the maximum is unique)."""
+    import torch
+    import torch.nn.functional as F
+    B, IH, IW, C, FH, FW, sy, sx = cfg
+    r = rng(sum(cfg))
+    x = r.permutation(B * IH * IW * C).astype(np.float32).reshape(B, IH, IW, C) - 100.0
+    for is_max in (True, False):
+        xt = torch.tensor(x).permute(0, 3, 1, 2).clone().requires_grad_(True)
+        yt = F.max_pool2d(xt, (FH, FW), (sy, sx)) if is_max else F.avg_pool2d(xt, (FH, FW), (sy, sx))
+        y = oracle_port.pool2d(is_max, x, FH, FW, False, sy, sx)
+        assert rel_fro(y, yt.detach().permute(0, 2, 3, 1).numpy()) <= 1e-6
+        dy = nrm(r, y.shape)
+        yt.backward(torch.tensor(dy).permute(0, 3, 1, 2))
+        want = xt.grad.permute(0, 2, 3, 1).numpy()
+        assert rel_fro(oracle_port.pool2d_grad(is_max, x, dy, FH, FW, False, sy, sx), want) <= 1e-6
+
+
+@pytest.mark.parametrize("cfg", [(2, 7, 7, 2, 3, 3, 2, 2), (1, 6, 6, 3, 3, 3, 1, 1), (1, 10, 10, 2, 4, 4, 3, 3), (1, 5, 5, 1, 2, 2, 2, 2)])
+def test_pooling_with_padding_against_padded_copy_and_reference(oracle_port, oracle_ref, cfg):
+    """covered = true: the forward pass equals pooling (inside the image) of a zero-padded copy -- so a
+    window of negative values that touches the border yields 0 -- while the max gradient ignores the
+    padding; ties go to the first element in scan order."""
+    B, IH, IW, C, FH, FW, sy, sx = cfg
+    r = rng(sum(cfg) + 1)
+    x = -np.abs(nrm(r, (B, IH, IW, C))) - 0.5  # all negative: padding zeros win every border window
+    OH, OW, pt, pl = oracle_port.conv2d_geometry(IH, IW, FH, FW, True, sy, sx, 1, 1)
+    py, px = max(0, (OH - 1) * sy + FH - IH), max(0, (OW - 1) * sx + FW - IW)
+    xp = np.zeros((B, IH + py, IW + px, C), np.float32)
+    xp[:, pt:pt + IH, pl:pl + IW] = x
+    for is_max in (True, False):
+        y = oracle_port.pool2d(is_max, x, FH, FW, True, sy, sx)
+        assert np.array_equal(y, oracle_port.pool2d(is_max, xp, FH, FW, False, sy, sx)[:, :OH, :OW])
+        if is_max and (py or px):
+            assert (y[:, -1] == 0).all()
+    # gradient: brute force over windows with numpy argmax on the clipped window
+    dy = ints(r, (B, OH, OW, C), 9) + 1
+    want = np.zeros_like(x)
+    wavg = np.zeros_like(x)
+    for b in range(B):
+        for oh in range(OH):
+            for ow in range(OW):
+                h0, h1 = max(0, oh * sy - pt), min(IH, oh * sy - pt + FH)
+                w0, w1 = max(0, ow * sx - pl), min(IW, ow * sx - pl + FW)
+                for c in range(C):
+                    win = x[b, h0:h1, w0:w1, c]
+                    k = int(np.argmax(win))  # first maximum in row-major order
+                    want[b, h0 + k // (w1 - w0), w0 + k % (w1 - w0), c] += dy[b, oh, ow, c]
+                    wavg[b, h0:h1, w0:w1, c] += dy[b, oh, ow, c] / np.float32(FH * FW)
+    assert np.array_equal(oracle_port.pool2d_grad(True, x, dy, FH, FW, True, sy, sx), want)
+    assert rel_fro(oracle_port.pool2d_grad(False, x, dy, FH, FW, True, sy, sx), wavg) <= 1e-6
+    # ties: a constant image sends every window's gradient to its first in-image element
+    k = np.ones((1, 4, 4, 1), np.float32)
+    g = oracle_port.pool2d_grad(True, k, np.ones((1, 2, 2, 1), np.float32), 2, 2, False, 2, 2)
+    assert np.array_equal(g[0, :, :, 0], np.array([[1, 0, 1, 0], [0, 0, 0, 0], [1, 0, 1, 0], [0, 0, 0, 0]], np.float32))
+    if oracle_ref is not None:
+        for is_max in (True, False):
+            assert rel_fro(oracle_ref.pool2d(is_max, x, FH, FW, True, sy, sx), oracle_port.pool2d(is_max, x, FH, FW, True, sy, sx)) <= 1e-6
+            assert rel_fro(oracle_ref.pool2d_grad(is_max, x, dy, FH, FW, True, sy, sx),
+                           oracle_port.pool2d_grad(is_max, x, dy, FH, FW, True, sy, sx)) <= 1e-6
