@@ -308,6 +308,32 @@ class BiasReluWorkload:
         check(L.d8_add_grad(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
 
 
+class PoolWorkload:
+    """MaxPooling2d 2x2 / 2 forward and gradient on config 4's activations.  HBM-bound gathers."""
+
+    def __init__(self, name, dtype, B, H, W, C, seed):
+        from deep8_amd import capi
+        self.name, self.dtype, self.key = name, np.dtype(dtype), name.split(":")[0]
+        self.lib = capi.init()
+        self.dt = capi.dtype_id(self.dtype)
+        r = np.random.default_rng(seed)
+        self.B, self.dims = B, (B, H, W, C)
+        self.x = _dev(r.standard_normal((B, H, W, C)).astype(np.float32).astype(dtype))
+        self.y = capi.DeviceArray((B, H // 2, W // 2, C), dtype)
+        self.gy = _dev(r.standard_normal((B, H // 2, W // 2, C)).astype(np.float32).astype(dtype))
+        self.gx = capi.DeviceArray((B, H, W, C), dtype)
+        n, es = B * H * W * C, self.dtype.itemsize
+        self.flops = 2.0 * n
+        # forward: r x, w y | fill gx | gradient: r x, r gy, rw gx
+        self.bytes = es * (n + n // 4 + n + n + n // 4 + 2 * n)
+
+    def step(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_maxpool2d(self.dt, self.x.ptr, self.y.ptr, *self.dims, 2, 2, 0, 2, 2, None))
+        self.gx.zero_()
+        check(self.lib.d8_maxpool2d_grad(self.dt, self.x.ptr, self.gx.ptr, self.gy.ptr, *self.dims, 2, 2, 0, 2, 2, None))
+
+
 def _uni(r, s):
     return r.uniform(-1, 1, s).astype(np.float32)
 
@@ -343,6 +369,8 @@ def make_workload(key):
                             np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
     if key == "e4":
         return BiasReluWorkload("e4: bias Add + ReLu fwd+bwd on config 4's output, fp32 B32 56x56x64", np.float32, 32, 56, 56, 64, 7)
+    if key == "p4":
+        return PoolWorkload("p4: MaxPooling2d 2x2/2 fwd+bwd on config 4's output, fp32 B32 56x56x64", np.float32, 32, 56, 56, 64, 8)
     raise SystemExit("unknown workload %r" % key)
 
 
@@ -489,7 +517,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5", "e4"):
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5", "e4", "p4"):
             if key == a.workload:
                 continue
             del wl
@@ -497,7 +525,7 @@ def main():
             oms = _time_steps(wl.step, 5, 2)
             o = {"ms_per_step": round(oms, 4), "tflops": round(wl.flops / (oms * 1e-3) / 1e12, 2),
                  "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
-            if isinstance(wl, (ConvWorkload, BiasReluWorkload)):
+            if isinstance(wl, (ConvWorkload, BiasReluWorkload, PoolWorkload)):
                 o["images_per_s"] = round(wl.B / (oms * 1e-3), 1)
             others[key] = o
         out["others"] = others
