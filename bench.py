@@ -36,8 +36,8 @@ EAGER_ZERO = False
 
 MEASURED_TRAFFIC = {
     "c3": int((192.2 + 224.2 + 224.2) / 3 * 2**20 + 32.0 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
-    "c4": int((26.5 + 24.5) * 2**20),                                # Conv2d forward kernel: fetch + write
-    "c5": int((17.6 + 24.5) * 2**20),                                # DeConv2d forward GEMM: fetch + write
+    "c4": int((2 * 14.1 + 2 * 13.0 + 2.0 + 0.5) * 2**20),            # Conv2d forward: tile launches (rows cut in two) fetch + write, + the band's split reduction
+    "c5": int((16.8 + 24.5) * 2**20),                                # DeConv2d forward GEMM: fetch + write
 }
 
 
@@ -246,8 +246,10 @@ class ConvWorkload:
 
     def gemm_roofline(self, reps):
         """The pass-forward GEMM launch, timed alone with HIP events, against the MFMA peak of its
-        element type.  Conv2d forward is ONE launch of the tiled kernel (its tile loader reads the
-        patch matrix straight from the image); DeConv2d forward's GEMM (one product per filter tap,
+        element type.  Conv2d forward runs the tiled kernel (its tile loader reads the patch matrix
+        straight from the image) over the rows that fill whole rounds of the chip, then over the
+        remaining band of rows with the reduction split, then the band's reduction: all three are
+        inside the timed call; DeConv2d forward's GEMM (one product per filter tap,
         a single batched launch) is issued here through d8_gemm with the operator's own arguments."""
         from deep8_amd import capi
         B, IH, IW, IC = self.xd
@@ -263,7 +265,7 @@ class ConvWorkload:
             name = "gemm_tiled_kernel<%s> (DeConv2d forward: %d per-tap products [%dx%d]x[%dx%d]^T, one launch)" % (dtype, T, M, IC, OC, IC)
         else:
             fn = self.fwd
-            name = "gemm_tiled_kernel<%s> (Conv2d forward, patch matrix read by the tile loader, one launch)" % dtype
+            name = "gemm_tiled_kernel<%s> (Conv2d forward, patch matrix read by the tile loader: whole rounds + split remainder band + its reduction, timed together)" % dtype
         ms = _time_events(fn, reps)
         ach = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "kernel": name, "achieved": round(ach, 2), "peak": PEAK[dtype], "unit": "TFLOP/s",
