@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libdeep8_hip.so")
 
 FLOAT16 = 10
 FLOAT32 = 11
+FLOAT64 = 12
 
 c_int, c_long, c_size_t, c_float, c_void_p = (ctypes.c_int, ctypes.c_long, ctypes.c_size_t, ctypes.c_float,
                                               ctypes.c_void_p)
@@ -140,6 +141,8 @@ def dtype_id(np_dtype):
         return FLOAT32
     if np_dtype == np.float16:
         return FLOAT16
+    if np_dtype == np.float64:  # the contraction path only; every other entry point rejects it
+        return FLOAT64
     raise Deep8HipError("type %s is not support" % np_dtype)
 
 

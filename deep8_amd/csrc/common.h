@@ -38,7 +38,7 @@ int fail(int code, const char *fmt, ...);
 
 inline hipStream_t as_stream(void *s) { return (hipStream_t)s; }
 
-inline size_t dtype_bytes(int dtype) { return dtype == D8_FLOAT16 ? 2 : (dtype == D8_FLOAT32 ? 4 : 0); }
+inline size_t dtype_bytes(int dtype) { return dtype == D8_FLOAT16 ? 2 : (dtype == D8_FLOAT32 ? 4 : (dtype == D8_FLOAT64 ? 8 : 0)); }
 
 // After a kernel launch: surface launch-configuration errors immediately.
 #define D8_LAUNCH_CHECK() D8_HIP(hipGetLastError())

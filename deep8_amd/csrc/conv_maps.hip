@@ -17,6 +17,16 @@ static inline int grid_for(long work, int block) {
 }
 
 // ---- im2col: pure copy, V is the raw vector moved per thread (bit-exact) -------------------
+// Sums are carried in fp32 for half and float images, in fp64 for double ones.
+template <typename T>
+struct Wide {
+    typedef float type;
+};
+template <>
+struct Wide<double> {
+    typedef double type;
+};
+
 template <typename V>
 __global__ __launch_bounds__(256) void im2col_kernel(const V *__restrict__ im, V *__restrict__ col,
                                                      MapGeom g, int CV, long total) {
@@ -57,13 +67,14 @@ __global__ __launch_bounds__(256) void col2im_kernel(const T *__restrict__ col, 
         const long q = p / g.IW;
         const int iy = (int)(q % g.IH), b = (int)(q / g.IH);
         T *dst = im + p * g.C + (long)cv * VEC;
-        float acc[VEC];
+        typedef typename Wide<T>::type W;
+        W acc[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+        for (int e = 0; e < VEC; ++e) acc[e] = 0;
         if (ACC) {
             VT v = *(const VT *)dst;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) acc[e] = (float)v[e];
+            for (int e = 0; e < VEC; ++e) acc[e] = (W)v[e];
         }
         for (int fy = 0; fy < g.FH; ++fy) {
             const int ty = iy + g.pt - fy * g.dy;
@@ -78,7 +89,7 @@ __global__ __launch_bounds__(256) void col2im_kernel(const T *__restrict__ col, 
                 const VT v = *(const VT *)(col + (((long)b * g.OH + oy) * g.OW + ox) * K +
                                            (long)(fy * g.FW + fx) * g.C + (long)cv * VEC);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) acc[e] += (float)v[e];
+                for (int e = 0; e < VEC; ++e) acc[e] += (W)v[e];
             }
         }
         VT o;
@@ -99,7 +110,8 @@ __global__ __launch_bounds__(256) void col2im_scalar_kernel(const T *__restrict_
         const int ix = (int)(p % g.IW);
         const long q = p / g.IW;
         const int iy = (int)(q % g.IH), b = (int)(q / g.IH);
-        float acc = ACC ? (float)im[idx] : 0.f;
+        typedef typename Wide<T>::type W;
+        W acc = ACC ? (W)im[idx] : (W)0;
         for (int fy = 0; fy < g.FH; ++fy) {
             const int ty = iy + g.pt - fy * g.dy;
             if (ty < 0 || ty % g.sy) continue;
@@ -110,7 +122,7 @@ __global__ __launch_bounds__(256) void col2im_scalar_kernel(const T *__restrict_
                 if (tx < 0 || tx % g.sx) continue;
                 const int ox = tx / g.sx;
                 if (ox >= g.OW) continue;
-                acc += (float)col[(((long)b * g.OH + oy) * g.OW + ox) * K + (long)(fy * g.FW + fx) * g.C + c];
+                acc += (W)col[(((long)b * g.OH + oy) * g.OW + ox) * K + (long)(fy * g.FW + fx) * g.C + c];
             }
         }
         im[idx] = (T)acc;
@@ -131,7 +143,8 @@ __global__ __launch_bounds__(256) void deconv_col2im_kernel(const T *__restrict_
         const int ox = (int)(p % g.OW);
         const long q = p / g.OW;
         const int oy = (int)(q % g.OH), b = (int)(q / g.OH);
-        float acc = 0.f;
+        typedef typename Wide<T>::type W;
+        W acc = 0;
         for (int fy = 0; fy < g.FH; ++fy) {
             const int ty = oy - g.pt + fy;
             if (ty < 0 || ty % g.sy) continue;
@@ -142,7 +155,7 @@ __global__ __launch_bounds__(256) void deconv_col2im_kernel(const T *__restrict_
                 if (tx < 0 || tx % g.sx) continue;
                 const int ix = tx / g.sx;
                 if (ix >= g.IW) continue;
-                acc += (float)zmat[(((long)b * g.IH + iy) * g.IW + ix) * N + (long)oc * taps + fy * g.FW + fx];
+                acc += (W)zmat[(((long)b * g.IH + iy) * g.IW + ix) * N + (long)oc * taps + fy * g.FW + fx];
             }
         }
         z[idx] = (T)acc;
@@ -174,7 +187,7 @@ __global__ __launch_bounds__(256) void deconv_im2col_kernel(const T *__restrict_
 }
 
 static int check_geom(const char *who, int dtype, const void *a, const void *b, const MapGeom &g) {
-    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
     D8_REQUIRE(g.B >= 0 && g.IH > 0 && g.IW > 0 && g.C > 0 && g.OH > 0 && g.OW > 0 && g.FH > 0 && g.FW > 0,
                "%s: sizes must be positive", who);
@@ -196,6 +209,9 @@ int launch_im2col(int dtype, const void *im, void *col, const MapGeom &g, hipStr
         const long total = elems / (16 / es);
         hipLaunchKernelGGL((im2col_kernel<uint4>), dim3(grid_for(total, 256)), dim3(256), 0, s,
                            (const uint4 *)im, (uint4 *)col, g, CV, total);
+    } else if (es == 8) {
+        hipLaunchKernelGGL((im2col_kernel<unsigned long long>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned long long *)im, (unsigned long long *)col, g, g.C, elems);
     } else if (es == 4) {
         hipLaunchKernelGGL((im2col_kernel<unsigned>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
                            (const unsigned *)im, (unsigned *)col, g, g.C, elems);
@@ -221,7 +237,10 @@ int launch_col2im(int dtype, const void *col, void *im, const MapGeom &g, bool a
     if (g.B == 0) return 0;
     const long elems = (long)g.B * g.IH * g.IW * g.C;
     const bool al = aligned16(im) && aligned16(col);
-    if (dtype == D8_FLOAT32) {
+    if (dtype == D8_FLOAT64) {
+        if (accumulate) launch_col2im_t<double, 2, true>(col, im, g, g.C % 2 == 0 && al, elems, s);
+        else launch_col2im_t<double, 2, false>(col, im, g, g.C % 2 == 0 && al, elems, s);
+    } else if (dtype == D8_FLOAT32) {
         if (accumulate) launch_col2im_t<float, 4, true>(col, im, g, g.C % 4 == 0 && al, elems, s);
         else launch_col2im_t<float, 4, false>(col, im, g, g.C % 4 == 0 && al, elems, s);
     } else {
@@ -262,7 +281,10 @@ int d8_deconv_col2im(int dtype, const void *zmat, void *z,
     if (B == 0) return 0;
     const long elems = (long)B * OH * OW * OC;
     hipStream_t s = as_stream(stream);
-    if (dtype == D8_FLOAT32)
+    if (dtype == D8_FLOAT64)
+        hipLaunchKernelGGL((deconv_col2im_kernel<double>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const double *)zmat, (double *)z, g, elems);
+    else if (dtype == D8_FLOAT32)
         hipLaunchKernelGGL((deconv_col2im_kernel<float>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
                            (const float *)zmat, (float *)z, g, elems);
     else
@@ -280,7 +302,10 @@ int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
     if (B == 0) return 0;
     const long elems = (long)B * IH * IW * OC * FH * FW;
     hipStream_t s = as_stream(stream);
-    if (dtype == D8_FLOAT32)
+    if (dtype == D8_FLOAT64)
+        hipLaunchKernelGGL((deconv_im2col_kernel<unsigned long long>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
+                           (const unsigned long long *)dz, (unsigned long long *)dzmat, g, elems);
+    else if (dtype == D8_FLOAT32)
         hipLaunchKernelGGL((deconv_im2col_kernel<unsigned>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
                            (const unsigned *)dz, (unsigned *)dzmat, g, elems);
     else

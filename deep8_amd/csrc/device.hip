@@ -125,14 +125,16 @@ int d8_memset(void *ptr, int value, size_t bytes, void *stream) {
 }
 
 int d8_fill(int dtype, void *ptr, size_t n, float scalar, void *stream) {
-    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "d8_fill: element type %d is not supported", dtype);
     if (!n) return 0;
     D8_REQUIRE(ptr, "d8_fill: ptr is null");
     if (scalar == 0.f) return d8_memset(ptr, 0, n * dtype_bytes(dtype), stream);
     int blocks = (int)((n + 255) / 256);
     if (blocks > 8192) blocks = 8192;
-    if (dtype == D8_FLOAT32)
+    if (dtype == D8_FLOAT64)
+        hipLaunchKernelGGL((fill_kernel<double>), dim3(blocks), dim3(256), 0, as_stream(stream), (double *)ptr, (double)scalar, n);
+    else if (dtype == D8_FLOAT32)
         hipLaunchKernelGGL((fill_kernel<float>), dim3(blocks), dim3(256), 0, as_stream(stream), (float *)ptr, scalar, n);
     else
         hipLaunchKernelGGL((fill_kernel<f16>), dim3(blocks), dim3(256), 0, as_stream(stream), (f16 *)ptr, (f16)scalar, n);

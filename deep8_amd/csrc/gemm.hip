@@ -335,7 +335,7 @@ size_t d8_gemm_workspace_bytes(int dtype, int transA, int transB, int M, int N, 
                                int batch, long strideC) {
     (void)transA;
     (void)transB;
-    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || dtype == D8_FLOAT64) return 0;
     const int red = (strideC == 0 && batch > 1) ? batch : 1;
     const int outs = red > 1 ? 1 : batch;
     // whichever kernel ends up running, the larger of the two plans fits
@@ -351,7 +351,7 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
             const void *B, int ldb, long strideB,
             float beta, void *C, int ldc, long strideC, int batch,
             void *workspace, size_t workspace_bytes, void *stream) {
-    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "d8_gemm: element type %d is not supported", dtype);
     D8_REQUIRE(!(transA && transB), "d8_gemm: transA and transB together are not supported");
     D8_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "d8_gemm: negative size");
@@ -386,6 +386,7 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     g.virt = VIRT_NONE;
     g.m_base = 0;
     memset(&g.pg, 0, sizeof(g.pg));
+    if (dtype == D8_FLOAT64) return gemm_f64_launch(g, transA, transB, as_stream(stream));
     const bool tiled = K > 0 && gemm_tiled_eligible(dtype, g, transA, transB);
     if (K > 0) {  // K == 0 is the empty reduction: C = beta * C
         const int BK = tiled ? gemm_tiled_k_step(dtype) : (dtype == D8_FLOAT16 ? Tile<f16>::BK : Tile<float>::BK);

@@ -56,6 +56,9 @@ int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipS
 bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB);
 int gemm_wide_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);
 
+// fp64 kernel (64 x 64 tiles, v_mfma_f64_16x16x4_f64): any shape, reduction never split.
+int gemm_f64_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);
+
 // Whether an unsplit product of this shape should run on 64 x 128 tiles: too few 128 x 128 tiles
 // for the chip, enough half-height ones, and a reduction (k_steps K steps in all) too short to
 // be worth splitting.

@@ -535,6 +535,7 @@ static int launch_any(const GemmArgs &g, int transA, int transB, hipStream_t str
 int gemm_tiled_k_step(int dtype) { return dtype == D8_FLOAT16 ? 64 : 32; }
 
 bool gemm_tiled_eligible(int dtype, const GemmArgs &g, int transA, int transB) {
+    if (dtype == D8_FLOAT64) return false;
     return dtype == D8_FLOAT16 ? eligible<f16>(g, transA, transB) : eligible<float>(g, transA, transB);
 }
 

@@ -37,7 +37,7 @@ static int run(int dtype, const Gemm &g, void *ws, size_t ws_bytes, void *stream
 }
 
 static int check_mm(const char *who, int dtype, int xb, int xr, int xc, int yb, int yr, int yc) {
-    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
     D8_REQUIRE(xb > 0 && xr > 0 && xc > 0 && yb > 0 && yr > 0 && yc > 0, "%s: sizes must be positive", who);
     D8_REQUIRE(xb == yb || xb == 1 || yb == 1, "%s: batch %d vs %d", who, xb, yb);
@@ -70,7 +70,7 @@ static Gemm mm_plan(int which, const void *x, int xb, int xr, int xc, const void
 
 static int check_conv(const char *who, int dtype, int B, int IH, int IW, int IC, int OC, int FH, int FW,
                       int sy, int sx, int dy, int dx) {
-    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
     D8_REQUIRE(B > 0 && IH > 0 && IW > 0 && IC > 0 && OC > 0 && FH > 0 && FW > 0, "%s: sizes must be positive", who);
     D8_REQUIRE(sy >= 1 && sx >= 1 && dy >= 1 && dx >= 1, "%s: the stride and dilation must >= 1", who);

@@ -192,6 +192,7 @@ public:
     GPUMemoryPool *memoryPool;
     int deviceId;
 
+    double *oneDouble;
     float *oneFloat, *zeroFloat, *minusOneFloat;
     half *oneHalf, *zeroHalf, *minusOneHalf;
 

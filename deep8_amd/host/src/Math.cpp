@@ -11,6 +11,7 @@ namespace {
 
 int dtypeOf(const Tensor &t) {
     switch (t.elementType.id) {
+    case DType::Float64: return D8_FLOAT64;  // MatrixMultiply, Conv2d, DeConv2d and Constant only
     case DType::Float32: return D8_FLOAT32;
     case DType::Float16: return D8_FLOAT16;
     default: DEEP8_RUNTIME_ERROR("type " << t.elementType.name << " is not support");

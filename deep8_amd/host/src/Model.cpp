@@ -263,9 +263,10 @@ GPUDevice::GPUDevice(int id, size_t poolBlockSize) : Device(DeviceType::GPU), me
     D8_CHECK(d8_device_init(deviceId));
     memoryPool = new GPUMemoryPool(deviceId, poolBlockSize);
 
-    // {1, 0, -1} in float and half, one pool allocation (the reference keeps the same constants)
-    void *ptr = memoryPool->malloc(sizeof(float) * 3 + sizeof(half) * 3);
-    oneFloat = (float *)ptr;
+    // {1, 0, -1} in double, float and half, one pool allocation (the reference keeps the same constants)
+    void *ptr = memoryPool->malloc(sizeof(double) * 3 + sizeof(float) * 3 + sizeof(half) * 3);
+    oneDouble = (double *)ptr;
+    oneFloat = (float *)(oneDouble + 3);
     zeroFloat = oneFloat + 1;
     minusOneFloat = zeroFloat + 1;
     oneHalf = (half *)(minusOneFloat + 1);
@@ -273,13 +274,15 @@ GPUDevice::GPUDevice(int id, size_t poolBlockSize) : Device(DeviceType::GPU), me
     minusOneHalf = zeroHalf + 1;
     const float numberF[3] = {1.f, 0.f, -1.f};
     const half numberH[3] = {half(1.f), half(0.f), half(-1.f)};
+    const double numberD[3] = {1., 0., -1.};
+    memoryPool->copyFromCPUToGPU(numberD, oneDouble, sizeof(numberD));
     memoryPool->copyFromCPUToGPU(numberF, oneFloat, sizeof(numberF));
     memoryPool->copyFromCPUToGPU(numberH, oneHalf, sizeof(numberH));
 }
 
 GPUDevice::~GPUDevice() {
     d8_stream_sync(nullptr);
-    memoryPool->free(oneFloat);
+    memoryPool->free(oneDouble);
     delete memoryPool;
 }
 
@@ -297,7 +300,7 @@ void GPUDevice::copyFromGPUToCPU(const void *from, void *to, size_t size) { memo
 void GPUDevice::copyFromGPUToGPU(const void *from, void *to, size_t size) { memoryPool->copyFromGPUToGPU(from, to, size); }
 void *GPUDevice::gpuOneHalf() { return oneHalf; }
 void *GPUDevice::gpuOneFloat() { return oneFloat; }
-void *GPUDevice::gpuOneDouble() { DEEP8_RUNTIME_ERROR("type float64 is not support"); }
+void *GPUDevice::gpuOneDouble() { return oneDouble; }
 void GPUDevice::synchronize() { D8_CHECK(d8_stream_sync(nullptr)); }
 
 void GPUDevice::zeroLater(void *ptr, size_t size) { pendingZero[ptr] = size; }
@@ -364,6 +367,7 @@ void Tensor::one() {
     DEEP8_ARGUMENT_CHECK(isScalar(), "the tensor is not a scalar");
     Device *dev = device();
     switch (elementType.id) {
+    case DType::Float64: dev->copyFromGPUToGPU(dev->gpuOneDouble(), raw(), elementType.byteWidth); break;
     case DType::Float32: dev->copyFromGPUToGPU(dev->gpuOneFloat(), raw(), elementType.byteWidth); break;
     case DType::Float16: dev->copyFromGPUToGPU(dev->gpuOneHalf(), raw(), elementType.byteWidth); break;
     default: DEEP8_RUNTIME_ERROR("the type is not support");
@@ -377,7 +381,8 @@ std::string Tensor::valueStr() {
     out << "[";
     for (size_t i = 0; i < size(); ++i) {
         if (i) out << ", ";
-        if (elementType.id == DType::Float32) out << ((float *)host.data())[i];
+        if (elementType.id == DType::Float64) out << ((double *)host.data())[i];
+        else if (elementType.id == DType::Float32) out << ((float *)host.data())[i];
         else if (elementType.id == DType::Float16) out << (float)((half *)host.data())[i];
         else DEEP8_RUNTIME_ERROR("the type is not support");
     }

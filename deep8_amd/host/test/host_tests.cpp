@@ -88,6 +88,9 @@ Tensor makeTensor(GPUDevice &dev, ElementType type, size_t batch, std::vector<si
 void upload(HostTensor &h) {
     if (h.t.elementType.id == DType::Float32) {
         h.t.device()->copyFromCPUToGPU(h.host.data(), h.t.raw(), h.t.byteCount());
+    } else if (h.t.elementType.id == DType::Float64) {
+        std::vector<double> tmp(h.host.begin(), h.host.end());
+        h.t.device()->copyFromCPUToGPU(tmp.data(), h.t.raw(), h.t.byteCount());
     } else {
         std::vector<half> tmp(h.host.begin(), h.host.end());
         h.t.device()->copyFromCPUToGPU(tmp.data(), h.t.raw(), h.t.byteCount());
@@ -97,6 +100,10 @@ void upload(HostTensor &h) {
 void download(HostTensor &h) {
     if (h.t.elementType.id == DType::Float32) {
         h.t.device()->copyFromGPUToCPU(h.t.raw(), h.host.data(), h.t.byteCount());
+    } else if (h.t.elementType.id == DType::Float64) {
+        std::vector<double> tmp(h.host.size());
+        h.t.device()->copyFromGPUToCPU(h.t.raw(), tmp.data(), h.t.byteCount());
+        for (size_t i = 0; i < tmp.size(); ++i) h.host[i] = (float)tmp[i];
     } else {
         std::vector<half> tmp(h.host.size());
         h.t.device()->copyFromGPUToCPU(h.t.raw(), tmp.data(), h.t.byteCount());
@@ -302,6 +309,18 @@ TEST_GPU(matrix_multiply_half) {
     matmulCase(ElementType::from<half>(), 3, {24, 16}, 3, {16, 8}, 3);
 }
 
+TEST_GPU(matrix_multiply_double) {  // the reference's Float64 branch (MatrixMultiply.cu:142-175)
+    matmulCase(ElementType::from<double>(), 10, {40, 20}, 1, {20, 30}, 50);
+    matmulCase(ElementType::from<double>(), 1, {30, 10}, 10, {10}, 50);
+    matmulCase(ElementType::from<double>(), 6, {33, 17}, 6, {17, 29}, 50);
+    matmulCase(ElementType::from<double>(), 1, {33, 17}, 6, {17, 29}, 50);
+    Tensor s = makeTensor(gpu(), ElementType::from<double>(), 1, {1});
+    s.one();
+    double one = 0;
+    gpu().copyFromGPUToCPU(s.raw(), &one, 8);
+    EXPECT(one == 1.0);
+}
+
 TEST_GPU(matrix_multiply_errors) {
     ElementType f32 = ElementType::from<float>();
     HostTensor x = randomTensor(f32, 1, {4, 5}, 5), y = randomTensor(f32, 1, {5, 6}, 5);
@@ -311,7 +330,7 @@ TEST_GPU(matrix_multiply_errors) {
     EXPECT(throws<std::invalid_argument>([&] { Math::MatrixMultiply(x.t, y.t, zh.t); }));
     EXPECT(throws<std::invalid_argument>([&] { Math::MatrixMultiplyGradX(x.t, bad.t, y.t, z.t, z.t); }));
     Tensor d64 = makeTensor(gpu(), ElementType::from<double>(), 1, {4, 4});
-    EXPECT(throws<std::runtime_error>([&] { Math::MatrixMultiply(d64, d64, d64); }));
+    EXPECT(throws<std::runtime_error>([&] { Math::ReLu(d64, d64); }));  // Float64 exists on the contraction path only
     Variable v0 = placeholder(f32);
     std::vector<Node *> one = {&v0};
     EXPECT(throws<std::invalid_argument>([&] { MatrixMultiply mm(one); }));
@@ -377,6 +396,7 @@ TEST_GPU(conv2d_float_covered_stride_dilation) {  // Conv2dTest forwardCPU_float
 }
 TEST_GPU(conv2d_float_covered_5x5) { convCase(ElementType::from<float>(), 2, 12, 12, 4, 4, 5, 5, true, 1, 1, 1, 1, 20); }
 TEST_GPU(conv2d_float_not_covered) { convCase(ElementType::from<float>(), 2, 13, 11, 5, 3, 3, 3, false, 1, 1, 1, 1, 20); }
+TEST_GPU(conv2d_double) { convCase(ElementType::from<double>(), 2, 13, 11, 5, 3, 3, 3, true, 2, 2, 1, 1, 20); }
 TEST_GPU(conv2d_half) { convCase(ElementType::from<half>(), 2, 8, 8, 8, 8, 3, 3, true, 1, 1, 1, 1, 2); }
 
 // ---- DeConv2d -----------------------------------------------------------------------------------------------------
@@ -432,6 +452,7 @@ void deconvCase(ElementType type, int B, int IH, int IW, int IC, int OC, int FH,
 TEST_GPU(deconv2d_float_not_covered_stride3) { deconvCase(ElementType::from<float>(), 2, 8, 8, 8, 4, 4, 4, false, 3, 3, 20); }
 TEST_GPU(deconv2d_float_covered_stride3) { deconvCase(ElementType::from<float>(), 2, 8, 8, 8, 4, 4, 4, true, 3, 3, 20); }
 TEST_GPU(deconv2d_float_stride2) { deconvCase(ElementType::from<float>(), 2, 7, 6, 4, 6, 4, 4, false, 2, 2, 20); }
+TEST_GPU(deconv2d_double) { deconvCase(ElementType::from<double>(), 2, 7, 6, 4, 6, 4, 4, false, 2, 2, 20); }
 TEST_GPU(deconv2d_half) { deconvCase(ElementType::from<half>(), 2, 6, 6, 8, 8, 4, 4, false, 2, 2, 2); }
 
 TEST_GPU(conv2d_errors) {

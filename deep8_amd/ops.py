@@ -3,7 +3,8 @@
 Every function copies its operands to the GPU, calls one entry point of libdeep8_hip.so and copies
 the result back.  Tensors follow Deep8's layout: first axis = Shape::batch, then Shape::dims
 (matrix: (batch, rows[, cols]); image: (B, H, W, C); filter: (OC, FH, FW, IC)).
-float32 and float16 arrays are accepted; all operands of one call must share the dtype.
+float32 and float16 arrays are accepted (float64 too by gemm, the gather maps, matmul*, conv2d* and
+deconv2d*); all operands of one call must share the dtype.
 """
 import ctypes
 

@@ -23,6 +23,7 @@ extern "C" {
 /* element types: the ids of Deep8's DType (deep8/include/model/ElementType.h:8-22) */
 #define D8_FLOAT16 10
 #define D8_FLOAT32 11
+#define D8_FLOAT64 12 /* the contraction path only: d8_fill, d8_gemm, the four gather maps, d8_matmul*, d8_conv2d*, d8_deconv2d* */
 
 #define D8_ERR_ARGUMENT 10001 /* bad shape / leading dimension / null pointer */
 #define D8_ERR_DTYPE    10002 /* element type not supported by this build     */

@@ -14,6 +14,7 @@ axes are ``Shape::dims`` (deep8/include/model/Shape.h:32-83): a matrix operand i
 or ``(batch, rows, cols)``, an image ``(B, H, W, C)``, a filter ``(1, OC, FH, FW, IC)`` or
 ``(OC, FH, FW, IC)``.
 """
+import contextlib
 import ctypes
 import os
 import subprocess
@@ -103,6 +104,39 @@ def _filt(w):
     return w
 
 
+# The working precision of the MatrixMultiply / gemm / Conv2d / DeConv2d checkers: float32, or
+# float64 inside ``with oracle.float64():`` (every other checker is float32 only).
+_WORK = [np.float32]
+
+
+def _cw(a):
+    return np.ascontiguousarray(a, dtype=_WORK[0])
+
+
+def _filtw(w):
+    w = _cw(w)
+    if w.ndim == 5:
+        assert w.shape[0] == 1
+        w = w[0]
+    return w
+
+
+@contextlib.contextmanager
+def float64():
+    """Inside the block, port.* and ref.* matmul / gemm / conv2d / deconv2d (and their gradients)
+    take and return float64: the port's double twins (orc_*_f64) and the reference's own double
+    path (deep8/src/math/MatrixMultiply.cpp:119-131 and the Float64 cases of Conv2d.cpp / DeConv2d.cpp)."""
+    _WORK[0] = np.float64
+    if ref is not None:
+        ref.lib.ref_set_double(1)
+    try:
+        yield
+    finally:
+        _WORK[0] = np.float32
+        if ref is not None:
+            ref.lib.ref_set_double(0)
+
+
 class _Port:
     name = "port"
 
@@ -113,37 +147,40 @@ class _Port:
     def threads(self):
         return self.lib.orc_threads()
 
+    def _f(self, name):
+        return getattr(self.lib, name + ("_f64" if _WORK[0] is np.float64 else ""))
+
     # -- MatrixMultiply ------------------------------------------------------------------
     def matmul(self, x, y):
-        x, y = _c(x), _c(y)
-        z = np.zeros(matmul_out_shape(x, y), np.float32)
+        x, y = _cw(x), _cw(y)
+        z = np.zeros(matmul_out_shape(x, y), _WORK[0])
         xb, _, xr, xc = _mat(x)
         yb, _, yr, yc = _mat(y)
-        self.lib.orc_matmul(_p(x), _i(xb), _i(xr), _i(xc), _p(y), _i(yb), _i(yr), _i(yc), _p(z))
+        self._f("orc_matmul")(_p(x), _i(xb), _i(xr), _i(xc), _p(y), _i(yb), _i(yr), _i(yc), _p(z))
         return z
 
     def matmul_grad_x(self, x, y, dz, dx=None):
-        x, y, dz = _c(x), _c(y), _c(dz)
-        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        x, y, dz = _cw(x), _cw(y), _cw(dz)
+        dx = np.zeros_like(x) if dx is None else _cw(dx).copy()
         xb, _, xr, xc = _mat(x)
         yb, _, yr, yc = _mat(y)
-        self.lib.orc_matmul_grad_x(_p(dx), _i(xb), _i(xr), _i(xc), _p(y), _i(yb), _i(yr), _i(yc), _p(dz))
+        self._f("orc_matmul_grad_x")(_p(dx), _i(xb), _i(xr), _i(xc), _p(y), _i(yb), _i(yr), _i(yc), _p(dz))
         return dx
 
     def matmul_grad_y(self, x, y, dz, dy=None):
-        x, y, dz = _c(x), _c(y), _c(dz)
-        dy = np.zeros_like(y) if dy is None else _c(dy).copy()
+        x, y, dz = _cw(x), _cw(y), _cw(dz)
+        dy = np.zeros_like(y) if dy is None else _cw(dy).copy()
         xb, _, xr, xc = _mat(x)
         yb, _, yr, yc = _mat(y)
-        self.lib.orc_matmul_grad_y(_p(x), _i(xb), _i(xr), _i(xc), _p(dy), _i(yb), _i(yr), _i(yc), _p(dz))
+        self._f("orc_matmul_grad_y")(_p(x), _i(xb), _i(xr), _i(xc), _p(dy), _i(yb), _i(yr), _i(yc), _p(dz))
         return dy
 
     def gemm(self, ta, tb, A, B, C=None, beta=0.0):
-        A, B = _c(A), _c(B)
+        A, B = _cw(A), _cw(B)
         M, K = (A.shape[1], A.shape[0]) if ta else A.shape
         N = B.shape[0] if tb else B.shape[1]
-        C = np.zeros((M, N), np.float32) if C is None else _c(C).copy()
-        self.lib.orc_gemm(_i(ta), _i(tb), _i(M), _i(N), _i(K), _p(A), _i(A.shape[1]), _p(B), _i(B.shape[1]),
+        C = np.zeros((M, N), _WORK[0]) if C is None else _cw(C).copy()
+        self._f("orc_gemm")(_i(ta), _i(tb), _i(M), _i(N), _i(K), _p(A), _i(A.shape[1]), _p(B), _i(B.shape[1]),
                           ctypes.c_float(beta), _p(C), _i(N))
         return C
 
@@ -160,54 +197,54 @@ class _Port:
 
     # -- Conv2d ----------------------------------------------------------------------------
     def conv2d(self, x, w, covered=True, sy=1, sx=1, dy=1, dx=1):
-        x, w = _c(x), _filt(w)
+        x, w = _cw(x), _filtw(w)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         OH, OW, _, _ = self.conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx)
-        z = np.zeros((B, OH, OW, OC), np.float32)
-        self.lib.orc_conv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), int(covered), sy, sx, dy, dx)
+        z = np.zeros((B, OH, OW, OC), _WORK[0])
+        self._f("orc_conv2d")(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), int(covered), sy, sx, dy, dx)
         return z
 
     def conv2d_grad_x(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
-        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
-        self.lib.orc_conv2d_grad_x(_p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(gz), int(covered), sy, sx, dy, dx)
+        gx = np.zeros_like(x) if gx is None else _cw(gx).copy()
+        self._f("orc_conv2d_grad_x")(_p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(gz), int(covered), sy, sx, dy, dx)
         return gx
 
     def conv2d_grad_y(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
-        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
-        self.lib.orc_conv2d_grad_y(_p(x), B, IH, IW, IC, _p(gw), OC, FH, FW, _p(gz), int(covered), sy, sx, dy, dx)
+        gw = np.zeros_like(w) if gw is None else _filtw(gw).copy()
+        self._f("orc_conv2d_grad_y")(_p(x), B, IH, IW, IC, _p(gw), OC, FH, FW, _p(gz), int(covered), sy, sx, dy, dx)
         return gw
 
     # -- DeConv2d --------------------------------------------------------------------------
     def deconv2d(self, x, w, covered=False, sy=1, sx=1):
-        x, w = _c(x), _filt(w)
+        x, w = _cw(x), _filtw(w)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         OH, OW, _, _ = self.deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx)
-        z = np.zeros((B, OH, OW, OC), np.float32)
-        self.lib.orc_deconv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), int(covered), sy, sx)
+        z = np.zeros((B, OH, OW, OC), _WORK[0])
+        self._f("orc_deconv2d")(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), int(covered), sy, sx)
         return z
 
     def deconv2d_grad_x(self, x, w, gz, covered=False, sy=1, sx=1, gx=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
-        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
-        self.lib.orc_deconv2d_grad_x(_p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(gz), int(covered), sy, sx)
+        gx = np.zeros_like(x) if gx is None else _cw(gx).copy()
+        self._f("orc_deconv2d_grad_x")(_p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(gz), int(covered), sy, sx)
         return gx
 
     def deconv2d_grad_y(self, x, w, gz, covered=False, sy=1, sx=1, gw=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
-        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
-        self.lib.orc_deconv2d_grad_y(_p(x), B, IH, IW, IC, _p(gw), OC, FH, FW, _p(gz), int(covered), sy, sx)
+        gw = np.zeros_like(w) if gw is None else _filtw(gw).copy()
+        self._f("orc_deconv2d_grad_y")(_p(x), B, IH, IW, IC, _p(gw), OC, FH, FW, _p(gz), int(covered), sy, sx)
         return gw
 
     # -- gather / scatter maps ---------------------------------------------------------------
@@ -349,7 +386,7 @@ class _Port:
 
 
 class _Ref:
-    """Deep8's own CPU path (float only)."""
+    """Deep8's own CPU path (float; double for the contraction path inside ``float64()``)."""
     name = "reference"
 
     def __init__(self, path):
@@ -367,86 +404,86 @@ class _Ref:
             raise RuntimeError(self.lib.ref_last_error().decode())
 
     def matmul(self, x, y, z_shape=None):
-        x, y = _c(x), _c(y)
-        z = np.zeros(matmul_out_shape(x, y) if z_shape is None else z_shape, np.float32)
+        x, y = _cw(x), _cw(y)
+        z = np.zeros(matmul_out_shape(x, y) if z_shape is None else z_shape, _WORK[0])
         self._chk(self.lib.ref_matmul(_p(x), *map(_i, _mat(x)), _p(y), *map(_i, _mat(y)), _p(z), *map(_i, _mat(z))))
         return z
 
     def matmul_grad_x(self, x, y, dz, dx=None):
-        x, y, dz = _c(x), _c(y), _c(dz)
-        dx = np.zeros_like(x) if dx is None else _c(dx).copy()
+        x, y, dz = _cw(x), _cw(y), _cw(dz)
+        dx = np.zeros_like(x) if dx is None else _cw(dx).copy()
         z = np.zeros_like(dz)
         self._chk(self.lib.ref_matmul_grad_x(_p(x), _p(dx), *map(_i, _mat(x)), _p(y), *map(_i, _mat(y)),
                                              _p(z), _p(dz), *map(_i, _mat(dz))))
         return dx
 
     def matmul_grad_y(self, x, y, dz, dy=None):
-        x, y, dz = _c(x), _c(y), _c(dz)
-        dy = np.zeros_like(y) if dy is None else _c(dy).copy()
+        x, y, dz = _cw(x), _cw(y), _cw(dz)
+        dy = np.zeros_like(y) if dy is None else _cw(dy).copy()
         z = np.zeros_like(dz)
         self._chk(self.lib.ref_matmul_grad_y(_p(x), *map(_i, _mat(x)), _p(y), _p(dy), *map(_i, _mat(y)),
                                              _p(z), _p(dz), *map(_i, _mat(dz))))
         return dy
 
     def conv2d(self, x, w, covered=True, sy=1, sx=1, dy=1, dx=1, out_hw=None):
-        x, w = _c(x), _filt(w)
+        x, w = _cw(x), _filtw(w)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         OH, OW = out_hw if out_hw else port.conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx)[:2]
-        z = np.zeros((B, OH, OW, OC), np.float32)
+        z = np.zeros((B, OH, OW, OC), _WORK[0])
         self._chk(self.lib.ref_conv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), OH, OW,
                                       int(covered), sy, sx, dy, dx))
         return z
 
     def conv2d_grad_x(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         _, OH, OW, _ = gz.shape
-        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
+        gx = np.zeros_like(x) if gx is None else _cw(gx).copy()
         z = np.zeros_like(gz)
         self._chk(self.lib.ref_conv2d_grad_x(_p(x), _p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), _p(gz),
                                              OH, OW, int(covered), sy, sx, dy, dx))
         return gx
 
     def conv2d_grad_y(self, x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gw=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         _, OH, OW, _ = gz.shape
-        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
+        gw = np.zeros_like(w) if gw is None else _filtw(gw).copy()
         z = np.zeros_like(gz)
         self._chk(self.lib.ref_conv2d_grad_y(_p(x), B, IH, IW, IC, _p(w), _p(gw), OC, FH, FW, _p(z), _p(gz),
                                              OH, OW, int(covered), sy, sx, dy, dx))
         return gw
 
     def deconv2d(self, x, w, covered=False, sy=1, sx=1, out_hw=None):
-        x, w = _c(x), _filt(w)
+        x, w = _cw(x), _filtw(w)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         OH, OW = out_hw if out_hw else port.deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx)[:2]
-        z = np.zeros((B, OH, OW, OC), np.float32)
+        z = np.zeros((B, OH, OW, OC), _WORK[0])
         self._chk(self.lib.ref_deconv2d(_p(x), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), OH, OW,
                                         int(covered), sy, sx))
         return z
 
     def deconv2d_grad_x(self, x, w, gz, covered=False, sy=1, sx=1, gx=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         _, OH, OW, _ = gz.shape
-        gx = np.zeros_like(x) if gx is None else _c(gx).copy()
+        gx = np.zeros_like(x) if gx is None else _cw(gx).copy()
         z = np.zeros_like(gz)
         self._chk(self.lib.ref_deconv2d_grad_x(_p(x), _p(gx), B, IH, IW, IC, _p(w), OC, FH, FW, _p(z), _p(gz),
                                                OH, OW, int(covered), sy, sx))
         return gx
 
     def deconv2d_grad_y(self, x, w, gz, covered=False, sy=1, sx=1, gw=None):
-        x, w, gz = _c(x), _filt(w), _c(gz)
+        x, w, gz = _cw(x), _filtw(w), _cw(gz)
         B, IH, IW, IC = x.shape
         OC, FH, FW, _ = w.shape
         _, OH, OW, _ = gz.shape
-        gw = np.zeros_like(w) if gw is None else _filt(gw).copy()
+        gw = np.zeros_like(w) if gw is None else _filtw(gw).copy()
         z = np.zeros_like(gz)
         self._chk(self.lib.ref_deconv2d_grad_y(_p(x), B, IH, IW, IC, _p(w), _p(gw), OC, FH, FW, _p(z), _p(gz),
                                                OH, OW, int(covered), sy, sx))

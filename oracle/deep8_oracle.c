@@ -300,79 +300,6 @@ int orc_threads(void) {
 static int imax(int a, int b) { return a > b ? a : b; }
 
 /* ---------------------------------------------------------------------------------------- */
-/* C[M,N] = op(A) * op(B) + beta * C; op(A) is M x K.  transA: A stored K x M (lda >= M).    */
-void orc_gemm(int transA, int transB, int M, int N, int K,
-              const float *A, int lda, const float *B, int ldb, float beta, float *C, int ldc) {
-#pragma omp parallel for schedule(static) if ((long)M * N * K > 1000000L)
-    for (int m = 0; m < M; ++m) {
-        for (int n = 0; n < N; ++n) {
-            double acc = 0.0;
-            for (int k = 0; k < K; ++k) {
-                float a = transA ? A[(size_t)k * lda + m] : A[(size_t)m * lda + k];
-                float b = transB ? B[(size_t)n * ldb + k] : B[(size_t)k * ldb + n];
-                acc += (double)a * (double)b;
-            }
-            float *c = C + (size_t)m * ldc + n;
-            *c = (float)(beta != 0.f ? (double)*c + acc : acc);
-        }
-    }
-}
-
-/* deep8/src/math/MatrixMultiply.cpp:94-116 */
-void orc_matmul(const float *x, int xb, int xr, int xc,
-                const float *y, int yb, int yr, int yc, float *z) {
-    int zb = imax(xb, yb);
-    (void)yr;
-    if (1 == yb) {
-        orc_gemm(0, 0, xb * xr, yc, xc, x, xc, y, yc, 0.f, z, yc);
-    } else if (1 == xb && 1 == yc) {
-        /* z[yb x xr] = Y[yb x K] * X^T */
-        orc_gemm(0, 1, yb, xr, xc, y, xc, x, xc, 0.f, z, xr);
-    } else {
-        for (int b = 0; b < zb; ++b) {
-            orc_gemm(0, 0, xr, yc, xc, x + (size_t)(b % xb) * xr * xc, xc,
-                     y + (size_t)(b % yb) * yr * yc, yc, 0.f, z + (size_t)b * xr * yc, yc);
-        }
-    }
-}
-
-/* deep8/src/math/MatrixMultiply.cpp:134-163 */
-void orc_matmul_grad_x(float *dx, int xb, int xr, int xc,
-                       const float *y, int yb, int yr, int yc, const float *dz) {
-    int zb = imax(xb, yb);
-    if (1 == yb) {
-        /* dX[(xb*xr) x xc] += dZ[(xb*xr) x yc] * Y^T */
-        orc_gemm(0, 1, xb * xr, xc, yc, dz, yc, y, yc, 1.f, dx, xc);
-    } else if (1 == xb && 1 == yc) {
-        /* dX[xr x xc] += dZ^T (dZ is [yb x xr]) * Y[yb x xc] */
-        orc_gemm(1, 0, xr, xc, yb, dz, xr, y, xc, 1.f, dx, xc);
-    } else {
-        for (int b = 0; b < zb; ++b) {
-            orc_gemm(0, 1, xr, xc, yc, dz + (size_t)b * xr * yc, yc,
-                     y + (size_t)(b % yb) * yr * yc, yc, 1.f, dx + (size_t)(b % xb) * xr * xc, xc);
-        }
-    }
-}
-
-/* deep8/src/math/MatrixMultiply.cpp:181-210 */
-void orc_matmul_grad_y(const float *x, int xb, int xr, int xc,
-                       float *dy, int yb, int yr, int yc, const float *dz) {
-    int zb = imax(xb, yb);
-    if (1 == yb) {
-        /* dY[yr x yc] += X^T (X is [(xb*xr) x xc]) * dZ[(xb*xr) x yc] */
-        orc_gemm(1, 0, yr, yc, xb * xr, x, xc, dz, yc, 1.f, dy, yc);
-    } else if (1 == xb && 1 == yc) {
-        /* dY[yb x K] += dZ[yb x xr] * X[xr x xc] */
-        orc_gemm(0, 0, yb, xc, xr, dz, xr, x, xc, 1.f, dy, xc);
-    } else {
-        for (int b = 0; b < zb; ++b) {
-            orc_gemm(1, 0, yr, yc, xr, x + (size_t)(b % xb) * xr * xc, xc,
-                     dz + (size_t)b * xr * yc, yc, 1.f, dy + (size_t)(b % yb) * yr * yc, yc);
-        }
-    }
-}
-
-/* ---------------------------------------------------------------------------------------- */
 /* deep8/src/math/Conv2d.cpp:20-32 (output size), :341-350 (padding) */
 void orc_conv2d_geometry(int IH, int IW, int FH, int FW, int covered,
                          int sy, int sx, int dy, int dx, int *out) {
@@ -409,187 +336,17 @@ void orc_deconv2d_geometry(int IH, int IW, int FH, int FW, int covered,
     out[3] = imax(0, OW + FW - (IW - 1) * sx - 2) / 2;
 }
 
-/* z[b,oy,ox,oc] = sum x[b, oy*sy+fy*dy-padTop, ox*sx+fx*dx-padLeft, ic] * w[oc,fy,fx,ic] */
-void orc_conv2d(const float *x, int B, int IH, int IW, int IC,
-                const float *w, int OC, int FH, int FW, float *z,
-                int covered, int sy, int sx, int dy, int dx) {
-    int g[4];
-    orc_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g);
-    int OH = g[0], OW = g[1], pt = g[2], pl = g[3];
-#pragma omp parallel for collapse(2) schedule(static)
-    for (int b = 0; b < B; ++b)
-        for (int oy = 0; oy < OH; ++oy)
-            for (int ox = 0; ox < OW; ++ox)
-                for (int oc = 0; oc < OC; ++oc) {
-                    double acc = 0.0;
-                    for (int fy = 0; fy < FH; ++fy) {
-                        int iy = oy * sy + fy * dy - pt;
-                        if (iy < 0 || iy >= IH) continue;
-                        for (int fx = 0; fx < FW; ++fx) {
-                            int ix = ox * sx + fx * dx - pl;
-                            if (ix < 0 || ix >= IW) continue;
-                            const float *xp = x + (((size_t)b * IH + iy) * IW + ix) * IC;
-                            const float *wp = w + (((size_t)oc * FH + fy) * FW + fx) * IC;
-                            for (int ic = 0; ic < IC; ++ic) acc += (double)xp[ic] * (double)wp[ic];
-                        }
-                    }
-                    z[(((size_t)b * OH + oy) * OW + ox) * OC + oc] = (float)acc;
-                }
-}
-
-/* gx[b,iy,ix,ic] += sum over (oc,fy,fx,oy,ox) hitting (iy,ix) of gz[b,oy,ox,oc] * w[oc,fy,fx,ic] */
-void orc_conv2d_grad_x(float *gx, int B, int IH, int IW, int IC,
-                       const float *w, int OC, int FH, int FW, const float *gz,
-                       int covered, int sy, int sx, int dy, int dx) {
-    int g[4];
-    orc_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g);
-    int OH = g[0], OW = g[1], pt = g[2], pl = g[3];
-#pragma omp parallel for collapse(2) schedule(static)
-    for (int b = 0; b < B; ++b)
-        for (int iy = 0; iy < IH; ++iy)
-            for (int ix = 0; ix < IW; ++ix)
-                for (int ic = 0; ic < IC; ++ic) {
-                    double acc = 0.0;
-                    for (int fy = 0; fy < FH; ++fy) {
-                        int ty = iy + pt - fy * dy;
-                        if (ty < 0 || ty % sy) continue;
-                        int oy = ty / sy;
-                        if (oy >= OH) continue;
-                        for (int fx = 0; fx < FW; ++fx) {
-                            int tx = ix + pl - fx * dx;
-                            if (tx < 0 || tx % sx) continue;
-                            int ox = tx / sx;
-                            if (ox >= OW) continue;
-                            const float *gp = gz + (((size_t)b * OH + oy) * OW + ox) * OC;
-                            for (int oc = 0; oc < OC; ++oc)
-                                acc += (double)gp[oc] *
-                                       (double)w[(((size_t)oc * FH + fy) * FW + fx) * IC + ic];
-                        }
-                    }
-                    float *p = gx + (((size_t)b * IH + iy) * IW + ix) * IC + ic;
-                    *p = (float)((double)*p + acc);
-                }
-}
-
-/* gw[oc,fy,fx,ic] += sum_{b,oy,ox} gz[b,oy,ox,oc] * x[b, oy*sy+fy*dy-padTop, ..., ic] */
-void orc_conv2d_grad_y(const float *x, int B, int IH, int IW, int IC,
-                       float *gw, int OC, int FH, int FW, const float *gz,
-                       int covered, int sy, int sx, int dy, int dx) {
-    int g[4];
-    orc_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g);
-    int OH = g[0], OW = g[1], pt = g[2], pl = g[3];
-#pragma omp parallel for collapse(2) schedule(static)
-    for (int oc = 0; oc < OC; ++oc)
-        for (int fy = 0; fy < FH; ++fy)
-            for (int fx = 0; fx < FW; ++fx)
-                for (int ic = 0; ic < IC; ++ic) {
-                    double acc = 0.0;
-                    for (int b = 0; b < B; ++b)
-                        for (int oy = 0; oy < OH; ++oy) {
-                            int iy = oy * sy + fy * dy - pt;
-                            if (iy < 0 || iy >= IH) continue;
-                            for (int ox = 0; ox < OW; ++ox) {
-                                int ix = ox * sx + fx * dx - pl;
-                                if (ix < 0 || ix >= IW) continue;
-                                acc += (double)gz[(((size_t)b * OH + oy) * OW + ox) * OC + oc] *
-                                       (double)x[(((size_t)b * IH + iy) * IW + ix) * IC + ic];
-                            }
-                        }
-                    float *p = gw + (((size_t)oc * FH + fy) * FW + fx) * IC + ic;
-                    *p = (float)((double)*p + acc);
-                }
-}
-
-/* ---------------------------------------------------------------------------------------- */
-/* z[b,oy,ox,oc] = sum_{fy,fx,ic : iy*sy == oy-padTop+fy} x[b,iy,ix,ic] * w[oc,fy,fx,ic]      */
-void orc_deconv2d(const float *x, int B, int IH, int IW, int IC,
-                  const float *w, int OC, int FH, int FW, float *z,
-                  int covered, int sy, int sx) {
-    int g[4];
-    orc_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g);
-    int OH = g[0], OW = g[1], pt = g[2], pl = g[3];
-#pragma omp parallel for collapse(2) schedule(static)
-    for (int b = 0; b < B; ++b)
-        for (int oy = 0; oy < OH; ++oy)
-            for (int ox = 0; ox < OW; ++ox)
-                for (int oc = 0; oc < OC; ++oc) {
-                    double acc = 0.0;
-                    for (int fy = 0; fy < FH; ++fy) {
-                        int ty = oy - pt + fy;
-                        if (ty < 0 || ty % sy) continue;
-                        int iy = ty / sy;
-                        if (iy >= IH) continue;
-                        for (int fx = 0; fx < FW; ++fx) {
-                            int tx = ox - pl + fx;
-                            if (tx < 0 || tx % sx) continue;
-                            int ix = tx / sx;
-                            if (ix >= IW) continue;
-                            const float *xp = x + (((size_t)b * IH + iy) * IW + ix) * IC;
-                            const float *wp = w + (((size_t)oc * FH + fy) * FW + fx) * IC;
-                            for (int ic = 0; ic < IC; ++ic) acc += (double)xp[ic] * (double)wp[ic];
-                        }
-                    }
-                    z[(((size_t)b * OH + oy) * OW + ox) * OC + oc] = (float)acc;
-                }
-}
-
-/* gx[b,iy,ix,ic] += sum_{oc,fy,fx} gz[b, iy*sy+padTop-fy, ix*sx+padLeft-fx, oc] * w[oc,fy,fx,ic] */
-void orc_deconv2d_grad_x(float *gx, int B, int IH, int IW, int IC,
-                         const float *w, int OC, int FH, int FW, const float *gz,
-                         int covered, int sy, int sx) {
-    int g[4];
-    orc_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g);
-    int OH = g[0], OW = g[1], pt = g[2], pl = g[3];
-#pragma omp parallel for collapse(2) schedule(static)
-    for (int b = 0; b < B; ++b)
-        for (int iy = 0; iy < IH; ++iy)
-            for (int ix = 0; ix < IW; ++ix)
-                for (int ic = 0; ic < IC; ++ic) {
-                    double acc = 0.0;
-                    for (int fy = 0; fy < FH; ++fy) {
-                        int oy = iy * sy + pt - fy;
-                        if (oy < 0 || oy >= OH) continue;
-                        for (int fx = 0; fx < FW; ++fx) {
-                            int ox = ix * sx + pl - fx;
-                            if (ox < 0 || ox >= OW) continue;
-                            const float *gp = gz + (((size_t)b * OH + oy) * OW + ox) * OC;
-                            for (int oc = 0; oc < OC; ++oc)
-                                acc += (double)gp[oc] *
-                                       (double)w[(((size_t)oc * FH + fy) * FW + fx) * IC + ic];
-                        }
-                    }
-                    float *p = gx + (((size_t)b * IH + iy) * IW + ix) * IC + ic;
-                    *p = (float)((double)*p + acc);
-                }
-}
-
-void orc_deconv2d_grad_y(const float *x, int B, int IH, int IW, int IC,
-                         float *gw, int OC, int FH, int FW, const float *gz,
-                         int covered, int sy, int sx) {
-    int g[4];
-    orc_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g);
-    int OH = g[0], OW = g[1], pt = g[2], pl = g[3];
-#pragma omp parallel for collapse(2) schedule(static)
-    for (int oc = 0; oc < OC; ++oc)
-        for (int fy = 0; fy < FH; ++fy)
-            for (int fx = 0; fx < FW; ++fx)
-                for (int ic = 0; ic < IC; ++ic) {
-                    double acc = 0.0;
-                    for (int b = 0; b < B; ++b)
-                        for (int iy = 0; iy < IH; ++iy) {
-                            int oy = iy * sy + pt - fy;
-                            if (oy < 0 || oy >= OH) continue;
-                            for (int ix = 0; ix < IW; ++ix) {
-                                int ox = ix * sx + pl - fx;
-                                if (ox < 0 || ox >= OW) continue;
-                                acc += (double)gz[(((size_t)b * OH + oy) * OW + ox) * OC + oc] *
-                                       (double)x[(((size_t)b * IH + iy) * IW + ix) * IC + ic];
-                            }
-                        }
-                    float *p = gw + (((size_t)oc * FH + fy) * FW + fx) * IC + ic;
-                    *p = (float)((double)*p + acc);
-                }
-}
+/* the contraction path, once per element type */
+#define REAL float
+#define ORC(name) orc_##name
+#include "deep8_oracle_path.inc"
+#undef REAL
+#undef ORC
+#define REAL double
+#define ORC(name) orc_##name##_f64
+#include "deep8_oracle_path.inc"
+#undef REAL
+#undef ORC
 
 /* ---------------------------------------------------------------------------------------- */
 /* deep8/src/math/Conv2d.cu:27-60 (padTop there is stored negated) */

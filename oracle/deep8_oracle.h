@@ -58,6 +58,38 @@ void orc_deconv2d_grad_y(const float *x, int B, int IH, int IW, int IC,
                          float *gw, int OC, int FH, int FW, const float *gz,
                          int covered, int sy, int sx);
 
+/* ---- the same contraction path on double operands (the reference's Float64 cases) ----------- */
+void orc_matmul_f64(const double *x, int xb, int xr, int xc,
+                const double *y, int yb, int yr, int yc, double *z);
+void orc_matmul_grad_x_f64(double *dx, int xb, int xr, int xc,
+                       const double *y, int yb, int yr, int yc, const double *dz);
+void orc_matmul_grad_y_f64(const double *x, int xb, int xr, int xc,
+                       double *dy, int yb, int yr, int yc, const double *dz);
+
+void orc_gemm_f64(int transA, int transB, int M, int N, int K,
+              const double *A, int lda, const double *B, int ldb, float beta, double *C, int ldc);
+
+void orc_conv2d_f64(const double *x, int B, int IH, int IW, int IC,
+                const double *w, int OC, int FH, int FW, double *z,
+                int covered, int sy, int sx, int dy, int dx);
+void orc_conv2d_grad_x_f64(double *gx, int B, int IH, int IW, int IC,
+                       const double *w, int OC, int FH, int FW, const double *gz,
+                       int covered, int sy, int sx, int dy, int dx);
+void orc_conv2d_grad_y_f64(const double *x, int B, int IH, int IW, int IC,
+                       double *gw, int OC, int FH, int FW, const double *gz,
+                       int covered, int sy, int sx, int dy, int dx);
+
+void orc_deconv2d_f64(const double *x, int B, int IH, int IW, int IC,
+                  const double *w, int OC, int FH, int FW, double *z,
+                  int covered, int sy, int sx);
+void orc_deconv2d_grad_x_f64(double *gx, int B, int IH, int IW, int IC,
+                         const double *w, int OC, int FH, int FW, const double *gz,
+                         int covered, int sy, int sx);
+void orc_deconv2d_grad_y_f64(const double *x, int B, int IH, int IW, int IC,
+                         double *gw, int OC, int FH, int FW, const double *gz,
+                         int covered, int sy, int sx);
+
+
 /* ---- the four gather/scatter maps, explicit geometry ---------------------------------------- */
 /* col[(b,oy,ox)][(fy,fx,c)] = im[b, oy*sy + fy*dy - padTop, ox*sx + fx*dx - padLeft, c] or +0 */
 void orc_im2col(const float *im, float *col, int B, int IH, int IW, int C, int OH, int OW,

@@ -66,11 +66,15 @@ struct Wrapped {
     std::unique_ptr<Tensor> t;
 };
 
+/* Element type of every tensor wrapped from now on: float, or double after ref_set_double(1)
+ * (the pointers then address doubles whatever the prototypes below say). */
+bool g_double = false;
+
 void wrap(Wrapped &w, const float *ptr, size_t batch, std::vector<size_t> dims) {
     Shape shape(batch, dims);
-    TensorStorage storage((void *)ptr, &w.ref, sizeof(float) * shape.size(), cpu());
+    TensorStorage storage((void *)ptr, &w.ref, (g_double ? sizeof(double) : sizeof(float)) * shape.size(), cpu());
     w.ref += 1;
-    w.t.reset(new Tensor(storage, 0, shape, ElementType::from<float>()));
+    w.t.reset(new Tensor(storage, 0, shape, g_double ? ElementType::from<double>() : ElementType::from<float>()));
 }
 
 std::vector<size_t> mdims(int nd, int r, int c) {
@@ -101,6 +105,10 @@ struct MM {
 extern "C" {
 
 const char *ref_last_error() { return g_error.c_str(); }
+
+/* Selects the reference's Float64 path for the calls that follow (used for MatrixMultiply, Conv2d
+ * and DeConv2d only). */
+void ref_set_double(int on) { g_double = on != 0; }
 
 /* thread count the reference's CPUDevice gives Eigen (deep8/src/model/Device.cpp:67-85) */
 int ref_threads() { return cpu()->getDeviceThreadNum(); }

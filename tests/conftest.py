@@ -23,6 +23,13 @@ def oracle_port():
 
 
 @pytest.fixture(scope="session")
+def oracle(oracle_port):
+    """The checker package itself (for its float64() switch)."""
+    import oracle
+    return oracle
+
+
+@pytest.fixture(scope="session")
 def oracle_ref():
     import oracle
     if oracle.ref is None:

@@ -193,7 +193,7 @@ def test_gemm_argument_errors():
     a = capi.DeviceArray((16, 16), np.float32, zero=True)
     rc = lib.d8_gemm(capi.FLOAT32, 1, 1, 16, 16, 16, a.ptr, 16, 0, a.ptr, 16, 0, 0.0, a.ptr, 16, 0, 1, None, 0, None)
     assert rc == 10001 and b"transA" in lib.d8_last_error()
-    rc = lib.d8_gemm(12, 0, 0, 16, 16, 16, a.ptr, 16, 0, a.ptr, 16, 0, 0.0, a.ptr, 16, 0, 1, None, 0, None)
+    rc = lib.d8_gemm(9, 0, 0, 16, 16, 16, a.ptr, 16, 0, a.ptr, 16, 0, 0.0, a.ptr, 16, 0, 1, None, 0, None)
     assert rc == 10002
     rc = lib.d8_gemm(capi.FLOAT32, 0, 0, 16, 16, 16, a.ptr, 8, 0, a.ptr, 16, 0, 0.0, a.ptr, 16, 0, 1, None, 0, None)
     assert rc == 10001 and b"lda" in lib.d8_last_error()

@@ -541,3 +541,151 @@ def test_pooling_with_padding_against_padded_copy_and_reference(oracle_port, ora
             assert rel_fro(oracle_ref.pool2d(is_max, x, FH, FW, True, sy, sx), oracle_port.pool2d(is_max, x, FH, FW, True, sy, sx)) <= 1e-6
             assert rel_fro(oracle_ref.pool2d_grad(is_max, x, dy, FH, FW, True, sy, sx),
                            oracle_port.pool2d_grad(is_max, x, dy, FH, FW, True, sy, sx)) <= 1e-6
+
+
+# ---- the double twins of the contraction path (orc_*_f64) ----------------------------------------------------
+# Same loops as the float functions, compiled for double.  Pinned by: the float path on integer inputs
+# (exact in both), numpy / torch in float64 on real inputs, and the reference's own Float64 CPU path live.
+F64_TOL = 1e-13
+
+
+def _torch_conv2d(port, x, w, gz, cfg):
+    import torch
+    F = torch.nn.functional
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    OH, OW, pt, pl = port.conv2d_geometry(IH, IW, FH, FW, cov, sy, sx, dy, dx)
+    rfh, rfw = FH + (FH - 1) * (dy - 1), FW + (FW - 1) * (dx - 1)
+    py, px = max(0, (OH - 1) * sy + rfh - IH), max(0, (OW - 1) * sx + rfw - IW)
+    tx = torch.tensor(x, dtype=torch.float64).permute(0, 3, 1, 2).requires_grad_(True)
+    tw = torch.tensor(w, dtype=torch.float64).permute(0, 3, 1, 2).requires_grad_(True)
+    tz = F.conv2d(F.pad(tx, (pl, px - pl, pt, py - pt)), tw, stride=(sy, sx), dilation=(dy, dx))
+    tz.backward(torch.tensor(gz, dtype=torch.float64).permute(0, 3, 1, 2))
+    return (tz.detach().permute(0, 2, 3, 1).numpy(), tx.grad.permute(0, 2, 3, 1).numpy(), tw.grad.permute(0, 2, 3, 1).numpy())
+
+
+def _torch_deconv2d(port, x, w, gz, cfg):
+    import torch
+    F = torch.nn.functional
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = cfg
+    OH, OW, pt, pl = port.deconv2d_geometry(IH, IW, FH, FW, cov, sy, sx)
+    tx = torch.tensor(x, dtype=torch.float64).permute(0, 3, 1, 2).requires_grad_(True)
+    tw = torch.tensor(w, dtype=torch.float64).requires_grad_(True)
+    full = F.conv_transpose2d(tx, torch.flip(tw, (1, 2)).permute(3, 0, 1, 2), stride=(sy, sx))
+    oy, ox = FH - 1 - pt, FW - 1 - pl
+    tz = full[:, :, oy:oy + OH, ox:ox + OW]
+    tz.backward(torch.tensor(gz, dtype=torch.float64).permute(0, 3, 1, 2))
+    return tz.detach().permute(0, 2, 3, 1).numpy(), tx.grad.permute(0, 2, 3, 1).numpy(), tw.grad.numpy()
+
+
+@pytest.mark.parametrize("xs,ys", MM_SHAPES)
+def test_double_matmul(oracle_port, oracle_ref, oracle, xs, ys):
+    r = rng(40)
+    xi, yi = ints(r, xs), ints(r, ys)
+    zi = oracle_port.matmul(xi, yi)
+    dzi = ints(r, zi.shape)
+    x, y = r.standard_normal(xs), r.standard_normal(ys)
+    x3 = x.reshape(xs[0], xs[1], xs[2] if len(xs) == 3 else 1)
+    y3 = y.reshape(ys[0], ys[1], ys[2] if len(ys) == 3 else 1)
+    zb = max(xs[0], ys[0])
+    X, Y = np.broadcast_to(x3, (zb,) + x3.shape[1:]), np.broadcast_to(y3, (zb,) + y3.shape[1:])
+    want = np.matmul(X, Y)
+    dz = r.standard_normal(zi.shape)
+    DZ = dz.reshape(want.shape)
+    dX, dY = np.matmul(DZ, Y.transpose(0, 2, 1)), np.matmul(X.transpose(0, 2, 1), DZ)
+    dX = dX.sum(0, keepdims=True) if xs[0] == 1 else dX
+    dY = dY.sum(0, keepdims=True) if ys[0] == 1 else dY
+    f32 = (zi, oracle_port.matmul_grad_x(xi, yi, dzi), oracle_port.matmul_grad_y(xi, yi, dzi))
+    with oracle.float64():
+        got_i = (oracle_port.matmul(xi, yi), oracle_port.matmul_grad_x(xi, yi, dzi), oracle_port.matmul_grad_y(xi, yi, dzi))
+        got = (oracle_port.matmul(x, y), oracle_port.matmul_grad_x(x, y, dz), oracle_port.matmul_grad_y(x, y, dz))
+        live = (oracle_ref.matmul(x, y), oracle_ref.matmul_grad_x(x, y, dz), oracle_ref.matmul_grad_y(x, y, dz))
+    for a, b in zip(got_i, f32):
+        assert a.dtype == np.float64 and np.array_equal(a, b.astype(np.float64))
+    for a, b, c in zip(got, (want, dX, dY), live):
+        assert rel_fro(a.reshape(b.shape), b) <= F64_TOL
+        assert c.dtype == np.float64 and rel_fro(a, c) <= F64_TOL
+    # beta = 1: the old value takes part
+    with oracle.float64():
+        twice = oracle_port.matmul_grad_x(x, y, dz, dx=got[1])
+    assert rel_fro(twice, 2 * got[1]) <= F64_TOL
+
+
+@pytest.mark.parametrize("cfg", CONV)
+def test_double_conv2d(oracle_port, oracle, cfg):
+    pytest.importorskip("torch")
+    B, IH, IW, IC, OC, FH, FW = cfg[:7]
+    a = cfg[7:]
+    r = rng(41)
+    xi, wi = ints(r, (B, IH, IW, IC), 8), ints(r, (OC, FH, FW, IC), 8)
+    zi = oracle_port.conv2d(xi, wi, *a)
+    gzi = ints(r, zi.shape, 8)
+    f32 = (zi, oracle_port.conv2d_grad_x(xi, wi, gzi, *a), oracle_port.conv2d_grad_y(xi, wi, gzi, *a))
+    x, w, gz = r.standard_normal(xi.shape), r.standard_normal(wi.shape), r.standard_normal(zi.shape)
+    want = _torch_conv2d(oracle_port, x, w, gz, cfg)
+    with oracle.float64():
+        got_i = (oracle_port.conv2d(xi, wi, *a), oracle_port.conv2d_grad_x(xi, wi, gzi, *a), oracle_port.conv2d_grad_y(xi, wi, gzi, *a))
+        got = (oracle_port.conv2d(x, w, *a), oracle_port.conv2d_grad_x(x, w, gz, *a), oracle_port.conv2d_grad_y(x, w, gz, *a))
+    for p, q in zip(got_i, f32):
+        assert p.dtype == np.float64 and np.array_equal(p, q.astype(np.float64))
+    for p, q in zip(got, want):
+        assert rel_fro(p, q) <= F64_TOL
+
+
+@pytest.mark.parametrize("cfg", DECONV)
+def test_double_deconv2d(oracle_port, oracle, cfg):
+    pytest.importorskip("torch")
+    B, IH, IW, IC, OC, FH, FW = cfg[:7]
+    a = cfg[7:]
+    r = rng(42)
+    xi, wi = ints(r, (B, IH, IW, IC), 8), ints(r, (OC, FH, FW, IC), 8)
+    zi = oracle_port.deconv2d(xi, wi, *a)
+    gzi = ints(r, zi.shape, 8)
+    f32 = (zi, oracle_port.deconv2d_grad_x(xi, wi, gzi, *a), oracle_port.deconv2d_grad_y(xi, wi, gzi, *a))
+    x, w, gz = r.standard_normal(xi.shape), r.standard_normal(wi.shape), r.standard_normal(zi.shape)
+    want = _torch_deconv2d(oracle_port, x, w, gz, cfg)
+    with oracle.float64():
+        got_i = (oracle_port.deconv2d(xi, wi, *a), oracle_port.deconv2d_grad_x(xi, wi, gzi, *a), oracle_port.deconv2d_grad_y(xi, wi, gzi, *a))
+        got = (oracle_port.deconv2d(x, w, *a), oracle_port.deconv2d_grad_x(x, w, gz, *a), oracle_port.deconv2d_grad_y(x, w, gz, *a))
+    for p, q in zip(got_i, f32):
+        assert p.dtype == np.float64 and np.array_equal(p, q.astype(np.float64))
+    for p, q in zip(got, want):
+        assert rel_fro(p, q) <= F64_TOL
+
+
+def test_double_gemm_against_numpy(oracle_port, oracle):
+    r = rng(43)
+    A, B, C = r.standard_normal((37, 23)), r.standard_normal((23, 41)), r.standard_normal((37, 41))
+    with oracle.float64():
+        assert rel_fro(oracle_port.gemm(0, 0, A, B), A @ B) <= F64_TOL
+        assert rel_fro(oracle_port.gemm(0, 1, A, np.ascontiguousarray(B.T)), A @ B) <= F64_TOL
+        assert rel_fro(oracle_port.gemm(1, 0, np.ascontiguousarray(A.T), B, C, 1.0), A @ B + C) <= F64_TOL
+
+
+# The reference's Float64 CPU path, live, on the shapes of the float live tests above (square images: its patch
+# expression pads the wrong axis when the two pads differ).
+@pytest.mark.parametrize("cov", [True, False])
+@pytest.mark.parametrize("s,d,F", [(1, 1, 3), (2, 2, 4), (2, 1, 3), (1, 2, 3), (3, 1, 5)])
+def test_double_conv2d_against_reference_live(oracle_port, oracle_ref, oracle, cov, s, d, F):
+    r = rng(44)
+    x, w = r.standard_normal((2, 17, 17, 5)), r.standard_normal((6, F, F, 5))
+    a = (cov, s, s, d, d)
+    with oracle.float64():
+        z = oracle_ref.conv2d(x, w, *a)
+        assert z.dtype == np.float64 and rel_fro(oracle_port.conv2d(x, w, *a), z) <= F64_TOL
+        gz = r.standard_normal(z.shape)
+        assert rel_fro(oracle_port.conv2d_grad_x(x, w, gz, *a), oracle_ref.conv2d_grad_x(x, w, gz, *a)) <= F64_TOL
+        assert rel_fro(oracle_port.conv2d_grad_y(x, w, gz, *a), oracle_ref.conv2d_grad_y(x, w, gz, *a)) <= F64_TOL
+
+
+@pytest.mark.parametrize("cov", [True, False])
+@pytest.mark.parametrize("s,F", [(1, 3), (2, 4), (3, 4), (2, 3), (3, 2)])
+def test_double_deconv2d_against_reference_live(oracle_port, oracle_ref, oracle, cov, s, F):
+    r = rng(45)
+    x, w = r.standard_normal((2, 9, 9, 5)), r.standard_normal((6, F, F, 5))
+    a = (cov, s, s)
+    with oracle.float64():
+        z = oracle_ref.deconv2d(x, w, *a)
+        assert z.dtype == np.float64 and rel_fro(oracle_port.deconv2d(x, w, *a), z) <= F64_TOL
+        gz = r.standard_normal(z.shape)
+        assert rel_fro(oracle_port.deconv2d_grad_x(x, w, gz, *a), oracle_ref.deconv2d_grad_x(x, w, gz, *a)) <= F64_TOL
+        assert rel_fro(oracle_port.deconv2d_grad_y(x, w, gz, *a), oracle_ref.deconv2d_grad_y(x, w, gz, *a)) <= F64_TOL
