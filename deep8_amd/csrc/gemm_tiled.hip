@@ -298,9 +298,23 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
 
     // ---- which tile: ids of one XCD (same id mod 8) form a contiguous run, runs are laid out in
     // bands of GM tile rows walked column by column
+    // blockIdx.z = output batch index * splits + piece of the reduction.  The reduction runs over
+    // `red` products (1 unless the whole batch is summed into one C) times K, cut into `splits`.
+    // The tiles of one piece read the same rows of A and B, so they should meet in one L2: the
+    // launch's workgroups (x fastest, then z) go to the XCDs in turn, and the ids one XCD receives
+    // are therefore dealt out piece by piece, all tiles of a piece before the next.
     int id = blockIdx.x;
     const int total = tilesM * tilesN;
-    if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    const int b = blockIdx.z / g.splits;
+    int split = blockIdx.z - b * g.splits;
+    const int linear = id + total * split, whole = total * (g.splits & ~7);
+    if (linear < whole) {
+        const int j = linear >> 3, piece = j / total;
+        split = (piece << 3) + (linear & 7);
+        id = j - piece * total;
+    } else if ((total & 7) == 0) {
+        id = (id & 7) * (total >> 3) + (id >> 3);
+    }
     constexpr int GM = 4;
     const int band = id / (GM * tilesN), first = band * GM;
     const int rows_in_band = min(GM, tilesM - first);
@@ -315,9 +329,6 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // number of rows below piece 0, in global memory and in LDS alike.  Global memory is read
     // through buffer descriptors: byte offset = uniform part (tile origin, K step, piece; scalar
     // registers) + per-thread part (one VGPR per operand).
-    // blockIdx.z = output batch index * splits + piece of the reduction.  The reduction runs over
-    // `red` products (1 unless the whole batch is summed into one C) times K, cut into `splits`.
-    const int b = blockIdx.z / g.splits, split = blockIdx.z - b * g.splits;
     constexpr int VIRT = T::VIRT, B_IT = T::B_IT;
     const PatchGeom &pg = g.pg;
     const long a_rows = A_KC ? g.M : g.K, b_rows = B_KC ? g.N : g.K;
