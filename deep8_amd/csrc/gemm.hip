@@ -228,7 +228,7 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     const long total = (long)red * ceil_div(K, BK);
     const int cus = cu_count();
     long splits = 1;
-    if (tiles < cus) splits = (2L * cus + tiles - 1) / tiles;
+    if (tiles < cus) splits = 2L * cus / tiles;  // at most two workgroups per CU: a third one would run alone, after the rest
     // A short reduction over an output that half-height tiles spread over most of the chip is better
     // left whole: the tiled kernel then takes 64 x 128 tiles (gemm_tiled_half_tiles) and the fp32
     // partial sums, their round trip through memory and the second launch are saved.

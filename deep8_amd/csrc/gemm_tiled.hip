@@ -52,8 +52,7 @@ struct Elem<f16> {
     static constexpr int MFMA_PER_FRAG = 1;  // MFMAs that consume one fragment pair
     static constexpr int TR_READS = 2;       // LDS instructions per fragment in the [k][row] layout
     static constexpr int TR_PAD = 64;        // bytes added to a [k][row] row: its 4 k-rows x 64 B hit different banks
-    // lane's element offset inside a [row][k] tile (row r0 + lane%32, its half of the k group)
-    __device__ static int kc_offset(int lane, int ld, int row0) { return (row0 + (lane & 31)) * ld + (lane >> 5) * 8; }
+    static constexpr int KC_HALF = 8;        // [row][k] tile: elements between what the two lane halves read
     // ... and inside a [k][row] tile: the lane whose index within its group of 16 is i addresses
     // k-row (i / 4), columns 4 * (i % 4) .. + 3 of its 16-column group, and receives column i
     __device__ static int tr_offset(int lane, int ld, int row0) {
@@ -77,8 +76,8 @@ struct Elem<float> {
     static constexpr int KG = 8;
     static constexpr int MFMA_PER_FRAG = 4;  // MFMA e pairs k = e with k = 4 + e
     static constexpr int TR_READS = 4;
-    static constexpr int TR_PAD = 160;  // rows 4 apart (the two lane halves) land in different bank halves
-    __device__ static int kc_offset(int lane, int ld, int row0) { return (row0 + (lane & 31)) * ld + (lane >> 5) * 4; }
+    static constexpr int TR_PAD = 32;  // k-rows 4 apart (the two lane halves) land in different bank halves
+    static constexpr int KC_HALF = 4;
     __device__ static int tr_offset(int lane, int ld, int row0) { return (lane >> 5) * 4 * ld + row0 + (lane & 31); }
     __device__ static Frag read_kc(const float *p) { return *(const f32x4 *)p; }
     __device__ static Frag read_tr(const float *p, int ld) {
@@ -110,18 +109,26 @@ struct Tile {
     static constexpr int NT = WGM * WGN * 64;
     static constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32;
     static constexpr int MQ = TM * TN * EL::MFMA_PER_FRAG;  // MFMAs per quarter step
-    // leading dimensions in elements: [row][k] rows get 16 bytes of padding so that consecutive
-    // rows start in different banks
-    static constexpr int A_LD = A_KC ? BK + EPV : BM + EL::TR_PAD / ES;
-    static constexpr int B_LD = B_KC ? BK + EPV : BN + EL::TR_PAD / ES;
-    static constexpr int A_SZ = A_KC ? BM * A_LD : BK * A_LD;
-    static constexpr int B_SZ = B_KC ? BN * B_LD : BK * B_LD;
+    // A [row][k] tile keeps its rows (128 bytes each) in order with 16 bytes of padding after every
+    // second row: the 16 rows that one cycle of a 16-byte LDS read touches then start in 16 different
+    // groups of four banks, and two workgroup tiles of the 64-wide shapes stay under a third of the
+    // CU's LDS.  A [k][row] tile has a leading dimension (A_LD / B_LD) with TR_PAD bytes of padding.
+    __device__ __host__ static constexpr int kc_row(int r) { return r * BK + (r >> 1) * EPV; }
+    static constexpr int KC_BLK = kc_row(32);  // elements between rows 32 apart (from an even row)
+    static constexpr int A_LD = BM + EL::TR_PAD / ES, B_LD = BN + EL::TR_PAD / ES;
+    static constexpr int A_SZ = A_KC ? kc_row(BM) : BK * A_LD;
+    static constexpr int B_SZ = B_KC ? kc_row(BN) : BK * B_LD;
     // 16-byte pieces each thread moves per K step, and the rows one pass of all threads covers
     static constexpr int A_IT = BM * 8 / NT, B_IT = BN * 8 / NT, NP = A_IT + B_IT;
     static constexpr int A_ROWS = A_KC ? NT / 8 : NT / (BM / EPV);
     static constexpr int B_ROWS = B_KC ? NT / 8 : NT / (BN / EPV);
+    static_assert(A_ROWS % 2 == 0 && B_ROWS % 2 == 0, "a pass of all threads starts on an even row");
+    // elements between the pieces two consecutive passes write, and between a wave's 32-row blocks
+    static constexpr int A_PASS = A_KC ? kc_row(A_ROWS) : A_ROWS * A_LD, B_PASS = B_KC ? kc_row(B_ROWS) : B_ROWS * B_LD;
+    static constexpr int A_BLK = A_KC ? KC_BLK : 32, B_BLK = B_KC ? KC_BLK : 32;
     static constexpr int A_RD = A_KC ? 1 : EL::TR_READS, B_RD = B_KC ? 1 : EL::TR_READS;
-    // the epilogue's transposing patches reuse the larger of the two operand areas
+    // the epilogue's transposing patches reuse the two halves of the larger operand area: the first
+    // half of the waves turn their blocks around in one, the rest in the other
     static constexpr bool PATCH_IN_A = A_SZ >= B_SZ;
     static constexpr int PATCH_SZ = PATCH_IN_A ? A_SZ : B_SZ;
 };
@@ -162,7 +169,7 @@ __device__ __forceinline__ void k_step(const typename T::E *Ar, const typename T
             for (int t = 0; t < w_n; ++t)
                 if (slot_of(t, w_n, MQ) == m) {
                     const int p = w_lo + t;
-                    E *dst = p < A_IT ? Aw + p * T::A_ROWS * T::A_LD : Bw + (p - A_IT) * T::B_ROWS * T::B_LD;
+                    E *dst = p < A_IT ? Aw + p * T::A_PASS : Bw + (p - A_IT) * T::B_PASS;
                     *(u32x4 *)dst = R[p];
                 }
 #pragma unroll
@@ -179,10 +186,10 @@ __device__ __forceinline__ void k_step(const typename T::E *Ar, const typename T
                     const int kk = q < 3 ? (q + 1) * T::KQ : 0;
                     const E *a_base = q < 3 ? Ar : An, *b_base = q < 3 ? Br : Bn;
                     if (f < TM)
-                        fa[(q + 1) & 1][f] = T::A_KC ? EL::read_kc(a_base + f * 32 * T::A_LD + kk)
+                        fa[(q + 1) & 1][f] = T::A_KC ? EL::read_kc(a_base + f * T::A_BLK + kk)
                                                      : EL::read_tr(a_base + kk * T::A_LD + f * 32, T::A_LD);
                     else
-                        fb[(q + 1) & 1][f - TM] = T::B_KC ? EL::read_kc(b_base + (f - TM) * 32 * T::B_LD + kk)
+                        fb[(q + 1) & 1][f - TM] = T::B_KC ? EL::read_kc(b_base + (f - TM) * T::B_BLK + kk)
                                                           : EL::read_tr(b_base + kk * T::B_LD + (f - TM) * 32, T::B_LD);
                 }
         }
@@ -220,14 +227,15 @@ struct Origin {
 // through the wave's own 32 x 36 float patch of LDS, so that a lane ends up with 8 consecutive
 // columns of one row: 16-byte loads of the old C and 16-byte stores.
 template <typename T, typename O>
-__device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *lds, O *C, int ldc, float beta,
+__device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *lds0, float *lds1, O *C, int ldc, float beta,
                                            bool aligned, int N, const Origin &o) {
     constexpr int TM = T::TM, TN = T::TN, OPV = 16 / sizeof(O);
     typedef O OV __attribute__((ext_vector_type(OPV)));
-    static_assert((size_t)T::PATCH_SZ * T::ES >= (size_t)T::NT / 64 * 32 * 36 * sizeof(float), "patch space");
+    constexpr int HALF_WAVES = T::NT / 128;
+    static_assert((size_t)T::PATCH_SZ * T::ES >= (size_t)HALF_WAVES * 32 * 36 * sizeof(float), "patch space");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lhi = lane >> 5;
     if (aligned && N % 8 == 0) {
-        float *patch = lds + wave * (32 * 36);
+        float *patch = (wave < HALF_WAVES ? lds0 + wave * (32 * 36) : lds1 + (wave - HALF_WAVES) * (32 * 36));
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -342,7 +350,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const unsigned Bu = (unsigned)ES * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
     const int a_r = A_KC ? tid >> 3 : tid / (BM / EPV), a_c = A_KC ? tid & 7 : tid % (BM / EPV);
     const int b_r = B_KC ? tid >> 3 : tid / (BN / EPV), b_c = B_KC ? tid & 7 : tid % (BN / EPV);
-    const int a_dst = a_r * A_LD + a_c * EPV, b_dst = b_r * B_LD + b_c * EPV;
+    const int a_dst = (A_KC ? T::kc_row(a_r) : a_r * A_LD) + a_c * EPV, b_dst = (B_KC ? T::kc_row(b_r) : b_r * B_LD) + b_c * EPV;
     const unsigned a_pass = VIRT == VIRT_A_ROWS ? 0u : (unsigned)ES * T::A_ROWS * g.lda;  // bytes
     const unsigned b_pass = VIRT == VIRT_B_KROWS ? 0u : (unsigned)ES * T::B_ROWS * g.ldb;
     const unsigned a_step = A_KC ? 128u : (unsigned)ES * BK * g.lda;
@@ -378,8 +386,8 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     }
 
     // ---- per-lane LDS offsets of its MFMA operands
-    const int a_frag = A_KC ? EL::kc_offset(lane, A_LD, wm * TM * 32) : EL::tr_offset(lane, A_LD, wm * TM * 32);
-    const int b_frag = B_KC ? EL::kc_offset(lane, B_LD, wn * TN * 32) : EL::tr_offset(lane, B_LD, wn * TN * 32);
+    const int a_frag = A_KC ? T::kc_row(wm * TM * 32 + (lane & 31)) + (lane >> 5) * EL::KC_HALF : EL::tr_offset(lane, A_LD, wm * TM * 32);
+    const int b_frag = B_KC ? T::kc_row(wn * TN * 32 + (lane & 31)) + (lane >> 5) * EL::KC_HALF : EL::tr_offset(lane, B_LD, wn * TN * 32);
 
     u32x4 R[NP];
     typename EL::Frag fa[2][TM], fb[2][TN];
@@ -442,7 +450,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     }
 #pragma unroll
     for (int p = 0; p < NP; ++p)
-        *(u32x4 *)(p < A_IT ? As0 + a_dst + p * T::A_ROWS * A_LD : Bs0 + b_dst + (p - A_IT) * T::B_ROWS * B_LD) = R[p];
+        *(u32x4 *)(p < A_IT ? As0 + a_dst + p * T::A_PASS : Bs0 + b_dst + (p - A_IT) * T::B_PASS) = R[p];
     {
         const unsigned pa = step_a(1), pb = step_b(1);
 #pragma unroll
@@ -453,10 +461,10 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-        fa[0][i] = A_KC ? EL::read_kc(As0 + a_frag + i * 32 * A_LD) : EL::read_tr(As0 + a_frag + i * 32, A_LD);
+        fa[0][i] = A_KC ? EL::read_kc(As0 + a_frag + i * T::A_BLK) : EL::read_tr(As0 + a_frag + i * 32, A_LD);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-        fb[0][j] = B_KC ? EL::read_kc(Bs0 + b_frag + j * 32 * B_LD) : EL::read_tr(Bs0 + b_frag + j * 32, B_LD);
+        fb[0][j] = B_KC ? EL::read_kc(Bs0 + b_frag + j * T::B_BLK) : EL::read_tr(Bs0 + b_frag + j * 32, B_LD);
 
     // ---- main loop, two steps per trip so that the LDS half of every access is known statically;
     for (int i = 0; i < nsteps; i += 2) {
@@ -475,11 +483,11 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // ---- epilogue: the result itself, or this piece's fp32 partial sums when the reduction is split
     __syncthreads();  // every wave is past the last step: the operand areas are free
     const Origin o = {m0, n0, m_own, n_own, (wm * TM) * 32, (wn * TN) * 32};
-    float *patches = (float *)(T::PATCH_IN_A ? As0 : Bs0);
+    float *patches = (float *)(T::PATCH_IN_A ? As0 : Bs0), *patches1 = (float *)(T::PATCH_IN_A ? As1 : Bs1);
     if (g.splits > 1)
-        store_tile<T, float>(acc, patches, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o);
+        store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o);
     else
-        store_tile<T, E>(acc, patches, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
+        store_tile<T, E>(acc, patches, patches1, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
                          g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o);
 }
 
