@@ -495,7 +495,12 @@ template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, in
 static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
     typedef Tile<E, BM, BN, WGM, WGN, A_KC, B_KC, VIRT> T;
     const int tilesM = ceil_div(g.M, BM), tilesN = ceil_div(g.N, BN);
-    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, g.batch * g.splits), dim3(T::NT), 0, stream, g, tilesM, tilesN);
+    // A launch of at most two workgroups per CU is spread evenly only if a CU cannot take a third:
+    // where the tile's own LDS would let three in, unused dynamic LDS is requested on top.
+    constexpr long lds = 2L * (T::A_SZ + T::B_SZ) * T::ES, third = 160 * 1024 / 3;
+    const long wgs = (long)tilesM * tilesN * g.batch * g.splits, cus = cu_count();
+    const unsigned pad = (lds <= third && wgs > cus && wgs <= 2 * cus) ? (unsigned)(third + 512 - lds) : 0u;
+    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, g.batch * g.splits), dim3(T::NT), pad, stream, g, tilesM, tilesN);
     D8_LAUNCH_CHECK();
     return 0;
 }
