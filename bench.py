@@ -257,7 +257,12 @@ class ConvWorkload:
         es = self.dtype.itemsize
         dtype = "f16" if self.dtype == np.float16 else "f32"
         flops = self.flops / 3
-        if self.deconv:
+        q = self.lib.d8_deconv2d_scratch_bytes
+        if self.deconv and q(self.dt, 0, B, IH, IW, IC, OC, FH, FW, *self.geo) == 0:
+            fn = self.fwd  # no interim matrix: the whole forward is one launch
+            name = ("gemm_tiled_kernel<%s> (DeConv2d forward: one launch over the %d residue classes of output pixels, "
+                    "patch rows read from x by the tile loader)" % (dtype, self.geo[1] * self.geo[2]))
+        elif self.deconv:
             T, M = FH * FW, B * IH * IW
             mat = capi.DeviceArray((M * T * OC,), self.dtype)
             fn = lambda: capi.check(self.lib.d8_gemm(self.dt, 0, 1, M, OC, IC, self.x.ptr, IC, 0, self.w.ptr, T * IC, IC, 0.0,

@@ -365,6 +365,7 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     D8_REQUIRE((long)ceil_div(M, 128) < 65536 && (long)batch * 128 < 65536, "d8_gemm: grid too large");
 
     GemmArgs g;
+    memset(&g, 0, sizeof(g));
     g.A = A;
     g.B = B;
     g.C = C;

@@ -20,7 +20,23 @@ struct PatchGeom {
     unsigned bytes;            // size of the image
 };
 
-enum { VIRT_NONE = 0, VIRT_A_ROWS = 1, VIRT_B_KROWS = 2 };
+enum { VIRT_NONE = 0, VIRT_A_ROWS = 1, VIRT_B_KROWS = 2, VIRT_A_CLASSES = 3 };
+
+// A strided transposed convolution, output pixel by output pixel: the output pixels whose
+// coordinates have one residue (py, px) modulo the stride form a class; a class is an ordinary
+// stride-1 patch product over the taps fy = f0y + sy * j, fx = f0x + sx * i that reach it:
+//   z[b][sy * y' + py][sx * x' + px][:] = sum over (j, i) of x[b][y' + j - pt][x' + i - pl][:] . w[:][fy][fx][:]
+// VIRT_A_CLASSES runs all classes in one launch (blockIdx.z = class): the patch grid, the taps, the
+// filter slice and the rows of C a class writes come from its OutClass, everything else from GemmArgs.
+struct OutClass {
+    int M;             // rows (b, y', x') of the class
+    int OH, OW;        // its grid of (y', x')
+    int taps_w, red;   // taps per filter row that reach it, and in all
+    int pt, pl;        // patch origin (may be negative)
+    int py, px;        // residue: output pixel = (sy * y' + py, sx * x' + px)
+    unsigned b_off;    // element offset of the filter slice of its first tap (f0y, f0x)
+};
+enum { MAX_CLASSES = 16 };
 
 struct GemmArgs {
     const void *A;
@@ -42,6 +58,12 @@ struct GemmArgs {
     int virt;
     PatchGeom pg;
     int m_base;  // VIRT_A_ROWS: row 0 of this product is patch row m_base (a product over a band of rows)
+    // VIRT_A_CLASSES: product (j, i) of a class reads B at b_off + j * sB_row + i * sB; row (b, y', x') of
+    // the class is row ((b * out_H + out_sy * y' + py) * out_W + out_sx * x' + px) of C
+    long sB_row;
+    int out_H, out_W, out_sy, out_sx;
+    int ncls;
+    OutClass cls[MAX_CLASSES];
 };
 
 // Tiled kernels (fp16 and fp32) for shapes whose operands can be moved in 16-byte pieces.

@@ -100,7 +100,7 @@ struct Tile {
     static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
     static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
     static constexpr int VIRT = VIRT_;  // which operand, if any, is a patch matrix read from its image
-    static_assert(VIRT != VIRT_A_ROWS || A_KC, "patch rows are K-contiguous");
+    static_assert((VIRT != VIRT_A_ROWS && VIRT != VIRT_A_CLASSES) || A_KC, "patch rows are K-contiguous");
     static_assert(VIRT != VIRT_B_KROWS || !B_KC, "patch k-rows are N-contiguous");
     static constexpr int ES = sizeof(E), EPV = 16 / ES;  // element size, elements per 16-byte piece
     static constexpr int BK = 128 / ES;                  // K step: 128 bytes of a row
@@ -226,9 +226,20 @@ struct Origin {
 // each 32x32 block.  Where rows of C can be moved 16 bytes at a time, each block is turned around
 // through the wave's own 32 x 36 float patch of LDS, so that a lane ends up with 8 consecutive
 // columns of one row: 16-byte loads of the old C and 16-byte stores.
+// C row of tile row m: m itself, or the output pixel of row (b, y', x') of a class of a transposed convolution
+struct RowMap {
+    int plane, OW;                           // 0: identity
+    int out_H, out_W, out_sy, out_sx, py, px;
+    __device__ long operator()(int m) const {
+        if (!plane) return m;
+        const int img = m / plane, rem = m - img * plane, y = rem / OW, x = rem - y * OW;
+        return ((long)img * out_H + out_sy * y + py) * out_W + out_sx * x + px;
+    }
+};
+
 template <typename T, typename O>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *lds0, float *lds1, O *C, int ldc, float beta,
-                                           bool aligned, int N, const Origin &o) {
+                                           bool aligned, int N, const Origin &o, const RowMap &crow) {
     constexpr int TM = T::TM, TN = T::TN, OPV = 16 / sizeof(O);
     typedef O OV __attribute__((ext_vector_type(OPV)));
     constexpr int HALF_WAVES = T::NT / 128;
@@ -250,7 +261,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
                     *(f32x4 *)&v[0] = *(const f32x4 *)(patch + row * 36 + cc);
                     *(f32x4 *)&v[4] = *(const f32x4 *)(patch + row * 36 + cc + 4);
                     if (m >= o.m_own && n >= o.n_own) {
-                        O *c = C + (long)m * ldc + n;
+                        O *c = C + crow(m) * ldc + n;
 #pragma unroll
                         for (int h = 0; h < 8 / OPV; ++h) {
                             OV out;
@@ -278,7 +289,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
             for (int r = 0; r < 16; ++r) {
                 const int m = o.m0 + o.wm0 + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
                 if (m >= o.m_own && n >= o.n_own) {
-                    O *c = C + (long)m * ldc + n;
+                    O *c = C + crow(m) * ldc + n;
                     float v = acc[i][j][r];
                     if (beta != 0.f) v += as_f32(*c);
                     *c = (O)v;
@@ -311,10 +322,24 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // The tiles of one piece read the same rows of A and B, so they should meet in one L2: the
     // launch's workgroups (x fastest, then z) go to the XCDs in turn, and the ids one XCD receives
     // are therefore dealt out piece by piece, all tiles of a piece before the next.
+    constexpr int VIRT = T::VIRT, B_IT = T::B_IT;
+    constexpr bool VA = VIRT == VIRT_A_ROWS || VIRT == VIRT_A_CLASSES;  // A's rows are patch rows
+    PatchGeom pg = g.pg;
+    int M = g.M, red = g.red;
+    unsigned b_cls = 0;
+    RowMap crow = {0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (VIRT == VIRT_A_CLASSES) {
+        const OutClass &c = g.cls[blockIdx.z];
+        M = c.M, red = c.red, b_cls = c.b_off;
+        pg.OH = c.OH, pg.OW = c.OW, pg.FW = c.taps_w, pg.pt = c.pt, pg.pl = c.pl;
+        crow = {c.OH * c.OW, c.OW, g.out_H, g.out_W, g.out_sy, g.out_sx, c.py, c.px};
+        tilesM = (M + BM - 1) / BM;
+        if ((int)blockIdx.x >= tilesM * tilesN) return;  // the grid is sized for the largest class
+    }
     int id = blockIdx.x;
     const int total = tilesM * tilesN;
-    const int b = blockIdx.z / g.splits;
-    int split = blockIdx.z - b * g.splits;
+    const int b = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z / g.splits;
+    int split = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z - b * g.splits;
     const int linear = id + total * split, whole = total * (g.splits & ~7);
     if (linear < whole) {
         const int j = linear >> 3, piece = j / total;
@@ -331,27 +356,26 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // A tile that would stick out of the matrix is moved back inside; the rows / columns it then
     // shares with its neighbour are computed twice but stored only by the neighbour.
     const int m_own = tm * BM, n_own = tn * BN;
-    const int m0 = min(m_own, g.M - BM), n0 = min(n_own, g.N - BN);
+    const int m0 = min(m_own, M - BM), n0 = min(n_own, g.N - BN);
 
     // ---- the 16-byte pieces this thread moves each K step: piece `it` of an operand lies a fixed
     // number of rows below piece 0, in global memory and in LDS alike.  Global memory is read
     // through buffer descriptors: byte offset = uniform part (tile origin, K step, piece; scalar
     // registers) + per-thread part (one VGPR per operand).
-    constexpr int VIRT = T::VIRT, B_IT = T::B_IT;
-    const PatchGeom &pg = g.pg;
     const long a_rows = A_KC ? g.M : g.K, b_rows = B_KC ? g.N : g.K;
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
         (void *)((const E *)g.A + (long)b * g.sA), 0,
-        VIRT == VIRT_A_ROWS ? (int)pg.bytes : (int)(ES * ((g.red - 1) * g.sA + a_rows * g.lda)), 0x00020000);
+        VA ? (int)pg.bytes : (int)(ES * ((g.red - 1) * g.sA + a_rows * g.lda)), 0x00020000);
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
         (void *)((const E *)g.B + (long)b * g.sB), 0,
-        VIRT == VIRT_B_KROWS ? (int)pg.bytes : (int)(ES * ((g.red - 1) * g.sB + b_rows * g.ldb)), 0x00020000);
+        VIRT == VIRT_B_KROWS ? (int)pg.bytes
+                             : (int)(ES * ((VIRT == VIRT_A_CLASSES ? 0 : (g.red - 1) * g.sB) + b_rows * g.ldb)), 0x00020000);
     const unsigned Au = (unsigned)ES * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0);
     const unsigned Bu = (unsigned)ES * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
     const int a_r = A_KC ? tid >> 3 : tid / (BM / EPV), a_c = A_KC ? tid & 7 : tid % (BM / EPV);
     const int b_r = B_KC ? tid >> 3 : tid / (BN / EPV), b_c = B_KC ? tid & 7 : tid % (BN / EPV);
     const int a_dst = (A_KC ? T::kc_row(a_r) : a_r * A_LD) + a_c * EPV, b_dst = (B_KC ? T::kc_row(b_r) : b_r * B_LD) + b_c * EPV;
-    const unsigned a_pass = VIRT == VIRT_A_ROWS ? 0u : (unsigned)ES * T::A_ROWS * g.lda;  // bytes
+    const unsigned a_pass = VA ? 0u : (unsigned)ES * T::A_ROWS * g.lda;  // bytes
     const unsigned b_pass = VIRT == VIRT_B_KROWS ? 0u : (unsigned)ES * T::B_ROWS * g.ldb;
     const unsigned a_step = A_KC ? 128u : (unsigned)ES * BK * g.lda;
     const unsigned b_step = B_KC ? 128u : (unsigned)ES * BK * g.ldb;
@@ -365,7 +389,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     for (int p = 0; p < B_IT; ++p) bv[p] = (unsigned)ES * ((unsigned)b_r * (unsigned)g.ldb + b_c * EPV);
     // patch rows as A: this thread's rows never change; a step selects the tap
     int va_base[A_IT], va_iy[A_IT], va_ix[A_IT];
-    if constexpr (VIRT == VIRT_A_ROWS) {
+    if constexpr (VA) {
         const int plane = pg.OH * pg.OW;
 #pragma unroll
         for (int p = 0; p < A_IT; ++p) {
@@ -402,11 +426,12 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // ---- this workgroup's steps x0 .. x0 + nsteps - 1 of the extended reduction; step x reads
     // product x / ktiles at K offset (x % ktiles) * BK (all uniform: scalar arithmetic)
     const int ktiles = g.K / BK;
-    const int x0 = split * g.tiles_per_split, nsteps = min(g.red * ktiles, x0 + g.tiles_per_split) - x0;
+    const int x0 = split * g.tiles_per_split, nsteps = min(red * ktiles, x0 + g.tiles_per_split) - x0;
     const unsigned a_prod = (unsigned)ES * (unsigned)g.sA, b_prod = (unsigned)ES * (unsigned)g.sB;
+    const unsigned b_prod_row = (unsigned)ES * (unsigned)g.sB_row, b_first = (unsigned)ES * b_cls;
     auto step_a = [&](int i) -> unsigned {
         const int x = x0 + min(i, nsteps - 1), r = x / ktiles;  // past the end: refetch the last step, never used
-        if constexpr (VIRT == VIRT_A_ROWS) {
+        if constexpr (VA) {
             const int fy = r / pg.FW, fx = r - fy * pg.FW, tdy = fy * pg.dy, tdx = fx * pg.dx;
             const int toff = ((tdy * pg.W + tdx) * pg.C + (x - r * ktiles) * BK) * ES;
 #pragma unroll
@@ -435,6 +460,9 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
                 bv[p] = inside ? (unsigned)(((((int)img * pg.H + iy) * pg.W + ix) * pg.C + vb_c) * ES) : OUTSIDE;
             }
             return 0u;
+        } else if constexpr (VIRT == VIRT_A_CLASSES) {
+            const int fy = r / pg.FW, fx = r - fy * pg.FW;
+            return Bu + b_first + fy * b_prod_row + fx * b_prod + (x - r * ktiles) * b_step;
         } else {
             return Bu + (g.red > 1 ? r * b_prod : 0u) + (x - r * ktiles) * b_step;
         }
@@ -485,10 +513,10 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const Origin o = {m0, n0, m_own, n_own, (wm * TM) * 32, (wn * TN) * 32};
     float *patches = (float *)(T::PATCH_IN_A ? As0 : Bs0), *patches1 = (float *)(T::PATCH_IN_A ? As1 : Bs1);
     if (g.splits > 1)
-        store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o);
+        store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o, crow);
     else
         store_tile<T, E>(acc, patches, patches1, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
-                         g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o);
+                         g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o, crow);
 }
 
 template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int VIRT>
@@ -498,9 +526,10 @@ static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
     // A launch of at most two workgroups per CU is spread evenly only if a CU cannot take a third:
     // where the tile's own LDS would let three in, unused dynamic LDS is requested on top.
     constexpr long lds = 2L * (T::A_SZ + T::B_SZ) * T::ES, third = 160 * 1024 / 3;
-    const long wgs = (long)tilesM * tilesN * g.batch * g.splits, cus = cu_count();
+    const int layers = VIRT == VIRT_A_CLASSES ? g.ncls : g.batch * g.splits;  // for classes g.M is the largest one's
+    const long wgs = (long)tilesM * tilesN * layers, cus = cu_count();
     const unsigned pad = (lds <= third && wgs > cus && wgs <= 2 * cus) ? (unsigned)(third + 512 - lds) : 0u;
-    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, g.batch * g.splits), dim3(T::NT), pad, stream, g, tilesM, tilesN);
+    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
     D8_LAUNCH_CHECK();
     return 0;
 }
@@ -530,7 +559,8 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
 template <typename E>
 static bool eligible(const GemmArgs &g, int transA, int transB) {
     constexpr long ES = sizeof(E), EPV = 16 / ES, BK = 128 / ES;
-    const bool va = g.virt == VIRT_A_ROWS, vb = g.virt == VIRT_B_KROWS;
+    const bool va = g.virt == VIRT_A_ROWS || g.virt == VIRT_A_CLASSES, vb = g.virt == VIRT_B_KROWS;
+    if (g.virt == VIRT_A_CLASSES && (!transB || g.splits > 1 || g.ncls < 1 || g.ncls > MAX_CLASSES || g.M < 128)) return false;
     if (va && (transA || g.K != g.pg.C)) return false;                       // a K step stays inside one tap
     if (vb && (!transA || transB || g.red != 1 || g.pg.C % EPV || g.N % g.pg.C)) return false;  // a piece stays inside one tap
     if ((va || vb) && (g.pg.bytes >= (1u << 31) || g.batch != 1)) return false;
@@ -549,6 +579,10 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
 
 template <typename E>
 static int launch_any(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
+    if (g.virt == VIRT_A_CLASSES) {  // every class has at least 128 rows (checked by eligible)
+        if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, true, true, VIRT_A_CLASSES>(g, stream);
+        return launch_tiled<E, 128, 128, 2, 2, true, true, VIRT_A_CLASSES>(g, stream);
+    }
     if (g.virt == VIRT_A_ROWS) return transB ? pick_tile<E, true, true, VIRT_A_ROWS>(g, stream) : pick_tile<E, true, false, VIRT_A_ROWS>(g, stream);
     if (g.virt == VIRT_B_KROWS) return pick_tile<E, false, false, VIRT_B_KROWS>(g, stream);
     if (!transA && !transB) return pick_tile<E, true, false>(g, stream);

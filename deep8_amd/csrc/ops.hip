@@ -359,6 +359,49 @@ static bool deconv_implicit_grad_x(int dtype, int B, int IH, int IW, int IC, int
     return gemm_tiled_eligible(dtype, g, 0, 0);
 }
 
+// z computed output pixel by output pixel: the sy * sx residue classes of output coordinates are each
+// a stride-1 patch product over the taps that reach them (OutClass), all in one launch; nothing
+// is staged.  Needs a tap for every class (FH >= sy, FW >= sx) and tile-sized classes.
+static bool deconv_implicit_fwd(int dtype, int B, int IH, int IW, int IC, int OC, int FH, int FW, int sy, int sx,
+                                const int *geo, const void *x, const void *w, const void *z, GemmArgs &g) {
+    if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
+    const long es = (long)dtype_bytes(dtype), T = (long)FH * FW;
+    const int OH = geo[0], OW = geo[1], pt = geo[2], pl = geo[3];
+    if (es == 8 || sy * sx > MAX_CLASSES || FH < sy || FW < sx || OH < sy || OW < sx) return false;
+    const long xbytes = (long)B * IH * IW * IC * es;
+    if (xbytes >= (1L << 31) || (long)B * OH * OW * OC * es >= (1L << 31) || T * IC * OC * es >= (1L << 31)) return false;
+    memset(&g, 0, sizeof(g));
+    g.pg = {IH, IW, IC, 0, 0, 0, 1, 1, 1, 1, 0, 0, 0, 0, (unsigned)xbytes};
+    g.virt = VIRT_A_CLASSES;
+    g.A = x, g.B = w, g.C = (void *)z;
+    g.N = OC, g.K = IC;
+    g.ldb = (int)(T * IC), g.sB = (long)sx * IC, g.sB_row = (long)sy * FW * IC, g.ldc = OC;
+    g.batch = 1, g.red = 1, g.splits = 1, g.beta = 0.f;
+    g.out_H = OH, g.out_W = OW, g.out_sy = sy, g.out_sx = sx;
+    int largest = 0, smallest = 0x7fffffff, most_taps = 0;
+    for (int py = 0; py < sy; ++py)
+        for (int px = 0; px < sx; ++px) {
+            OutClass &c = g.cls[g.ncls++];
+            c.OH = (OH - py + sy - 1) / sy, c.OW = (OW - px + sx - 1) / sx;
+            c.M = B * c.OH * c.OW;
+            // taps fy with (py - pt + fy) a multiple of sy: fy = f0y + sy * j
+            const int f0y = (((pt - py) % sy) + sy) % sy, f0x = (((pl - px) % sx) + sx) % sx;
+            const int nty = (FH - f0y + sy - 1) / sy, ntx = (FW - f0x + sx - 1) / sx;
+            c.taps_w = ntx, c.red = nty * ntx;
+            c.pt = -((py - pt + f0y) / sy), c.pl = -((px - pl + f0x) / sx);  // input row = y' + j + (py - pt + f0y) / sy
+            c.py = py, c.px = px;
+            c.b_off = (unsigned)((f0y * FW + f0x) * IC);
+            largest = c.M > largest ? c.M : largest;
+            smallest = c.M < smallest ? c.M : smallest;
+            most_taps = c.red > most_taps ? c.red : most_taps;
+        }
+    g.tiles_per_split = most_taps * (IC / gemm_tiled_k_step(dtype) + 1);  // never the limit: a class walks all its taps
+    g.M = smallest;
+    const bool ok = gemm_tiled_eligible(dtype, g, 0, 1);
+    g.M = largest;
+    return ok;
+}
+
 size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                  int OC, int FH, int FW, int covered, int sy, int sx) {
     int geo[4];
@@ -368,6 +411,7 @@ size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, in
     GemmArgs ga;
     if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
         return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
+    if (which == 0 && deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga)) return 0;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     return mat + gemm_ws(dtype, deconv_plan(which, M, T, OC, IC, nullptr, nullptr, nullptr));
 }
@@ -381,7 +425,13 @@ int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
-    D8_REQUIRE(x && w && z && scratch, "d8_deconv2d: null tensor");
+    D8_REQUIRE(x && w && z, "d8_deconv2d: null tensor");
+    {
+        GemmArgs ga;
+        if (deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, w, z, ga))
+            return gemm_tiled_launch(dtype, ga, 0, 1, as_stream(stream));
+    }
+    D8_REQUIRE(scratch, "d8_deconv2d: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d: scratch too small");
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
     if (int rc = run(dtype, deconv_plan(0, M, T, OC, IC, scratch, w, x), ws ? (char *)scratch + mat : nullptr, ws, stream))

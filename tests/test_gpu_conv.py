@@ -304,3 +304,61 @@ def test_conv2d_implicit_route(oracle_port, monkeypatch, cfg, imp32, imp16, dtyp
         got = (ops.conv2d(x, w, *a), ops.conv2d_grad_x(x, w, gz, *a), ops.conv2d_grad_y(x, w, gz, *a))
         for k, (g_, w_) in enumerate(zip(got, want)):
             assert rel_fro(f(g_), w_) <= tol, (route, k)
+
+
+# ---- DeConv2d forward by residue classes of output pixels (no interim matrix): shapes that take it (channel
+# counts that are multiples of the K step, 64 or more output channels, every class tile-sized, a tap for
+# every class) and, last, shapes that must fall back.  (B, IH, IW, IC, OC, FH, FW, covered, sy, sx), fp32?, half?
+DECONV_CLASSES = [
+    ((2, 9, 8, 64, 64, 4, 4, False, 2, 2), True, True),
+    ((3, 9, 8, 64, 96, 4, 4, True, 2, 2), True, True),      # covered: pads shift the classes' taps
+    ((2, 12, 11, 64, 64, 4, 4, False, 3, 3), True, True),   # stride 3: classes with 2x2, 2x1, 1x2 and 1x1 taps
+    ((2, 12, 11, 64, 64, 4, 4, True, 3, 3), True, True),
+    ((2, 10, 10, 128, 128, 3, 3, True, 2, 2), True, True),  # 3x3 stride 2: 2 or 1 taps per axis; 128-wide tiles
+    ((2, 9, 9, 64, 64, 5, 3, False, 2, 1), True, True),     # different strides per axis, 5x3 filter
+    ((3, 8, 8, 32, 64, 2, 2, False, 2, 2), True, False),    # 32 channels: one fp32 K step, too few for half
+    ((1, 16, 16, 64, 64, 4, 4, False, 1, 1), True, True),   # stride 1: a single class with all 16 taps
+    ((2, 16, 16, 64, 72, 4, 4, True, 4, 4), True, True),    # 16 classes of one tap each
+    ((2, 9, 8, 64, 64, 2, 2, False, 3, 3), False, False),   # stride > filter: some classes have no tap
+    ((1, 6, 6, 64, 64, 4, 4, False, 2, 2), False, False),   # classes smaller than a tile
+]
+
+
+@pytest.mark.parametrize("cfg,imp32,imp16", DECONV_CLASSES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_deconv2d_forward_by_classes(oracle_port, monkeypatch, cfg, imp32, imp16, dtype):
+    from deep8_amd import capi, ops
+    from deep8_amd.capi import DeviceArray, check
+    lib = capi.init()
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = cfg
+    dt = capi.dtype_id(np.dtype(dtype))
+    OH, OW, _, _ = ops.deconv2d_geometry(IH, IW, FH, FW, cov, sy, sx)
+    nb = lib.d8_deconv2d_scratch_bytes(dt, 0, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx)
+    assert (nb == 0) == (imp32 if dtype == np.float32 else imp16)
+    monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+    assert lib.d8_deconv2d_scratch_bytes(dt, 0, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx) >= B * IH * IW * FH * FW * OC * np.dtype(dtype).itemsize
+    monkeypatch.delenv("D8_CONV_EXPLICIT")
+
+    def forward(x, w):  # into an output pre-filled with NaN: every pixel must be written
+        dx_, dw_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w)
+        dz_ = DeviceArray.from_numpy(np.full((B, OH, OW, OC), np.nan, dtype))
+        ws = DeviceArray((max(nb, 16),), np.uint8)
+        check(lib.d8_deconv2d(dt, dx_.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dz_.ptr, int(cov), sy, sx, ws.ptr if nb else None, nb, None))
+        return dz_.numpy()
+
+    r = rng(B + IH + OC + 91)
+    c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
+    hi = 3 if dtype == np.float16 else 20
+    x, w = ints(r, (B, IH, IW, IC), hi), ints(r, (OC, FH, FW, IC), hi)
+    if dtype == np.float16:
+        x, w = x * (r.random(x.shape) < 0.3), w * (r.random(w.shape) < 0.3)
+    want = oracle_port.deconv2d(x, w, cov, sy, sx)
+    assert dtype == np.float32 or np.abs(want).max() < 2048
+    got = forward(c(x), c(w))
+    assert got.shape == want.shape and np.array_equal(f(got), want)
+    x, w = c(nrm(r, (B, IH, IW, IC))), c(nrm(r, (OC, FH, FW, IC), np.sqrt(2.0 / (FH * FW * IC))))
+    want = oracle_port.deconv2d(f(x), f(w), cov, sy, sx)
+    tol = FP16_TOL if dtype == np.float16 else FP32_TOL
+    assert rel_fro(f(forward(x, w)), want) <= tol
+    monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+    assert rel_fro(f(ops.deconv2d(x, w, cov, sy, sx)), want) <= tol
