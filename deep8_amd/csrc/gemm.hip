@@ -163,6 +163,15 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(GemmArgs g) {
         }
 }
 
+// Where element (m, n) of an output lives (GemmArgs::perm_OC: a filter gradient stored transposed per tap).
+__device__ inline long c_index(const GemmArgs &g, int m, int n) {
+    if (g.perm_OC) {
+        const int t = n / g.perm_OC, oc = n - t * g.perm_OC;
+        return ((long)oc * g.perm_T + t) * g.ldc + m;
+    }
+    return (long)m * g.ldc + n;
+}
+
 // C[b][m][n] = beta * C + sum_s ws[b][s][m][n].  A workgroup covers 32 groups of 4 consecutive
 // outputs; its 8 thread rows each add every 8th partial (16-byte loads), and the 8 sums meet in
 // LDS in a fixed order, so the result does not depend on scheduling.
@@ -186,12 +195,13 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(GemmArgs g) {
 #pragma unroll
         for (int k = 1; k < 8; ++k) v += part[k][lane];
         const int m = (int)(r / g.N), n = (int)(r - (long)m * g.N);
-        T *c = (T *)g.C + (long)b * g.sC + (long)m * g.ldc + n;
+        T *c0 = (T *)g.C + (long)b * g.sC;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
+            T *c = c0 + c_index(g, m, n + k);
             float o = v[k];
-            if (g.beta != 0.f) o += to_f32(c[k]);
-            c[k] = (T)o;
+            if (g.beta != 0.f) o += to_f32(*c);
+            *c = (T)o;
         }
     }
 }
@@ -208,7 +218,7 @@ __global__ void gemm_split_reduce_scalar_kernel(GemmArgs g) {
         const float *p = g.ws + (long)b * g.splits * mn + e;
         float v = 0.f;
         for (int s = 0; s < g.splits; ++s) v += p[(long)s * mn];
-        T *c = (T *)g.C + (long)b * g.sC + (long)m * g.ldc + n;
+        T *c = (T *)g.C + (long)b * g.sC + c_index(g, m, n);
         if (g.beta != 0.f) v += to_f32(*c);
         *c = (T)v;
     }
@@ -233,7 +243,13 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     // left whole: the tiled kernel then takes 64 x 128 tiles (gemm_tiled_half_tiles) and the fp32
     // partial sums, their round trip through memory and the second launch are saved.
     if (gemm_tiled_half_tiles(M, N, batch, total)) splits = 1;
-    const long max_by_len = total / 4 > 0 ? total / 4 : 1;  // at least 4 K steps per piece
+    static const char *force = getenv("D8_GEMM_SPLITS");  // tuning aid
+    if (force && splits > 1) splits = atoi(force);
+    // Every piece costs a tile's prologue, a tile of fp32 partial sums written and read back: at least 8 K steps
+    // per piece, or 4 where 8 would leave more than half of the CUs without a workgroup.
+    long max_by_len = total / 8;
+    if (max_by_len * tiles < cus / 2) max_by_len = total / 4;
+    if (max_by_len < 1) max_by_len = 1;
     if (splits > max_by_len) splits = max_by_len;
     if (splits > 128) splits = 128;
     // no more pieces than the caller's workspace holds

@@ -64,6 +64,9 @@ struct GemmArgs {
     int out_H, out_W, out_sy, out_sx;
     int ncls;
     OutClass cls[MAX_CLASSES];
+    // perm_OC > 0: the result is stored transposed per filter tap: element (m, n = t * perm_OC + oc) of the
+    // product goes to C[(oc * perm_T + t) * ldc + m] (a filter gradient [OC][taps][IC] computed as [IC][taps x OC])
+    int perm_T, perm_OC;
 };
 
 // Tiled kernels (fp16 and fp32) for shapes whose operands can be moved in 16-byte pieces.

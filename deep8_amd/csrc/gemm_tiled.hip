@@ -230,10 +230,18 @@ struct Origin {
 struct RowMap {
     int plane, OW;                           // 0: identity
     int out_H, out_W, out_sy, out_sx, py, px;
+    int perm_T, perm_OC;                     // perm_OC > 0: stored transposed per tap (GemmArgs::perm_OC)
     __device__ long operator()(int m) const {
         if (!plane) return m;
         const int img = m / plane, rem = m - img * plane, y = rem / OW, x = rem - y * OW;
         return ((long)img * out_H + out_sy * y + py) * out_W + out_sx * x + px;
+    }
+    __device__ long at(int m, int n, int ldc) const {
+        if (perm_OC) {
+            const int t = n / perm_OC, oc = n - t * perm_OC;
+            return ((long)oc * perm_T + t) * ldc + m;
+        }
+        return (*this)(m) * ldc + n;
     }
 };
 
@@ -245,7 +253,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
     constexpr int HALF_WAVES = T::NT / 128;
     static_assert((size_t)T::PATCH_SZ * T::ES >= (size_t)HALF_WAVES * 32 * 36 * sizeof(float), "patch space");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lhi = lane >> 5;
-    if (aligned && N % 8 == 0) {
+    if (aligned && N % 8 == 0 && !crow.perm_OC) {
         float *patch = (wave < HALF_WAVES ? lds0 + wave * (32 * 36) : lds1 + (wave - HALF_WAVES) * (32 * 36));
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -289,7 +297,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
             for (int r = 0; r < 16; ++r) {
                 const int m = o.m0 + o.wm0 + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
                 if (m >= o.m_own && n >= o.n_own) {
-                    O *c = C + crow(m) * ldc + n;
+                    O *c = C + crow.at(m, n, ldc);
                     float v = acc[i][j][r];
                     if (beta != 0.f) v += as_f32(*c);
                     *c = (O)v;
@@ -327,12 +335,13 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     PatchGeom pg = g.pg;
     int M = g.M, red = g.red;
     unsigned b_cls = 0;
-    RowMap crow = {0, 0, 0, 0, 0, 0, 0, 0};
+    RowMap crow = {0, 0, 0, 0, 0, 0, 0, 0, g.perm_T, g.perm_OC};
+    const RowMap plain = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     if constexpr (VIRT == VIRT_A_CLASSES) {
         const OutClass &c = g.cls[blockIdx.z];
         M = c.M, red = c.red, b_cls = c.b_off;
         pg.OH = c.OH, pg.OW = c.OW, pg.FW = c.taps_w, pg.pt = c.pt, pg.pl = c.pl;
-        crow = {c.OH * c.OW, c.OW, g.out_H, g.out_W, g.out_sy, g.out_sx, c.py, c.px};
+        crow = {c.OH * c.OW, c.OW, g.out_H, g.out_W, g.out_sy, g.out_sx, c.py, c.px, 0, 0};
         tilesM = (M + BM - 1) / BM;
         if ((int)blockIdx.x >= tilesM * tilesN) return;  // the grid is sized for the largest class
     }
@@ -513,7 +522,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const Origin o = {m0, n0, m_own, n_own, (wm * TM) * 32, (wn * TN) * 32};
     float *patches = (float *)(T::PATCH_IN_A ? As0 : Bs0), *patches1 = (float *)(T::PATCH_IN_A ? As1 : Bs1);
     if (g.splits > 1)
-        store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o, crow);
+        store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o, plain);
     else
         store_tile<T, E>(acc, patches, patches1, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
                          g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o, crow);

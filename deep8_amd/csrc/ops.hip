@@ -402,6 +402,27 @@ static bool deconv_implicit_fwd(int dtype, int B, int IH, int IW, int IC, int OC
     return ok;
 }
 
+// dw[oc][tap][ic] += sum over input pixels m of dz gathered for (m, tap)[oc] . x[m][ic], computed as the
+// transposed product [IC] x [taps x OC] = x^T . patch(dz) -- the patch matrix of dz read by the tile loader, as
+// for Conv2d's filter gradient -- and stored transposed per tap by the reduction.
+static bool deconv_implicit_grad_y(int dtype, int B, int IH, int IW, int IC, int OC, int FH, int FW, int sy, int sx,
+                                   const int *geo, const void *x, const void *gw, const void *gz, GemmArgs &g) {
+    if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
+    const long es = (long)dtype_bytes(dtype), T = (long)FH * FW;
+    const long zbytes = (long)B * geo[0] * geo[1] * OC * es;
+    if (es == 8 || zbytes >= (1L << 31) || (long)B * IH * IW >= (1L << 31) || T * OC >= (1L << 31)) return false;
+    memset(&g, 0, sizeof(g));
+    g.pg = {geo[0], geo[1], OC, IH, IW, FW, sy, sx, -1, -1, -geo[2], -geo[3],
+            magic_of((unsigned)IH * IW), magic_of((unsigned)IW), (unsigned)zbytes};
+    g.virt = VIRT_B_KROWS;
+    g.A = x, g.B = gz, g.C = (void *)gw;
+    g.M = IC, g.N = (int)(T * OC), g.K = B * IH * IW;
+    g.lda = IC, g.ldc = IC;
+    g.batch = 1, g.red = 1, g.splits = 1, g.beta = 1.f;
+    g.perm_T = (int)T, g.perm_OC = OC;
+    return gemm_tiled_eligible(dtype, g, 1, 0);
+}
+
 size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                  int OC, int FH, int FW, int covered, int sy, int sx) {
     int geo[4];
@@ -412,6 +433,8 @@ size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, in
     if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
         return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
     if (which == 0 && deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga)) return 0;
+    if (which == 2 && deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
+        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     return mat + gemm_ws(dtype, deconv_plan(which, M, T, OC, IC, nullptr, nullptr, nullptr));
 }
@@ -475,7 +498,15 @@ static int d8_deconv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int 
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
-    D8_REQUIRE(x && gw && gz && scratch, "d8_deconv2d_grad_y: null tensor");
+    D8_REQUIRE(x && gw && gz, "d8_deconv2d_grad_y: null tensor");
+    {
+        GemmArgs ga;
+        if (deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, gw, gz, ga)) {
+            ga.beta = beta;
+            return gemm_tiled_run(dtype, ga, 1, 0, scratch, scratch_bytes, as_stream(stream));
+        }
+    }
+    D8_REQUIRE(scratch, "d8_deconv2d_grad_y: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d_grad_y: scratch too small");
     if (int rc = launch_im2col(dtype, gz, scratch, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), as_stream(stream)))
         return rc;

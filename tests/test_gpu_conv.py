@@ -362,3 +362,51 @@ def test_deconv2d_forward_by_classes(oracle_port, monkeypatch, cfg, imp32, imp16
     assert rel_fro(f(forward(x, w)), want) <= tol
     monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
     assert rel_fro(f(ops.deconv2d(x, w, cov, sy, sx)), want) <= tol
+
+
+# ---- DeConv2d filter gradient without the interim matrix (the patch matrix of dz read by the tile loader, the
+# result stored transposed per tap): needs B*IH*IW a multiple of the K step and 64 or more input channels
+DECONV_DW = [
+    ((2, 8, 8, 64, 64, 4, 4, False, 2, 2), True, True),
+    ((4, 8, 8, 64, 96, 4, 4, True, 2, 2), True, True),
+    ((2, 8, 8, 128, 64, 3, 3, True, 2, 2), True, True),
+    ((1, 16, 8, 64, 64, 4, 4, False, 3, 3), True, True),
+    ((2, 8, 8, 64, 64, 5, 3, False, 2, 1), True, True),
+    ((2, 16, 16, 64, 64, 2, 2, False, 3, 3), True, True),   # stride > filter
+    ((1, 8, 4, 64, 64, 4, 4, False, 2, 2), True, False),    # 32 input pixels: one fp32 K step
+    ((2, 7, 7, 64, 64, 4, 4, False, 2, 2), False, False),   # 98 input pixels: not a multiple of the K step
+]
+
+
+@pytest.mark.parametrize("cfg,imp32,imp16", DECONV_DW)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_deconv2d_filter_gradient_without_interim(oracle_port, monkeypatch, cfg, imp32, imp16, dtype):
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = cfg
+    a = (cov, sy, sx)
+    dt = capi.dtype_id(np.dtype(dtype))
+    OH, OW, _, _ = ops.deconv2d_geometry(IH, IW, FH, FW, *a)
+    q = lambda: lib.d8_deconv2d_scratch_bytes(dt, 2, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx)
+    interim = B * IH * IW * FH * FW * OC * np.dtype(dtype).itemsize
+    monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+    assert q() >= interim
+    monkeypatch.delenv("D8_CONV_EXPLICIT")
+    expect = imp32 if dtype == np.float32 else imp16
+    assert (q() < interim) == expect or (not expect and q() >= interim)
+    r = rng(B + IH + OC + 93)
+    c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
+    hi = 3 if dtype == np.float16 else 20
+    x, w, gz = ints(r, (B, IH, IW, IC), hi), ints(r, (OC, FH, FW, IC), hi), ints(r, (B, OH, OW, OC), hi)
+    if dtype == np.float16:
+        x, gz = x * (r.random(x.shape) < 0.3), gz * (r.random(gz.shape) < 0.2)
+    want = oracle_port.deconv2d_grad_y(x, w, gz, *a, w)
+    assert dtype == np.float32 or np.abs(want).max() < 2048
+    assert np.array_equal(f(ops.deconv2d_grad_y(c(x), c(w), c(gz), *a, c(w))), want)
+    assert np.array_equal(f(ops.deconv2d_grad_y(c(x), c(w), c(gz), *a, c(w) - 2, overwrite=True)), want - w)
+    x, w, gz = c(nrm(r, (B, IH, IW, IC))), c(nrm(r, (OC, FH, FW, IC))), c(nrm(r, (B, OH, OW, OC)))
+    want = oracle_port.deconv2d_grad_y(f(x), f(w), f(gz), *a)
+    tol = FP16_TOL if dtype == np.float16 else FP32_TOL
+    assert rel_fro(f(ops.deconv2d_grad_y(x, w, gz, *a)), want) <= tol
+    monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+    assert rel_fro(f(ops.deconv2d_grad_y(x, w, gz, *a)), want) <= tol
