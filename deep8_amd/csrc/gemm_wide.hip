@@ -277,7 +277,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
 #pragma unroll
                     for (int e = 0; e < 8; ++e) out[e] = (f16)v[e];
                 }
-                *(f16x8 *)c = out;
+                // streamed past the L2: the whole output leaves the chip during the kernel's last microseconds
+                // either way, and lines left dirty in L2 are written back only after the last wave has ended
+                __builtin_nontemporal_store(out, (f16x8 *)c);
             }
         }
     }
