@@ -569,7 +569,7 @@ template <typename E>
 static bool eligible(const GemmArgs &g, int transA, int transB) {
     constexpr long ES = sizeof(E), EPV = 16 / ES, BK = 128 / ES;
     const bool va = g.virt == VIRT_A_ROWS || g.virt == VIRT_A_CLASSES, vb = g.virt == VIRT_B_KROWS;
-    if (g.virt == VIRT_A_CLASSES && (!transB || g.splits > 1 || g.ncls < 1 || g.ncls > MAX_CLASSES || g.M < 128)) return false;
+    if (g.virt == VIRT_A_CLASSES && (g.splits > 1 || g.ncls < 1 || g.ncls > MAX_CLASSES || g.M < 128)) return false;
     if (va && (transA || g.K != g.pg.C)) return false;                       // a K step stays inside one tap
     if (vb && (!transA || transB || g.red != 1 || g.pg.C % EPV || g.N % g.pg.C)) return false;  // a piece stays inside one tap
     if ((va || vb) && (g.pg.bytes >= (1u << 31) || g.batch != 1)) return false;
@@ -589,8 +589,12 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
 template <typename E>
 static int launch_any(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
     if (g.virt == VIRT_A_CLASSES) {  // every class has at least 128 rows (checked by eligible)
-        if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, true, true, VIRT_A_CLASSES>(g, stream);
-        return launch_tiled<E, 128, 128, 2, 2, true, true, VIRT_A_CLASSES>(g, stream);
+        if (transB) {
+            if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, true, true, VIRT_A_CLASSES>(g, stream);
+            return launch_tiled<E, 128, 128, 2, 2, true, true, VIRT_A_CLASSES>(g, stream);
+        }
+        if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, true, false, VIRT_A_CLASSES>(g, stream);
+        return launch_tiled<E, 128, 128, 2, 2, true, false, VIRT_A_CLASSES>(g, stream);
     }
     if (g.virt == VIRT_A_ROWS) return transB ? pick_tile<E, true, true, VIRT_A_ROWS>(g, stream) : pick_tile<E, true, false, VIRT_A_ROWS>(g, stream);
     if (g.virt == VIRT_B_KROWS) return pick_tile<E, false, false, VIRT_B_KROWS>(g, stream);

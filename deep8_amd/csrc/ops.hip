@@ -130,6 +130,49 @@ static bool conv_implicit_plan(int dtype, int which, const ConvShape &c, const v
     return gemm_tiled_eligible(dtype, g, ta, tb);
 }
 
+// Conv2d's gradient of x for a stride above 1 (dilation 1), input pixel by input pixel: the pixels of dx with
+// one residue (py, px) modulo the stride receive the taps fy = f0y + sy * j, f0y = (py + pt) mod sy, from
+// dz[b][y' + (py + pt - f0y) / sy - j][..] -- a stride-1 patch product with dilation -1 per class (OutClass),
+// all classes in one launch, nothing staged.
+static bool conv_classes_grad_x(int dtype, const ConvShape &c, const void *gx, const void *w, const void *gz, GemmArgs &g) {
+    if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
+    if ((c.sy == 1 && c.sx == 1) || c.dy != 1 || c.dx != 1 || c.sy * c.sx > MAX_CLASSES) return false;
+    if (c.FH < c.sy || c.FW < c.sx || c.IH < c.sy || c.IW < c.sx) return false;  // every class needs a tap
+    const long es = (long)dtype_bytes(dtype), T = (long)c.FH * c.FW;
+    const long zbytes = (long)c.B * c.OH * c.OW * c.OC * es;
+    if (es == 8 || zbytes >= (1L << 31) || (long)c.B * c.IH * c.IW * c.IC * es >= (1L << 31) || T * c.IC * c.OC * es >= (1L << 31))
+        return false;
+    memset(&g, 0, sizeof(g));
+    g.pg = {c.OH, c.OW, c.OC, 0, 0, 0, 1, 1, -1, -1, 0, 0, 0, 0, (unsigned)zbytes};
+    g.virt = VIRT_A_CLASSES;
+    g.A = gz, g.B = w, g.C = (void *)gx;
+    g.N = c.IC, g.K = c.OC;
+    g.ldb = (int)(T * c.IC), g.sB = (long)c.sx * c.IC, g.sB_row = (long)c.sy * c.FW * c.IC, g.ldc = c.IC;
+    g.batch = 1, g.red = 1, g.splits = 1, g.beta = 1.f;
+    g.out_H = c.IH, g.out_W = c.IW, g.out_sy = c.sy, g.out_sx = c.sx;
+    int largest = 0, smallest = 0x7fffffff, most_taps = 0;
+    for (int py = 0; py < c.sy; ++py)
+        for (int px = 0; px < c.sx; ++px) {
+            OutClass &k = g.cls[g.ncls++];
+            k.OH = (c.IH - py + c.sy - 1) / c.sy, k.OW = (c.IW - px + c.sx - 1) / c.sx;
+            k.M = c.B * k.OH * k.OW;
+            const int f0y = (py + c.pt) % c.sy, f0x = (px + c.pl) % c.sx;
+            k.taps_w = (c.FW - f0x + c.sx - 1) / c.sx;
+            k.red = ((c.FH - f0y + c.sy - 1) / c.sy) * k.taps_w;
+            k.pt = -((py + c.pt - f0y) / c.sy), k.pl = -((px + c.pl - f0x) / c.sx);  // dz row = y' - j + (py + pt - f0y) / sy
+            k.py = py, k.px = px;
+            k.b_off = (unsigned)((f0y * c.FW + f0x) * c.IC);
+            largest = k.M > largest ? k.M : largest;
+            smallest = k.M < smallest ? k.M : smallest;
+            most_taps = k.red > most_taps ? k.red : most_taps;
+        }
+    g.tiles_per_split = most_taps * (c.OC / gemm_tiled_k_step(dtype) + 1);
+    g.M = smallest;
+    const bool ok = gemm_tiled_eligible(dtype, g, 0, 0);
+    g.M = largest;
+    return ok;
+}
+
 }  // namespace d8
 
 using namespace d8;
@@ -237,6 +280,7 @@ size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int 
     int ta, tb;
     if (conv_implicit_plan(dtype, which, cs, nullptr, nullptr, nullptr, ga, ta, tb))
         return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
+    if (which == 1 && conv_classes_grad_x(dtype, cs, nullptr, nullptr, nullptr, ga)) return 0;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
     return col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
 }
@@ -283,6 +327,10 @@ static int d8_conv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int
         if (conv_implicit_plan(dtype, 1, cs, gx, w, gz, ga, ta, tb)) {
             ga.beta = beta;
             return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+        }
+        if (conv_classes_grad_x(dtype, cs, gx, w, gz, ga)) {
+            ga.beta = beta;
+            return gemm_tiled_launch(dtype, ga, 0, 0, as_stream(stream));
         }
     }
     D8_REQUIRE(scratch, "d8_conv2d_grad_x: null scratch");

@@ -410,3 +410,44 @@ def test_deconv2d_filter_gradient_without_interim(oracle_port, monkeypatch, cfg,
     assert rel_fro(f(ops.deconv2d_grad_y(x, w, gz, *a)), want) <= tol
     monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
     assert rel_fro(f(ops.deconv2d_grad_y(x, w, gz, *a)), want) <= tol
+
+
+# ---- Conv2d gradient of x for a stride above 1, by residue classes of input pixels (no patch matrix)
+CONV_DX_CLASSES = [
+    ((2, 16, 16, 64, 64, 3, 3, True, 2, 2, 1, 1), True),
+    ((3, 17, 15, 64, 128, 3, 3, False, 2, 2, 1, 1), True),   # not covered: border pixels that no patch reaches
+    ((4, 18, 18, 128, 64, 4, 4, True, 3, 3, 1, 1), True),
+    ((2, 16, 16, 64, 64, 5, 3, True, 2, 1, 1, 1), True),     # stride 2 down, 1 across
+    ((4, 16, 16, 64, 64, 2, 2, False, 2, 2, 1, 1), True),    # filter == stride: one tap per class
+    ((2, 16, 16, 64, 64, 3, 3, True, 2, 2, 2, 2), False),    # dilation: im2col route
+    ((2, 16, 16, 64, 64, 1, 1, True, 2, 2, 1, 1), False),    # filter smaller than the stride: classes without a tap
+]
+
+
+@pytest.mark.parametrize("cfg,classes", CONV_DX_CLASSES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_conv2d_strided_gradient_of_x(oracle_port, monkeypatch, cfg, classes, dtype):
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    a = (cov, sy, sx, dy, dx)
+    OH, OW, _, _ = ops.conv2d_geometry(IH, IW, FH, FW, *a)
+    nb = lib.d8_conv2d_scratch_bytes(capi.dtype_id(np.dtype(dtype)), 1, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx, dy, dx)
+    assert (nb == 0) == classes
+    r = rng(B + IH + OC + 95)
+    c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
+    hi = 3 if dtype == np.float16 else 20
+    x, w, gz = ints(r, (B, IH, IW, IC), hi), ints(r, (OC, FH, FW, IC), hi), ints(r, (B, OH, OW, OC), hi)
+    if dtype == np.float16:
+        w, gz = w * (r.random(w.shape) < 0.3), gz * (r.random(gz.shape) < 0.3)
+    want = oracle_port.conv2d_grad_x(x, w, gz, *a, x)
+    assert dtype == np.float32 or np.abs(want).max() < 2048
+    assert np.array_equal(f(ops.conv2d_grad_x(c(x), c(w), c(gz), *a, c(x))), want)
+    nan = np.full(x.shape, np.nan, dtype)  # the overwrite form must write every pixel, reached by a patch or not
+    assert np.array_equal(f(ops.conv2d_grad_x(c(x), c(w), c(gz), *a, nan, overwrite=True)), want - x)
+    x, w, gz = c(nrm(r, (B, IH, IW, IC))), c(nrm(r, (OC, FH, FW, IC), np.sqrt(2.0 / (FH * FW * IC)))), c(nrm(r, (B, OH, OW, OC)))
+    want = oracle_port.conv2d_grad_x(f(x), f(w), f(gz), *a)
+    tol = FP16_TOL if dtype == np.float16 else FP32_TOL
+    assert rel_fro(f(ops.conv2d_grad_x(x, w, gz, *a)), want) <= tol
+    monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+    assert rel_fro(f(ops.conv2d_grad_x(x, w, gz, *a)), want) <= tol
