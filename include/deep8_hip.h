@@ -122,7 +122,10 @@ int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
  * DeConv2d.h:18,28,38): shape cases, pad formulas, scratch use and accumulate-vs-overwrite
  * semantics are Deep8's.  A matrix operand is (batch, rows, cols) with cols = 1 for a 1-D
  * tensor.  `scratch` is the interim buffer the node allocates (size from the *_scratch_bytes
- * function, which already includes any split-reduction workspace).                          */
+ * function, which already includes any split-reduction workspace).  Where that function
+ * returns 0 the operator stages nothing (its patch matrix is read by the GEMM's tile loader)
+ * and `scratch` may be NULL; a scratch smaller than asked for is an error only when the
+ * operator has to stage.                                                                     */
 size_t d8_matmul_scratch_bytes(int dtype, int which /*0 fwd, 1 gradX, 2 gradY*/,
                                int xb, int xr, int xc, int yb, int yr, int yc);
 int d8_matmul(int dtype, const void *x, int xb, int xr, int xc,
