@@ -9,6 +9,7 @@
 // Prints "PASS <name>" / "FAIL <name>: <why>" per test; exit code = number of failures.
 #include <cmath>
 #include <cstdio>
+#include <chrono>
 #include <cstring>
 #include <functional>
 #include <iostream>
@@ -902,6 +903,63 @@ TEST_GPU(two_layer_convnet_trains_with_sgd) {
 }
 
 }  // namespace
+
+// Node-level step times at the three large configurations: forward + both gradients through Function::forward /
+// backward, i.e. with the scratch buffer taken from and returned to the device pool inside every call and the
+// gradients zeroed before the backward pass (lazily: Tensor::zero defers the fill).  Printed, not asserted.
+template <typename NodeT>
+void timeNode(const char *what, NodeT &node, HostTensor &a, HostTensor &b, HostTensor &z, HostTensor &gz, HostTensor &ga,
+              HostTensor &gb, double flops) {
+    std::vector<const Tensor *> tin = {&a.t, &b.t};
+    auto step = [&] {
+        node.forward(tin, &z.t);
+        ga.t.zero();
+        gb.t.zero();
+        node.backward(tin, &z.t, &gz.t, 0, &ga.t);
+        node.backward(tin, &z.t, &gz.t, 1, &gb.t);
+    };
+    for (int i = 0; i < 3; ++i) step();
+    gpu().synchronize();
+    const int reps = 20;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < reps; ++i) step();
+    gpu().synchronize();
+    const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count() / reps;
+    printf("     %-58s %8.1f us / step  %8.1f TFLOP/s\n", what, us, flops / us * 1e-6);
+}
+
+TEST_GPU(node_level_step_times) {
+    {
+        ElementType h16 = ElementType::from<half>();
+        HostTensor x = randomTensor(h16, 1, {4096, 4096}, 2), y = randomTensor(h16, 1, {4096, 4096}, 2);
+        HostTensor z = randomTensor(h16, 1, {4096, 4096}, 0), dz = randomTensor(h16, 1, {4096, 4096}, 2);
+        HostTensor dx = randomTensor(h16, 1, {4096, 4096}, 0), dy = randomTensor(h16, 1, {4096, 4096}, 0);
+        Variable v0 = placeholder(h16), v1 = placeholder(h16);
+        std::vector<Node *> in = {&v0, &v1};
+        MatrixMultiply mm(in);
+        timeNode("MatrixMultiply half 4096^3 (0/1-valued operands)", mm, x, y, z, dz, dx, dy, 3 * 2.0 * 4096.0 * 4096.0 * 4096.0);
+    }
+    {
+        ElementType f32 = ElementType::from<float>();
+        HostTensor x = randomTensor(f32, 32, {56, 56, 64}, 5), w = randomTensor(f32, 1, {64, 3, 3, 64}, 5);
+        HostTensor z = randomTensor(f32, 32, {56, 56, 64}, 0), gz = randomTensor(f32, 32, {56, 56, 64}, 5);
+        HostTensor gx = randomTensor(f32, 32, {56, 56, 64}, 0), gw = randomTensor(f32, 1, {64, 3, 3, 64}, 0);
+        Variable v0 = placeholder(f32), v1 = placeholder(f32);
+        std::vector<Node *> in = {&v0, &v1};
+        Conv2d conv(in, true, 1, 1, 1, 1);
+        timeNode("Conv2d fp32 B32 56x56x64 3x3 -> 64", conv, x, w, z, gz, gx, gw, 3 * 2.0 * 32 * 56 * 56 * 576.0 * 64);
+    }
+    {
+        ElementType h16 = ElementType::from<half>();
+        HostTensor x = randomTensor(h16, 16, {28, 28, 128}, 2), w = randomTensor(h16, 1, {64, 4, 4, 128}, 2);
+        HostTensor z = randomTensor(h16, 16, {58, 58, 64}, 0), gz = randomTensor(h16, 16, {58, 58, 64}, 2);
+        HostTensor gx = randomTensor(h16, 16, {28, 28, 128}, 0), gw = randomTensor(h16, 1, {64, 4, 4, 128}, 0);
+        Variable v0 = placeholder(h16), v1 = placeholder(h16);
+        std::vector<Node *> in = {&v0, &v1};
+        DeConv2d deconv(in, false, 2, 2);
+        timeNode("DeConv2d half B16 28x28x128 4x4 s2 -> 58x58x64", deconv, x, w, z, gz, gx, gw, 3 * 2.0 * 16 * 28 * 28 * 128.0 * 64 * 16);
+    }
+}
 
 int main(int argc, char **argv) {
     bool cpuOnly = false, list = false;
