@@ -301,18 +301,23 @@ class BiasReluWorkload:
         self.ws = capi.DeviceArray((max(self.ws_bytes, 16),), np.uint8)
         es = self.dtype.itemsize
         self.flops = 4.0 * self.n
-        # add: r z, w pre | relu: r pre, w act | relu_grad: r pre, r gy, rw gpre | bias grad: r gpre
-        self.bytes = es * self.n * 9
+        # add: r z, w pre | relu: r pre, w act | relu_grad: r pre, r gy, w gpre (+ fill and read-back of gpre
+        # with --eager-zero) | bias grad: r gpre
+        self.bytes = es * self.n * (10 if EAGER_ZERO else 8)
 
     def step(self):
         from deep8_amd.capi import check
         L = self.lib
         check(L.d8_add(self.dt, self.z.ptr, self.zd, self.b.ptr, self.bd, self.pre.ptr, self.zd, None))
         check(L.d8_relu(self.dt, self.pre.ptr, self.act.ptr, self.n, None))
-        self.gpre.zero_()
-        self.gb.zero_()
-        check(L.d8_relu_grad(self.dt, self.pre.ptr, self.gpre.ptr, self.gy.ptr, self.n, None))
-        check(L.d8_add_grad(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
+        if EAGER_ZERO:
+            self.gpre.zero_()
+            self.gb.zero_()
+            check(L.d8_relu_grad(self.dt, self.pre.ptr, self.gpre.ptr, self.gy.ptr, self.n, None))
+            check(L.d8_add_grad(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
+        else:  # gradients whose zero fill is still pending are written, not added to
+            check(L.d8_relu_grad_overwrite(self.dt, self.pre.ptr, self.gpre.ptr, self.gy.ptr, self.n, None))
+            check(L.d8_add_grad_overwrite(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
 
 
 class PoolWorkload:
@@ -331,14 +336,17 @@ class PoolWorkload:
         self.gx = capi.DeviceArray((B, H, W, C), dtype)
         n, es = B * H * W * C, self.dtype.itemsize
         self.flops = 2.0 * n
-        # forward: r x, w y | fill gx | gradient: r x, r gy, rw gx
-        self.bytes = es * (n + n // 4 + n + n + n // 4 + 2 * n)
+        # forward: r x, w y | gradient: r x, r gy, w gx (+ fill and read-back of gx with --eager-zero)
+        self.bytes = es * (n + n // 4 + n + n // 4 + n + (2 * n if EAGER_ZERO else 0))
 
     def step(self):
         from deep8_amd.capi import check
         check(self.lib.d8_maxpool2d(self.dt, self.x.ptr, self.y.ptr, *self.dims, 2, 2, 0, 2, 2, None))
-        self.gx.zero_()
-        check(self.lib.d8_maxpool2d_grad(self.dt, self.x.ptr, self.gx.ptr, self.gy.ptr, *self.dims, 2, 2, 0, 2, 2, None))
+        if EAGER_ZERO:
+            self.gx.zero_()
+            check(self.lib.d8_maxpool2d_grad(self.dt, self.x.ptr, self.gx.ptr, self.gy.ptr, *self.dims, 2, 2, 0, 2, 2, None))
+        else:
+            check(self.lib.d8_maxpool2d_grad_overwrite(self.dt, self.x.ptr, self.gx.ptr, self.gy.ptr, *self.dims, 2, 2, 0, 2, 2, None))
 
 
 def _uni(r, s):

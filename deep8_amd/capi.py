@@ -72,8 +72,10 @@ SIGNATURES = {
     "d8_add": (_I, [_I, _P, _IP, _P, _IP, _P, _IP, _P]),
     "d8_add_grad_scratch_bytes": (_Z, [_I, _IP, _IP]),
     "d8_add_grad": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
+    "d8_add_grad_overwrite": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
     "d8_relu": (_I, [_I, _P, _P, ctypes.c_long, _P]),
     "d8_relu_grad": (_I, [_I, _P, _P, _P, ctypes.c_long, _P]),
+    "d8_relu_grad_overwrite": (_I, [_I, _P, _P, _P, ctypes.c_long, _P]),
     "d8_minus": (_I, [_I, _P, _IP, _P, _IP, _P, _IP, _P]),
     "d8_minus_grad_y": (_I, [_I, _P, _IP, _P, _IP, _P, _Z, _P]),
     "d8_l1norm": (_I, [_I, _P, _P, _I, ctypes.c_long, _P, _Z, _P]),
@@ -85,8 +87,10 @@ SIGNATURES = {
     "d8_axpby": (_I, [_I, _P, _F, _P, _F, _P, ctypes.c_long, _P]),
     "d8_maxpool2d": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
     "d8_maxpool2d_grad": (_I, [_I, _P, _P, _P] + [_I] * 9 + [_P]),
+    "d8_maxpool2d_grad_overwrite": (_I, [_I, _P, _P, _P] + [_I] * 9 + [_P]),
     "d8_avgpool2d": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
     "d8_avgpool2d_grad": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
+    "d8_avgpool2d_grad_overwrite": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
     "d8_adam_update": (_I, [_I, _P, _P, _P, _P, _F, _F, _F, _F, _F, ctypes.c_long, ctypes.c_long, _P]),
     "d8_mfma_stream_out_bytes": (_Z, []),
     "d8_mfma_stream": (_I, [_I, _P, _Z, _P, _I, ctypes.POINTER(ctypes.c_double), _P]),

@@ -85,12 +85,18 @@ enum { LOAD_ID = 0, LOAD_ABS = 1, LOAD_SQUARE = 2 };
 template <int OP>
 __device__ inline float ew_load(float v) { return OP == LOAD_ABS ? fabsf(v) : (OP == LOAD_SQUARE ? v * v : v); }
 
-// g += scale * op(dz), same shape.
+// g = keep * g + scale * op(dz), same shape.  keep is 1 (the reference's accumulate) or 0 (g's old contents are
+// not read: the overwrite forms).  The same convention holds for every kernel below that takes `keep`.
 template <typename T, int VEC, int OP>
-__global__ __launch_bounds__(256) void accumulate_kernel(T *__restrict__ g, const T *__restrict__ dz, long total, float scale) {
+__global__ __launch_bounds__(256) void accumulate_kernel(T *__restrict__ g, const T *__restrict__ dz, long total, float scale,
+                                                         float keep) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-        const VT a = *(const VT *)(g + idx * VEC), b = *(const VT *)(dz + idx * VEC);
+        VT a;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) a[e] = (T)0;
+        if (keep != 0.f) a = *(const VT *)(g + idx * VEC);
+        const VT b = *(const VT *)(dz + idx * VEC);
         VT o;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(a[e]) + scale * ew_load<OP>(ew_f32(b[e])));
@@ -105,7 +111,7 @@ __global__ __launch_bounds__(256) void accumulate_kernel(T *__restrict__ g, cons
 template <typename T, int VEC, int OP>
 __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ dz, T *__restrict__ g,
                                                          float *__restrict__ partial, int R, int C, int TX,
-                                                         int rows_per_chunk, int chunks, float scale) {
+                                                         int rows_per_chunk, int chunks, float scale, float keep) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
     __shared__ float part[256][VEC];
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX, lanes = 256 / TX;
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
         if (chunks == 1) {
             T *o = g + (long)k0 * C + (long)cv * VEC;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(o[e]) + scale * acc[e]);
+            for (int e = 0; e < VEC; ++e) o[e] = (T)((keep != 0.f ? ew_f32(o[e]) : 0.f) + scale * acc[e]);
         } else {
             float *o = partial + ((long)k0 * chunks + chunk) * C + (long)cv * VEC;
 #pragma unroll
@@ -147,7 +153,7 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
 // output each add every 8th chunk and meet in LDS in a fixed order.
 template <typename T>
 __global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__restrict__ partial, T *__restrict__ g,
-                                                                int C, int chunks, long total, float scale) {
+                                                                int C, int chunks, long total, float scale, float keep) {
     __shared__ float part[8][32];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const long idx = (long)blockIdx.x * 32 + tx;
@@ -163,7 +169,7 @@ __global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__r
     if (ty == 0 && idx < total) {
 #pragma unroll
         for (int k = 1; k < 8; ++k) v += part[k][tx];
-        g[idx] = (T)(ew_f32(g[idx]) + scale * v);
+        g[idx] = (T)((keep != 0.f ? ew_f32(g[idx]) : 0.f) + scale * v);
     }
 }
 
@@ -176,7 +182,7 @@ struct ReduceGeom {
 
 template <typename T, int OP>
 __global__ __launch_bounds__(256) void broadcast_sum_kernel(const T *__restrict__ dz, T *__restrict__ g, ReduceGeom q,
-                                                            long total, float scale) {
+                                                            long total, float scale, float keep) {
     long zs[5];
     zs[4] = 1;
     for (int a = 3; a >= 0; --a) zs[a] = zs[a + 1] * q.n[a + 1];
@@ -202,7 +208,7 @@ __global__ __launch_bounds__(256) void broadcast_sum_kernel(const T *__restrict_
             }
             if (a < 0) break;
         }
-        g[idx] = (T)(ew_f32(g[idx]) + scale * acc);
+        g[idx] = (T)((keep != 0.f ? ew_f32(g[idx]) : 0.f) + scale * acc);
     }
 }
 
@@ -220,10 +226,14 @@ __global__ __launch_bounds__(256) void relu_kernel(const T *__restrict__ x, T *_
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void relu_grad_kernel(const T *__restrict__ x, T *__restrict__ dx,
-                                                        const T *__restrict__ dy, long total) {
+                                                        const T *__restrict__ dy, long total, float keep) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-        const VT v = *(const VT *)(x + idx * VEC), d = *(const VT *)(dy + idx * VEC), old = *(const VT *)(dx + idx * VEC);
+        const VT v = *(const VT *)(x + idx * VEC), d = *(const VT *)(dy + idx * VEC);
+        VT old;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) old[e] = (T)0;
+        if (keep != 0.f) old = *(const VT *)(dx + idx * VEC);
         VT o;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o[e] = (T)(ew_f32(old[e]) + (v[e] > (T)0 ? ew_f32(d[e]) : 0.f));
@@ -360,17 +370,17 @@ static ReducePlan plan_reduce(const int *d, const int *zd) {
     return p;
 }
 
-// g += scale * (op(dz) summed over the axes where g has extent 1 and dz does not)
+// g = keep * g + scale * (op(dz) summed over the axes where g has extent 1 and dz does not)
 template <typename T, int WIDE, int OP = LOAD_ID>
 static int reduce_t(T *g, const int *d, const T *dz, const int *zd, void *scratch, size_t scratch_bytes, hipStream_t s,
-                    float scale = 1.f) {
+                    float scale = 1.f, float keep = 1.f) {
     const ReducePlan p = plan_reduce(d, zd);
     const long ng = prod5(d);
     if (p.kind == 0) {
         if (ng % WIDE == 0 && al16(g) && al16(dz))
-            hipLaunchKernelGGL((accumulate_kernel<T, WIDE, OP>), dim3(ew_grid(ng / WIDE, 256)), dim3(256), 0, s, g, dz, ng / WIDE, scale);
+            hipLaunchKernelGGL((accumulate_kernel<T, WIDE, OP>), dim3(ew_grid(ng / WIDE, 256)), dim3(256), 0, s, g, dz, ng / WIDE, scale, keep);
         else
-            hipLaunchKernelGGL((accumulate_kernel<T, 1, OP>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, g, dz, ng, scale);
+            hipLaunchKernelGGL((accumulate_kernel<T, 1, OP>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, g, dz, ng, scale, keep);
     } else if (p.kind == 1) {
         int chunks = p.chunks, rpc = p.rows_per_chunk;
         const size_t need = (size_t)p.K0 * chunks * p.C * sizeof(float);
@@ -383,19 +393,19 @@ static int reduce_t(T *g, const int *d, const T *dz, const int *zd, void *scratc
         dim3 grid((unsigned)((cvs + TX - 1) / TX), (unsigned)chunks, (unsigned)p.K0);
         if (wide)
             hipLaunchKernelGGL((column_sum_kernel<T, WIDE, OP>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
-                               TX, rpc, chunks, scale);
+                               TX, rpc, chunks, scale, keep);
         else
             hipLaunchKernelGGL((column_sum_kernel<T, 1, OP>), grid, dim3(256), 0, s, dz, g, (float *)scratch, (int)p.R, (int)p.C,
-                               TX, rpc, chunks, scale);
+                               TX, rpc, chunks, scale, keep);
         if (chunks > 1) {
             D8_LAUNCH_CHECK();
             hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3((unsigned)((ng + 31) / 32)), dim3(256), 0, s,
-                               (const float *)scratch, g, (int)p.C, chunks, ng, scale);
+                               (const float *)scratch, g, (int)p.C, chunks, ng, scale, keep);
         }
     } else {
         ReduceGeom q;
         for (int a = 0; a < 5; ++a) q.n[a] = zd[a], q.kept[a] = (d[a] == zd[a] && zd[a] > 1) ? 1 : 0;
-        hipLaunchKernelGGL((broadcast_sum_kernel<T, OP>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, dz, g, q, ng, scale);
+        hipLaunchKernelGGL((broadcast_sum_kernel<T, OP>), dim3(ew_grid(ng, 256)), dim3(256), 0, s, dz, g, q, ng, scale, keep);
     }
     D8_LAUNCH_CHECK();
     return 0;
@@ -489,15 +499,25 @@ size_t d8_add_grad_scratch_bytes(int dtype, const int *gdims, const int *zdims) 
     return p.kind == 1 && p.chunks > 1 ? (size_t)p.K0 * p.chunks * p.C * sizeof(float) : 0;
 }
 
-int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
-                void *scratch, size_t scratch_bytes, void *stream) {
+static int add_grad_impl(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                         void *scratch, size_t scratch_bytes, void *stream, float keep) {
     if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
         return fail(D8_ERR_DTYPE, "d8_add_grad: element type %d is not supported", dtype);
     D8_REQUIRE(g && dz && gdims && zdims, "d8_add_grad: null argument");
     if (int rc = check_dims("d8_add_grad", gdims, zdims)) return rc;
     return dtype == D8_FLOAT32
-               ? reduce_t<float, 4>((float *)g, gdims, (const float *)dz, zdims, scratch, scratch_bytes, as_stream(stream))
-               : reduce_t<f16, 8>((f16 *)g, gdims, (const f16 *)dz, zdims, scratch, scratch_bytes, as_stream(stream));
+               ? reduce_t<float, 4>((float *)g, gdims, (const float *)dz, zdims, scratch, scratch_bytes, as_stream(stream), 1.f, keep)
+               : reduce_t<f16, 8>((f16 *)g, gdims, (const f16 *)dz, zdims, scratch, scratch_bytes, as_stream(stream), 1.f, keep);
+}
+
+int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                void *scratch, size_t scratch_bytes, void *stream) {
+    return add_grad_impl(dtype, g, gdims, dz, zdims, scratch, scratch_bytes, stream, 1.f);
+}
+
+int d8_add_grad_overwrite(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                          void *scratch, size_t scratch_bytes, void *stream) {
+    return add_grad_impl(dtype, g, gdims, dz, zdims, scratch, scratch_bytes, stream, 0.f);
 }
 
 int d8_relu(int dtype, const void *x, void *y, long n, void *stream) {
@@ -518,7 +538,7 @@ int d8_relu(int dtype, const void *x, void *y, long n, void *stream) {
     return 0;
 }
 
-int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, void *stream) {
+static int relu_grad_impl(int dtype, const void *x, void *dx, const void *dy, long n, void *stream, float keep) {
     if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
         return fail(D8_ERR_DTYPE, "d8_relu_grad: element type %d is not supported", dtype);
     D8_REQUIRE(n >= 0, "d8_relu_grad: negative size");
@@ -527,14 +547,22 @@ int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, voi
     hipStream_t s = as_stream(stream);
     const bool al = al16(x) && al16(dx) && al16(dy);
     if (dtype == D8_FLOAT32) {
-        if (al && n % 4 == 0) hipLaunchKernelGGL((relu_grad_kernel<float, 4>), dim3(ew_grid(n / 4, 256)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, n / 4);
-        else hipLaunchKernelGGL((relu_grad_kernel<float, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, n);
+        if (al && n % 4 == 0) hipLaunchKernelGGL((relu_grad_kernel<float, 4>), dim3(ew_grid(n / 4, 256)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, n / 4, keep);
+        else hipLaunchKernelGGL((relu_grad_kernel<float, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, n, keep);
     } else {
-        if (al && n % 8 == 0) hipLaunchKernelGGL((relu_grad_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n / 8);
-        else hipLaunchKernelGGL((relu_grad_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n);
+        if (al && n % 8 == 0) hipLaunchKernelGGL((relu_grad_kernel<f16, 8>), dim3(ew_grid(n / 8, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n / 8, keep);
+        else hipLaunchKernelGGL((relu_grad_kernel<f16, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, n, keep);
     }
     D8_LAUNCH_CHECK();
     return 0;
+}
+
+int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, void *stream) {
+    return relu_grad_impl(dtype, x, dx, dy, n, stream, 1.f);
+}
+
+int d8_relu_grad_overwrite(int dtype, const void *x, void *dx, const void *dy, long n, void *stream) {
+    return relu_grad_impl(dtype, x, dx, dy, n, stream, 0.f);
 }
 
 int d8_minus(int dtype, const void *x, const int *xdims, const void *y, const int *ydims, void *z, const int *zdims,

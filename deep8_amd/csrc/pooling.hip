@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void pool_forward_kernel(const T *__restrict__
 //   AVG: dy[oh][ow][c] / (FH * FW)
 template <typename T, int VEC, bool MAX>
 __global__ __launch_bounds__(256) void pool_backward_kernel(const T *__restrict__ x, T *__restrict__ dx, const T *__restrict__ dy,
-                                                            PoolGeom g, long total) {
+                                                            PoolGeom g, long total, float keep) {
     typedef T VT __attribute__((ext_vector_type(VEC)));
     const int cv = g.C / VEC;
     const float inv = 1.0f / ((float)g.FH * (float)g.FW);
@@ -129,7 +129,10 @@ __global__ __launch_bounds__(256) void pool_backward_kernel(const T *__restrict_
                 for (int e = 0; e < VEC; ++e)
                     if (win[e]) acc[e] += pool_f32(d[e]);
             }
-        VT o = *(const VT *)(dx + idx * VEC);
+        VT o;  // keep = 1: added to what dx holds (the reference's accumulate); 0: dx's old contents are not read
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = (T)0;
+        if (keep != 0.f) o = *(const VT *)(dx + idx * VEC);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) o[e] = (T)(pool_f32(o[e]) + acc[e]);
         *(VT *)(dx + idx * VEC) = o;
@@ -164,15 +167,15 @@ static int pool_forward(int dtype, const void *x, void *y, const PoolGeom &g, hi
 }
 
 template <bool MAX>
-static int pool_backward(int dtype, const void *x, void *dx, const void *dy, const PoolGeom &g, hipStream_t s) {
+static int pool_backward(int dtype, const void *x, void *dx, const void *dy, const PoolGeom &g, hipStream_t s, float keep) {
     const long pixels = (long)g.B * g.IH * g.IW;
     const bool al = (((size_t)x | (size_t)dx | (size_t)dy) & 15) == 0;
     if (dtype == D8_FLOAT32) {
-        if (al && g.C % 4 == 0) hipLaunchKernelGGL((pool_backward_kernel<float, 4, MAX>), dim3(pool_grid(pixels * g.C / 4)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, pixels * g.C / 4);
-        else hipLaunchKernelGGL((pool_backward_kernel<float, 1, MAX>), dim3(pool_grid(pixels * g.C)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, pixels * g.C);
+        if (al && g.C % 4 == 0) hipLaunchKernelGGL((pool_backward_kernel<float, 4, MAX>), dim3(pool_grid(pixels * g.C / 4)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, pixels * g.C / 4, keep);
+        else hipLaunchKernelGGL((pool_backward_kernel<float, 1, MAX>), dim3(pool_grid(pixels * g.C)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, pixels * g.C, keep);
     } else {
-        if (al && g.C % 8 == 0) hipLaunchKernelGGL((pool_backward_kernel<f16, 8, MAX>), dim3(pool_grid(pixels * g.C / 8)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, g, pixels * g.C / 8);
-        else hipLaunchKernelGGL((pool_backward_kernel<f16, 1, MAX>), dim3(pool_grid(pixels * g.C)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, g, pixels * g.C);
+        if (al && g.C % 8 == 0) hipLaunchKernelGGL((pool_backward_kernel<f16, 8, MAX>), dim3(pool_grid(pixels * g.C / 8)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, g, pixels * g.C / 8, keep);
+        else hipLaunchKernelGGL((pool_backward_kernel<f16, 1, MAX>), dim3(pool_grid(pixels * g.C)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, g, pixels * g.C, keep);
     }
     D8_LAUNCH_CHECK();
     return 0;
@@ -197,7 +200,15 @@ int d8_maxpool2d_grad(int dtype, const void *x, void *dx, const void *dy, int B,
     PoolGeom g;
     if (int rc = pool_geometry("d8_maxpool2d_grad", dtype, B, IH, IW, C, FH, FW, covered, sy, sx, g)) return rc;
     D8_REQUIRE(x && dx && dy, "d8_maxpool2d_grad: null tensor");
-    return pool_backward<true>(dtype, x, dx, dy, g, as_stream(stream));
+    return pool_backward<true>(dtype, x, dx, dy, g, as_stream(stream), 1.f);
+}
+
+int d8_maxpool2d_grad_overwrite(int dtype, const void *x, void *dx, const void *dy, int B, int IH, int IW, int C, int FH, int FW,
+                                int covered, int sy, int sx, void *stream) {
+    PoolGeom g;
+    if (int rc = pool_geometry("d8_maxpool2d_grad_overwrite", dtype, B, IH, IW, C, FH, FW, covered, sy, sx, g)) return rc;
+    D8_REQUIRE(x && dx && dy, "d8_maxpool2d_grad_overwrite: null tensor");
+    return pool_backward<true>(dtype, x, dx, dy, g, as_stream(stream), 0.f);
 }
 
 int d8_avgpool2d(int dtype, const void *x, void *y, int B, int IH, int IW, int C, int FH, int FW, int covered, int sy, int sx,
@@ -213,7 +224,15 @@ int d8_avgpool2d_grad(int dtype, void *dx, const void *dy, int B, int IH, int IW
     PoolGeom g;
     if (int rc = pool_geometry("d8_avgpool2d_grad", dtype, B, IH, IW, C, FH, FW, covered, sy, sx, g)) return rc;
     D8_REQUIRE(dx && dy, "d8_avgpool2d_grad: null tensor");
-    return pool_backward<false>(dtype, dx, dx, dy, g, as_stream(stream));
+    return pool_backward<false>(dtype, dx, dx, dy, g, as_stream(stream), 1.f);
+}
+
+int d8_avgpool2d_grad_overwrite(int dtype, void *dx, const void *dy, int B, int IH, int IW, int C, int FH, int FW, int covered,
+                                int sy, int sx, void *stream) {
+    PoolGeom g;
+    if (int rc = pool_geometry("d8_avgpool2d_grad_overwrite", dtype, B, IH, IW, C, FH, FW, covered, sy, sx, g)) return rc;
+    D8_REQUIRE(dx && dy, "d8_avgpool2d_grad_overwrite: null tensor");
+    return pool_backward<false>(dtype, dx, dx, dy, g, as_stream(stream), 0.f);
 }
 
 }  // extern "C"

@@ -345,7 +345,8 @@ void addGradGPU(Tensor &g, const Tensor &dz) {
     const Dims5 ga = enlargeShapeToMaxDim(g.shape), za = enlargeShapeToMaxDim(dz.shape);
     const int dt = dtypeOf(g);
     PoolScratch ws(g.device(), d8_add_grad_scratch_bytes(dt, ga.d, za.d));
-    D8_CHECK(d8_add_grad(dt, g.raw(), ga.d, dz.raw(), za.d, ws.ptr, ws.bytes, nullptr));
+    const bool fresh = g.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_add_grad_overwrite : d8_add_grad)(dt, g.raw(), ga.d, dz.raw(), za.d, ws.ptr, ws.bytes, nullptr));
 }
 
 }  // namespace
@@ -416,7 +417,8 @@ void ReLuGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &dy) {
 }
 
 void ReLuGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy) {
-    D8_CHECK(d8_relu_grad(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), (long)x.shape.size(), nullptr));
+    const bool fresh = dx.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_relu_grad_overwrite : d8_relu_grad)(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), (long)x.shape.size(), nullptr));
 }
 
 // ---- Minus / L1Norm / L2Norm / ReduceMean / AXPBY ---------------------------------------------------------------
@@ -661,7 +663,9 @@ void MaxPooling2dGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor
     MaxPooling2dGradGPU(x, dx, y, dy, POOL_ARGS);
 }
 void MaxPooling2dGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
-    D8_CHECK(d8_maxpool2d_grad(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), POOL_DIMS(x), filterHeight, filterWidth, covered, strideY, strideX, nullptr));
+    const bool fresh = dx.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_maxpool2d_grad_overwrite : d8_maxpool2d_grad)(dtypeOf(x), x.raw(), dx.raw(), dy.raw(), POOL_DIMS(x), filterHeight, filterWidth,
+                                                                      covered, strideY, strideX, nullptr));
 }
 void AvgPooling2d(const Tensor &x, Tensor &y, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
     checkPool(x, y, POOL_ARGS);
@@ -675,7 +679,9 @@ void AvgPooling2dGrad(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor
     AvgPooling2dGradGPU(x, dx, y, dy, POOL_ARGS);
 }
 void AvgPooling2dGradGPU(const Tensor &x, Tensor &dx, const Tensor &, const Tensor &dy, bool covered, int filterHeight, int filterWidth, int strideY, int strideX) {
-    D8_CHECK(d8_avgpool2d_grad(dtypeOf(x), dx.raw(), dy.raw(), POOL_DIMS(x), filterHeight, filterWidth, covered, strideY, strideX, nullptr));
+    const bool fresh = dx.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK((fresh ? d8_avgpool2d_grad_overwrite : d8_avgpool2d_grad)(dtypeOf(x), dx.raw(), dy.raw(), POOL_DIMS(x), filterHeight, filterWidth, covered,
+                                                                      strideY, strideX, nullptr));
 }
 #undef POOL_ARGS
 #undef POOL_DIMS

@@ -287,8 +287,9 @@ def add(x, y):
     return dz_.numpy()
 
 
-def add_grad(g, dz, use_scratch=True):
-    """returns g + dz summed over the axes g is broadcast along (g: (batch, dims..), right-aligned to dz)"""
+def add_grad(g, dz, use_scratch=True, overwrite=False):
+    """returns g + dz summed over the axes g is broadcast along (g: (batch, dims..), right-aligned to dz);
+    overwrite: g's contents are ignored"""
     lib = capi.init()
     g, dz = np.ascontiguousarray(g), np.ascontiguousarray(dz)
     dt = _same_dtype(g, dz)
@@ -297,7 +298,8 @@ def add_grad(g, dz, use_scratch=True):
     dg, ddz = DeviceArray.from_numpy(g), DeviceArray.from_numpy(dz)
     nb = lib.d8_add_grad_scratch_bytes(dt, gd, zd) if use_scratch else 0
     ws = _scratch(nb)
-    check(lib.d8_add_grad(dt, dg.ptr, gd, ddz.ptr, zd, ws.ptr if nb else None, nb, None))
+    fn = lib.d8_add_grad_overwrite if overwrite else lib.d8_add_grad
+    check(fn(dt, dg.ptr, gd, ddz.ptr, zd, ws.ptr if nb else None, nb, None))
     return dg.numpy()
 
 
@@ -309,13 +311,13 @@ def relu(x):
     return dy_.numpy()
 
 
-def relu_grad(x, dy, dx=None):
+def relu_grad(x, dy, dx=None, overwrite=False):
     lib = capi.init()
     x, dy = np.ascontiguousarray(x), np.ascontiguousarray(dy)
     dt = _same_dtype(x, dy)
     dx = np.zeros_like(x) if dx is None else np.ascontiguousarray(dx)
     a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
-    check(lib.d8_relu_grad(dt, a.ptr, b.ptr, c.ptr, x.size, None))
+    check((lib.d8_relu_grad_overwrite if overwrite else lib.d8_relu_grad)(dt, a.ptr, b.ptr, c.ptr, x.size, None))
     return b.numpy()
 
 
@@ -456,7 +458,7 @@ def avgpool2d(x, FH, FW, covered=False, sy=1, sx=1):
     return _pool("avg", x, FH, FW, covered, sy, sx)
 
 
-def maxpool2d_grad(x, dy, FH, FW, covered=False, sy=1, sx=1, dx=None):
+def maxpool2d_grad(x, dy, FH, FW, covered=False, sy=1, sx=1, dx=None, overwrite=False):
     """returns dx + the gradient of maxpool2d at x"""
     lib = capi.init()
     x, dy = np.ascontiguousarray(x), np.ascontiguousarray(dy)
@@ -464,16 +466,18 @@ def maxpool2d_grad(x, dy, FH, FW, covered=False, sy=1, sx=1, dx=None):
     dx = np.zeros_like(x) if dx is None else np.ascontiguousarray(dx)
     B, IH, IW, C = x.shape
     a, b, c = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
-    check(lib.d8_maxpool2d_grad(dt, a.ptr, b.ptr, c.ptr, B, IH, IW, C, FH, FW, int(covered), sy, sx, None))
+    fn = lib.d8_maxpool2d_grad_overwrite if overwrite else lib.d8_maxpool2d_grad
+    check(fn(dt, a.ptr, b.ptr, c.ptr, B, IH, IW, C, FH, FW, int(covered), sy, sx, None))
     return b.numpy()
 
 
-def avgpool2d_grad(xshape, dy, FH, FW, covered=False, sy=1, sx=1, dx=None):
+def avgpool2d_grad(xshape, dy, FH, FW, covered=False, sy=1, sx=1, dx=None, overwrite=False):
     lib = capi.init()
     dy = np.ascontiguousarray(dy)
     dx = np.zeros(xshape, dy.dtype) if dx is None else np.ascontiguousarray(dx)
     dt = _same_dtype(dx, dy)
     B, IH, IW, C = dx.shape
     b, c = DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
-    check(lib.d8_avgpool2d_grad(dt, b.ptr, c.ptr, B, IH, IW, C, FH, FW, int(covered), sy, sx, None))
+    fn = lib.d8_avgpool2d_grad_overwrite if overwrite else lib.d8_avgpool2d_grad
+    check(fn(dt, b.ptr, c.ptr, B, IH, IW, C, FH, FW, int(covered), sy, sx, None))
     return b.numpy()

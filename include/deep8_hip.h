@@ -224,6 +224,12 @@ int d8_add_grad(int dtype, void *g, const int *gdims, const void *dz, const int 
                 void *scratch, size_t scratch_bytes, void *stream);
 int d8_relu(int dtype, const void *x, void *y, long n, void *stream);
 int d8_relu_grad(int dtype, const void *x, void *dx, const void *dy, long n, void *stream);
+/* Overwrite forms of the two gradients: the destination's old contents are not read (what "zero the
+ * gradient, then accumulate" leaves, deep8/src/model/EagerExecutor.cpp:51-65, without the fill and
+ * the read-back).                                                                                   */
+int d8_add_grad_overwrite(int dtype, void *g, const int *gdims, const void *dz, const int *zdims,
+                          void *scratch, size_t scratch_bytes, void *stream);
+int d8_relu_grad_overwrite(int dtype, const void *x, void *dx, const void *dy, long n, void *stream);
 
 /* ---- Minus, L1Norm / L2Norm, ReduceMean, AXPBY ------------------------------------------------
  * What a loss and a trainer step need on top of the operators above.  Shapes as for d8_add.
@@ -288,6 +294,11 @@ int d8_avgpool2d(int dtype, const void *x, void *y, int B, int IH, int IW, int C
                  int FH, int FW, int covered, int sy, int sx, void *stream);
 int d8_avgpool2d_grad(int dtype, void *dx, const void *dy, int B, int IH, int IW, int C,
                       int FH, int FW, int covered, int sy, int sx, void *stream);
+/* The two pooling gradients written over dx instead of added to it (see d8_relu_grad_overwrite). */
+int d8_maxpool2d_grad_overwrite(int dtype, const void *x, void *dx, const void *dy, int B, int IH, int IW, int C,
+                                int FH, int FW, int covered, int sy, int sx, void *stream);
+int d8_avgpool2d_grad_overwrite(int dtype, void *dx, const void *dy, int B, int IH, int IW, int C,
+                                int FH, int FW, int covered, int sy, int sx, void *stream);
 
 /* ---- measurement aid (no counterpart in the reference) ---------------------------------------
  * d8_mfma_stream issues the tiled GEMM's MFMA instruction back to back on operands taken from

@@ -50,6 +50,9 @@ def test_add_forward_and_gradients(oracle_port, xs, ys, dtype):
         assert dtype == np.float32 or np.abs(w).max() < 2048
         for use_scratch in (True, False):
             assert np.array_equal(f(ops.add_grad(c(g0), c(dz), use_scratch)), w), (like.shape, use_scratch)
+            # the overwrite form never reads what the destination held
+            nan = np.full(g0.shape, np.nan, dtype)
+            assert np.array_equal(f(ops.add_grad(nan, c(dz), use_scratch, overwrite=True)), w - g0), (like.shape, use_scratch)
     # reals within tolerance
     dzr = c(nrm(r, want.shape))
     tol = FP16_TOL if dtype == np.float16 else FP32_TOL
@@ -73,6 +76,8 @@ def test_relu_forward_and_gradient(oracle_port, shape, dtype):
     dy, dx0 = c(nrm(r, shape)), c(nrm(r, shape))
     want = oracle_port.relu_grad(f(x), f(dy), f(dx0))
     assert np.array_equal(ops.relu_grad(x, dy, dx0), want.astype(dtype))
+    nan = np.full(shape, np.nan, dtype)
+    assert np.array_equal(ops.relu_grad(x, dy, nan, overwrite=True), oracle_port.relu_grad(f(x), f(dy)).astype(dtype))
 
 
 def test_full_size_bias_and_relu_after_config4(oracle_port):

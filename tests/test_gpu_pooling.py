@@ -32,6 +32,9 @@ def test_pooling_forward_and_gradients(oracle_port, cfg, dtype):
     OH, OW = oracle_port.pool2d(True, f(xi), *a).shape[1:3]
     dy, dx0 = c(ints(r, (B, OH, OW, C), 4)), c(ints(r, (B, IH, IW, C), 4))
     assert np.array_equal(f(ops.maxpool2d_grad(xi, dy, *a, dx=dx0)), oracle_port.pool2d_grad(True, f(xi), f(dy), *a, dx=f(dx0)))
+    nan = np.full(xi.shape, np.nan, dtype)  # the overwrite forms never read what the destination held
+    assert np.array_equal(f(ops.maxpool2d_grad(xi, dy, *a, dx=nan, overwrite=True)), oracle_port.pool2d_grad(True, f(xi), f(dy), *a))
+    assert np.array_equal(f(ops.avgpool2d_grad(xi.shape, c(np.zeros((B, OH, OW, C))), *a, dx=nan, overwrite=True)), np.zeros(xi.shape, np.float32))
     dyr = c(nrm(r, (B, OH, OW, C)))
     assert rel_fro(f(ops.avgpool2d_grad(x.shape, dyr, *a, dx=dx0)), oracle_port.pool2d_grad(False, f(x), f(dyr), *a, dx=f(dx0))) <= tol
     assert rel_fro(f(ops.maxpool2d_grad(x, dyr, *a)), oracle_port.pool2d_grad(True, f(x), f(dyr), *a)) <= tol
