@@ -463,6 +463,50 @@ def calibrate_copy(mib):
     print(json.dumps({"copy_kernel": "im2col_kernel (1x1 filter)", "bytes_read": rows * 256, "bytes_written": rows * 256}))
 
 
+def phase_record(launches=12):
+    """The fp16 4096^3 launches of workload c3 with the kernel's own phase record switched on (D8_GEMM_STAMPS):
+    every workgroup notes the wall clock (100 MHz, common to the chip) at its start, after its prologue, after
+    its K loop and after its last store was acknowledged, and the shader clock around the loop.  Prints, per
+    product, the phases in microseconds and the shader clock per XCD (workgroup id mod 8).  A diagnostic: it
+    shows how much of a launch is the loop and at which clock the loop runs on the config's data."""
+    from deep8_amd import capi
+    lib = capi.init()
+    wl = make_workload("c3")
+    n = 4096
+    forms = (("forward NN", 0, 0, wl.x, wl.y), ("dX NT", 0, 1, wl.dz, wl.y), ("dY TN", 1, 0, wl.x, wl.dz))
+    out = capi.DeviceArray((n, n), np.float16)
+    recs = [capi.DeviceArray((256 * 6,), np.uint64, zero=True) for _ in range(launches)]
+    for name, ta, tb, A, B in forms:
+        def launch(i):
+            capi.check(lib.d8_gemm(wl.dt, ta, tb, n, n, n, A.ptr, n, 0, B.ptr, n, 0, 0.0, out.ptr, n, 0, 1,
+                                   recs[i].ptr, 256 * 6 * 8, None))
+        for i in range(launches):
+            launch(i)
+        capi.sync()
+        t = capi.Timer(None)
+        t.start()
+        for i in range(launches):
+            launch(i)
+        ms = t.stop_ms() / launches
+        d = [r.numpy().astype(np.int64).reshape(256, 6) for r in recs]
+        if not d[-1][:, 3].all():
+            raise SystemExit("no phase record was written: is D8_GEMM_STAMPS set and does the product take gemm_wide_kernel?")
+        print("%s: %.1f us per launch by HIP events over %d launches (%.0f TFLOP/s)" % (name, ms * 1e3, launches, 2.0 * n**3 / ms / 1e9))
+        r = d[-1]
+        t0 = r[:, 0].min()
+        us = lambda v: v / 100.0
+        pro, loop, epi = us(r[:, 1] - r[:, 0]), us(r[:, 2] - r[:, 1]), us(r[:, 3] - r[:, 2])
+        ghz = (r[:, 5] - r[:, 4]) / (loop * 1e3)
+        gap = us(r[:, 0].min() - d[-2][:, 3].max())
+        print("  last launch: prologue %.1f us, loop %.1f-%.1f (mean %.1f), epilogue until the last store is acknowledged "
+              "%.1f-%.1f; last workgroup done %.1f us after the first started; %.1f us from the end of the previous launch "
+              "to the first workgroup of this one" % (pro.mean(), loop.min(), loop.max(), loop.mean(), epi.min(), epi.max(),
+                                                      us(r[:, 3].max() - t0), gap))
+        print("  shader clock during the loop, per XCD: " + ", ".join(
+            "%.2f" % ghz[np.arange(256) % 8 == x].mean() for x in range(8)) + " GHz; cycles per K step %.0f" % (
+            (r[:, 5] - r[:, 4]).mean() / (n // 64)))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -477,6 +521,8 @@ def main():
     ap.add_argument("--eager-zero", action="store_true",
                     help="zero-fill the gradients and accumulate (the reference's literal "
                          "sequence) instead of the executor's deferred zeroing + overwrite")
+    ap.add_argument("--phases", action="store_true",
+                    help="only print the phase record of workload c3's three products (see phase_record)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
@@ -487,10 +533,14 @@ def main():
         raise SystemExit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, "
                          "no second device anywhere in the path)" % a.gpus)
 
+    if a.phases:
+        os.environ["D8_GEMM_STAMPS"] = "1"  # read by the library at its first launch
     from deep8_amd import capi
     capi.init()
     if a.calibrate_copy:
         return calibrate_copy(a.calibrate_copy)
+    if a.phases:
+        return phase_record()
 
     wl = make_workload(a.workload)
     ms = _time_steps(wl.step, a.steps, a.warmup)

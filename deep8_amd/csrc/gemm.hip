@@ -386,6 +386,7 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     g.B = B;
     g.C = C;
     g.ws = (float *)workspace;
+    g.ws_bytes = workspace_bytes;
     g.M = M;
     g.N = N;
     g.K = K;

@@ -67,6 +67,10 @@ struct GemmArgs {
     // perm_OC > 0: the result is stored transposed per filter tap: element (m, n = t * perm_OC + oc) of the
     // product goes to C[(oc * perm_T + t) * ldc + m] (a filter gradient [OC][taps][IC] computed as [IC][taps x OC])
     int perm_T, perm_OC;
+    // measurement aid (gemm_wide only, set by its launcher when the environment asks for it and a workspace
+    // is given): every workgroup records when its prologue, K loop and epilogue ended into ws
+    int stamps;
+    size_t ws_bytes;  // size of ws as d8_gemm received it (0 where a planner filled the block in)
 };
 
 // Tiled kernels (fp16 and fp32) for shapes whose operands can be moved in 16-byte pieces.

@@ -136,6 +136,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // optional phase record: wall clock (100 MHz, the same on every CU) and shader clock
+    unsigned long long wall[4] = {0, 0, 0, 0}, clk[2] = {0, 0};
+    if (g.stamps) wall[0] = wall_clock64();
     const int wm = wave >> 1, wn = wave & 1;
 
     // ---- which tile: the workgroups of one XCD (ids congruent mod 8) take a contiguous run of
@@ -192,6 +195,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces are in LDS
     __syncthreads();
+    if (g.stamps) wall[1] = wall_clock64(), clk[0] = __builtin_readcyclecounter();
 #pragma unroll
     for (int n = 0; n < 8; ++n) {
         fb[0][n] = ob.read(lds + OPERAND_BYTES, 0, n);
@@ -248,6 +252,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
 
     // ---- epilogue: 16 rows of the wave's 128 x 128 at a time through a patch of LDS, so that C
     // is read (beta = 1) and written 16 bytes per lane, 256 contiguous bytes per 16 lanes
+    if (g.stamps) wall[2] = wall_clock64(), clk[1] = __builtin_readcyclecounter();
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();  // no load is still on its way into LDS, every wave is past its last read
     float *patch = (float *)lds + wave * (16 * PATCH_LD);
@@ -283,6 +288,14 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
             }
         }
     }
+    if (g.stamps) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // this wave's stores have been acknowledged
+        wall[3] = wall_clock64();
+        if (tid == 0) {
+            unsigned long long *rec = (unsigned long long *)g.ws + 6 * (blockIdx.x + gridDim.x * blockIdx.z);
+            rec[0] = wall[0], rec[1] = wall[1], rec[2] = wall[2], rec[3] = wall[3], rec[4] = clk[0], rec[5] = clk[1];
+        }
+    }
 }
 
 bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB) {
@@ -296,7 +309,14 @@ bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB) {
     return true;
 }
 
-int gemm_wide_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
+size_t gemm_wide_stamp_bytes(const GemmArgs &g) {
+    return (size_t)ceil_div(g.M, 256) * ceil_div(g.N, 256) * g.batch * 6 * sizeof(unsigned long long);
+}
+
+int gemm_wide_launch(const GemmArgs &g0, int transA, int transB, hipStream_t stream) {
+    static const bool stamps = getenv("D8_GEMM_STAMPS") != nullptr;  // measurement aid, see GemmArgs::stamps
+    GemmArgs g = g0;
+    g.stamps = stamps && g.ws && ((size_t)g.ws & 7) == 0 && g.ws_bytes >= gemm_wide_stamp_bytes(g);
     const int tilesM = ceil_div(g.M, 256), tilesN = ceil_div(g.N, 256);
     const dim3 grid(tilesM * tilesN, 1, g.batch), block(256);
     if (!transA && !transB) hipLaunchKernelGGL((gemm_wide_kernel<true, false>), grid, block, 0, stream, g, tilesM, tilesN);
