@@ -306,6 +306,11 @@ int d8_avgpool2d_grad_overwrite(int dtype, void *dx, const void *dy, int B, int 
  * every CU, no LDS or global traffic in the loop.  Timing one launch gives the rate the matrix
  * pipe sustains on those operand bits, i.e. the ceiling a GEMM has on that data.  `out` takes
  * d8_mfma_stream_out_bytes() bytes; *flops receives the flops one launch performs.             */
+/* A second aid needs no entry point: with D8_GEMM_STAMPS set in the environment before the first launch, a
+ * d8_gemm call that runs the large-output fp16 kernel and is given an 8-byte aligned workspace of at least
+ * 48 bytes per 256 x 256 tile of C leaves there, per workgroup, six 64-bit values: the chip's 100 MHz wall
+ * clock at its start, after its prologue, after its K loop and after its last store was acknowledged, and
+ * the shader clock before and after the loop.                                                          */
 size_t d8_mfma_stream_out_bytes(void);
 int d8_mfma_stream(int dtype, const void *operands, size_t operand_bytes, void *out, int iters,
                    double *flops, void *stream);
