@@ -172,6 +172,112 @@ __device__ inline long c_index(const GemmArgs &g, int m, int n) {
     return (long)m * g.ldc + n;
 }
 
+// ------------------------------------------------------------------------------------------
+// Small products: a handful of 128 x 128 tiles would leave the chip to a few workgroups, each
+// walking its whole reduction at one MFMA per 64 (fp32) cycles behind one load latency per K step.
+// Here a workgroup owns a 32 x 32 tile of C and its four waves take every fourth chunk of the
+// reduction each (8 k values for fp32, 16 for fp16: one MFMA operand per lane).  A lane fetches
+// its operand values of ALL its chunks straight from global memory into registers before the
+// first MFMA, so the whole product costs one load latency; the four partial tiles meet in LDS in
+// wave order, so the result does not depend on scheduling.  Any M, N, K, leading dimension and
+// alignment; element-wise, bounds-checked loads.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+struct SmallOp;
+template <>
+struct SmallOp<float> {
+    static constexpr int PER = 4, KG = 8, MAXC = 16;  // values per lane and chunk, k per chunk, chunks per wave
+    typedef f32x4 Frag;
+    __device__ static void mma(const Frag &a, const Frag &b, f32x16 &acc) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+    }
+};
+template <>
+struct SmallOp<f16> {
+    static constexpr int PER = 8, KG = 16, MAXC = 8;
+    typedef f16x8 Frag;
+    __device__ static void mma(const Frag &a, const Frag &b, f32x16 &acc) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+    }
+};
+
+template <typename T, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
+    typedef SmallOp<T> OP;
+    constexpr int BT = 32, PER = OP::PER, KG = OP::KG, MAXC = OP::MAXC;
+    __shared__ float part[3][BT * BT];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int b = blockIdx.z;
+    const int gm = blockIdx.y * BT + l32, gn = blockIdx.x * BT + l32;  // this lane's row of A and column of B
+    const int kchunks = (g.K + KG - 1) / KG, total = g.red * kchunks;   // total <= 4 * MAXC (gemm_is_small)
+
+    // a K-contiguous operand whose rows can be read 16 bytes at a time gives a lane its values in one load
+    const bool vec_a = !TA && g.lda % PER == 0 && g.sA % PER == 0 && g.K % PER == 0 && ((size_t)g.A & 15) == 0;
+    const bool vec_b = TB && g.ldb % PER == 0 && g.sB % PER == 0 && g.K % PER == 0 && ((size_t)g.B & 15) == 0;
+    typename OP::Frag fa[MAXC], fb[MAXC];
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        const int t = wave + 4 * c;
+#pragma unroll
+        for (int e = 0; e < PER; ++e) fa[c][e] = (T)0, fb[c][e] = (T)0;
+        if (t < total) {
+            const int r = t / kchunks, k0 = (t - r * kchunks) * KG + lhi * PER;
+            const T *Ap = (const T *)g.A + (long)(b + r) * g.sA;
+            const T *Bp = (const T *)g.B + (long)(b + r) * g.sB;
+            if (vec_a) {
+                if (gm < g.M && k0 < g.K) fa[c] = *(const typename OP::Frag *)(Ap + (long)gm * g.lda + k0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < PER; ++e)
+                    if (gm < g.M && k0 + e < g.K) fa[c][e] = TA ? Ap[(long)(k0 + e) * g.lda + gm] : Ap[(long)gm * g.lda + k0 + e];
+            }
+            if (vec_b) {
+                if (gn < g.N && k0 < g.K) fb[c] = *(const typename OP::Frag *)(Bp + (long)gn * g.ldb + k0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < PER; ++e)
+                    if (gn < g.N && k0 + e < g.K) fb[c][e] = TB ? Bp[(long)gn * g.ldb + k0 + e] : Bp[(long)(k0 + e) * g.ldb + gn];
+            }
+        }
+    }
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c)
+        if (wave + 4 * c < total) OP::mma(fa[c], fb[c], acc);
+
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part[wave - 1][((r >> 2) * 8 + lhi * 4 + (r & 3)) * BT + l32] = acc[r];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = (r >> 2) * 8 + lhi * 4 + (r & 3), m = blockIdx.y * BT + row;
+            float v = acc[r];
+#pragma unroll
+            for (int w = 0; w < 3; ++w) v += part[w][row * BT + l32];
+            if (m < g.M && gn < g.N) {
+                T *c = (T *)g.C + (long)b * g.sC + (long)m * g.ldc + gn;
+                if (g.beta != 0.f) v += to_f32(*c);
+                *c = (T)v;
+            }
+        }
+    }
+}
+
+// Whether a product is small in the sense above: at most four 128 x 128 tiles of output and a reduction of
+// at most 512 (summed products included) in at most 64 chunks of 8.
+static bool gemm_is_small(int M, int N, int K, int batch, int red) {
+    return (long)ceil_div(M, 128) * ceil_div(N, 128) * batch <= 4 && (long)K * red <= 512 && (long)red * ceil_div(K, 8) <= 64 &&
+           batch * 1L < 65536;
+}
+
 // C[b][m][n] = beta * C + sum_s ws[b][s][m][n].  A workgroup covers 32 groups of 4 consecutive
 // outputs; its 8 thread rows each add every 8th partial (16-byte loads), and the 8 sums meet in
 // LDS in a fixed order, so the result does not depend on scheduling.
@@ -236,6 +342,10 @@ bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps) {
 static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t workspace_bytes, int *tiles_per_split) {
     const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
     const long total = (long)red * ceil_div(K, BK);
+    if (gemm_is_small(M, N, K, batch, red)) {  // runs whole on gemm_small_kernel
+        *tiles_per_split = (int)total;
+        return 1;
+    }
     const int cus = cu_count();
     long splits = 1;
     if (tiles < cus) splits = 2L * cus / tiles;  // at most two workgroups per CU: a third one would run alone, after the rest
@@ -264,6 +374,17 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
 
 template <typename T>
 static int launch(GemmArgs &g, int transA, int transB, bool tiled, hipStream_t stream) {
+    if (g.virt == VIRT_NONE && g.splits == 1 && gemm_is_small(g.M, g.N, g.K, g.batch, g.red)) {
+        dim3 grid(ceil_div(g.N, 32), ceil_div(g.M, 32), g.batch);
+        if (!transA && !transB)
+            hipLaunchKernelGGL((gemm_small_kernel<T, false, false>), grid, dim3(256), 0, stream, g);
+        else if (!transA && transB)
+            hipLaunchKernelGGL((gemm_small_kernel<T, false, true>), grid, dim3(256), 0, stream, g);
+        else
+            hipLaunchKernelGGL((gemm_small_kernel<T, true, false>), grid, dim3(256), 0, stream, g);
+        D8_LAUNCH_CHECK();
+        return 0;
+    }
     if (tiled) {
         if (int rc = gemm_tiled_launch(sizeof(T) == 2 ? D8_FLOAT16 : D8_FLOAT32, g, transA, transB, stream)) return rc;
     } else {
