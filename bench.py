@@ -94,9 +94,10 @@ class MatMulWorkload:
         m, k, n = xs[1], xs[2], ys[2]
         self.flops = 3 * 2.0 * zb * m * k * n
         wide = self.dtype == np.float16 and m >= 256 and n >= 256 and k % 64 == 0 and zb * (-(-m // 256)) * (-(-n // 256)) >= 192
+        small = zb * (-(-m // 128)) * (-(-n // 128)) <= 4 and max(m, n, k) * (zb if 1 in (xs[0], ys[0]) else 1) <= 512
         self.kernel = "%s (one launch each for fwd, dX, dY)" % (
             "gemm_wide_kernel (fp16, 256x256 tiles)" if wide else
-            "gemm_tiled_kernel<%s>" % ("f16" if self.dtype == np.float16 else "f32"))
+            "gemm_%s_kernel<%s>" % ("small" if small else "tiled", "f16" if self.dtype == np.float16 else "f32"))
         es = self.dtype.itemsize
         nx, ny, nz = np.prod(xs), np.prod(ys), np.prod(self.zs)
         # fwd reads x,y writes z; dX reads dz,y and read-modify-writes dx; dY likewise
