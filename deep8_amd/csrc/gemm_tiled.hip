@@ -26,6 +26,13 @@
 // Workgroup ids are remapped so that the workgroups one XCD receives (ids congruent mod 8) cover
 // a compact block of tiles and share A / B panels in that XCD's L2.  The epilogue turns each
 // 32 x 32 accumulator block around through LDS so that C is read and written 16 bytes per lane.
+//
+// An operand may be a patch matrix that is never written out (GemmArgs::virt): its loader turns
+// row / column numbers into image offsets, and an offset outside the image makes the buffer load
+// return zeros, which is the padding.  That carries the convolutions: Conv2d forward and its two
+// gradients, DeConv2d's gradient of x and of the filter, and -- one residue class of output
+// pixels per grid layer (OutClass) -- DeConv2d forward and Conv2d's gradient of x for strides
+// above 1, whose rows of C are then pixels of the output image rather than consecutive rows.
 #include "gemm_args.h"
 
 namespace d8 {
