@@ -78,6 +78,7 @@ class MatMulWorkload:
         from deep8_amd import capi
         self.name, self.dtype = name, np.dtype(dtype)
         self.lib = capi.init()
+        self.stream = None  # a hipStream_t as an integer, or None for the default stream
         self.dt = capi.dtype_id(self.dtype)
         r = np.random.default_rng(seed)
         self.xs, self.ys = xs, ys
@@ -106,27 +107,27 @@ class MatMulWorkload:
     def fwd(self):
         from deep8_amd.capi import check
         check(self.lib.d8_matmul(self.dt, self.x.ptr, *self.xs, self.y.ptr, *self.ys, self.z.ptr,
-                                 self.ws.ptr, self.ws_bytes, None))
+                                 self.ws.ptr, self.ws_bytes, self.stream))
 
     def grad_x(self):
         from deep8_amd.capi import check
         check(self.lib.d8_matmul_grad_x(self.dt, self.dx.ptr, *self.xs, self.y.ptr, *self.ys, self.dz.ptr,
-                                        self.ws.ptr, self.ws_bytes, None))
+                                        self.ws.ptr, self.ws_bytes, self.stream))
 
     def grad_y(self):
         from deep8_amd.capi import check
         check(self.lib.d8_matmul_grad_y(self.dt, self.x.ptr, *self.xs, self.dy.ptr, *self.ys, self.dz.ptr,
-                                        self.ws.ptr, self.ws_bytes, None))
+                                        self.ws.ptr, self.ws_bytes, self.stream))
 
     def grad_x_first(self):
         from deep8_amd.capi import check
         check(self.lib.d8_matmul_grad_x_overwrite(self.dt, self.dx.ptr, *self.xs, self.y.ptr, *self.ys, self.dz.ptr,
-                                                  self.ws.ptr, self.ws_bytes, None))
+                                                  self.ws.ptr, self.ws_bytes, self.stream))
 
     def grad_y_first(self):
         from deep8_amd.capi import check
         check(self.lib.d8_matmul_grad_y_overwrite(self.dt, self.x.ptr, *self.xs, self.dy.ptr, *self.ys, self.dz.ptr,
-                                                  self.ws.ptr, self.ws_bytes, None))
+                                                  self.ws.ptr, self.ws_bytes, self.stream))
 
     def step(self):
         """One forward + backward of a MatrixMultiply node as the executor issues it: forward, then the
@@ -464,6 +465,38 @@ def calibrate_copy(mib):
     print(json.dumps({"copy_kernel": "im2col_kernel (1x1 filter)", "bytes_read": rows * 256, "bytes_written": rows * 256}))
 
 
+def graph_replay_ms(wl, steps, warmup):
+    """ms per step of a MatrixMultiply workload whose step is captured once into a HIP graph (d8_graph_begin /
+    d8_graph_end) and replayed: what a caller gets who removes the per-launch latency of a small product that way."""
+    import ctypes
+    from deep8_amd import capi
+    lib = capi.init()
+    capi.sync()
+    side, graph = ctypes.c_void_p(), ctypes.c_void_p()
+    capi.check(lib.d8_stream_create(ctypes.byref(side)))
+    wl.stream = side
+    try:
+        for _ in range(3):
+            wl.step()
+        capi.sync(side)
+        capi.check(lib.d8_graph_begin(side))
+        wl.step()
+        capi.check(lib.d8_graph_end(side, ctypes.byref(graph)))
+        for _ in range(warmup):
+            capi.check(lib.d8_graph_launch(graph, side))
+        capi.sync(side)
+        t = capi.Timer(side)
+        t.start()
+        for _ in range(steps):
+            capi.check(lib.d8_graph_launch(graph, side))
+        return t.stop_ms() / steps
+    finally:
+        wl.stream = None
+        capi.sync(side)
+        lib.d8_graph_destroy(graph)
+        lib.d8_stream_destroy(side)
+
+
 def phase_record(launches=12):
     """The fp16 4096^3 launches of workload c3 with the kernel's own phase record switched on (D8_GEMM_STAMPS):
     every workgroup notes the wall clock (100 MHz, common to the chip) at its start, after its prologue, after
@@ -593,6 +626,8 @@ def main():
                  "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
             if isinstance(wl, (ConvWorkload, BiasReluWorkload, PoolWorkload)):
                 o["images_per_s"] = round(wl.B / (oms * 1e-3), 1)
+            if key == "c1":  # launch-latency bound: the same three launches replayed from a HIP graph
+                o["ms_per_step_graph_replay"] = round(graph_replay_ms(wl, 50, 5), 4)
             others[key] = o
         out["others"] = others
     print(json.dumps(out), flush=True)

@@ -39,6 +39,10 @@ SIGNATURES = {
     "d8_stream_create": (_I, [_PP]),
     "d8_stream_destroy": (_I, [_P]),
     "d8_stream_sync": (_I, [_P]),
+    "d8_graph_begin": (_I, [_P]),
+    "d8_graph_end": (_I, [_P, _PP]),
+    "d8_graph_launch": (_I, [_P, _P]),
+    "d8_graph_destroy": (_I, [_P]),
     "d8_event_create": (_I, [_PP]),
     "d8_event_destroy": (_I, [_P]),
     "d8_event_record": (_I, [_P, _P]),

@@ -196,6 +196,35 @@ int d8_event_record(void *event, void *stream) {
     return 0;
 }
 
+int d8_graph_begin(void *stream) {
+    D8_REQUIRE(stream, "d8_graph_begin: a graph is captured on a stream of its own, not on the default stream");
+    D8_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return 0;
+}
+
+int d8_graph_end(void *stream, void **graph) {
+    D8_REQUIRE(stream && graph, "d8_graph_end: null argument");
+    hipGraph_t captured = nullptr;
+    D8_HIP(hipStreamEndCapture(as_stream(stream), &captured));
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, captured, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(captured);
+    if (e != hipSuccess) return fail((int)e, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    *graph = (void *)exec;
+    return 0;
+}
+
+int d8_graph_launch(void *graph, void *stream) {
+    D8_REQUIRE(graph, "d8_graph_launch: graph is null");
+    D8_HIP(hipGraphLaunch((hipGraphExec_t)graph, as_stream(stream)));
+    return 0;
+}
+
+int d8_graph_destroy(void *graph) {
+    if (graph) D8_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+    return 0;
+}
+
 int d8_event_elapsed_ms(void *start, void *stop, float *ms) {
     D8_REQUIRE(ms, "ms is null");
     D8_HIP(hipEventSynchronize((hipEvent_t)stop));

@@ -51,6 +51,16 @@ int d8_fill(int dtype, void *ptr, size_t n, float scalar, void *stream);
 int d8_stream_create(void **stream);
 int d8_stream_destroy(void *stream);
 int d8_stream_sync(void *stream);
+/* Every entry point of this header only launches kernels on the stream it is given (no allocation, no
+ * synchronisation, no memset node), so a sequence of calls can be captured once and replayed: for products
+ * so small that the launches cost more than the arithmetic.  d8_graph_begin starts capturing on `stream`
+ * (not the default stream); the calls that follow, given the same stream, are recorded instead of run;
+ * d8_graph_end returns the instantiated graph; d8_graph_launch replays it on a stream.  No counterpart in
+ * the reference (hipStreamBeginCapture / hipStreamEndCapture / hipGraphInstantiate / hipGraphLaunch). */
+int d8_graph_begin(void *stream);
+int d8_graph_end(void *stream, void **graph);
+int d8_graph_launch(void *graph, void *stream);
+int d8_graph_destroy(void *graph);
 int d8_event_create(void **event);
 int d8_event_destroy(void *event);
 int d8_event_record(void *event, void *stream);

@@ -140,3 +140,49 @@ def test_config3_large_half_properties(oracle_port):
     t = ip(f(C), f(dC))
     assert abs(ip(f(A), f(dA)) - t) <= 2e-3 * abs(t) + 1.0
     assert abs(ip(f(B), f(dB)) - t) <= 2e-3 * abs(t) + 1.0
+
+
+def test_matmul_step_replayed_from_a_hip_graph(oracle_port):
+    """The entry points only launch kernels on the stream they are given, so a caller can capture a step into a
+    HIP graph (d8_graph_begin / d8_graph_end): three replays, with eager work and synchronisations between
+    them, must each reproduce the eager result (BASELINE config 1's shapes, integer inputs: bit-exact)."""
+    import ctypes
+    from deep8_amd import capi
+    from deep8_amd.capi import DeviceArray, check
+    lib = capi.init()
+    r = rng(2024)
+    xs, ys = (1, 64, 128), (1, 128, 256)
+    x, y = ints(r, xs), ints(r, ys)
+    dz = ints(r, (1, 64, 256))
+    want = (oracle_port.matmul(x, y), oracle_port.matmul_grad_x(x, y, dz), oracle_port.matmul_grad_y(x, y, dz))
+    dx_, dy_, ddz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray.from_numpy(dz)
+    z_, gx_, gy_ = DeviceArray((1, 64, 256), np.float32), DeviceArray(xs, np.float32), DeviceArray(ys, np.float32)
+    nb = max(lib.d8_matmul_scratch_bytes(capi.FLOAT32, w, *xs, *ys) for w in range(3))
+    ws = DeviceArray((max(nb, 16),), np.uint8)
+
+    def step(stream):
+        check(lib.d8_matmul(capi.FLOAT32, dx_.ptr, *xs, dy_.ptr, *ys, z_.ptr, ws.ptr, nb, stream))
+        gx_.zero_(stream)  # the fill is a kernel, not a memset node
+        check(lib.d8_matmul_grad_x(capi.FLOAT32, gx_.ptr, *xs, dy_.ptr, *ys, ddz.ptr, ws.ptr, nb, stream))
+        check(lib.d8_matmul_grad_y_overwrite(capi.FLOAT32, dx_.ptr, *xs, gy_.ptr, *ys, ddz.ptr, ws.ptr, nb, stream))
+
+    side, graph = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.d8_stream_create(ctypes.byref(side)))
+    assert lib.d8_graph_begin(None) == 10001  # not on the default stream
+    step(side)
+    capi.sync(side)
+    check(lib.d8_graph_begin(side))
+    step(side)
+    check(lib.d8_graph_end(side, ctypes.byref(graph)))
+    for replay in range(3):
+        for out in (z_, gx_, gy_):
+            out.copy_from(np.full(out.shape, -7.0, np.float32))
+        check(lib.d8_graph_launch(graph, side))
+        capi.sync(side)
+        got = (z_.numpy(), gx_.numpy(), gy_.numpy())
+        for g_, w_ in zip(got, want):
+            assert np.array_equal(g_, w_), replay
+        step(None)  # eager work between the replays
+        capi.sync()
+    check(lib.d8_graph_destroy(graph))
+    check(lib.d8_stream_destroy(side))
