@@ -199,3 +199,23 @@ def test_gemm_argument_errors():
     assert rc == 10001 and b"lda" in lib.d8_last_error()
     rc = lib.d8_gemm(capi.FLOAT32, 0, 0, 16, 16, 16, a.ptr, 16, 0, a.ptr, 16, 0, 0.5, a.ptr, 16, 0, 1, None, 0, None)
     assert rc == 10001 and b"beta" in lib.d8_last_error()
+
+
+def test_gemm_operand_beyond_2_gib():
+    """An operand whose byte offsets do not fit 32 bits (2.15 GB) is outside what the tiled kernels' buffer
+    descriptors address: the product must take the any-shape kernel's 64-bit addressing and still be exact
+    (integer inputs, every partial sum below 2^24)."""
+    from deep8_amd import ops
+    r = rng(31)
+    M, K, N = 16400, 32800, 64
+    A = r.integers(0, 4, size=(M, K), dtype=np.int8).astype(np.float32)
+    B = r.integers(0, 4, size=(K, N), dtype=np.int8).astype(np.float32)
+    assert A.nbytes > 2**31
+    got = ops.gemm(0, 0, A, B)
+    assert np.array_equal(got[0] if got.ndim == 3 else got, A @ B)
+    # and as the transposed operand of a TN product (rows of the result come from columns of A)
+    At = A[:4100].T.copy()                      # [K x 4100]: 538 MB, fits; the 2 GiB case again through B
+    Bbig = np.ascontiguousarray(A.T[:, :16384])  # [K x 16384] fp32 = 2.15 GB
+    got = ops.gemm(1, 0, np.ascontiguousarray(At[:, :128]), Bbig)
+    want = At[:, :128].T @ Bbig
+    assert np.array_equal(got[0] if got.ndim == 3 else got, want)
