@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--no-cpu] [--no-others]
 
 A step is one forward + both backward passes of the workload over one batch of synthetic input that
-already sits in HBM.  The headline workload is BASELINE config 3 (MatrixMultiply, half,
+already sits in HBM.  The headline workload is benchmark configuration 3 (MatrixMultiply, half,
 4096 x 4096 x 4096); the other configs are timed briefly and reported under "others".
 Prints ONE JSON line.
 

@@ -21,14 +21,14 @@ CONV = [
     (1, 9, 9, 4, 4, 3, 3, True, 2, 2, 1, 1),
     (3, 12, 12, 16, 8, 3, 3, False, 2, 2, 2, 2),
     (2, 8, 8, 16, 16, 1, 1, True, 1, 1, 1, 1),      # 1x1: conv == GEMM
-    (2, 14, 14, 32, 24, 3, 3, True, 1, 1, 1, 1),    # same padding like BASELINE config 4
+    (2, 14, 14, 32, 24, 3, 3, True, 1, 1, 1, 1),    # same padding like benchmark configuration 4
     (1, 10, 10, 3, 5, 2, 2, True, 3, 3, 1, 1),      # stride > filter: holes in col2im
 ]
 # (B, IH, IW, IC, OC, FH, FW, covered, sy, sx)
 DECONV = [
     (2, 8, 8, 16, 8, 4, 4, False, 3, 3),    # DeConv2dTest forwardCPU geometry (smaller)
     (2, 8, 8, 16, 8, 4, 4, True, 3, 3),     # backwardCPU geometry
-    (2, 7, 7, 8, 16, 4, 4, False, 2, 2),    # BASELINE config 5 family -> 2*7+2
+    (2, 7, 7, 8, 16, 4, 4, False, 2, 2),    # benchmark configuration 5 family -> 2*7+2
     (2, 7, 7, 8, 16, 4, 4, True, 2, 2),
     (1, 5, 6, 3, 5, 3, 3, False, 1, 1),
     (2, 6, 5, 4, 3, 3, 2, True, 2, 2),
@@ -175,7 +175,7 @@ def test_deconv2d_real_tolerance(oracle_port, cfg):
 
 
 def test_config4_full_size_properties(oracle_port):
-    """BASELINE config 4 (Conv2d fp32, B32 56x56x64, 3x3x64 -> 64, same padding) at full size:
+    """benchmark configuration 4 (Conv2d fp32, B32 56x56x64, 3x3x64 -> 64, same padding) at full size:
     two sampled images against the oracle (forward and dX are independent per image), dW through
     its additivity over the batch, and the adjoint identity <z, dz> == <x, dx> == <w, dw>."""
     from deep8_amd import ops
@@ -199,7 +199,7 @@ def test_config4_full_size_properties(oracle_port):
 
 @pytest.mark.parametrize("cov", [False, True])
 def test_config5_full_size_properties(oracle_port, cov):
-    """BASELINE config 5 (DeConv2d half, B16 28x28x128, 4x4 stride 2 -> 64 channels) at Deep8's two
+    """benchmark configuration 5 (DeConv2d half, B16 28x28x128, 4x4 stride 2 -> 64 channels) at Deep8's two
     legal output sizes (58 when not covered, 55 when covered)."""
     from deep8_amd import ops
     r = rng(55)

@@ -81,7 +81,7 @@ def test_relu_forward_and_gradient(oracle_port, shape, dtype):
 
 
 def test_full_size_bias_and_relu_after_config4(oracle_port):
-    """The element-wise steps at BASELINE config 4's output size (32 x 56 x 56 x 64, fp32)."""
+    """The element-wise steps at benchmark configuration 4's output size (32 x 56 x 56 x 64, fp32)."""
     from deep8_amd import ops
     r = rng(404)
     z, b = nrm(r, (32, 56, 56, 64)), nrm(r, (1, 64))

@@ -1,6 +1,6 @@
 """MatrixMultiply forward / GradX / GradY through the C ABI against the oracle: the three shape
 cases of deep8/src/math/MatrixMultiply.cpp:94-116 (collapsed batch, vector-by-batch, batched with
-broadcast), the reference's own test shapes (test/MatrixMultiplyTest.h), and BASELINE configs."""
+broadcast), the reference's own test shapes (test/MatrixMultiplyTest.h), and benchmark configurations."""
 import numpy as np
 import pytest
 
@@ -15,7 +15,7 @@ CASES = [
     ((6, 40, 30), (6, 30, 50)),        # batched both (F3/X3/Y3)
     ((1, 40, 30), (6, 30, 50)),        # x broadcast: dX sums over the batch
     ((6, 40, 30), (6, 30)),            # batched matrix-vector (1-D y, both batched)
-    ((1, 64, 128), (1, 128, 256)),     # BASELINE config 1
+    ((1, 64, 128), (1, 128, 256)),     # benchmark configuration 1
     ((3, 17), (1, 1, 9)),              # 1-D x (column vector) times a row: outer products
 ]
 
@@ -105,7 +105,7 @@ def _against_reference_or_port(oracle_port, name, *args):
 
 @pytest.mark.parametrize("yb", [32, 1])
 def test_config2_batched_fp32(oracle_port, yb):
-    """BASELINE config 2: batch 32 of 512x512x512 (and the shared-weight broadcast case), uniform(-1,1)."""
+    """benchmark configuration 2: batch 32 of 512x512x512 (and the shared-weight broadcast case), uniform(-1,1)."""
     from deep8_amd import ops
     r = rng(2024)
     x, y, dz = uni(r, (32, 512, 512)), uni(r, (yb, 512, 512)), uni(r, (32, 512, 512))
@@ -117,7 +117,7 @@ def test_config2_batched_fp32(oracle_port, yb):
 
 
 def test_config3_large_half_properties(oracle_port):
-    """BASELINE config 3 (4096^3 half) at full size, checked through size-independent properties:
+    """benchmark configuration 3 (4096^3 half) at full size, checked through size-independent properties:
     sampled rows/columns against the oracle's GEMM on the half-rounded inputs, and linearity."""
     from deep8_amd import ops
     r = rng(4096)
@@ -145,7 +145,7 @@ def test_config3_large_half_properties(oracle_port):
 def test_matmul_step_replayed_from_a_hip_graph(oracle_port):
     """The entry points only launch kernels on the stream they are given, so a caller can capture a step into a
     HIP graph (d8_graph_begin / d8_graph_end): three replays, with eager work and synchronisations between
-    them, must each reproduce the eager result (BASELINE config 1's shapes, integer inputs: bit-exact)."""
+    them, must each reproduce the eager result (benchmark configuration 1's shapes, integer inputs: bit-exact)."""
     import ctypes
     from deep8_amd import capi
     from deep8_amd.capi import DeviceArray, check

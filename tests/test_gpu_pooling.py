@@ -41,7 +41,7 @@ def test_pooling_forward_and_gradients(oracle_port, cfg, dtype):
 
 
 def test_pooling_after_config4_full_size(oracle_port):
-    """2 x 2 / 2 pooling at BASELINE config 4's activation size, against numpy reshapes."""
+    """2 x 2 / 2 pooling at benchmark configuration 4's activation size, against numpy reshapes."""
     from deep8_amd import ops
     r = rng(56)
     x = nrm(r, (32, 56, 56, 64))

@@ -284,7 +284,7 @@ def test_special_cases(oracle_port):
     col = ints(r, (9, 2 * 2 * 2)) + 1
     out = oracle_port.col2im(col, im, 3, 3, 2, 2, 2, 2, 1, 1, 0, 0)
     assert sorted(out.ravel()) == sorted(col.ravel())
-    # geometry of the BASELINE configs
+    # geometry of the benchmark configurations
     assert oracle_port.conv2d_geometry(56, 56, 3, 3, True, 1, 1, 1, 1) == (56, 56, 1, 1)
     assert oracle_port.deconv2d_geometry(28, 28, 4, 4, False, 2, 2) == (58, 58, 3, 3)
     assert oracle_port.deconv2d_geometry(28, 28, 4, 4, True, 2, 2) == (55, 55, 1, 1)
