@@ -35,7 +35,7 @@ HBM_PEAK = 8000.0                      # GB/s
 EAGER_ZERO = False
 
 MEASURED_TRAFFIC = {
-    "c3": int((192.2 + 224.2 + 224.2) / 3 * 2**20 + 32.0 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
+    "c3": int((192.2 + 192.2 + 192.3) / 3 * 2**20 + 32.0 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
     "c4": int((2 * 13.9 + 2 * 13.0 + 2.0 + 0.5) * 2**20),            # Conv2d forward: tile launches (rows cut in two) fetch + write, + the band's split reduction
     "c5": int((17.4 + 6.6) * 2**20),                                 # DeConv2d forward (one launch over the output classes): fetch + write
 }
