@@ -8,6 +8,12 @@ already sits in HBM.  The headline workload is benchmark configuration 3 (Matrix
 4096 x 4096 x 4096); the other configs are timed briefly and reported under "others".
 Prints ONE JSON line.
 
+Every measurement is preceded by --settle-ms (default 60) milliseconds of the same work, untimed: the chip's
+power management raises the shader clock over the first tens of milliseconds of sustained load, so a run that
+starts on an idle device and times 20 steps after 3 warm-up steps measures the ramp, not the rate a training
+loop sees (MatrixMultiply half 4096^3: about 1150 TFLOP/s from idle, about 1400 sustained, same box, same
+binary).  --settle-ms 0 gives the from-idle number; the JSON line reports the value used as "settle_ms".
+
   value          whole-step throughput: algorithmic FLOPs of fwd + dX + dY / wall time of a step
                  (gradient destinations are zeroed inside the step, as Deep8's executor does)
   roofline       the slowest of the step's GEMM launches, timed alone with HIP events on the stream
@@ -46,9 +52,31 @@ def _dev(a):
     return DeviceArray.from_numpy(a)
 
 
+# Milliseconds of untimed, uninterrupted work issued before every measurement (--settle-ms).  The chip's power
+# management raises the shader clock over the first tens of milliseconds of sustained load: a measurement that
+# starts on an idle device runs its first steps 15-20 % slower than the sustained rate (by the fp16 kernel's own
+# clock record 1.4 GHz after 4 ms of load, 1.65 GHz after 40 ms), and a few warm-up steps do not cover that ramp.
+SETTLE_MS = 60.0
+
+
+def _settle(fn):
+    """keeps the device busy with fn for about SETTLE_MS, untimed; returns with the work still queued"""
+    from deep8_amd import capi
+    if SETTLE_MS <= 0:
+        return
+    capi.sync()
+    t0 = time.perf_counter()
+    fn()
+    capi.sync()
+    one = max(time.perf_counter() - t0, 1e-6)
+    for _ in range(min(20000, int(SETTLE_MS * 1e-3 / one) + 1)):
+        fn()
+
+
 def _time_steps(fn, steps, warmup):
     """wall-clock ms per step over exactly `steps` calls, device idle on both sides"""
     from deep8_amd import capi
+    _settle(fn)
     for _ in range(warmup):
         fn()
     capi.sync()
@@ -62,6 +90,7 @@ def _time_steps(fn, steps, warmup):
 def _time_events(fn, reps):
     """average ms per call measured with HIP events on the launch stream"""
     from deep8_amd import capi
+    _settle(fn)
     fn()
     capi.sync()
     t = capi.Timer(None)
@@ -514,6 +543,7 @@ def phase_record(launches=12):
         def launch(i):
             capi.check(lib.d8_gemm(wl.dt, ta, tb, n, n, n, A.ptr, n, 0, B.ptr, n, 0, 0.0, out.ptr, n, 0, 1,
                                    recs[i].ptr, 256 * 6 * 8, None))
+        _settle(lambda: launch(0))
         for i in range(launches):
             launch(i)
         capi.sync()
@@ -542,6 +572,7 @@ def phase_record(launches=12):
 
 
 def main():
+    global ZERO_OPERANDS, EAGER_ZERO, SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -555,12 +586,15 @@ def main():
     ap.add_argument("--eager-zero", action="store_true",
                     help="zero-fill the gradients and accumulate (the reference's literal "
                          "sequence) instead of the executor's deferred zeroing + overwrite")
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="untimed work issued before every measurement so that it runs at the sustained clock "
+                         "(0: start from an idle device)")
     ap.add_argument("--phases", action="store_true",
                     help="only print the phase record of workload c3's three products (see phase_record)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
-    global ZERO_OPERANDS, EAGER_ZERO
+    SETTLE_MS = a.settle_ms
     ZERO_OPERANDS = a.operands == "zeros"
     EAGER_ZERO = a.eager_zero
     if a.gpus != 1:
@@ -602,7 +636,7 @@ def main():
         "metric": "Conv2d fwd+bwd images/s" if is_conv else "MatrixMultiply fwd+bwd TFLOP/s",
         "value": round(wl.B / (ms * 1e-3), 1) if is_conv else round(tflops, 2),
         "unit": "images/s" if is_conv else "TFLOP/s",
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "settle_ms": SETTLE_MS, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "ALL-ZERO OPERANDS (diagnostic run, not a benchmark value)" if ZERO_OPERANDS else
         "synthetic (seeded numpy generators, resident in HBM before timing)",
@@ -621,7 +655,7 @@ def main():
                 continue
             del wl
             wl = make_workload(key)
-            oms = _time_steps(wl.step, 5, 2)
+            oms = _time_steps(wl.step, 20, 3)
             o = {"ms_per_step": round(oms, 4), "tflops": round(wl.flops / (oms * 1e-3) / 1e12, 2),
                  "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
             if isinstance(wl, (ConvWorkload, BiasReluWorkload, PoolWorkload)):
