@@ -32,7 +32,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK = {"f16": 2500.0, "f32": 157.3}   # dense MFMA TFLOP/s, MI355X
+PEAK = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}   # dense MFMA TFLOP/s, MI355X
 HBM_PEAK = 8000.0                      # GB/s
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this file (each counter scaled by what it reads for a plain copy of known size; the
@@ -44,6 +44,11 @@ MEASURED_TRAFFIC = {
     "c3": int((192.2 + 192.2 + 192.3) / 3 * 2**20 + 32.0 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
     "c4": int((2 * 13.9 + 2 * 13.0 + 2.0 + 0.5) * 2**20),            # Conv2d forward: tile launches (rows cut in two) fetch + write, + the band's split reduction
     "c5": int((17.4 + 6.6) * 2**20),                                 # DeConv2d forward (one launch over the output classes): fetch + write
+    "d3": int((288.1 + 32.0) * 2**20),                               # fp64 128 x 128 tiles: fetch + write
+    # element-wise and pooling steps: per kernel of the step (fetch + write)
+    "e4": {"add (bias broadcast)": int((24.5 + 24.5) * 2**20), "relu": int((24.5 + 24.5) * 2**20),
+           "relu_grad": int((49.0 + 24.5) * 2**20), "bias_grad (sum over rows)": int((24.5 + 0.3 + 0.1) * 2**20)},
+    "p4": {"maxpool2d": int((24.6 + 6.1) * 2**20), "maxpool2d_grad": int((30.7 + 24.5) * 2**20)},
 }
 
 
@@ -126,6 +131,8 @@ class MatMulWorkload:
         wide = self.dtype == np.float16 and m >= 256 and n >= 256 and k % 64 == 0 and zb * (-(-m // 256)) * (-(-n // 256)) >= 192
         small = zb * (-(-m // 128)) * (-(-n // 128)) <= 4 and max(m, n, k) * (zb if 1 in (xs[0], ys[0]) else 1) <= 512
         self.kernel = "%s (one launch each for fwd, dX, dY)" % (
+            "gemm_f64_kernel (%s tiles, v_mfma_f64_16x16x4_f64)" % ("128x128" if zb * (-(-m // 128)) * (-(-n // 128)) >= 192 else "64x64")
+            if self.dtype == np.float64 else
             "gemm_wide_kernel (fp16, 256x256 tiles)" if wide else
             "gemm_%s_kernel<%s>" % ("small" if small else "tiled", "f16" if self.dtype == np.float16 else "f32"))
         es = self.dtype.itemsize
@@ -189,7 +196,7 @@ def mfma_stream_ceiling(wl, dtype_name):
     lib = wl.lib
     out = capi.DeviceArray((lib.d8_mfma_stream_out_bytes(),), np.uint8)
     flops = ctypes.c_double(0)
-    iters = 200 if wl.dtype == np.float16 else 100  # 100-200 us per launch, like the GEMMs
+    iters = {2: 200, 4: 100, 8: 1000}[wl.dtype.itemsize]  # 100-400 us per launch, like the GEMMs
 
     def run():
         capi.check(lib.d8_mfma_stream(wl.dt, wl.x.ptr, wl.x.nbytes, out.ptr, iters, ctypes.byref(flops), None))
@@ -336,19 +343,43 @@ class BiasReluWorkload:
         # with --eager-zero) | bias grad: r gpre
         self.bytes = es * self.n * (10 if EAGER_ZERO else 8)
 
-    def step(self):
+    def add(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_add(self.dt, self.z.ptr, self.zd, self.b.ptr, self.bd, self.pre.ptr, self.zd, None))
+
+    def relu(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_relu(self.dt, self.pre.ptr, self.act.ptr, self.n, None))
+
+    def relu_grad(self):
         from deep8_amd.capi import check
         L = self.lib
-        check(L.d8_add(self.dt, self.z.ptr, self.zd, self.b.ptr, self.bd, self.pre.ptr, self.zd, None))
-        check(L.d8_relu(self.dt, self.pre.ptr, self.act.ptr, self.n, None))
         if EAGER_ZERO:
             self.gpre.zero_()
-            self.gb.zero_()
             check(L.d8_relu_grad(self.dt, self.pre.ptr, self.gpre.ptr, self.gy.ptr, self.n, None))
-            check(L.d8_add_grad(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
-        else:  # gradients whose zero fill is still pending are written, not added to
+        else:  # a gradient whose zero fill is still pending is written, not added to
             check(L.d8_relu_grad_overwrite(self.dt, self.pre.ptr, self.gpre.ptr, self.gy.ptr, self.n, None))
+
+    def bias_grad(self):
+        from deep8_amd.capi import check
+        L = self.lib
+        if EAGER_ZERO:
+            self.gb.zero_()
+            check(L.d8_add_grad(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
+        else:
             check(L.d8_add_grad_overwrite(self.dt, self.gb.ptr, self.bd, self.gpre.ptr, self.zd, self.ws.ptr, self.ws_bytes, None))
+
+    def step(self):
+        self.add()
+        self.relu()
+        self.relu_grad()
+        self.bias_grad()
+
+    def parts(self):
+        """name -> (call, algorithmic bytes): what each kernel must read and write once"""
+        nb = self.dtype.itemsize * self.n
+        return {"add (bias broadcast)": (self.add, 2 * nb), "relu": (self.relu, 2 * nb),
+                "relu_grad": (self.relu_grad, (5 if EAGER_ZERO else 3) * nb), "bias_grad (sum over rows)": (self.bias_grad, nb)}
 
 
 class PoolWorkload:
@@ -370,14 +401,26 @@ class PoolWorkload:
         # forward: r x, w y | gradient: r x, r gy, w gx (+ fill and read-back of gx with --eager-zero)
         self.bytes = es * (n + n // 4 + n + n // 4 + n + (2 * n if EAGER_ZERO else 0))
 
-    def step(self):
+    def fwd(self):
         from deep8_amd.capi import check
         check(self.lib.d8_maxpool2d(self.dt, self.x.ptr, self.y.ptr, *self.dims, 2, 2, 0, 2, 2, None))
+
+    def grad(self):
+        from deep8_amd.capi import check
         if EAGER_ZERO:
             self.gx.zero_()
             check(self.lib.d8_maxpool2d_grad(self.dt, self.x.ptr, self.gx.ptr, self.gy.ptr, *self.dims, 2, 2, 0, 2, 2, None))
         else:
             check(self.lib.d8_maxpool2d_grad_overwrite(self.dt, self.x.ptr, self.gx.ptr, self.gy.ptr, *self.dims, 2, 2, 0, 2, 2, None))
+
+    def step(self):
+        self.fwd()
+        self.grad()
+
+    def parts(self):
+        """name -> (call, algorithmic bytes)"""
+        nb = self.dtype.itemsize * int(np.prod(self.dims))
+        return {"maxpool2d": (self.fwd, nb + nb // 4), "maxpool2d_grad": (self.grad, nb + nb // 4 + nb + (2 * nb if EAGER_ZERO else 0))}
 
 
 def _uni(r, s):
@@ -413,6 +456,9 @@ def make_workload(key):
     if key == "c5":
         return ConvWorkload("c5: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 58x58x64 (Deep8 covered=false)",
                             np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
+    if key == "d3":
+        return MatMulWorkload("d3: MatrixMultiply fwd+dX+dY double [2048x2048]x[2048x2048]", np.float64,
+                              (1, 2048, 2048), (1, 2048, 2048), U, 10)
     if key == "e4":
         return BiasReluWorkload("e4: bias Add + ReLu fwd+bwd on config 4's output, fp32 B32 56x56x64", np.float32, 32, 56, 56, 64, 7)
     if key == "p4":
@@ -439,6 +485,28 @@ def cpu_baseline(key, seconds=12.0):
     src = oracle.ref if oracle.ref is not None else oracle.port
     kind = "reference" if oracle.ref is not None else "port"
     r = np.random.default_rng(9)
+    if key in ("e4", "p4"):
+        # element-wise and pooling operators run on the CPU device's Eigen thread pool in the reference
+        B = 8
+        x = r.standard_normal((B, 56, 56, 64)).astype(np.float32)
+        if key == "e4":
+            b, gy = r.standard_normal((1, 64)).astype(np.float32), r.standard_normal(x.shape).astype(np.float32)
+
+            def one():
+                pre = src.add(x, b)
+                src.relu(pre)
+                gpre = src.relu_grad(pre, gy)
+                src.add_grad(1, x, b, gpre) if kind == "reference" else src.add_grad(b, gpre)
+        else:
+            gy = r.standard_normal((B, 28, 28, 64)).astype(np.float32)
+
+            def one():
+                src.pool2d(True, x, 2, 2, False, 2, 2)
+                src.pool2d_grad(True, x, gy, 2, 2, False, 2, 2)
+        n, dt = _repeat_for(one, seconds)
+        return {"value": n * B / dt, "unit": "images/s", "cores": src.threads(), "kind": kind,
+                "sample": "%s fwd+bwd on %d images x %d repeats (fp32 CPU path, host-side array copies included), %.1f s"
+                          % (key, B, n, dt)}
     if key in ("c4", "c5"):
         # the reference runs Conv2d/DeConv2d on Eigen's thread pool: all host cores
         B = 8
@@ -458,25 +526,32 @@ def cpu_baseline(key, seconds=12.0):
         return {"value": n * B / dt, "unit": "images/s", "cores": src.threads(), "kind": kind,
                 "sample": "%s fwd+dX+dW on %d images x %d repeats (fp32 CPU path), %.1f s" % (key, B, n, dt)}
     # MatrixMultiply: Eigen's dense product is single-threaded in the reference build
-    if key == "c3":
+    wide = np.float64 if key == "d3" else np.float32
+    if key == "d3":
+        m, k, n_, b = 256, 2048, 2048, 1
+    elif key == "c3":
         m, k, n_, b = 256, 4096, 4096, 1
     elif key in ("c2a", "c2b"):
         m, k, n_, b = 512, 512, 512, 8
     else:
         m, k, n_, b = 64, 128, 256, 1
-    x, y = r.uniform(-1, 1, (b, m, k)).astype(np.float32), r.uniform(-1, 1, (1 if key != "c2a" else b, k, n_)).astype(np.float32)
-    dz = r.uniform(-1, 1, (b, m, n_)).astype(np.float32)
+    x, y = r.uniform(-1, 1, (b, m, k)).astype(wide), r.uniform(-1, 1, (1 if key != "c2a" else b, k, n_)).astype(wide)
+    dz = r.uniform(-1, 1, (b, m, n_)).astype(wide)
 
     def one():
         src.matmul(x, y)
         src.matmul_grad_x(x, y, dz)
         src.matmul_grad_y(x, y, dz)
-    n, dt = _repeat_for(one, seconds)
+    if key == "d3":
+        with oracle.float64():
+            n, dt = _repeat_for(one, seconds)
+    else:
+        n, dt = _repeat_for(one, seconds)
     flops = n * 3 * 2.0 * b * m * k * n_
     return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1 if kind == "reference" else src.threads(),
             "kind": kind,
-            "sample": "fwd+dX+dY of %d x [%dx%d]x[%dx%d] fp32 (the reference has no CPU half) x %d repeats, %.1f s"
-                      % (b, m, k, k, n_, n, dt)}
+            "sample": "fwd+dX+dY of %d x [%dx%d]x[%dx%d] %s x %d repeats, %.1f s"
+                      % (b, m, k, k, n_, "fp64" if key == "d3" else "fp32 (the reference has no CPU half)", n, dt)}
 
 
 def calibrate_copy(mib):
@@ -612,16 +687,28 @@ def main():
 
     wl = make_workload(a.workload)
     ms = _time_steps(wl.step, a.steps, a.warmup)
-    dtype = "f16" if wl.dtype == np.float16 else "f32"
+    dtype = {2: "f16", 4: "f32", 8: "f64"}[wl.dtype.itemsize]
     is_conv = isinstance(wl, ConvWorkload)
+    is_stream = isinstance(wl, (BiasReluWorkload, PoolWorkload))  # element-wise / pooling: HBM-bound kernels
     tflops = wl.flops / (ms * 1e-3) / 1e12
 
     parts = {}
-    for pname, (fn, fl) in wl.parts().items():
-        pms = _time_events(fn, max(5, a.steps))
-        parts[pname] = {"ms": round(pms, 4), "tflops": round(fl / (pms * 1e-3) / 1e12, 2)}
+    for pname, (fn, amount) in wl.parts().items():
+        pms = _time_events(fn, max(200, a.steps) if is_stream else max(5, a.steps))  # 10 us kernels: more launches per timing
+        if is_stream:
+            parts[pname] = {"ms": round(pms, 4), "algorithmic_GBps": round(amount / (pms * 1e-3) / 1e9, 1)}
+        else:
+            parts[pname] = {"ms": round(pms, 4), "tflops": round(amount / (pms * 1e-3) / 1e12, 2)}
     if is_conv:
         roof = wl.gemm_roofline(max(5, a.steps))
+    elif is_stream:
+        # the kernel the step spends most of its time in, against the HBM peak: the bytes it must read
+        # and write once / its duration alone (HIP events on the launch stream)
+        pname = max(parts, key=lambda k: parts[k]["ms"])
+        ach = parts[pname]["algorithmic_GBps"]
+        roof = {"bound": "hbm", "kernel": pname, "achieved": ach, "peak": HBM_PEAK, "unit": "GB/s",
+                "frac": round(ach / HBM_PEAK, 4), "launch_us": round(parts[pname]["ms"] * 1e3, 2),
+                "traffic": MEASURED_TRAFFIC.get(a.workload, {}).get(pname)}
     else:
         # each of fwd / dX / dY is ONE launch of the same tiled GEMM kernel (its NN, NT and TN
         # instances): flops per launch / average launch duration, HIP events on the launch stream
@@ -633,16 +720,18 @@ def main():
         roof["mfma_stream_ceiling"] = mfma_stream_ceiling(wl, dtype)
 
     out = {
-        "metric": "Conv2d fwd+bwd images/s" if is_conv else "MatrixMultiply fwd+bwd TFLOP/s",
-        "value": round(wl.B / (ms * 1e-3), 1) if is_conv else round(tflops, 2),
-        "unit": "images/s" if is_conv else "TFLOP/s",
+        "metric": "Conv2d fwd+bwd images/s" if is_conv else "%s fwd+bwd images/s" % wl.key if is_stream
+        else "MatrixMultiply fwd+bwd TFLOP/s",
+        "value": round(wl.B / (ms * 1e-3), 1) if is_conv or is_stream else round(tflops, 2),
+        "unit": "images/s" if is_conv or is_stream else "TFLOP/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "settle_ms": SETTLE_MS, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "ALL-ZERO OPERANDS (diagnostic run, not a benchmark value)" if ZERO_OPERANDS else
         "synthetic (seeded numpy generators, resident in HBM before timing)",
         "config": {"workload": wl.name},
-        "pct_mfma_peak": round(100.0 * tflops / PEAK[dtype], 2),
+        "pct_mfma_peak": None if is_stream else round(100.0 * tflops / PEAK[dtype], 2),
         "tflops": round(tflops, 2),
+        "algorithmic_GBps": round(wl.bytes / (ms * 1e-3) / 1e9, 1),
         "parts": parts,
         "roofline": roof,
     }

@@ -124,7 +124,18 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
     if (live) {
         const int r1 = min(R, (chunk + 1) * rows_per_chunk);
         const T *p = dz + ((long)k0 * R) * C + (long)cv * VEC;
-        for (int r = chunk * rows_per_chunk + ty; r < r1; r += lanes) {
+        int r = chunk * rows_per_chunk + ty;
+        // four rows in flight per thread; the adds keep the order of the plain loop
+        for (; r + 3 * lanes < r1; r += 4 * lanes) {
+            VT v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *(const VT *)(p + (long)(r + u * lanes) * C);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] += ew_load<OP>(ew_f32(v[u][e]));
+        }
+        for (; r < r1; r += lanes) {
             const VT v = *(const VT *)(p + (long)r * C);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc[e] += ew_load<OP>(ew_f32(v[e]));
@@ -149,26 +160,34 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const T *__restrict__ d
     }
 }
 
-// g[k0][c] += sum over chunks of partial[k0][chunk][c].  A block covers 32 outputs; 8 lanes per
-// output each add every 8th chunk and meet in LDS in a fixed order.
+// g[k0][c] += sum over chunks of partial[k0][chunk][c].  A block covers 16 outputs; 16 lanes per
+// output each add every 16th chunk (eight loads in flight) and meet in LDS in a fixed order.
 template <typename T>
 __global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__restrict__ partial, T *__restrict__ g,
                                                                 int C, int chunks, long total, float scale, float keep) {
-    __shared__ float part[8][32];
-    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    const long idx = (long)blockIdx.x * 32 + tx;
+    __shared__ float part[16][16];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const long idx = (long)blockIdx.x * 16 + tx;
     float v = 0.f;
     if (idx < total) {
         const long k0 = idx / C;
         const int c = (int)(idx - k0 * C);
         const float *p = partial + k0 * chunks * C + c;
-        for (int k = ty; k < chunks; k += 8) v += p[(long)k * C];
+        int k = ty;
+        for (; k + 7 * 16 < chunks; k += 8 * 16) {
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = p[(long)(k + u * 16) * C];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v += t[u];
+        }
+        for (; k < chunks; k += 16) v += p[(long)k * C];
     }
     part[ty][tx] = v;
     __syncthreads();
     if (ty == 0 && idx < total) {
 #pragma unroll
-        for (int k = 1; k < 8; ++k) v += part[k][tx];
+        for (int k = 1; k < 16; ++k) v += part[k][tx];
         g[idx] = (T)((keep != 0.f ? ew_f32(g[idx]) : 0.f) + scale * v);
     }
 }
@@ -362,7 +381,7 @@ static ReducePlan plan_reduce(const int *d, const int *zd) {
         long chunks = (4L * cu_count()) / (colblocks * p.K0);
         const long max_chunks = (p.R + 63) / 64;
         if (chunks > max_chunks) chunks = max_chunks;
-        if (chunks > 256) chunks = 256;
+        if (chunks > 512) chunks = 512;
         if (chunks < 1) chunks = 1;
         p.rows_per_chunk = (int)((p.R + chunks - 1) / chunks);
         p.chunks = (int)((p.R + p.rows_per_chunk - 1) / p.rows_per_chunk);
@@ -399,7 +418,7 @@ static int reduce_t(T *g, const int *d, const T *dz, const int *zd, void *scratc
                                TX, rpc, chunks, scale, keep);
         if (chunks > 1) {
             D8_LAUNCH_CHECK();
-            hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3((unsigned)((ng + 31) / 32)), dim3(256), 0, s,
+            hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3((unsigned)((ng + 15) / 16)), dim3(256), 0, s,
                                (const float *)scratch, g, (int)p.C, chunks, ng, scale, keep);
         }
     } else {

@@ -13,14 +13,22 @@ namespace d8 {
 
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 
-// 64 x 64 tile, 4 waves in a 2 x 2 arrangement, 32 x 32 per wave (2 x 2 instruction blocks),
-// K step 16.  Both LDS tiles are [row][k] with an odd row pitch, so the 16 rows one operand read
-// touches fall into different banks.  Tile loads are element-wise and bounds-checked.
-template <bool TA, bool TB>
+// BM x BN tile (64 x 64 or 128 x 128), 4 waves in a 2 x 2 arrangement, each wave WT x WT instruction
+// blocks (WT = 2 or 4), K step 16.  Both LDS tiles are [row][k] with an odd row pitch, so the 16 rows
+// one operand read touches fall into different banks.  Tile loads are element-wise and
+// bounds-checked.  Everything that is not a matrix instruction is issued under one: the next K
+// step's elements are fetched into registers before the current step is multiplied (a step is
+// 4 * WT * WT matrix instructions of 64 cycles per wave, which covers the fetch) and written to the
+// other half of the double-buffered LDS tiles half-way through it, and the operand fragments of
+// the next group of four k are read from LDS before the current group is multiplied.  One barrier
+// per K step.  The 128 x 128 tile halves the operand traffic per flop; it keeps 64 accumulator
+// doubles per lane, one wave per SIMD.
+template <bool TA, bool TB, int WT>
 __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
-    constexpr int BM = 64, BN = 64, BK = 16, LD = 17;
-    __shared__ double As[BM * LD];
-    __shared__ double Bs[BN * LD];
+    constexpr int BM = 32 * WT, BN = 32 * WT, BK = 16, LD = 17;
+    constexpr int NA = BM * BK / 256, NB = BN * BK / 256;  // elements a thread moves per K step
+    __shared__ double As[2][BM * LD];
+    __shared__ double Bs[2][BN * LD];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -30,71 +38,93 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
     const int ktiles = (g.K + BK - 1) / BK;
     const int total = g.red * ktiles;
 
-    f64x4 acc[2][2];
+    f64x4 acc[WT][WT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = f64x4{0., 0., 0., 0.};
+        for (int j = 0; j < WT; ++j) acc[i][j] = f64x4{0., 0., 0., 0.};
 
-    const int l16 = lane & 15, kq = lane >> 4;
-    for (int t = 0; t < total; ++t) {
+    // element u of this thread: A (m, k) and B (n, k) inside the tile, the same for every K step
+    int am[NA], ak[NA], bn[NB], bk[NB];
+#pragma unroll
+    for (int u = 0; u < NA; ++u) {
+        const int i = tid + 256 * u;
+        am[u] = TA ? i % BM : i / BK;
+        ak[u] = TA ? i / BM : i % BK;
+    }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const int i = tid + 256 * u;
+        bn[u] = TB ? i / BK : i % BN;
+        bk[u] = TB ? i % BK : i / BN;
+    }
+    double pa[NA], pb[NB];
+    auto fetch = [&](int t) {
         const int r = t / ktiles, k0 = (t - r * ktiles) * BK;
         const double *Ap = (const double *)g.A + (long)(b + r) * g.sA;
         const double *Bp = (const double *)g.B + (long)(b + r) * g.sB;
+#pragma unroll
+        for (int u = 0; u < NA; ++u) {
+            const int gm = m0 + am[u], gk = k0 + ak[u];
+            pa[u] = 0.;
+            if (gm < g.M && gk < g.K) pa[u] = TA ? Ap[(long)gk * g.lda + gm] : Ap[(long)gm * g.lda + gk];
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int gn = n0 + bn[u], gk = k0 + bk[u];
+            pb[u] = 0.;
+            if (gn < g.N && gk < g.K) pb[u] = TB ? Bp[(long)gn * g.ldb + gk] : Bp[(long)gk * g.ldb + gn];
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < NA; ++u) As[buf][am[u] * LD + ak[u]] = pa[u];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) Bs[buf][bn[u] * LD + bk[u]] = pb[u];
+    };
 
-        for (int i = tid; i < BM * BK; i += 256) {
-            int m, k;
-            if (!TA) {
-                m = i / BK;
-                k = i % BK;
-            } else {
-                k = i / BM;
-                m = i % BM;
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int a_row = (wm * 16 * WT + l16) * LD + kq, b_row = (wn * 16 * WT + l16) * LD + kq;
+    if (total > 0) {
+        fetch(0);
+        stage(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < total; ++t) {
+        const bool more = t + 1 < total;
+        const int cur = t & 1;
+        if (more) fetch(t + 1);
+        double fa[2][WT], fb[2][WT];
+#pragma unroll
+        for (int i = 0; i < WT; ++i) fa[0][i] = As[cur][a_row + i * 16 * LD];
+#pragma unroll
+        for (int j = 0; j < WT; ++j) fb[0][j] = Bs[cur][b_row + j * 16 * LD];
+#pragma unroll
+        for (int s = 0; s < BK / 4; ++s) {
+            if (s + 1 < BK / 4) {
+#pragma unroll
+                for (int i = 0; i < WT; ++i) fa[(s + 1) & 1][i] = As[cur][a_row + i * 16 * LD + 4 * (s + 1)];
+#pragma unroll
+                for (int j = 0; j < WT; ++j) fb[(s + 1) & 1][j] = Bs[cur][b_row + j * 16 * LD + 4 * (s + 1)];
             }
-            const int gm = m0 + m, gk = k0 + k;
-            double v = 0.;
-            if (gm < g.M && gk < g.K) v = TA ? Ap[(long)gk * g.lda + gm] : Ap[(long)gm * g.lda + gk];
-            As[m * LD + k] = v;
-        }
-        for (int i = tid; i < BN * BK; i += 256) {
-            int n, k;
-            if (TB) {
-                n = i / BK;
-                k = i % BK;
-            } else {
-                k = i / BN;
-                n = i % BN;
-            }
-            const int gn = n0 + n, gk = k0 + k;
-            double v = 0.;
-            if (gn < g.N && gk < g.K) v = TB ? Bp[(long)gn * g.ldb + gk] : Bp[(long)gk * g.ldb + gn];
-            Bs[n * LD + k] = v;
-        }
-        __syncthreads();
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 4) {
-            double a[2], bb[2];
+            for (int i = 0; i < WT; ++i)
 #pragma unroll
-            for (int i = 0; i < 2; ++i) a[i] = As[(wm * 32 + i * 16 + l16) * LD + kk + kq];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) bb[j] = Bs[(wn * 32 + j * 16 + l16) * LD + kk + kq];
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], bb[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < WT; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+            if (s == 1 && more) stage(cur ^ 1);  // the other half: nobody reads it before the barrier below
         }
         __syncthreads();
     }
 
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int n = n0 + wn * 32 + j * 16 + l16;
+        for (int j = 0; j < WT; ++j) {
+            const int n = n0 + wn * 16 * WT + j * 16 + l16;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int m = m0 + wm * 32 + i * 16 + 4 * r + kq;
+                const int m = m0 + wm * 16 * WT + i * 16 + 4 * r + kq;
                 if (m < g.M && n < g.N) {
                     double *c = (double *)g.C + (long)b * g.sC + (long)m * g.ldc + n;
                     double v = acc[i][j][r];
@@ -105,15 +135,23 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
         }
 }
 
+template <int WT>
+static void launch_f64(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
+    dim3 grid(ceil_div(g.M, 32 * WT), ceil_div(g.N, 32 * WT), g.batch);
+    if (!transA && !transB)
+        hipLaunchKernelGGL((gemm_f64_kernel<false, false, WT>), grid, dim3(256), 0, stream, g);
+    else if (!transA && transB)
+        hipLaunchKernelGGL((gemm_f64_kernel<false, true, WT>), grid, dim3(256), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemm_f64_kernel<true, false, WT>), grid, dim3(256), 0, stream, g);
+}
+
 int gemm_f64_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
     D8_REQUIRE(ceil_div(g.N, 64) < 65536 && g.batch < 65536, "d8_gemm: grid too large");
-    dim3 grid(ceil_div(g.M, 64), ceil_div(g.N, 64), g.batch);
-    if (!transA && !transB)
-        hipLaunchKernelGGL((gemm_f64_kernel<false, false>), grid, dim3(256), 0, stream, g);
-    else if (!transA && transB)
-        hipLaunchKernelGGL((gemm_f64_kernel<false, true>), grid, dim3(256), 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_f64_kernel<true, false>), grid, dim3(256), 0, stream, g);
+    // 128 x 128 tiles when they alone fill most of the chip
+    const long big = (long)ceil_div(g.M, 128) * ceil_div(g.N, 128) * g.batch;
+    if (big >= (long)cu_count() * 3 / 4) launch_f64<4>(g, transA, transB, stream);
+    else launch_f64<2>(g, transA, transB, stream);
     D8_LAUNCH_CHECK();
     return 0;
 }

@@ -139,6 +139,70 @@ __global__ __launch_bounds__(256) void pool_backward_kernel(const T *__restrict_
     }
 }
 
+// The same gradients when the windows do not overlap (stride >= filter in both directions, the usual
+// 2x2 / 2 pooling): a thread per window and channel vector reads the window once, finds the first
+// maximum exactly as the reference scans for it (start from the first element of the clipped window,
+// replace on strict >, deep8/src/math/MaxPooling2d.cpp:228-243), reads dy once and writes the stride
+// cell the window sits in -- the image is cut into OH x OW cells, cell (oh, ow) starting where window
+// (oh, ow) starts and the border cells reaching the image's edges, so that every element of dx is
+// written by exactly one thread.  Elements of a cell outside its window receive nothing: untouched
+// with keep = 1, zero with keep = 0.  Every tensor is read or written once.
+template <typename T, int VEC, bool MAX>
+__global__ __launch_bounds__(256) void pool_backward_cells_kernel(const T *__restrict__ x, T *__restrict__ dx,
+                                                                  const T *__restrict__ dy, PoolGeom g, long total, float keep) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    const int cv = g.C / VEC;
+    const float inv = 1.0f / ((float)g.FH * (float)g.FW);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int c = (int)(idx % cv) * VEC;
+        long p = idx / cv;
+        const int ow = (int)(p % g.OW);
+        p /= g.OW;
+        const int oh = (int)(p % g.OH), b = (int)(p / g.OH);
+        const int wh0 = max(0, oh * g.sy - g.pt), wh1 = min(g.IH, oh * g.sy - g.pt + g.FH);
+        const int ww0 = max(0, ow * g.sx - g.pl), ww1 = min(g.IW, ow * g.sx - g.pl + g.FW);
+        const int ch0 = oh == 0 ? 0 : oh * g.sy - g.pt, ch1 = oh == g.OH - 1 ? g.IH : (oh + 1) * g.sy - g.pt;
+        const int cw0 = ow == 0 ? 0 : ow * g.sx - g.pl, cw1 = ow == g.OW - 1 ? g.IW : (ow + 1) * g.sx - g.pl;
+        const long img = (long)b * g.IH * g.IW * g.C + c;
+        const VT d = *(const VT *)(dy + idx * VEC);
+        int pos[VEC];  // h * IW + w of the winner, per channel
+        if (MAX) {
+            float best[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) best[e] = 0.f, pos[e] = -1;
+            bool first = true;
+            for (int h = wh0; h < wh1; ++h)
+                for (int w = ww0; w < ww1; ++w) {
+                    const VT t = *(const VT *)(x + img + ((long)h * g.IW + w) * g.C);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const float v = pool_f32(t[e]);
+                        if (first || v > best[e]) best[e] = v, pos[e] = h * g.IW + w;
+                    }
+                    first = false;
+                }
+        }
+        for (int h = ch0; h < ch1; ++h)
+            for (int w = cw0; w < cw1; ++w) {
+                const bool inwin = h >= wh0 && h < wh1 && w >= ww0 && w < ww1;
+                if (!inwin && keep != 0.f) continue;
+                T *q = dx + img + ((long)h * g.IW + w) * g.C;
+                VT o;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o[e] = (T)0;
+                if (keep != 0.f) o = *(const VT *)q;
+                if (inwin) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const float add = MAX ? (pos[e] == h * g.IW + w ? pool_f32(d[e]) : 0.f) : pool_f32(d[e]) * inv;
+                        o[e] = (T)(pool_f32(o[e]) + add);
+                    }
+                }
+                *(VT *)q = o;
+            }
+    }
+}
+
 static int pool_geometry(const char *who, int dtype, int B, int IH, int IW, int C, int FH, int FW, int covered, int sy, int sx,
                          PoolGeom &g) {
     if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32) return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
@@ -170,6 +234,19 @@ template <bool MAX>
 static int pool_backward(int dtype, const void *x, void *dx, const void *dy, const PoolGeom &g, hipStream_t s, float keep) {
     const long pixels = (long)g.B * g.IH * g.IW;
     const bool al = (((size_t)x | (size_t)dx | (size_t)dy) & 15) == 0;
+    // windows that do not overlap, and an image that fits the cell kernel's 32-bit pixel index
+    if (g.sy >= g.FH && g.sx >= g.FW && g.pt < g.sy && g.pl < g.sx && (long)g.IH * g.IW < (1L << 31)) {
+        const long wins = (long)g.B * g.OH * g.OW;
+        if (dtype == D8_FLOAT32) {
+            if (al && g.C % 4 == 0) hipLaunchKernelGGL((pool_backward_cells_kernel<float, 4, MAX>), dim3(pool_grid(wins * g.C / 4)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, wins * g.C / 4, keep);
+            else hipLaunchKernelGGL((pool_backward_cells_kernel<float, 1, MAX>), dim3(pool_grid(wins * g.C)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, wins * g.C, keep);
+        } else {
+            if (al && g.C % 8 == 0) hipLaunchKernelGGL((pool_backward_cells_kernel<f16, 8, MAX>), dim3(pool_grid(wins * g.C / 8)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, g, wins * g.C / 8, keep);
+            else hipLaunchKernelGGL((pool_backward_cells_kernel<f16, 1, MAX>), dim3(pool_grid(wins * g.C)), dim3(256), 0, s, (const f16 *)x, (f16 *)dx, (const f16 *)dy, g, wins * g.C, keep);
+        }
+        D8_LAUNCH_CHECK();
+        return 0;
+    }
     if (dtype == D8_FLOAT32) {
         if (al && g.C % 4 == 0) hipLaunchKernelGGL((pool_backward_kernel<float, 4, MAX>), dim3(pool_grid(pixels * g.C / 4)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, pixels * g.C / 4, keep);
         else hipLaunchKernelGGL((pool_backward_kernel<float, 1, MAX>), dim3(pool_grid(pixels * g.C)), dim3(256), 0, s, (const float *)x, (float *)dx, (const float *)dy, g, pixels * g.C, keep);

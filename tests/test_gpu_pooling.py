@@ -11,7 +11,10 @@ pytestmark = pytest.mark.gpu
 # B, IH, IW, C, FH, FW, covered, sy, sx
 CASES = [(2, 8, 8, 3, 2, 2, False, 2, 2), (1, 9, 9, 4, 3, 3, False, 2, 2), (2, 7, 7, 2, 3, 3, True, 2, 2), (1, 6, 6, 5, 3, 3, True, 1, 1),
          (1, 10, 10, 8, 4, 4, True, 3, 3), (2, 12, 10, 16, 3, 2, False, 1, 2), (1, 5, 5, 1, 5, 5, False, 1, 1), (1, 1, 1, 4, 1, 1, False, 1, 1),
-         (4, 28, 28, 64, 2, 2, False, 2, 2), (2, 15, 15, 24, 3, 3, True, 2, 2)]
+         (4, 28, 28, 64, 2, 2, False, 2, 2), (2, 15, 15, 24, 3, 3, True, 2, 2),
+         # windows that do not overlap: rows and columns no window reaches, strides above the filter, padded borders
+         (2, 9, 9, 8, 2, 2, False, 2, 2), (2, 11, 10, 8, 2, 2, False, 3, 3), (1, 7, 9, 4, 3, 3, True, 3, 3), (1, 9, 7, 4, 2, 2, True, 2, 2),
+         (1, 10, 12, 4, 2, 3, True, 3, 4), (3, 13, 13, 3, 1, 1, False, 2, 2), (2, 8, 8, 5, 2, 2, True, 4, 4), (1, 6, 6, 16, 3, 3, False, 3, 3)]
 
 
 @pytest.mark.parametrize("cfg", CASES)
@@ -36,6 +39,8 @@ def test_pooling_forward_and_gradients(oracle_port, cfg, dtype):
     assert np.array_equal(f(ops.maxpool2d_grad(xi, dy, *a, dx=nan, overwrite=True)), oracle_port.pool2d_grad(True, f(xi), f(dy), *a))
     assert np.array_equal(f(ops.avgpool2d_grad(xi.shape, c(np.zeros((B, OH, OW, C))), *a, dx=nan, overwrite=True)), np.zeros(xi.shape, np.float32))
     dyr = c(nrm(r, (B, OH, OW, C)))
+    assert rel_fro(f(ops.avgpool2d_grad(x.shape, dyr, *a, dx=nan, overwrite=True)), oracle_port.pool2d_grad(False, f(x), f(dyr), *a)) <= tol
+    assert rel_fro(f(ops.maxpool2d_grad(x, dyr, *a, dx=nan, overwrite=True)), oracle_port.pool2d_grad(True, f(x), f(dyr), *a)) <= tol
     assert rel_fro(f(ops.avgpool2d_grad(x.shape, dyr, *a, dx=dx0)), oracle_port.pool2d_grad(False, f(x), f(dyr), *a, dx=f(dx0))) <= tol
     assert rel_fro(f(ops.maxpool2d_grad(x, dyr, *a)), oracle_port.pool2d_grad(True, f(x), f(dyr), *a)) <= tol
 
