@@ -472,9 +472,14 @@ size_t d8_gemm_workspace_bytes(int dtype, int transA, int transB, int M, int N, 
                                int batch, long strideC) {
     (void)transA;
     (void)transB;
-    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || dtype == D8_FLOAT64) return 0;
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
     const int red = (strideC == 0 && batch > 1) ? batch : 1;
     const int outs = red > 1 ? 1 : batch;
+    if (dtype == D8_FLOAT64) {
+        int tps64 = 0;
+        const int pieces = gemm_f64_splits(M, N, K, outs, red, (size_t)-1, &tps64);
+        return pieces > 1 ? (size_t)pieces * outs * M * N * sizeof(double) : 0;
+    }
     // whichever kernel ends up running, the larger of the two plans fits
     int tps = 0;
     const int a = plan_splits(gemm_tiled_k_step(dtype), M, N, K, outs, red, (size_t)-1, &tps);

@@ -85,8 +85,11 @@ int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipS
 bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB);
 int gemm_wide_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);
 
-// fp64 kernel (64 x 64 tiles, v_mfma_f64_16x16x4_f64): any shape, reduction never split.
+// fp64 kernel (64 x 64 or 128 x 128 tiles, v_mfma_f64_16x16x4_f64): any shape; plans its own split of the
+// reduction from g.ws / g.ws_bytes (double partial sums) and reduces.
 int gemm_f64_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);
+// Pieces it would cut the reduction into given that much workspace.
+int gemm_f64_splits(int M, int N, int K, int batch, int red, size_t workspace_bytes, int *tiles_per_split);
 
 // Whether an unsplit product of this shape should run on 64 x 128 tiles: too few 128 x 128 tiles
 // for the chip, enough half-height ones, and a reduction (k_steps K steps in all) too short to

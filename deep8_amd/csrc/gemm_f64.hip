@@ -1,6 +1,8 @@
 // Row-major fp64 GEMM for gfx950 on v_mfma_f64_16x16x4_f64: C_b = op(A_b) op(B_b) + beta C_b,
 // NN / NT / TN, any size and leading dimension, strided batch with broadcast operands, optional
-// summation of the whole batch into one C.  The reduction is never split (no workspace).
+// summation of the whole batch into one C.  A long reduction over a small output (a filter
+// gradient) is cut into pieces that write double partial sums to the caller's workspace, added up
+// in a fixed order by a second kernel.
 //
 // Replaces the cublasDgemm call sites of deep8/src/math/MatrixMultiply.cu, Conv2d.cu and
 // DeConv2d.cu (the `double` twins of the calls listed in include/deep8_hip.h).
@@ -33,10 +35,11 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
-    const int b = blockIdx.z;
+    const int b = blockIdx.z / g.splits, piece = blockIdx.z - b * g.splits;
 
     const int ktiles = (g.K + BK - 1) / BK;
-    const int total = g.red * ktiles;
+    // this workgroup's share of the extended reduction (products x K steps)
+    const int t0 = piece * g.tiles_per_split, t1 = min(g.red * ktiles, t0 + g.tiles_per_split);
 
     f64x4 acc[WT][WT];
 #pragma unroll
@@ -85,14 +88,14 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
 
     const int l16 = lane & 15, kq = lane >> 4;
     const int a_row = (wm * 16 * WT + l16) * LD + kq, b_row = (wn * 16 * WT + l16) * LD + kq;
-    if (total > 0) {
-        fetch(0);
+    if (t0 < t1) {
+        fetch(t0);
         stage(0);
     }
     __syncthreads();
-    for (int t = 0; t < total; ++t) {
-        const bool more = t + 1 < total;
-        const int cur = t & 1;
+    for (int t = t0; t < t1; ++t) {
+        const bool more = t + 1 < t1;
+        const int cur = (t - t0) & 1;
         if (more) fetch(t + 1);
         double fa[2][WT], fb[2][WT];
 #pragma unroll
@@ -126,6 +129,10 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
             for (int r = 0; r < 4; ++r) {
                 const int m = m0 + wm * 16 * WT + i * 16 + 4 * r + kq;
                 if (m < g.M && n < g.N) {
+                    if (g.splits > 1) {  // partial sums [piece][b][M][N]
+                        ((double *)g.ws)[((long)piece * g.batch + b) * g.M * g.N + (long)m * g.N + n] = acc[i][j][r];
+                        continue;
+                    }
                     double *c = (double *)g.C + (long)b * g.sC + (long)m * g.ldc + n;
                     double v = acc[i][j][r];
                     if (g.beta != 0.f) v += *c;
@@ -135,9 +142,40 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
         }
 }
 
+// C = beta C + the pieces' partial sums, piece 0 first.
+__global__ __launch_bounds__(256) void gemm_f64_reduce_kernel(GemmArgs g) {
+    const long mn = (long)g.M * g.N, total = mn * g.batch;
+    for (long idx = (long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long)gridDim.x * 256) {
+        const long b = idx / mn, e = idx - b * mn;
+        const int m = (int)(e / g.N), n = (int)(e - (long)m * g.N);
+        const double *p = (const double *)g.ws + idx;
+        double v = 0.;
+        for (int s = 0; s < g.splits; ++s) v += p[(long)s * total];
+        double *c = (double *)g.C + b * g.sC + (long)m * g.ldc + n;
+        if (g.beta != 0.f) v += *c;
+        *c = v;
+    }
+}
+
+// Pieces for the fp64 kernel: only when 64 x 64 tiles leave most CUs idle, at least 16 K steps (256 k) per
+// piece, no more than the workspace holds.
+int gemm_f64_splits(int M, int N, int K, int batch, int red, size_t workspace_bytes, int *tiles_per_split) {
+    const long tiles = (long)ceil_div(M, 64) * ceil_div(N, 64) * batch, cus = cu_count();
+    const long total = (long)red * ceil_div(K, 16);
+    long splits = tiles * 2 <= cus ? 2 * cus / tiles : 1;
+    if (splits > total / 16) splits = total / 16;
+    if (splits > 256) splits = 256;
+    const size_t per = (size_t)batch * M * N * sizeof(double);
+    if (per && splits > (long)(workspace_bytes / per)) splits = (long)(workspace_bytes / per);
+    if (splits < 2) splits = 1;
+    const long tps = (total + splits - 1) / splits;
+    *tiles_per_split = (int)(tps < 1 ? 1 : tps);
+    return tps > 0 ? (int)((total + tps - 1) / tps) : 1;
+}
+
 template <int WT>
 static void launch_f64(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
-    dim3 grid(ceil_div(g.M, 32 * WT), ceil_div(g.N, 32 * WT), g.batch);
+    dim3 grid(ceil_div(g.M, 32 * WT), ceil_div(g.N, 32 * WT), g.batch * g.splits);
     if (!transA && !transB)
         hipLaunchKernelGGL((gemm_f64_kernel<false, false, WT>), grid, dim3(256), 0, stream, g);
     else if (!transA && transB)
@@ -146,13 +184,22 @@ static void launch_f64(const GemmArgs &g, int transA, int transB, hipStream_t st
         hipLaunchKernelGGL((gemm_f64_kernel<true, false, WT>), grid, dim3(256), 0, stream, g);
 }
 
-int gemm_f64_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream) {
-    D8_REQUIRE(ceil_div(g.N, 64) < 65536 && g.batch < 65536, "d8_gemm: grid too large");
+int gemm_f64_launch(const GemmArgs &args, int transA, int transB, hipStream_t stream) {
+    GemmArgs g = args;
+    const bool ws_ok = g.ws && ((size_t)g.ws & 7) == 0;
+    g.splits = gemm_f64_splits(g.M, g.N, g.K, g.batch, g.red, ws_ok ? g.ws_bytes : 0, &g.tiles_per_split);
+    D8_REQUIRE(ceil_div(g.N, 64) < 65536 && (long)g.batch * g.splits < 65536, "d8_gemm: grid too large");
     // 128 x 128 tiles when they alone fill most of the chip
     const long big = (long)ceil_div(g.M, 128) * ceil_div(g.N, 128) * g.batch;
     if (big >= (long)cu_count() * 3 / 4) launch_f64<4>(g, transA, transB, stream);
     else launch_f64<2>(g, transA, transB, stream);
     D8_LAUNCH_CHECK();
+    if (g.splits > 1) {
+        long blocks = ((long)g.M * g.N * g.batch + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(gemm_f64_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, g);
+        D8_LAUNCH_CHECK();
+    }
     return 0;
 }
 

@@ -311,9 +311,9 @@ int d8_avgpool2d_grad_overwrite(int dtype, void *dx, const void *dy, int B, int 
                                 int FH, int FW, int covered, int sy, int sx, void *stream);
 
 /* ---- measurement aid (no counterpart in the reference) ---------------------------------------
- * d8_mfma_stream issues the tiled GEMM's MFMA instruction back to back on operands taken from
- * `operands` (any device buffer; 16-byte aligned) and held in registers: two waves per SIMD on
- * every CU, no LDS or global traffic in the loop.  Timing one launch gives the rate the matrix
+ * d8_mfma_stream issues the GEMM kernels' MFMA instruction for `dtype` (D8_FLOAT16, D8_FLOAT32 or
+ * D8_FLOAT64) back to back on operands taken from `operands` (any device buffer; 16-byte aligned)
+ * and held in registers, on every CU, no LDS or global traffic in the loop.  Timing one launch gives the rate the matrix
  * pipe sustains on those operand bits, i.e. the ceiling a GEMM has on that data.  `out` takes
  * d8_mfma_stream_out_bytes() bytes; *flops receives the flops one launch performs.             */
 /* A second aid needs no entry point: with D8_GEMM_STAMPS set in the environment before the first launch, a

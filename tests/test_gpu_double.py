@@ -47,6 +47,35 @@ def test_gemm_f64_batched_broadcast_and_summed():
     assert np.array_equal(ops.gemm(1, 0, np.ascontiguousarray(Ai.transpose(0, 2, 1)), Bi), Ai @ Bi)
 
 
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("M,N,K,batch", [(64, 576, 20000, 1), (70, 33, 9001, 1), (40, 50, 5000, 3), (128, 128, 70000, 1)])
+def test_gemm_f64_long_reduction_is_split(ta, tb, M, N, K, batch):
+    """A small output with a long reduction runs in pieces through the workspace; the pieces must add up to the
+    same result as the whole (bit for bit on integers), with beta = 1 too, and without a workspace."""
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    assert lib.d8_gemm_workspace_bytes(capi.FLOAT64, ta, tb, M, N, K, batch, M * N if batch > 1 else 0) >= 2 * batch * M * N * 8
+    r = rng(M + N + K + batch)
+    sa, sb = ((batch, K, M) if ta else (batch, M, K)), ((batch, N, K) if tb else (batch, K, N))
+    Ai, Bi, Ci = d(ints(r, sa, 4)), d(ints(r, sb, 4)), d(ints(r, (batch, M, N)))
+    want = (Ai.transpose(0, 2, 1) if ta else Ai) @ (Bi.transpose(0, 2, 1) if tb else Bi)
+    assert np.array_equal(ops.gemm(ta, tb, Ai, Bi), want)
+    assert np.array_equal(ops.gemm(ta, tb, Ai, Bi, Ci, 1.0), want + Ci)
+    assert np.array_equal(ops.gemm(ta, tb, Ai, Bi, use_workspace=False), want)
+    A, B = r.standard_normal(sa), r.standard_normal(sb)
+    wantr = (A.transpose(0, 2, 1) if ta else A) @ (B.transpose(0, 2, 1) if tb else B)
+    assert rel_fro(ops.gemm(ta, tb, A, B), wantr) <= F64_TOL
+
+
+def test_gemm_f64_summed_batch_is_split():
+    """strideC = 0: the products of the whole batch are summed into one C, in pieces over products x K steps"""
+    from deep8_amd import ops
+    r = rng(79)
+    Ai, Bi = d(ints(r, (9, 48, 1000), 4)), d(ints(r, (9, 1000, 40), 4))
+    C0 = d(ints(r, (48, 40)))
+    assert np.array_equal(ops.gemm(0, 0, Ai, Bi, C0, 1.0), np.einsum("bmk,bkn->mn", Ai, Bi) + C0)
+
+
 def test_gemm_f64_large_against_numpy():
     from deep8_amd import ops
     r = rng(78)
