@@ -65,17 +65,24 @@ SETTLE_MS = 60.0
 
 
 def _settle(fn):
-    """keeps the device busy with fn for about SETTLE_MS, untimed; returns with the work still queued"""
+    """keeps the device busy with fn for SETTLE_MS of wall time, untimed.  The loop is bounded by the clock, not
+    by a call count derived from one timed call: the first call of an entry point in a process also loads its
+    code object, which would make that estimate far too small."""
     from deep8_amd import capi
     if SETTLE_MS <= 0:
         return
+    fn()
     capi.sync()
     t0 = time.perf_counter()
     fn()
     capi.sync()
     one = max(time.perf_counter() - t0, 1e-6)
-    for _ in range(min(20000, int(SETTLE_MS * 1e-3 / one) + 1)):
-        fn()
+    burst = max(1, min(64, int(2e-3 / one)))  # about 2 ms of work between two looks at the clock
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(burst):
+            fn()
+        capi.sync()
 
 
 def _time_steps(fn, steps, warmup):

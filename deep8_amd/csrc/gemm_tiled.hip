@@ -354,15 +354,24 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     }
     int id = blockIdx.x;
     const int total = tilesM * tilesN;
-    const int b = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z / g.splits;
+    int b = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z / g.splits;
     int split = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z - b * g.splits;
-    const int linear = id + total * split, whole = total * (g.splits & ~7);
-    if (linear < whole) {
-        const int j = linear >> 3, piece = j / total;
-        split = (piece << 3) + (linear & 7);
-        id = j - piece * total;
-    } else if ((total & 7) == 0) {
-        id = (id & 7) * (total >> 3) + (id >> 3);
+    {
+        // an unsplit batched product is dealt out the same way over its batch index: one XCD takes all
+        // tiles of a batch element, whose A and B it then reads once
+        const bool by_batch = g.splits == 1;
+        int layer = by_batch ? b : split;
+        const int layers = by_batch ? g.batch : g.splits;
+        const int linear = id + total * layer, whole = total * (layers & ~7);
+        if (linear < whole) {
+            const int j = linear >> 3, piece = j / total;
+            layer = (piece << 3) + (linear & 7);
+            id = j - piece * total;
+        } else if ((total & 7) == 0) {
+            id = (id & 7) * (total >> 3) + (id >> 3);
+        }
+        if (by_batch) b = layer;
+        else split = layer;
     }
     constexpr int GM = 4;
     const int band = id / (GM * tilesN), first = band * GM;
