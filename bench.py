@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Deep8 dense-contraction hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--no-cpu] [--no-others]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--no-cpu] [--no-others] [--settle-ms 60]
 
 A step is one forward + both backward passes of the workload over one batch of synthetic input that
 already sits in HBM.  The headline workload is benchmark configuration 3 (MatrixMultiply, half,
@@ -9,15 +9,16 @@ already sits in HBM.  The headline workload is benchmark configuration 3 (Matrix
 Prints ONE JSON line.
 
 Every measurement is preceded by --settle-ms (default 60) milliseconds of the same work, untimed: the chip's
-power management raises the shader clock over the first tens of milliseconds of sustained load, so a run that
+power management raises the shader clock over the first 35-50 milliseconds of sustained load, so a run that
 starts on an idle device and times 20 steps after 3 warm-up steps measures the ramp, not the rate a training
-loop sees (MatrixMultiply half 4096^3: about 1150 TFLOP/s from idle, about 1400 sustained, same box, same
+loop sees (MatrixMultiply half 4096^3: about 1185 TFLOP/s from idle, about 1425 sustained, same box, same
 binary).  --settle-ms 0 gives the from-idle number; the JSON line reports the value used as "settle_ms".
 
   value          whole-step throughput: algorithmic FLOPs of fwd + dX + dY / wall time of a step
                  (gradient destinations are zeroed inside the step, as Deep8's executor does)
-  roofline       the slowest of the step's GEMM launches, timed alone with HIP events on the stream
-                 it runs on, against the dense FP16 MFMA peak
+  roofline       flops of one GEMM launch / the average duration of the step's launches, each timed alone
+                 with HIP events on the stream it runs on, against the dense MFMA peak of the element type
+                 (element-wise and pooling workloads: the longest kernel's bytes / its duration, against HBM)
   cpu_baseline   Deep8's own CPU (Eigen) path from oracle/_ref -- or the C restatement when that was
                  not built -- on a bounded sample of the same workload, on this host's cores
 """
