@@ -323,6 +323,66 @@ class ConvWorkload:
                 "frac": round(ach / PEAK[dtype], 4), "launch_us": round(ms * 1e3, 2), "traffic": MEASURED_TRAFFIC.get(self.key)}
 
 
+class DeconvLiteralWorkload:
+    """Benchmark configuration 5 at its literal geometry (28 -> 56, PyTorch's ConvTranspose2d(k=4, s=2, p=1)),
+    which Deep8's DeConv2d does not admit (deep8/src/nodes/DeConv2d.cpp:36-52 allows 58 or 55): kernel level only,
+    through the explicit pads of the gather maps, the route the reference's GPU path takes
+    (deep8/src/math/DeConv2d.cu:251-308, 557-622, 826-891):
+      forward  zmat = X W^T (one GEMM)  ->  d8_deconv_col2im (padTop = padLeft = 2)
+      dX       d8_deconv_im2col(dz)     ->  dX = dzmat W
+      dW       d8_deconv_im2col(dz)     ->  dW = dzmat^T X"""
+
+    def __init__(self, name, seed):
+        from deep8_amd import capi
+        self.name, self.dtype, self.key = name, np.dtype(np.float16), name.split(":")[0]
+        self.lib = capi.init()
+        self.dt = capi.dtype_id(self.dtype)
+        r = np.random.default_rng(seed)
+        B, IH, IC, OC, F, S, OH, P = 16, 28, 128, 64, 4, 2, 56, 2
+        self.B, self.geo = B, (B, IH, IH, OH, OH, OC, F, F, S, S, P, P)
+        self.M, self.N, self.K = B * IH * IH, OC * F * F, IC
+        h = lambda a: _dev(a.astype(np.float32).astype(np.float16))
+        self.x = h(r.standard_normal((self.M, IC)))
+        self.w = h(r.standard_normal((self.N, IC)) * np.sqrt(2.0 / (F * F * IC)))
+        self.dz = h(r.standard_normal((B, OH, OH, OC)))
+        self.zmat = capi.DeviceArray((self.M, self.N), np.float16)
+        self.z = capi.DeviceArray((B, OH, OH, OC), np.float16)
+        self.dx = capi.DeviceArray((self.M, IC), np.float16)
+        self.dw = capi.DeviceArray((self.N, IC), np.float16)
+        self.ws_bytes = max(self.lib.d8_gemm_workspace_bytes(self.dt, ta, tb, m, n, k, 1, 0) for ta, tb, m, n, k in
+                            ((0, 1, self.M, self.N, self.K), (0, 0, self.M, self.K, self.N), (1, 0, self.N, self.K, self.M)))
+        self.ws = capi.DeviceArray((max(self.ws_bytes, 16),), np.uint8)
+        self.flops = 3 * 2.0 * self.M * self.N * self.K
+        nx, nw, nz, nm = self.M * IC, self.N * IC, B * OH * OH * OC, self.M * self.N
+        # GEMM operands and results once, the interim matrix written and read once per pass
+        self.bytes = 2 * ((nx + nw + 2 * nm + nz) + (nz + 2 * nm + nw + nx) + (nz + 2 * nm + nx + nw))
+
+    def _gemm(self, ta, tb, m, n, k, a, lda, b, ldb, c, ldc):
+        from deep8_amd.capi import check
+        check(self.lib.d8_gemm(self.dt, ta, tb, m, n, k, a.ptr, lda, 0, b.ptr, ldb, 0, 0.0, c.ptr, ldc, 0, 1,
+                               self.ws.ptr, self.ws_bytes, None))
+
+    def fwd(self):
+        from deep8_amd.capi import check
+        self._gemm(0, 1, self.M, self.N, self.K, self.x, self.K, self.w, self.K, self.zmat, self.N)
+        check(self.lib.d8_deconv_col2im(self.dt, self.zmat.ptr, self.z.ptr, *self.geo, None))
+
+    def grad_x(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_deconv_im2col(self.dt, self.dz.ptr, self.zmat.ptr, *self.geo, None))
+        self._gemm(0, 0, self.M, self.K, self.N, self.zmat, self.N, self.w, self.K, self.dx, self.K)
+
+    def grad_y(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_deconv_im2col(self.dt, self.dz.ptr, self.zmat.ptr, *self.geo, None))
+        self._gemm(1, 0, self.N, self.K, self.M, self.zmat, self.N, self.x, self.K, self.dw, self.K)
+
+    def step(self):
+        self.fwd()
+        self.grad_x()
+        self.grad_y()
+
+
 class BiasReluWorkload:
     """The element-wise steps after a convolution: Add (per-channel bias, broadcast) -> ReLu, and back:
     ReLuGrad -> AddGradY (bias gradient: a sum over batch, rows and columns).  HBM-bound."""
@@ -464,6 +524,9 @@ def make_workload(key):
     if key == "c5":
         return ConvWorkload("c5: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 58x58x64 (Deep8 covered=false)",
                             np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
+    if key == "c5l":
+        return DeconvLiteralWorkload("c5l: DeConv2d half B16 28x28x128 4x4 s2 -> 56x56x64 (the literal geometry of configuration 5; "
+                                     "kernel level: GEMM + gather maps with explicit pads)", 9)
     if key == "d3":
         return MatMulWorkload("d3: MatrixMultiply fwd+dX+dY double [2048x2048]x[2048x2048]", np.float64,
                               (1, 2048, 2048), (1, 2048, 2048), U, 10)
@@ -747,7 +810,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5", "e4", "p4"):
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5", "c5l", "e4", "p4", "d3"):
             if key == a.workload:
                 continue
             del wl
@@ -755,7 +818,7 @@ def main():
             oms = _time_steps(wl.step, 20, 3)
             o = {"ms_per_step": round(oms, 4), "tflops": round(wl.flops / (oms * 1e-3) / 1e12, 2),
                  "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
-            if isinstance(wl, (ConvWorkload, BiasReluWorkload, PoolWorkload)):
+            if isinstance(wl, (ConvWorkload, DeconvLiteralWorkload, BiasReluWorkload, PoolWorkload)):
                 o["images_per_s"] = round(wl.B / (oms * 1e-3), 1)
             if key == "c1":  # launch-latency bound: the same three launches replayed from a HIP graph
                 o["ms_per_step_graph_replay"] = round(graph_replay_ms(wl, 50, 5), 4)
