@@ -75,8 +75,8 @@ int d8_event_elapsed_ms(void *start, void *stop, float *ms);  /* synchronises on
  * strideA/strideB 0 broadcasts that operand over the batch.  strideC == 0 with batch > 1
  * sums all batch products into the one C (Deep8's gradient of a batch-1 operand).
  * fp16 operands accumulate in fp32 and are rounded once; beta = 1 adds the old C in fp32.
- * D8_FLOAT64 operands accumulate in fp64 (the cublasDgemm twins of the call sites below); their
- * reduction is never split, so d8_gemm_workspace_bytes is 0 for them.
+ * D8_FLOAT64 operands accumulate in fp64 (the cublasDgemm twins of the call sites below); a split
+ * reduction keeps its partial sums in fp64 too.
  *
  * `workspace` (may be NULL) lets the kernel split the reduction (long K / summed batch, small
  * M x N) over more workgroups; d8_gemm_workspace_bytes says how much it can use.  It must be
