@@ -84,3 +84,56 @@ def test_random_shapes_against_the_oracle(oracle_port, seed):
         for k, (g, w) in enumerate(zip(got, want)):
             assert np.array_equal(g, w), (desc, k)
     assert ran > 150
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_pooling_geometries_against_the_oracle(oracle_port, seed):
+    """Pooling gradients over drawn geometries, overlapping windows (the gather kernel) and non-overlapping ones
+    (a thread per window writes its stride cell), accumulate and overwrite forms, fp32 and half; integer inputs
+    with many ties, so the first maximum must win: bit-exact."""
+    from deep8_amd import ops
+    r = np.random.default_rng(seed)
+    pick = lambda *o: o[r.integers(0, len(o))]
+    ran = 0
+    for _ in range(120):
+        B, IH, IW, C = int(pick(1, 2, 3)), int(pick(1, 4, 7, 8, 13, 16)), int(pick(1, 5, 8, 9, 16)), int(pick(1, 3, 4, 8, 16, 24))
+        FH, FW, sy, sx, cov = int(pick(1, 2, 3)), int(pick(1, 2, 3)), int(pick(1, 2, 3, 4)), int(pick(1, 2, 3)), bool(pick(0, 1))
+        if FH > IH or FW > IW:
+            continue
+        half = r.random() < 0.4
+        c = h if half else (lambda a: np.asarray(a, np.float32))
+        a = (FH, FW, cov, sy, sx)
+        x = c(r.integers(-2, 3, size=(B, IH, IW, C)).astype(np.float32))
+        y = oracle_port.pool2d(True, f(x), *a)
+        dy = c(r.integers(0, 4, size=y.shape).astype(np.float32))
+        dx0 = c(r.integers(0, 4, size=x.shape).astype(np.float32))
+        nan = np.full(x.shape, np.nan, x.dtype)
+        desc = (B, IH, IW, C, FH, FW, cov, sy, sx, half)
+        assert np.array_equal(f(ops.maxpool2d(x, *a)), y), desc
+        assert np.array_equal(f(ops.maxpool2d_grad(x, dy, *a, dx=dx0)), oracle_port.pool2d_grad(True, f(x), f(dy), *a, dx=f(dx0))), desc
+        assert np.array_equal(f(ops.maxpool2d_grad(x, dy, *a, dx=nan, overwrite=True)), oracle_port.pool2d_grad(True, f(x), f(dy), *a)), desc
+        if FH * FW in (1, 2, 4):  # dy / (FH * FW) is exact
+            assert np.array_equal(f(ops.avgpool2d_grad(x.shape, dy, *a, dx=dx0)), oracle_port.pool2d_grad(False, f(x), f(dy), *a, dx=f(dx0))), desc
+            assert np.array_equal(f(ops.avgpool2d_grad(x.shape, dy, *a, dx=nan, overwrite=True)), oracle_port.pool2d_grad(False, f(x), f(dy), *a)), desc
+        ran += 1
+    assert ran > 80
+
+
+@pytest.mark.parametrize("seed", [31])
+def test_random_double_products_against_numpy(seed):
+    """fp64 d8_gemm over drawn shapes, among them small outputs with long reductions (split through the workspace)
+    and outputs large enough for the 128 x 128 tiles; integer inputs: bit-exact."""
+    from deep8_amd import ops
+    r = np.random.default_rng(seed)
+    pick = lambda *o: o[r.integers(0, len(o))]
+    for _ in range(60):
+        M, N = int(pick(1, 7, 33, 64, 100, 128, 257, 700, 1800)), int(pick(1, 5, 64, 72, 136, 576, 1700))
+        K = int(pick(1, 15, 16, 17, 100, 1000, 4097, 30000))
+        if M * N * K > 3e9:
+            continue
+        ta, tb = pick((0, 0), (0, 1), (1, 0))
+        A = r.integers(0, 9, size=(K, M) if ta else (M, K)).astype(np.float64)
+        B = r.integers(0, 9, size=(N, K) if tb else (K, N)).astype(np.float64)
+        C0, beta = r.integers(0, 9, size=(M, N)).astype(np.float64), float(pick(0, 1))
+        want = (A.T if ta else A) @ (B.T if tb else B) + beta * C0
+        assert np.array_equal(ops.gemm(ta, tb, A, B, C0, beta), want), (ta, tb, M, N, K, beta)
