@@ -907,6 +907,8 @@ TEST_GPU(two_layer_convnet_trains_with_sgd) {
 // Node-level step times at the three large configurations: forward + both gradients through Function::forward /
 // backward, i.e. with the scratch buffer taken from and returned to the device pool inside every call and the
 // gradients zeroed before the backward pass (lazily: Tensor::zero defers the fill).  Printed, not asserted.
+// The device is kept busy with the same steps for 60 ms first: the chip raises its shader clock over the first
+// 35-50 ms of sustained load, and a loop timed from an idle device measures that ramp.
 template <typename NodeT>
 void timeNode(const char *what, NodeT &node, HostTensor &a, HostTensor &b, HostTensor &z, HostTensor &gz, HostTensor &ga,
               HostTensor &gb, double flops) {
@@ -918,6 +920,12 @@ void timeNode(const char *what, NodeT &node, HostTensor &a, HostTensor &b, HostT
         node.backward(tin, &z.t, &gz.t, 0, &ga.t);
         node.backward(tin, &z.t, &gz.t, 1, &gb.t);
     };
+    step();
+    gpu().synchronize();
+    for (const auto s0 = std::chrono::steady_clock::now(); std::chrono::steady_clock::now() - s0 < std::chrono::milliseconds(60);) {
+        for (int i = 0; i < 4; ++i) step();
+        gpu().synchronize();
+    }
     for (int i = 0; i < 3; ++i) step();
     gpu().synchronize();
     const int reps = 20;
