@@ -450,7 +450,11 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
 
     // ---- this workgroup's steps x0 .. x0 + nsteps - 1 of the extended reduction; step x reads
     // product x / ktiles at K offset (x % ktiles) * BK (all uniform: scalar arithmetic)
-    const int ktiles = g.K / BK;
+    // K need not be a multiple of the K step for real matrices: the last step of a product is then partly past
+    // K, and the pieces that lie past it are fetched at an offset beyond the buffer, i.e. as zeros.
+    const int ktiles = (g.K + BK - 1) / BK, tail_len = g.K % BK;
+    const unsigned av_plain = (unsigned)ES * ((unsigned)a_r * (unsigned)g.lda + a_c * EPV);
+    const unsigned bv_plain = (unsigned)ES * ((unsigned)b_r * (unsigned)g.ldb + b_c * EPV);
     const int x0 = split * g.tiles_per_split, nsteps = min(red * ktiles, x0 + g.tiles_per_split) - x0;
     const unsigned a_prod = (unsigned)ES * (unsigned)g.sA, b_prod = (unsigned)ES * (unsigned)g.sB;
     const unsigned b_prod_row = (unsigned)ES * (unsigned)g.sB_row, b_first = (unsigned)ES * b_cls;
@@ -466,7 +470,18 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
             }
             return 0u;
         } else {
-            return Au + (g.red > 1 ? r * a_prod : 0u) + (x - r * ktiles) * a_step;
+            const int kx = x - r * ktiles;
+            if constexpr (VIRT == VIRT_NONE) {
+                if (tail_len) {
+                    const bool tail = kx == ktiles - 1;
+#pragma unroll
+                    for (int p = 0; p < A_IT; ++p) {
+                        const bool past = A_KC ? a_c * EPV >= tail_len : a_r + p * T::A_ROWS >= tail_len;
+                        av[p] = tail && past ? OUTSIDE : av_plain;
+                    }
+                }
+            }
+            return Au + (g.red > 1 ? r * a_prod : 0u) + kx * a_step;
         }
     };
     auto step_b = [&](int i) -> unsigned {
@@ -489,7 +504,18 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
             const int fy = r / pg.FW, fx = r - fy * pg.FW;
             return Bu + b_first + fy * b_prod_row + fx * b_prod + (x - r * ktiles) * b_step;
         } else {
-            return Bu + (g.red > 1 ? r * b_prod : 0u) + (x - r * ktiles) * b_step;
+            const int kx = x - r * ktiles;
+            if constexpr (VIRT == VIRT_NONE) {
+                if (tail_len) {
+                    const bool tail = kx == ktiles - 1;
+#pragma unroll
+                    for (int p = 0; p < B_IT; ++p) {
+                        const bool past = B_KC ? b_c * EPV >= tail_len : b_r + p * T::B_ROWS >= tail_len;
+                        bv[p] = tail && past ? OUTSIDE : bv_plain;
+                    }
+                }
+            }
+            return Bu + (g.red > 1 ? r * b_prod : 0u) + kx * b_step;
         }
     };
 
@@ -576,7 +602,7 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     // a 64-wide side gets a tile of that width (im2col products with 64 output channels)
     if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
     if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
-    if (g.splits == 1 && gemm_tiled_half_tiles(g.M, g.N, g.batch, (long)g.red * (g.K / (128 / (int)sizeof(E)))))
+    if (g.splits == 1 && gemm_tiled_half_tiles(g.M, g.N, g.batch, (long)g.red * ceil_div(g.K, 128 / (int)sizeof(E))))
         return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
     return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
 }
@@ -592,7 +618,10 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
     // byte offsets inside one operand (all summed products of it included) are 32-bit
     if (!va && ((g.red - 1) * g.sA + (long)(transA ? g.K : g.M) * g.lda) * ES >= (1L << 31)) return false;
     if (!vb && ((g.red - 1) * g.sB + (long)(transB ? g.N : g.K) * g.ldb) * ES >= (1L << 31)) return false;
-    if (g.M < 64 || g.N < 64 || (g.M < 128 && g.N < 128) || g.K < BK || g.K % BK) return false;
+    if (g.M < 64 || g.N < 64 || (g.M < 128 && g.N < 128) || g.K < BK) return false;
+    // a last K step that is partly past K: real matrices only, and a 16-byte piece of an operand stored along K
+    // must lie wholly on one side of K
+    if (g.K % BK && (g.virt != VIRT_NONE || ((!transA || transB) && g.K % EPV))) return false;
     if (!va && (g.lda % EPV || g.sA % EPV)) return false;
     if (!vb && (g.ldb % EPV || g.sB % EPV)) return false;
     if (((size_t)g.A | (size_t)g.B) & 15) return false;

@@ -219,3 +219,41 @@ def test_gemm_operand_beyond_2_gib():
     got = ops.gemm(1, 0, np.ascontiguousarray(At[:, :128]), Bbig)
     want = At[:, :128].T @ Bbig
     assert np.array_equal(got[0] if got.ndim == 3 else got, want)
+
+
+@pytest.mark.parametrize("ta,tb", TRANS)
+@pytest.mark.parametrize("M,N,K", [(256, 1000, 784), (300, 264, 100), (136, 130, 72), (128, 128, 40), (512, 256, 1000),
+                                   (2000, 64, 200), (64, 520, 328), (1024, 1024, 4000)])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_gemm_reduction_not_a_multiple_of_the_k_step(ta, tb, M, N, K, dtype):
+    """K ends inside a K step of the tiled kernels: what lies past K must count as zero whatever the memory there
+    holds.  Operands stored along K are given a leading dimension of K + 8 with NaN in the padding, operands stored
+    K-row-major are followed by rows of NaN; two products are summed into one C as well (strideC = 0), where the
+    rows past K of the first are the second's."""
+    from deep8_amd import capi
+    lib = capi.init()
+    r = rng(M + 3 * N + 7 * K)
+    hi = 2 if dtype == np.float16 else 30
+    dt = capi.dtype_id(np.dtype(dtype))
+    for batch in (1, 2):
+        A = r.integers(0, hi, size=(batch, K, M) if ta else (batch, M, K)).astype(np.float64)
+        B = r.integers(0, hi, size=(batch, N, K) if tb else (batch, K, N)).astype(np.float64)
+        if dtype == np.float16:  # thin the operands so that every sum stays below 2048
+            A *= r.random(A.shape) < 0.3
+            B *= r.random(B.shape) < 0.3
+        want = np.einsum("bmk,bkn->mn", A.transpose(0, 2, 1) if ta else A, B.transpose(0, 2, 1) if tb else B)
+        assert dtype == np.float32 or want.max() < 2048
+
+        def padded(X, along_k):
+            b, rows, cols = X.shape
+            P = np.full((b, rows + (0 if along_k else 8), cols + (8 if along_k else 0)), np.nan)
+            P[:, :rows, :cols] = X
+            return P.astype(dtype)
+        Ap, Bp = padded(A, not ta), padded(B, bool(tb))
+        dA, dB = capi.DeviceArray.from_numpy(Ap), capi.DeviceArray.from_numpy(Bp)
+        dC = capi.DeviceArray.from_numpy(np.full((M, N), np.nan, dtype))
+        wsb = lib.d8_gemm_workspace_bytes(dt, ta, tb, M, N, K, batch, 0)
+        ws = capi.DeviceArray((max(wsb, 16),), np.uint8)
+        capi.check(lib.d8_gemm(dt, ta, tb, M, N, K, dA.ptr, Ap.shape[2], Ap.shape[1] * Ap.shape[2], dB.ptr, Bp.shape[2],
+                               Bp.shape[1] * Bp.shape[2], 0.0, dC.ptr, N, 0, batch, ws.ptr, wsb, None))
+        assert np.array_equal(dC.numpy().astype(np.float64), want), (ta, tb, M, N, K, batch)
