@@ -226,6 +226,7 @@ __device__ inline float as_f32(f16 v) { return (float)v; }
 struct Origin {
     int m0, n0;        // where the computed tile starts (moved inside the matrix)
     int m_own, n_own;  // rows / columns from here on are this workgroup's to store
+    int m_end, n_end;  // ... up to the matrix's own (a tile may be larger than a matrix with fewer than BM rows or BN columns)
     int wm0, wn0;      // this wave's offset inside the tile
 };
 
@@ -275,7 +276,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
                     float v[8];
                     *(f32x4 *)&v[0] = *(const f32x4 *)(patch + row * 36 + cc);
                     *(f32x4 *)&v[4] = *(const f32x4 *)(patch + row * 36 + cc + 4);
-                    if (m >= o.m_own && n >= o.n_own) {
+                    if (m >= o.m_own && n >= o.n_own && m < o.m_end && n < o.n_end) {
                         O *c = C + crow(m) * ldc + n;
 #pragma unroll
                         for (int h = 0; h < 8 / OPV; ++h) {
@@ -303,7 +304,7 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = o.m0 + o.wm0 + i * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-                if (m >= o.m_own && n >= o.n_own) {
+                if (m >= o.m_own && n >= o.n_own && m < o.m_end && n < o.n_end) {
                     O *c = C + crow.at(m, n, ldc);
                     float v = acc[i][j][r];
                     if (beta != 0.f) v += as_f32(*c);
@@ -381,7 +382,10 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     // A tile that would stick out of the matrix is moved back inside; the rows / columns it then
     // shares with its neighbour are computed twice but stored only by the neighbour.
     const int m_own = tm * BM, n_own = tn * BN;
-    const int m0 = min(m_own, M - BM), n0 = min(n_own, g.N - BN);
+    // (a matrix with fewer rows or columns than the tile: the tile starts at 0 and reaches past it; what the loads
+    // bring in from there -- zeros past the end of the buffer, otherwise whatever follows -- only ever enters
+    // results of rows / columns past the matrix, which are not stored)
+    const int m0 = max(0, min(m_own, M - BM)), n0 = max(0, min(n_own, g.N - BN));
 
     // ---- the 16-byte pieces this thread moves each K step: piece `it` of an operand lies a fixed
     // number of rows below piece 0, in global memory and in LDS alike.  Global memory is read
@@ -561,7 +565,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
 
     // ---- epilogue: the result itself, or this piece's fp32 partial sums when the reduction is split
     __syncthreads();  // every wave is past the last step: the operand areas are free
-    const Origin o = {m0, n0, m_own, n_own, (wm * TM) * 32, (wn * TN) * 32};
+    const Origin o = {m0, n0, m_own, n_own, M, g.N, (wm * TM) * 32, (wn * TN) * 32};
     float *patches = (float *)(T::PATCH_IN_A ? As0 : Bs0), *patches1 = (float *)(T::PATCH_IN_A ? As1 : Bs1);
     if (g.splits > 1)
         store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o, plain);
@@ -618,7 +622,10 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
     // byte offsets inside one operand (all summed products of it included) are 32-bit
     if (!va && ((g.red - 1) * g.sA + (long)(transA ? g.K : g.M) * g.lda) * ES >= (1L << 31)) return false;
     if (!vb && ((g.red - 1) * g.sB + (long)(transB ? g.N : g.K) * g.ldb) * ES >= (1L << 31)) return false;
-    if (g.M < 64 || g.N < 64 || (g.M < 128 && g.N < 128) || g.K < BK) return false;
+    // one side may be shorter than any tile (a few rows against a wide matrix: the 64 x 128 / 128 x 64 tile
+    // then reaches past it) when the other side fills a tile
+    if ((g.M < 128 && g.N < 128) || g.K < BK) return false;
+    if ((g.M < 64 || g.N < 64) && g.virt != VIRT_NONE) return false;
     // a last K step that is partly past K: real matrices only, and a 16-byte piece of an operand stored along K
     // must lie wholly on one side of K
     if (g.K % BK && (g.virt != VIRT_NONE || ((!transA || transB) && g.K % EPV))) return false;

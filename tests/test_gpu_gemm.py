@@ -51,7 +51,10 @@ def test_gemm_f16_integer_exact(oracle_port, ta, tb, M, N, K):
 @pytest.mark.parametrize("ta,tb", TRANS)
 @pytest.mark.parametrize("M,N,K", [(300, 264, 128), (136, 130, 64), (512, 520, 256), (1000, 392, 192), (304, 261, 128),
                                    (256, 256, 64), (768, 1280, 448), (1000, 64, 192), (64, 520, 256), (300, 72, 128),
-                                   (96, 264, 64), (128, 64, 64), (64, 128, 128), (2000, 120, 576)])
+                                   (96, 264, 64), (128, 64, 64), (64, 128, 128), (2000, 120, 576),
+                                   # fewer rows or columns than any tile against a wide other side
+                                   (32, 520, 256), (1, 256, 128), (8, 136, 64), (300, 16, 128), (48, 1000, 192), (200, 24, 64),
+                                   (16, 4096, 512), (640, 8, 256)])
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 def test_gemm_tiled_kernels_edge_tiles(oracle_port, ta, tb, M, N, K, dtype):
     """Shapes that take the tiled kernels (K a multiple of 64, rows movable in 16-byte pieces) with
@@ -223,7 +226,7 @@ def test_gemm_operand_beyond_2_gib():
 
 @pytest.mark.parametrize("ta,tb", TRANS)
 @pytest.mark.parametrize("M,N,K", [(256, 1000, 784), (300, 264, 100), (136, 130, 72), (128, 128, 40), (512, 256, 1000),
-                                   (2000, 64, 200), (64, 520, 328), (1024, 1024, 4000)])
+                                   (2000, 64, 200), (64, 520, 328), (1024, 1024, 4000), (32, 520, 200), (304, 16, 72), (8, 256, 1000)])
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 def test_gemm_reduction_not_a_multiple_of_the_k_step(ta, tb, M, N, K, dtype):
     """K ends inside a K step of the tiled kernels: what lies past K must count as zero whatever the memory there
