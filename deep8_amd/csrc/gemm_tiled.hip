@@ -624,7 +624,7 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
     if (!vb && ((g.red - 1) * g.sB + (long)(transB ? g.N : g.K) * g.ldb) * ES >= (1L << 31)) return false;
     // one side may be shorter than any tile (a few rows against a wide matrix: the 64 x 128 / 128 x 64 tile
     // then reaches past it) when the other side fills a tile
-    if ((g.M < 128 && g.N < 128) || g.K < BK) return false;
+    if ((g.M < 128 && g.N < 128) || g.K < 1) return false;  // (a K below one K step is a lone partial step)
     if ((g.M < 64 || g.N < 64) && g.virt != VIRT_NONE) return false;
     // a last K step that is partly past K: real matrices only, and a 16-byte piece of an operand stored along K
     // must lie wholly on one side of K

@@ -226,7 +226,8 @@ def test_gemm_operand_beyond_2_gib():
 
 @pytest.mark.parametrize("ta,tb", TRANS)
 @pytest.mark.parametrize("M,N,K", [(256, 1000, 784), (300, 264, 100), (136, 130, 72), (128, 128, 40), (512, 256, 1000),
-                                   (2000, 64, 200), (64, 520, 328), (1024, 1024, 4000), (32, 520, 200), (304, 16, 72), (8, 256, 1000)])
+                                   (2000, 64, 200), (64, 520, 328), (1024, 1024, 4000), (32, 520, 200), (304, 16, 72), (8, 256, 1000),
+                                   (300, 264, 32), (2000, 64, 8), (136, 130, 16), (64, 520, 24)])
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
 def test_gemm_reduction_not_a_multiple_of_the_k_step(ta, tb, M, N, K, dtype):
     """K ends inside a K step of the tiled kernels: what lies past K must count as zero whatever the memory there
