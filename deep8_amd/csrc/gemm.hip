@@ -81,8 +81,8 @@ __device__ inline void wave_mma(const float *As, const float *Bs, int arow, int 
 template <typename T, bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_general_kernel(GemmArgs g) {
     constexpr int BM = 128, BN = 128, BK = Tile<T>::BK, LD = Tile<T>::LD;
-    __shared__ __attribute__((aligned(16))) T As[BM * LD];
-    __shared__ __attribute__((aligned(16))) T Bs[BN * LD];
+    __shared__ __attribute__((aligned(16))) T As[2][BM * LD];
+    __shared__ __attribute__((aligned(16))) T Bs[2][BN * LD];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -102,41 +102,63 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    for (int t = t0; t < t1; ++t) {
+    // A thread moves NE elements of each operand per K step; element u is tile element tid + 256 u.  Stored
+    // along K (A not transposed, B transposed): k = tid % BK for every u, row tid / BK + u * (256 / BK); stored
+    // K-row-major: row or column tid % 128, k = tid / 128 + 2 u.  The next step's elements are fetched into
+    // registers before the current step is multiplied and written to the other LDS half after it.
+    constexpr int NE = BM * BK / 256;
+    static_assert(BM == BN && 256 % BK == 0 && BM == 128, "element map");
+    const int kc_k = tid % BK, kc_row = tid / BK, tr_col = tid % 128, tr_k = tid / 128;
+    const bool a_in = TA ? m0 + tr_col < g.M : true, b_in = TB ? true : n0 + tr_col < g.N;
+    T pa[NE], pb[NE];
+    auto fetch = [&](int t) {
         const int r = t / ktiles, k0 = (t - r * ktiles) * BK;
         const T *Ap = (const T *)g.A + (long)(b + r) * g.sA;
         const T *Bp = (const T *)g.B + (long)(b + r) * g.sB;
-
-        for (int i = tid; i < BM * BK; i += 256) {
-            int m, k;
-            if (!TA) {
-                m = i / BK;
-                k = i % BK;
+#pragma unroll
+        for (int u = 0; u < NE; ++u) {
+            pa[u] = (T)0;
+            if (TA) {
+                const int gk = k0 + tr_k + 2 * u;
+                if (a_in && gk < g.K) pa[u] = Ap[(long)gk * g.lda + m0 + tr_col];
             } else {
-                k = i / BM;
-                m = i % BM;
+                const int gm = m0 + kc_row + u * (256 / BK);
+                if (gm < g.M && k0 + kc_k < g.K) pa[u] = Ap[(long)gm * g.lda + k0 + kc_k];
             }
-            const int gm = m0 + m, gk = k0 + k;
-            T v = (T)0;
-            if (gm < g.M && gk < g.K) v = TA ? Ap[(long)gk * g.lda + gm] : Ap[(long)gm * g.lda + gk];
-            As[m * LD + k] = v;
         }
-        for (int i = tid; i < BN * BK; i += 256) {
-            int n, k;
+#pragma unroll
+        for (int u = 0; u < NE; ++u) {
+            pb[u] = (T)0;
             if (TB) {
-                n = i / BK;
-                k = i % BK;
+                const int gn = n0 + kc_row + u * (256 / BK);
+                if (gn < g.N && k0 + kc_k < g.K) pb[u] = Bp[(long)gn * g.ldb + k0 + kc_k];
             } else {
-                k = i / BN;
-                n = i % BN;
+                const int gk = k0 + tr_k + 2 * u;
+                if (b_in && gk < g.K) pb[u] = Bp[(long)gk * g.ldb + n0 + tr_col];
             }
-            const int gn = n0 + n, gk = k0 + k;
-            T v = (T)0;
-            if (gn < g.N && gk < g.K) v = TB ? Bp[(long)gn * g.ldb + gk] : Bp[(long)gk * g.ldb + gn];
-            Bs[n * LD + k] = v;
         }
-        __syncthreads();
-        wave_mma<2, 2, LD, BK>(As, Bs, wm * 64, wn * 64, lane, acc);
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < NE; ++u) {
+            if (TA) As[buf][tr_col * LD + tr_k + 2 * u] = pa[u];
+            else As[buf][(kc_row + u * (256 / BK)) * LD + kc_k] = pa[u];
+            if (TB) Bs[buf][(kc_row + u * (256 / BK)) * LD + kc_k] = pb[u];
+            else Bs[buf][tr_col * LD + tr_k + 2 * u] = pb[u];
+        }
+    };
+
+    if (t0 < t1) {
+        fetch(t0);
+        stage(0);
+    }
+    __syncthreads();
+    for (int t = t0; t < t1; ++t) {
+        const int cur = (t - t0) & 1;
+        const bool more = t + 1 < t1;
+        if (more) fetch(t + 1);
+        wave_mma<2, 2, LD, BK>(As[cur], Bs[cur], wm * 64, wn * 64, lane, acc);
+        if (more) stage(cur ^ 1);  // nobody reads that half before the barrier below
         __syncthreads();
     }
 
