@@ -334,18 +334,36 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(GemmArgs g) {
     }
 }
 
-// The same for N not a multiple of 4: one output per thread, partials added in split order.
+// The same for N not a multiple of 4: a workgroup covers 32 outputs; its 8 thread rows each add every 8th
+// partial (four loads in flight) and the 8 sums meet in LDS in a fixed order.
 template <typename T>
-__global__ void gemm_split_reduce_scalar_kernel(GemmArgs g) {
+__global__ __launch_bounds__(256) void gemm_split_reduce_scalar_kernel(GemmArgs g) {
+    __shared__ float part[8][32];
     const long mn = (long)g.M * g.N;
-    const long total = mn * g.batch;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-        const int b = (int)(i / mn);
-        const long e = i - (long)b * mn;
-        const int m = (int)(e / g.N), n = (int)(e - (long)m * g.N);
+    const int lane = threadIdx.x & 31, row = threadIdx.x >> 5;
+    const long i = (long)blockIdx.x * 32 + lane;
+    const bool live = i < mn * g.batch;
+    const int b = live ? (int)(i / mn) : 0;
+    const long e = i - (long)b * mn;
+    float v = 0.f;
+    if (live) {
         const float *p = g.ws + (long)b * g.splits * mn + e;
-        float v = 0.f;
-        for (int s = 0; s < g.splits; ++s) v += p[(long)s * mn];
+        int s = row;
+        for (; s + 24 < g.splits; s += 32) {
+            float t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = p[(long)(s + 8 * u) * mn];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v += t[u];
+        }
+        for (; s < g.splits; s += 8) v += p[(long)s * mn];
+    }
+    part[row][lane] = v;
+    __syncthreads();
+    if (row == 0 && live) {
+#pragma unroll
+        for (int k = 1; k < 8; ++k) v += part[k][lane];
+        const int m = (int)(e / g.N), n = (int)(e - (long)m * g.N);
         T *c = (T *)g.C + (long)b * g.sC + c_index(g, m, n);
         if (g.beta != 0.f) v += to_f32(*c);
         *c = (T)v;
@@ -383,7 +401,7 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     if (max_by_len * tiles < cus / 2) max_by_len = total / 4;
     if (max_by_len < 1) max_by_len = 1;
     if (splits > max_by_len) splits = max_by_len;
-    if (splits > 128) splits = 128;
+    if (splits > 512) splits = 512;
     // no more pieces than the caller's workspace holds
     const size_t per_split = (size_t)batch * M * N * sizeof(float);
     const long fit = (long)(workspace_bytes / per_split);
@@ -424,9 +442,7 @@ static int launch(GemmArgs &g, int transA, int transB, bool tiled, hipStream_t s
         if (g.N % 4 == 0 && ((size_t)g.ws & 15) == 0) {
             hipLaunchKernelGGL((gemm_split_reduce_kernel<T>), dim3((unsigned)((total / 4 + 31) / 32)), dim3(256), 0, stream, g);
         } else {
-            int blocks = (int)((total + 255) / 256);
-            if (blocks > 4096) blocks = 4096;
-            hipLaunchKernelGGL((gemm_split_reduce_scalar_kernel<T>), dim3(blocks), dim3(256), 0, stream, g);
+            hipLaunchKernelGGL((gemm_split_reduce_scalar_kernel<T>), dim3((unsigned)((total + 31) / 32)), dim3(256), 0, stream, g);
         }
         D8_LAUNCH_CHECK();
     }
