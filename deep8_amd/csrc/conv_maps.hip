@@ -51,6 +51,45 @@ __global__ __launch_bounds__(256) void im2col_kernel(const V *__restrict__ im, V
     }
 }
 
+// The same with rows padded to `pitch` elements (a patch row whose own length cannot be moved in 16-byte
+// pieces: 1- and 3-channel images); the padding is written as zeros.  A thread gathers the NV elements of one
+// 16-byte piece of a row (the pitch is a multiple of that) and stores them at once.
+template <typename V, int NV>
+__global__ __launch_bounds__(256) void im2col_padded_kernel(const V *__restrict__ im, V *__restrict__ col, MapGeom g, long total) {
+    typedef V VV __attribute__((ext_vector_type(NV)));
+    const int K = g.FH * g.FW * g.C, pieces = g.pitch / NV;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int j0 = (int)(idx % pieces) * NV;
+        const long r = idx / pieces;
+        const int ox = (int)(r % g.OW);
+        const long q = r / g.OW;
+        const int oy = (int)(q % g.OH), b = (int)(q / g.OH);
+        const V *img = im + (long)b * g.IH * g.IW * g.C;
+        VV v;
+#pragma unroll
+        for (int e = 0; e < NV; ++e) {
+            const int j = j0 + e;
+            V s = 0;
+            if (j < K) {
+                const int tap = j / g.C, c = j - tap * g.C, fx = tap % g.FW, fy = tap / g.FW;
+                const int iy = oy * g.sy + fy * g.dy - g.pt, ix = ox * g.sx + fx * g.dx - g.pl;
+                if (iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW) s = img[((long)iy * g.IW + ix) * g.C + c];
+            }
+            v[e] = s;
+        }
+        *(VV *)(col + r * g.pitch + j0) = v;
+    }
+}
+
+template <typename V>
+__global__ __launch_bounds__(256) void pad_rows_kernel(const V *__restrict__ src, V *__restrict__ dst, int K, int pitch, long total) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const int j = (int)(idx % pitch);
+        const long r = idx / pitch;
+        dst[idx] = j < K ? src[r * K + j] : (V)0;
+    }
+}
+
 // ---- col2im: one thread owns VEC channels of one image pixel; taps are added in (fy, fx)
 // ascending order into registers, then the pixel is written once. -----------------------------
 template <typename T, int VEC, bool ACC>
@@ -102,7 +141,7 @@ __global__ __launch_bounds__(256) void col2im_kernel(const T *__restrict__ col, 
 template <typename T, bool ACC>
 __global__ __launch_bounds__(256) void col2im_scalar_kernel(const T *__restrict__ col, T *__restrict__ im,
                                                             MapGeom g, long total) {
-    const long K = (long)g.FH * g.FW * g.C;
+    const long K = g.pitch ? (long)g.pitch : (long)g.FH * g.FW * g.C;  // row pitch of col
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
          idx += (long)gridDim.x * blockDim.x) {
         const int c = (int)(idx % g.C);
@@ -199,9 +238,52 @@ static int check_geom(const char *who, int dtype, const void *a, const void *b, 
 
 static inline bool aligned16(const void *p) { return ((size_t)p & 15) == 0; }
 
+template <typename T>
+__global__ __launch_bounds__(256) void unpad_add_kernel(const T *__restrict__ src, T *__restrict__ dst, int K, int pitch, long total, float beta) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / K;
+        const int j = (int)(idx - r * K);
+        float v = (float)src[r * pitch + j];
+        if (beta != 0.f) v += (float)dst[idx];
+        dst[idx] = (T)v;
+    }
+}
+
+int launch_unpad_add(int dtype, const void *src, void *dst, long rows, int K, int pitch, float beta, hipStream_t s) {
+    const long total = rows * K;
+    if (total == 0) return 0;
+    if (dtype == D8_FLOAT32)
+        hipLaunchKernelGGL((unpad_add_kernel<float>), dim3(grid_for(total, 256)), dim3(256), 0, s, (const float *)src, (float *)dst, K, pitch, total, beta);
+    else
+        hipLaunchKernelGGL((unpad_add_kernel<f16>), dim3(grid_for(total, 256)), dim3(256), 0, s, (const f16 *)src, (f16 *)dst, K, pitch, total, beta);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_pad_rows(int dtype, const void *src, void *dst, long rows, int K, int pitch, hipStream_t s) {
+    const long total = rows * pitch;
+    if (total == 0) return 0;
+    if (dtype_bytes(dtype) == 4)
+        hipLaunchKernelGGL((pad_rows_kernel<unsigned>), dim3(grid_for(total, 256)), dim3(256), 0, s, (const unsigned *)src, (unsigned *)dst, K, pitch, total);
+    else
+        hipLaunchKernelGGL((pad_rows_kernel<unsigned short>), dim3(grid_for(total, 256)), dim3(256), 0, s, (const unsigned short *)src, (unsigned short *)dst, K, pitch, total);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
 int launch_im2col(int dtype, const void *im, void *col, const MapGeom &g, hipStream_t s) {
     if (g.B == 0) return 0;
     const size_t es = dtype_bytes(dtype);
+    if (g.pitch) {  // padded rows: fp32 and half only (the callers' choice)
+        // the pitch is a multiple of 16 bytes and col is 16-byte aligned (the operator's own scratch)
+        const long total = (long)g.B * g.OH * g.OW * (g.pitch / (int)(16 / es));
+        if (es == 4)
+            hipLaunchKernelGGL((im2col_padded_kernel<unsigned, 4>), dim3(grid_for(total, 256)), dim3(256), 0, s, (const unsigned *)im, (unsigned *)col, g, total);
+        else
+            hipLaunchKernelGGL((im2col_padded_kernel<unsigned short, 8>), dim3(grid_for(total, 256)), dim3(256), 0, s, (const unsigned short *)im, (unsigned short *)col, g, total);
+        D8_LAUNCH_CHECK();
+        return 0;
+    }
     const long elems = (long)g.B * g.OH * g.OW * g.FH * g.FW * g.C;
     const size_t row_bytes = (size_t)g.C * es;
     if (row_bytes % 16 == 0 && aligned16(im) && aligned16(col)) {
@@ -238,14 +320,14 @@ int launch_col2im(int dtype, const void *col, void *im, const MapGeom &g, bool a
     const long elems = (long)g.B * g.IH * g.IW * g.C;
     const bool al = aligned16(im) && aligned16(col);
     if (dtype == D8_FLOAT64) {
-        if (accumulate) launch_col2im_t<double, 2, true>(col, im, g, g.C % 2 == 0 && al, elems, s);
-        else launch_col2im_t<double, 2, false>(col, im, g, g.C % 2 == 0 && al, elems, s);
+        if (accumulate) launch_col2im_t<double, 2, true>(col, im, g, g.C % 2 == 0 && al && !g.pitch, elems, s);
+        else launch_col2im_t<double, 2, false>(col, im, g, g.C % 2 == 0 && al && !g.pitch, elems, s);
     } else if (dtype == D8_FLOAT32) {
-        if (accumulate) launch_col2im_t<float, 4, true>(col, im, g, g.C % 4 == 0 && al, elems, s);
-        else launch_col2im_t<float, 4, false>(col, im, g, g.C % 4 == 0 && al, elems, s);
+        if (accumulate) launch_col2im_t<float, 4, true>(col, im, g, g.C % 4 == 0 && al && !g.pitch, elems, s);
+        else launch_col2im_t<float, 4, false>(col, im, g, g.C % 4 == 0 && al && !g.pitch, elems, s);
     } else {
-        if (accumulate) launch_col2im_t<f16, 8, true>(col, im, g, g.C % 8 == 0 && al, elems, s);
-        else launch_col2im_t<f16, 8, false>(col, im, g, g.C % 8 == 0 && al, elems, s);
+        if (accumulate) launch_col2im_t<f16, 8, true>(col, im, g, g.C % 8 == 0 && al && !g.pitch, elems, s);
+        else launch_col2im_t<f16, 8, false>(col, im, g, g.C % 8 == 0 && al && !g.pitch, elems, s);
     }
     D8_LAUNCH_CHECK();
     return 0;

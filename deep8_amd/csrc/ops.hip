@@ -269,6 +269,31 @@ static Gemm conv_plan(int which, int M, int K, int OC, const void *col, const vo
     return {1, 0, OC, K, M, zz, OC, 0, col, K, 0, 1.f, (void *)w, K, 0, 1};                   // dW += dz^T xcol
 }
 
+// A patch row of K = FH * FW * IC elements that cannot be moved in 16-byte pieces (1- and 3-channel images) keeps
+// all three products off the tiled kernels.  Such a layer runs on a patch matrix whose rows are padded with zeros
+// to the next multiple of 16 bytes, against a copy of the filter in the same pitch: the products then have
+// K (forward) or N (gradients) = the pitch, and the padding contributes exact zeros.  Returns that pitch, or 0
+// where the plain route applies (K already fits, OC would not, Float64, or a patch row so short -- below 64
+// elements -- that the products stay small either way and the extra copies cost more than they save).
+static int conv_padded_pitch(int dtype, int K, int OC) {
+    if (dtype == D8_FLOAT64) return 0;
+    const int epv = 16 / (int)dtype_bytes(dtype);
+    if (K % epv == 0 || OC % epv != 0 || K < 64) return 0;
+    return (K + epv - 1) / epv * epv;
+}
+
+// scratch of the padded route: patch matrix [M][pitch] | filter or filter gradient [OC][pitch] | GEMM workspace
+struct PaddedScratch {
+    size_t col, filt, total;
+};
+static PaddedScratch conv_padded_scratch(int dtype, int which, int M, int OC, int pitch) {
+    PaddedScratch s;
+    s.col = align256((size_t)M * pitch * dtype_bytes(dtype));
+    s.filt = align256((size_t)OC * pitch * dtype_bytes(dtype));
+    s.total = s.col + s.filt + gemm_ws(dtype, conv_plan(which, M, pitch, OC, nullptr, nullptr, nullptr));
+    return s;
+}
+
 size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                int OC, int FH, int FW, int covered, int sy, int sx, int dy, int dx) {
     int g[4];
@@ -282,7 +307,12 @@ size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int 
         return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
     if (which == 1 && conv_classes_grad_x(dtype, cs, nullptr, nullptr, nullptr, ga)) return 0;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
-    return col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
+    const size_t plain = col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
+    if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
+        const size_t padded = conv_padded_scratch(dtype, which, M, OC, pitch).total;
+        return padded > plain ? padded : plain;
+    }
+    return plain;
 }
 
 int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
@@ -304,6 +334,17 @@ int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
     }
     D8_REQUIRE(scratch, "d8_conv2d: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d: scratch too small");
+    if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
+        const PaddedScratch ps = conv_padded_scratch(dtype, 0, M, OC, pitch);
+        if (scratch_bytes >= ps.total && ((size_t)scratch & 15) == 0) {  // a smaller scratch still serves the plain route
+            char *colp = (char *)scratch, *wp = colp + ps.col, *ws = wp + ps.filt;
+            const MapGeom mg = {B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], pitch};
+            if (int rc = launch_im2col(dtype, x, colp, mg, as_stream(stream))) return rc;
+            if (int rc = launch_pad_rows(dtype, w, wp, OC, K, pitch, as_stream(stream))) return rc;
+            Gemm plan = conv_plan(0, M, pitch, OC, colp, wp, z);  // z = xcol W^T over K = pitch
+            return run(dtype, plan, ws, scratch_bytes - ps.col - ps.filt, stream);
+        }
+    }
     if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
         return rc;
     const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
@@ -335,6 +376,19 @@ static int d8_conv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int
     }
     D8_REQUIRE(scratch, "d8_conv2d_grad_x: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_x: scratch too small");
+    if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
+        const PaddedScratch ps = conv_padded_scratch(dtype, 1, M, OC, pitch);
+        if (scratch_bytes >= ps.total && ((size_t)scratch & 15) == 0) {
+            char *colp = (char *)scratch, *wp = colp + ps.col, *ws = wp + ps.filt;
+            if (int rc = launch_pad_rows(dtype, w, wp, OC, K, pitch, as_stream(stream))) return rc;
+            Gemm plan = conv_plan(1, M, pitch, OC, colp, wp, gz);  // dxcol [M][pitch] = dz W, the padding columns come out 0
+            if (int rc = run(dtype, plan, ws, scratch_bytes - ps.col - ps.filt, stream)) return rc;
+            if (beta == 0.f)  // col2im adds into its destination
+                if (int rc = d8_fill(dtype, gx, (size_t)B * IH * IW * IC, 0.f, stream)) return rc;
+            const MapGeom mg = {B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], pitch};
+            return launch_col2im(dtype, colp, gx, mg, true, as_stream(stream));
+        }
+    }
     const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
     if (int rc = run(dtype, conv_plan(1, M, K, OC, scratch, w, gz), ws ? (char *)scratch + col : nullptr, ws, stream))
         return rc;
@@ -364,6 +418,18 @@ static int d8_conv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int IW
     }
     D8_REQUIRE(scratch, "d8_conv2d_grad_y: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_y: scratch too small");
+    if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
+        const PaddedScratch ps = conv_padded_scratch(dtype, 2, M, OC, pitch);
+        if (scratch_bytes >= ps.total && ((size_t)scratch & 15) == 0) {
+            char *colp = (char *)scratch, *gwp = colp + ps.col, *ws = gwp + ps.filt;
+            const MapGeom mg = {B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], pitch};
+            if (int rc = launch_im2col(dtype, x, colp, mg, as_stream(stream))) return rc;
+            Gemm plan = conv_plan(2, M, pitch, OC, colp, gwp, gz);  // [OC][pitch] = dz^T xcol
+            plan.beta = 0.f;
+            if (int rc = run(dtype, plan, ws, scratch_bytes - ps.col - ps.filt, stream)) return rc;
+            return launch_unpad_add(dtype, gwp, gw, OC, K, pitch, beta, as_stream(stream));  // gw (+)= its first K columns
+        }
+    }
     if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
         return rc;
     const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;

@@ -451,3 +451,44 @@ def test_conv2d_strided_gradient_of_x(oracle_port, monkeypatch, cfg, classes, dt
     assert rel_fro(f(ops.conv2d_grad_x(x, w, gz, *a)), want) <= tol
     monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
     assert rel_fro(f(ops.conv2d_grad_x(x, w, gz, *a)), want) <= tol
+
+
+# first layers: a patch row of 25, 27, 54, 147 ... elements cannot be moved in 16-byte pieces; with an output channel
+# count that can, the operator pads the patch matrix's rows (and a copy of the filter) to the next multiple
+FIRST_LAYERS = [(2, 12, 12, 3, 8, 3, 3, True, 1, 1, 1, 1), (2, 16, 16, 1, 16, 5, 5, True, 1, 1, 1, 1),
+                (1, 20, 20, 3, 64, 7, 7, True, 2, 2, 1, 1), (1, 12, 12, 3, 8, 3, 3, False, 1, 1, 2, 2),
+                (2, 9, 11, 6, 24, 3, 3, True, 2, 1, 1, 1), (3, 28, 28, 1, 32, 5, 5, False, 1, 1, 1, 1),
+                (16, 32, 32, 3, 32, 3, 3, True, 1, 1, 1, 1), (2, 10, 10, 3, 8, 5, 5, True, 1, 1, 1, 1),
+                (1, 14, 14, 3, 16, 6, 6, True, 1, 1, 1, 1), (2, 13, 9, 5, 40, 4, 4, False, 1, 2, 1, 1)]
+
+
+@pytest.mark.parametrize("cfg", FIRST_LAYERS)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_conv2d_first_layers_padded_patch_rows(oracle_port, cfg, dtype):
+    from deep8_amd import ops
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    a = (cov, sy, sx, dy, dx)
+    r = rng(B + IH + OC + 31)
+    half = dtype == np.float16
+    c = h if half else (lambda t: t)
+    hi = 2 if half else 20
+    thin = (lambda t, p: t * (r.random(t.shape) < p)) if half else (lambda t, p: t)
+    x, w = thin(ints(r, (B, IH, IW, IC), hi), 0.5), thin(ints(r, (OC, FH, FW, IC), hi), 0.5)
+    want = oracle_port.conv2d(x, w, *a)
+    gz = thin(ints(r, want.shape, hi), 0.1 if half else 1.0)
+    gx0, gw0 = ints(r, x.shape, hi), ints(r, w.shape, hi)
+    wants = [want, oracle_port.conv2d_grad_x(x, w, gz, *a, gx0), oracle_port.conv2d_grad_y(x, w, gz, *a, gw0),
+             oracle_port.conv2d_grad_x(x, w, gz, *a), oracle_port.conv2d_grad_y(x, w, gz, *a)]
+    assert not half or max(np.abs(t).max() for t in wants) < 2048
+    nan = lambda t: np.full(t.shape, np.nan, dtype)
+    gots = [ops.conv2d(c(x), c(w), *a), ops.conv2d_grad_x(c(x), c(w), c(gz), *a, c(gx0)), ops.conv2d_grad_y(c(x), c(w), c(gz), *a, c(gw0)),
+            ops.conv2d_grad_x(c(x), c(w), c(gz), *a, nan(x), overwrite=True), ops.conv2d_grad_y(c(x), c(w), c(gz), *a, nan(w), overwrite=True)]
+    for k, (g, t) in enumerate(zip(gots, wants)):
+        assert np.array_equal(f(g), t), (cfg, k)
+    # reals within the tolerance
+    xr, wr = c(nrm(r, x.shape)), c(nrm(r, w.shape, np.sqrt(2.0 / (FH * FW * IC))))
+    gzr = c(nrm(r, want.shape))
+    tol = FP16_TOL if half else FP32_TOL
+    assert rel_fro(f(ops.conv2d(xr, wr, *a)), oracle_port.conv2d(f(xr), f(wr), *a)) <= tol
+    assert rel_fro(f(ops.conv2d_grad_x(xr, wr, gzr, *a)), oracle_port.conv2d_grad_x(f(xr), f(wr), f(gzr), *a)) <= tol
+    assert rel_fro(f(ops.conv2d_grad_y(xr, wr, gzr, *a)), oracle_port.conv2d_grad_y(f(xr), f(wr), f(gzr), *a)) <= tol
