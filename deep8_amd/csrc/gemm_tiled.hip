@@ -398,7 +398,8 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
         (void *)((const E *)g.B + (long)b * g.sB), 0,
         VIRT == VIRT_B_KROWS ? (int)pg.bytes
-                             : (int)(ES * ((VIRT == VIRT_A_CLASSES ? 0 : (g.red - 1) * g.sB) + b_rows * g.ldb)), 0x00020000);
+                             // (the taps of a filter interleave inside its rows: the filter ends with its last row)
+                             : (int)(ES * ((VA ? 0 : (g.red - 1) * g.sB) + b_rows * g.ldb)), 0x00020000);
     const unsigned Au = (unsigned)ES * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0);
     const unsigned Bu = (unsigned)ES * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
     const int a_r = A_KC ? tid >> 3 : tid / (BM / EPV), a_c = A_KC ? tid & 7 : tid % (BM / EPV);
@@ -625,7 +626,8 @@ static bool eligible(const GemmArgs &g, int transA, int transB) {
     // one side may be shorter than any tile (a few rows against a wide matrix: the 64 x 128 / 128 x 64 tile
     // then reaches past it) when the other side fills a tile
     if ((g.M < 128 && g.N < 128) || g.K < 1) return false;  // (a K below one K step is a lone partial step)
-    if ((g.M < 64 || g.N < 64) && g.virt != VIRT_NONE) return false;
+    // (patch rows as A: a filter with few output channels is fine, its rows past the last read as zeros)
+    if (g.virt != VIRT_NONE && (g.M < 64 || (g.N < 64 && g.virt == VIRT_B_KROWS))) return false;
     // a last K step that is partly past K: real matrices only, and a 16-byte piece of an operand stored along K
     // must lie wholly on one side of K
     if (g.K % BK && (g.virt != VIRT_NONE || ((!transA || transB) && g.K % EPV))) return false;

@@ -26,6 +26,8 @@ CONV = [
 ]
 # (B, IH, IW, IC, OC, FH, FW, covered, sy, sx)
 DECONV = [
+    (2, 8, 8, 64, 3, 4, 4, False, 2, 2),    # few output channels (an RGB output)
+    (2, 10, 10, 128, 1, 3, 3, True, 1, 1),
     (2, 8, 8, 16, 8, 4, 4, False, 3, 3),    # DeConv2dTest forwardCPU geometry (smaller)
     (2, 8, 8, 16, 8, 4, 4, True, 3, 3),     # backwardCPU geometry
     (2, 7, 7, 8, 16, 4, 4, False, 2, 2),    # benchmark configuration 5 family -> 2*7+2
@@ -254,7 +256,7 @@ def test_config5_literal_56x56_through_explicit_pads(oracle_port):
 IMPLICIT = [
     ((2, 16, 16, 64, 64, 3, 3, True, 1, 1, 1, 1), (0, 1, 2), (0, 1, 2)),
     ((2, 16, 16, 64, 128, 3, 3, False, 1, 1, 1, 1), (0, 1), (0, 1)),       # 392 patch rows: ragged tiles, explicit dW
-    ((4, 16, 16, 32, 64, 3, 3, True, 2, 2, 1, 1), (0, 2), (2,)),           # stride 2: dX stays explicit
+    ((4, 16, 16, 32, 64, 3, 3, True, 2, 2, 1, 1), (0, 1, 2), (1, 2)),      # stride 2: dX by residue classes of input pixels (32 channels wide)
     ((2, 20, 12, 64, 96, 5, 3, True, 1, 1, 2, 2), (0, 1, 2), (0,)),       # dilation, 5x3 filter, non-square image
     ((8, 8, 8, 64, 192, 2, 2, False, 1, 1, 1, 1), (0, 1), (0, 1)),
     ((1, 16, 16, 128, 64, 3, 3, True, 1, 1, 1, 1), (0, 1, 2), (0, 1, 2)),
@@ -462,7 +464,14 @@ FIRST_LAYERS = [(2, 12, 12, 3, 8, 3, 3, True, 1, 1, 1, 1), (2, 16, 16, 1, 16, 5,
                 (1, 14, 14, 3, 16, 6, 6, True, 1, 1, 1, 1), (2, 13, 9, 5, 40, 4, 4, False, 1, 2, 1, 1)]
 
 
-@pytest.mark.parametrize("cfg", FIRST_LAYERS)
+# last layers: few output channels (an RGB or a one-channel output); the forward pass still reads its patch rows
+# straight from the image, the filter's rows past the last one arriving as zeros
+LAST_LAYERS = [(2, 16, 16, 64, 3, 3, 3, True, 1, 1, 1, 1), (2, 12, 12, 32, 1, 1, 1, True, 1, 1, 1, 1),
+               (1, 16, 16, 64, 5, 3, 3, False, 1, 1, 1, 1), (2, 14, 14, 128, 3, 5, 5, True, 1, 1, 1, 1),
+               (4, 20, 20, 64, 16, 3, 3, True, 2, 2, 1, 1), (2, 16, 16, 16, 64, 3, 3, True, 1, 1, 1, 1)]
+
+
+@pytest.mark.parametrize("cfg", FIRST_LAYERS + LAST_LAYERS)
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_conv2d_first_layers_padded_patch_rows(oracle_port, cfg, dtype):
     from deep8_amd import ops
