@@ -314,7 +314,9 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
         }
 }
 
-template <typename T>
+// TAIL: K is not a multiple of the K step (an instantiation of its own, so that the per-piece offsets of the
+// ordinary case stay constants)
+template <typename T, bool TAIL = false>
 __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tilesM, int tilesN) {
     typedef typename T::E E;
     typedef typename T::EL EL;
@@ -477,7 +479,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         } else {
             const int kx = x - r * ktiles;
             if constexpr (VIRT == VIRT_NONE) {
-                if (tail_len) {
+                if constexpr (TAIL) {
                     const bool tail = kx == ktiles - 1;
 #pragma unroll
                     for (int p = 0; p < A_IT; ++p) {
@@ -511,7 +513,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         } else {
             const int kx = x - r * ktiles;
             if constexpr (VIRT == VIRT_NONE) {
-                if (tail_len) {
+                if constexpr (TAIL) {
                     const bool tail = kx == ktiles - 1;
 #pragma unroll
                     for (int p = 0; p < B_IT; ++p) {
@@ -585,7 +587,10 @@ static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
     const int layers = VIRT == VIRT_A_CLASSES ? g.ncls : g.batch * g.splits;  // for classes g.M is the largest one's
     const long wgs = (long)tilesM * tilesN * layers, cus = cu_count();
     const unsigned pad = (lds <= third && wgs > cus && wgs <= 2 * cus) ? (unsigned)(third + 512 - lds) : 0u;
-    hipLaunchKernelGGL((gemm_tiled_kernel<T>), dim3(tilesM * tilesN, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
+    if (VIRT == VIRT_NONE && g.K % T::BK)
+        hipLaunchKernelGGL((gemm_tiled_kernel<T, VIRT == VIRT_NONE>), dim3(tilesM * tilesN, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
+    else
+        hipLaunchKernelGGL((gemm_tiled_kernel<T, false>), dim3(tilesM * tilesN, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
     D8_LAUNCH_CHECK();
     return 0;
 }
