@@ -33,6 +33,11 @@
 // gradients, DeConv2d's gradient of x and of the filter, and -- one residue class of output
 // pixels per grid layer (OutClass) -- DeConv2d forward and Conv2d's gradient of x for strides
 // above 1, whose rows of C are then pixels of the output image rather than consecutive rows.
+//
+// The same device covers ragged reductions and skinny matrices of real operands: in a last K step that is
+// partly past K the pieces beyond K are fetched at an offset outside the buffer (zeros), and a matrix with
+// fewer rows or columns than the tile is covered by a tile that starts at 0 and reaches past it -- what
+// its loads bring in from there only enters results that are not stored.
 #include "gemm_args.h"
 
 namespace d8 {
