@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libdeep8_hip.so")
 FLOAT16 = 10
 FLOAT32 = 11
 FLOAT64 = 12
+STATIC_SCRATCH_BYTES = 32 << 20  # D8_STATIC_SCRATCH_BYTES of include/deep8_hip.h
 
 c_int, c_long, c_size_t, c_float, c_void_p = (ctypes.c_int, ctypes.c_long, ctypes.c_size_t, ctypes.c_float,
                                               ctypes.c_void_p)
@@ -57,6 +58,7 @@ SIGNATURES = {
     "d8_matmul": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_x": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_y": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "d8_matmul_grad_y_static": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P]),
     "d8_matmul_grad_x_overwrite": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_y_overwrite": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_conv2d_geometry": (_I, [_I] * 9 + [ctypes.POINTER(_I)]),

@@ -48,6 +48,10 @@ inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
 // Number of compute units of the current device (cached).
 int cu_count();
 
+// Looks up, once per device, where the current device keeps its copy of the static scratch array
+// (static_scratch.hip).  Called by d8_device_init and, failing that, by the first call that needs it.
+int static_scratch_setup();
+
 }  // namespace d8
 
 #endif

@@ -58,7 +58,7 @@ int d8_device_init(int device_id) {
     D8_HIP(hipGetDeviceProperties(&prop, device_id));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(D8_ERR_ARCH, "device %d is %s; this library holds gfx950 code only", device_id, prop.gcnArchName);
-    return 0;
+    return static_scratch_setup();  // this device's address of the static scratch array
 }
 
 int d8_device_info(int *cus, int *clock_khz, size_t *hbm_bytes, char *name, int name_len) {

@@ -158,6 +158,18 @@ int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc,
                                void *dy, int yb, int yr, int yc, const void *dz,
                                void *scratch, size_t scratch_bytes, void *stream);
 
+/* d8_matmul_grad_y for callers that cannot allocate and have no scratch to pass.  No counterpart in the
+ * reference: it is for code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc.  Same arguments, checks and result (bit for bit) as d8_matmul_grad_y given a scratch of
+ * d8_matmul_scratch_bytes(dtype, 2, ...) bytes, but the split reduction's partial sums go to a device
+ * array of D8_STATIC_SCRATCH_BYTES that lives in the library (each GPU the library runs on holds one
+ * until the process ends).  A shape that would need more is refused with D8_ERR_ARGUMENT.  The call
+ * allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that overlap in time
+ * on one GPU (different streams or host threads) race.                                                  */
+#define D8_STATIC_SCRATCH_BYTES (32u << 20)
+int d8_matmul_grad_y_static(int dtype, const void *x, int xb, int xr, int xc,
+                            void *dy, int yb, int yr, int yc, const void *dz, void *stream);
+
 /* out[0..3] = OH, OW, padTop, padLeft (deep8/src/math/Conv2d.cpp:20-32, Conv2d.cu:332-336;
  * deep8/src/math/DeConv2d.cpp:23-29, DeConv2d.cu:99-100) */
 int d8_conv2d_geometry(int IH, int IW, int FH, int FW, int covered,
