@@ -35,22 +35,61 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}   # dense MFMA TFLOP/s, MI355X
 HBM_PEAK = 8000.0                      # GB/s
-# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of this file (each counter scaled by what it reads for a plain copy of known size; the
-# summaries are kept under profiles/).  None where no counter run has been made.
 # --eager-zero: fill both gradients and accumulate into them (the reference executor's literal sequence)
 EAGER_ZERO = False
 
-MEASURED_TRAFFIC = {
-    "c3": int((192.2 + 192.2 + 192.3) / 3 * 2**20 + 32.0 * 2**20),  # fetch (NN, NT, TN average) + write, bytes
-    "c4": int((2 * 13.9 + 2 * 13.0 + 2.0 + 0.5) * 2**20),            # Conv2d forward: tile launches (rows cut in two) fetch + write, + the band's split reduction
-    "c5": int((17.4 + 6.6) * 2**20),                                 # DeConv2d forward (one launch over the output classes): fetch + write
-    "d3": int((288.1 + 32.0) * 2**20),                               # fp64 128 x 128 tiles: fetch + write
-    # element-wise and pooling steps: per kernel of the step (fetch + write)
-    "e4": {"add (bias broadcast)": int((24.5 + 24.5) * 2**20), "relu": int((24.5 + 24.5) * 2**20),
-           "relu_grad": int((49.0 + 24.5) * 2**20), "bias_grad (sum over rows)": int((24.5 + 0.3 + 0.1) * 2**20)},
-    "p4": {"maxpool2d": int((24.6 + 6.1) * 2**20), "maxpool2d_grad": int((30.7 + 24.5) * 2**20)},
+# HBM-side bytes per launch of the dominant kernel: read from the "HBM-side traffic per dispatch" table of the
+# rocprofv3 summary kept under profiles/ for the workload (FETCH_SIZE / WRITE_SIZE runs of this file, each counter
+# scaled by what it reads for a plain copy of known size).  workload -> (summary, rows of the table that make
+# up one launch of the roofline kernel: substrings of the kernel column, each with the number of dispatches
+# of that row per launch; a list of alternatives is averaged).  None where the summary or a row is missing.
+TRAFFIC_ROWS = {
+    "c3": ("gemm_wide_f16_matmul_4096_half.txt", [("gemm_wide_kernel", 1.0 / 3)]),           # NN, NT, TN averaged
+    "c4": ("conv2d_fp32_b32_56x56x64_3x3.txt", [("NT, A = patch rows", 2), ("gemm_split_reduce", 1)]),  # forward: rows cut in two + the band's reduction
+    "c5": ("deconv2d_half_b16_28x28x128_4x4s2.txt", [("one class of output pixels", 1)]),    # forward: one launch over the classes
+    "d3": ("gemm_f64_matmul_2048_double.txt", [("gemm_f64_kernel", 1.0 / 3)]),
+    "e4": ("elementwise_bias_relu_b32_56x56x64.txt", {"add (bias broadcast)": [("add_kernel", 1)], "relu": [("relu_kernel", 1)],
+                                                       "relu_grad": [("relu_grad_kernel", 1)],
+                                                       "bias_grad (sum over rows)": [("column_sum_kernel", 1), ("column_sum_finish", 1)]}),
+    "p4": ("maxpool2d_b32_56x56x64.txt", {"maxpool2d": [("pool_forward_kernel", 1)], "maxpool2d_grad": [("pool_backward", 1)]}),
+    "i4": ("im2col_col2im_fp32_b32_56x56x64_3x3.txt", {"im2col": [("im2col_kernel", 1)], "col2im": [("col2im_kernel", 1)]}),
 }
+
+
+def profile_traffic(key, part=None):
+    """{"bytes": fetch + write bytes per launch, "source": file} from the committed summary, or None"""
+    ent = TRAFFIC_ROWS.get(key)
+    if ent is None:
+        return None
+    fname, rows = ent
+    if isinstance(rows, dict):
+        rows = rows.get(part)
+        if rows is None:
+            return None
+    path = os.path.join(ROOT, "profiles", fname)
+    if not os.path.exists(path):
+        return None
+    table, seen = [], False
+    for line in open(path):
+        if line.startswith("HBM-side traffic per dispatch"):
+            seen = True
+            continue
+        if seen:
+            f = line.split(None, 4)
+            if len(f) == 5 and f[0].replace(".", "").isdigit():
+                table.append((float(f[1]), float(f[3]), f[4].strip()))  # fetch MiB, write MiB, kernel
+    total = 0.0
+    for sub, count in rows:
+        hit = [t for t in table if sub in t[2]]
+        if not hit:
+            return None
+        total += count * sum(t[0] + t[1] for t in hit) * 2**20
+    return {"bytes": int(total), "source": "profiles/" + fname}
+
+
+def _traffic_fields(key, part=None):
+    t = profile_traffic(key, part)
+    return {"traffic": t["bytes"] if t else None, "traffic_source": t["source"] if t else None}
 
 
 def _dev(a):
@@ -86,18 +125,26 @@ def _settle(fn):
         capi.sync()
 
 
-def _time_steps(fn, steps, warmup):
-    """wall-clock ms per step over exactly `steps` calls, device idle on both sides"""
+REPS = 5   # --reps: the timed region (exactly --steps steps) is repeated this often; the median is reported
+
+
+def _time_steps(fn, steps, warmup, reps=None):
+    """wall-clock ms per step over exactly `steps` calls, device idle on both sides; the region is timed
+    `reps` times back to back (the device stays under load in between) and the median is returned together
+    with every sample"""
     from deep8_amd import capi
     _settle(fn)
-    for _ in range(warmup):
-        fn()
-    capi.sync()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    capi.sync()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    samples = []
+    for _ in range(reps or REPS):
+        for _ in range(warmup):
+            fn()
+        capi.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        capi.sync()
+        samples.append((time.perf_counter() - t0) * 1e3 / steps)
+    return float(np.median(samples)), samples
 
 
 def _time_events(fn, reps):
@@ -174,25 +221,35 @@ class MatMulWorkload:
                                                   self.ws.ptr, self.ws_bytes, self.stream))
 
     def step(self):
-        """One forward + backward of a MatrixMultiply node as the executor issues it: forward, then the
+        """One forward + backward of a MatrixMultiply node as this build's executor issues it: forward, then the
         two gradient products.  The executor's zeroGradient() before a backward pass is deferred
         (Device::zeroLater), so the first product into each gradient is the overwrite form: same
         result as fill + accumulate, without the fill and without reading the zeros back."""
-        self.fwd()
         if EAGER_ZERO:
-            self.dx.zero_()
-            self.dy.zero_()
-            self.grad_x()
-            self.grad_y()
-        else:
-            self.grad_x_first()
-            self.grad_y_first()
+            return self.step_eager_zero()
+        self.fwd()
+        self.grad_x_first()
+        self.grad_y_first()
+
+    def step_eager_zero(self):
+        """The reference executor's literal sequence (deep8/src/model/EagerExecutor.cpp:51-65, then
+        MatrixMultiply.cu:203 with beta = 1): forward, fill both gradients with zeros, accumulate into them."""
+        self.fwd()
+        self.dx.zero_()
+        self.dy.zero_()
+        self.grad_x()
+        self.grad_y()
 
     def parts(self):
         f = self.flops / 3
         if EAGER_ZERO:
             return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
         return {"fwd": (self.fwd, f), "grad_x": (self.grad_x_first, f), "grad_y": (self.grad_y_first, f)}
+
+    def parts_accumulate(self):
+        """the two gradient launches in their beta = 1 form (read the destination, add, write)"""
+        f = self.flops / 3
+        return {"grad_x_accumulate": (self.grad_x, f), "grad_y_accumulate": (self.grad_y, f)}
 
 
 def mfma_stream_ceiling(wl, dtype_name):
@@ -219,9 +276,14 @@ def mfma_stream_ceiling(wl, dtype_name):
 class ConvWorkload:
     """Conv2d or DeConv2d forward + GradX + GradY through d8_conv2d* / d8_deconv2d*."""
 
-    def __init__(self, name, dtype, deconv, B, IH, IW, IC, OC, FH, FW, covered, sy, sx, seed):
+    def __init__(self, name, dtype, deconv, B, IH, IW, IC, OC, FH, FW, covered, sy, sx, seed, explicit=False):
         from deep8_amd import capi, ops
         self.name, self.dtype, self.deconv = name, np.dtype(dtype), deconv
+        # explicit: the reference's own lowering (im2col -> GEMM, GEMM -> col2im through the interim matrix);
+        # the library reads D8_CONV_EXPLICIT at every call
+        self.explicit = explicit
+        if explicit:
+            os.environ["D8_CONV_EXPLICIT"] = "1"
         self.key = name.split(":")[0]
         self.lib = capi.init()
         self.dt = capi.dtype_id(self.dtype)
@@ -242,7 +304,8 @@ class ConvWorkload:
         self.gw = capi.DeviceArray((OC, FH, FW, IC), dtype)
         q = self.lib.d8_deconv2d_scratch_bytes if deconv else self.lib.d8_conv2d_scratch_bytes
         self.ws_bytes = max(q(self.dt, w, B, IH, IW, IC, OC, FH, FW, *self.geo) for w in range(3))
-        self.ws = capi.DeviceArray((self.ws_bytes,), np.uint8)
+        self.ws = capi.DeviceArray((max(self.ws_bytes, 16),), np.uint8)
+        os.environ.pop("D8_CONV_EXPLICIT", None)
         if deconv:
             self.flops = 3 * 2.0 * (B * IH * IW) * IC * (OC * FH * FW)
             mat = B * IH * IW * OC * FH * FW
@@ -260,7 +323,13 @@ class ConvWorkload:
         from deep8_amd.capi import check
         B, IH, IW, IC = self.xd
         OC, FH, FW, _ = self.wd
-        check(fn(self.dt, a, B, IH, IW, IC, b, OC, FH, FW, c, *self.geo, self.ws.ptr, self.ws_bytes, None))
+        if self.explicit:
+            os.environ["D8_CONV_EXPLICIT"] = "1"
+        try:
+            check(fn(self.dt, a, B, IH, IW, IC, b, OC, FH, FW, c, *self.geo, self.ws.ptr, self.ws_bytes, None))
+        finally:
+            if self.explicit:
+                os.environ.pop("D8_CONV_EXPLICIT", None)
 
     def fwd(self):
         self._call(self.lib.d8_deconv2d if self.deconv else self.lib.d8_conv2d, self.x.ptr, self.w.ptr, self.z.ptr)
@@ -320,7 +389,7 @@ class ConvWorkload:
         ms = _time_events(fn, reps)
         ach = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "kernel": name, "achieved": round(ach, 2), "peak": PEAK[dtype], "unit": "TFLOP/s",
-                "frac": round(ach / PEAK[dtype], 4), "launch_us": round(ms * 1e3, 2), "traffic": MEASURED_TRAFFIC.get(self.key)}
+                "frac": round(ach / PEAK[dtype], 4), "launch_us": round(ms * 1e3, 2), **_traffic_fields(self.key)}
 
 
 class DeconvLiteralWorkload:
@@ -381,6 +450,45 @@ class DeconvLiteralWorkload:
         self.fwd()
         self.grad_x()
         self.grad_y()
+
+
+class GatherMapsWorkload:
+    """d8_im2col and d8_col2im alone at config 4's size (fp32 B32 56x56x64, 3x3, stride 1, pad 1): the
+    gather / scatter kernels of the reference's Conv2d lowering (deep8/src/math/Conv2d.cu:10-61, 64-118).
+    HBM-bound: im2col reads the image and writes the patch matrix once; col2im reads the patch matrix once and
+    read-modify-writes the image gradient."""
+
+    def __init__(self, name, dtype, B, H, W, C, F, seed):
+        from deep8_amd import capi
+        self.name, self.dtype, self.key = name, np.dtype(dtype), name.split(":")[0]
+        self.lib = capi.init()
+        self.dt = capi.dtype_id(self.dtype)
+        r = np.random.default_rng(seed)
+        self.B = B
+        self.geo = (B, H, W, C, H, W, F, F, 1, 1, 1, 1, F // 2, F // 2)
+        self.x = _dev(r.standard_normal((B, H, W, C)).astype(np.float32).astype(dtype))
+        self.col = capi.DeviceArray((B * H * W, F * F * C), dtype)
+        self.gx = capi.DeviceArray((B, H, W, C), dtype, zero=True)
+        es = self.dtype.itemsize
+        self.im_bytes, self.col_bytes = es * B * H * W * C, es * B * H * W * F * F * C
+        self.flops = float(B * H * W * F * F * C)  # the additions of col2im
+        self.bytes = (self.im_bytes + self.col_bytes) + (self.col_bytes + 2 * self.im_bytes)
+
+    def im2col(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_im2col(self.dt, self.x.ptr, self.col.ptr, *self.geo, None))
+
+    def col2im(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_col2im(self.dt, self.col.ptr, self.gx.ptr, *self.geo, None))
+
+    def step(self):
+        self.im2col()
+        self.col2im()
+
+    def parts(self):
+        """name -> (call, algorithmic bytes)"""
+        return {"im2col": (self.im2col, self.im_bytes + self.col_bytes), "col2im": (self.col2im, self.col_bytes + 2 * self.im_bytes)}
 
 
 class BiasReluWorkload:
@@ -521,6 +629,13 @@ def make_workload(key):
     if key == "c4":
         return ConvWorkload("c4: Conv2d fwd+dX+dW fp32 B32 56x56x64 3x3x64->64 s1 same", np.float32, False,
                             32, 56, 56, 64, 64, 3, 3, True, 1, 1, 5)
+    if key == "c4x":
+        return ConvWorkload("c4x: Conv2d fwd+dX+dW fp32 B32 56x56x64 3x3x64->64 s1 same, the reference's lowering "
+                            "(im2col -> GEMM, GEMM -> col2im, 231 MB interim matrix)", np.float32, False,
+                            32, 56, 56, 64, 64, 3, 3, True, 1, 1, 5, explicit=True)
+    if key == "i4":
+        return GatherMapsWorkload("i4: d8_im2col + d8_col2im alone at config 4's size, fp32 B32 56x56x64 3x3 s1 pad 1",
+                                  np.float32, 32, 56, 56, 64, 3, 11)
     if key == "c5":
         return ConvWorkload("c5: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 58x58x64 (Deep8 covered=false)",
                             np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
@@ -578,10 +693,24 @@ def cpu_baseline(key, seconds=12.0):
         return {"value": n * B / dt, "unit": "images/s", "cores": src.threads(), "kind": kind,
                 "sample": "%s fwd+bwd on %d images x %d repeats (fp32 CPU path, host-side array copies included), %.1f s"
                           % (key, B, n, dt)}
-    if key in ("c4", "c5"):
+    if key == "i4":
+        # the reference's CPU path never materialises the patch matrix (it is a lazy Eigen expression), so the
+        # two maps are timed on the C restatement of the reference's GPU kernels' index maps
+        port = oracle.port
+        B = 8
+        x = r.standard_normal((B, 56, 56, 64)).astype(np.float32)
+        gx = np.zeros_like(x)
+
+        def one():
+            col = port.im2col(x, 56, 56, 3, 3, 1, 1, 1, 1, 1, 1)
+            port.col2im(col, gx, 56, 56, 3, 3, 1, 1, 1, 1, 1, 1)
+        n, dt = _repeat_for(one, seconds)
+        return {"value": n * B / dt, "unit": "images/s", "cores": port.threads(), "kind": "port",
+                "sample": "im2col + col2im on %d images x %d repeats (fp32, C restatement), %.1f s" % (B, n, dt)}
+    if key in ("c4", "c4x", "c5"):
         # the reference runs Conv2d/DeConv2d on Eigen's thread pool: all host cores
         B = 8
-        if key == "c4":
+        if key in ("c4", "c4x"):
             x, w = r.standard_normal((B, 56, 56, 64)).astype(np.float32), r.standard_normal((64, 3, 3, 64)).astype(np.float32)
             args, f3 = (True, 1, 1, 1, 1), (src.conv2d, src.conv2d_grad_x, src.conv2d_grad_y)
         else:
@@ -718,7 +847,7 @@ def phase_record(launches=12):
 
 
 def main():
-    global ZERO_OPERANDS, EAGER_ZERO, SETTLE_MS
+    global ZERO_OPERANDS, EAGER_ZERO, SETTLE_MS, REPS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -732,6 +861,8 @@ def main():
     ap.add_argument("--eager-zero", action="store_true",
                     help="zero-fill the gradients and accumulate (the reference's literal "
                          "sequence) instead of the executor's deferred zeroing + overwrite")
+    ap.add_argument("--reps", type=int, default=REPS,
+                    help="repetitions of the timed region of --steps steps; ms_per_step is their median")
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                     help="untimed work issued before every measurement so that it runs at the sustained clock "
                          "(0: start from an idle device)")
@@ -741,6 +872,7 @@ def main():
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
     SETTLE_MS = a.settle_ms
+    REPS = max(1, a.reps)
     ZERO_OPERANDS = a.operands == "zeros"
     EAGER_ZERO = a.eager_zero
     if a.gpus != 1:
@@ -757,19 +889,25 @@ def main():
         return phase_record()
 
     wl = make_workload(a.workload)
-    ms = _time_steps(wl.step, a.steps, a.warmup)
+    ms, samples = _time_steps(wl.step, a.steps, a.warmup)
     dtype = {2: "f16", 4: "f32", 8: "f64"}[wl.dtype.itemsize]
     is_conv = isinstance(wl, ConvWorkload)
-    is_stream = isinstance(wl, (BiasReluWorkload, PoolWorkload))  # element-wise / pooling: HBM-bound kernels
+    is_mm = isinstance(wl, MatMulWorkload)
+    is_stream = isinstance(wl, (BiasReluWorkload, PoolWorkload, GatherMapsWorkload))  # HBM-bound kernels
     tflops = wl.flops / (ms * 1e-3) / 1e12
 
-    parts = {}
-    for pname, (fn, amount) in wl.parts().items():
-        pms = _time_events(fn, max(200, a.steps) if is_stream else max(5, a.steps))  # 10 us kernels: more launches per timing
-        if is_stream:
-            parts[pname] = {"ms": round(pms, 4), "algorithmic_GBps": round(amount / (pms * 1e-3) / 1e9, 1)}
-        else:
-            parts[pname] = {"ms": round(pms, 4), "tflops": round(amount / (pms * 1e-3) / 1e12, 2)}
+    def time_parts(table):
+        res = {}
+        for pname, (fn, amount) in table.items():
+            pms = _time_events(fn, max(200, a.steps) if is_stream else max(5, a.steps))  # 10 us kernels: more launches per timing
+            if is_stream:
+                res[pname] = {"ms": round(pms, 4), "algorithmic_GBps": round(amount / (pms * 1e-3) / 1e9, 1)}
+            else:
+                res[pname] = {"ms": round(pms, 4), "tflops": round(amount / (pms * 1e-3) / 1e12, 2)}
+        return res
+
+    parts = time_parts(wl.parts())
+    eager = None
     if is_conv:
         roof = wl.gemm_roofline(max(5, a.steps))
     elif is_stream:
@@ -779,7 +917,9 @@ def main():
         ach = parts[pname]["algorithmic_GBps"]
         roof = {"bound": "hbm", "kernel": pname, "achieved": ach, "peak": HBM_PEAK, "unit": "GB/s",
                 "frac": round(ach / HBM_PEAK, 4), "launch_us": round(parts[pname]["ms"] * 1e3, 2),
-                "traffic": MEASURED_TRAFFIC.get(a.workload, {}).get(pname)}
+                **_traffic_fields(a.workload, pname)}
+        for k, v in parts.items():  # every kernel of the step against the HBM peak
+            v["frac_of_hbm_peak"] = round(v["algorithmic_GBps"] / HBM_PEAK, 4)
     else:
         # each of fwd / dX / dY is ONE launch of the same tiled GEMM kernel (its NN, NT and TN
         # instances): flops per launch / average launch duration, HIP events on the launch stream
@@ -787,39 +927,66 @@ def main():
         ach = wl.flops / 3 / (avg_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "kernel": wl.kernel, "achieved": round(ach, 2), "peak": PEAK[dtype],
                 "unit": "TFLOP/s", "frac": round(ach / PEAK[dtype], 4), "launch_us": round(avg_ms * 1e3, 2),
-                "traffic": MEASURED_TRAFFIC.get(a.workload)}
+                **_traffic_fields(a.workload)}
         roof["mfma_stream_ceiling"] = mfma_stream_ceiling(wl, dtype)
+        if is_mm and not EAGER_ZERO:
+            # the reference executor's literal sequence beside the deferred-zeroing one `value` is quoted on:
+            # forward, fill both gradients, two beta = 1 products (same flops, same result)
+            ems, esamples = _time_steps(wl.step_eager_zero, a.steps, a.warmup)
+            acc = time_parts(wl.parts_accumulate())
+            parts.update(acc)
+            eavg = (parts["fwd"]["ms"] + sum(p["ms"] for p in acc.values())) / 3
+            et = wl.flops / (ems * 1e-3) / 1e12
+            eager = {"sequence": "forward, zero-fill dX and dY, dX += dZ.Y^T, dY += X^T.dZ (beta = 1): the reference "
+                                 "executor's literal calls",
+                     "ms_per_step": round(ems, 4), "ms_per_step_samples": [round(v, 4) for v in esamples],
+                     "tflops": round(et, 2), "pct_mfma_peak": round(100.0 * et / PEAK[dtype], 2),
+                     "frac": round(wl.flops / 3 / (eavg * 1e-3) / 1e12 / PEAK[dtype], 4), "launch_us": round(eavg * 1e3, 2)}
 
+    form = ""
+    if is_mm or is_conv:
+        form = ("; gradients: zero fill + accumulate (beta = 1), the reference executor's literal sequence" if EAGER_ZERO else
+                "; gradients: written by the overwrite form (beta = 0) that this build's executor issues while the zero fill "
+                "of a gradient is still deferred -- same flops, same result as fill + accumulate"
+                + (", which is reported beside it under eager_zero" if eager else ""))
     out = {
         "metric": "Conv2d fwd+bwd images/s" if is_conv else "%s fwd+bwd images/s" % wl.key if is_stream
         else "MatrixMultiply fwd+bwd TFLOP/s",
         "value": round(wl.B / (ms * 1e-3), 1) if is_conv or is_stream else round(tflops, 2),
         "unit": "images/s" if is_conv or is_stream else "TFLOP/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "settle_ms": SETTLE_MS, "ms_per_step": round(ms, 4),
+        "reps": len(samples), "ms_per_step_samples": [round(v, 4) for v in samples],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "ALL-ZERO OPERANDS (diagnostic run, not a benchmark value)" if ZERO_OPERANDS else
         "synthetic (seeded numpy generators, resident in HBM before timing)",
-        "config": {"workload": wl.name},
+        "config": {"workload": wl.name + form},
         "pct_mfma_peak": None if is_stream else round(100.0 * tflops / PEAK[dtype], 2),
         "tflops": round(tflops, 2),
         "algorithmic_GBps": round(wl.bytes / (ms * 1e-3) / 1e9, 1),
         "parts": parts,
         "roofline": roof,
     }
+    if eager:
+        out["eager_zero"] = eager
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c5", "c5l", "e4", "p4", "d3"):
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4x", "i4", "c5", "c5l", "e4", "p4", "d3"):
             if key == a.workload:
                 continue
             del wl
             wl = make_workload(key)
-            oms = _time_steps(wl.step, 20, 3)
+            oms, _ = _time_steps(wl.step, 20, 3, reps=3)
             o = {"ms_per_step": round(oms, 4), "tflops": round(wl.flops / (oms * 1e-3) / 1e12, 2),
                  "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
-            if isinstance(wl, (ConvWorkload, DeconvLiteralWorkload, BiasReluWorkload, PoolWorkload)):
+            if isinstance(wl, (ConvWorkload, DeconvLiteralWorkload, BiasReluWorkload, PoolWorkload, GatherMapsWorkload)):
                 o["images_per_s"] = round(wl.B / (oms * 1e-3), 1)
+            if isinstance(wl, GatherMapsWorkload):  # the two kernels alone, against the HBM peak
+                for pname, (fn, amount) in wl.parts().items():
+                    pms = _time_events(fn, 100)
+                    o[pname] = {"launch_us": round(pms * 1e3, 2), "algorithmic_GBps": round(amount / (pms * 1e-3) / 1e9, 1),
+                                "frac_of_hbm_peak": round(amount / (pms * 1e-3) / 1e9 / HBM_PEAK, 4), **_traffic_fields(key, pname)}
             if key == "c1":  # launch-latency bound: the same three launches replayed from a HIP graph
                 o["ms_per_step_graph_replay"] = round(graph_replay_ms(wl, 50, 5), 4)
             others[key] = o

@@ -51,6 +51,74 @@ __global__ __launch_bounds__(256) void im2col_kernel(const V *__restrict__ im, V
     }
 }
 
+// Division of a number below 2^31 by a runtime constant as a multiply-high, an add and a shift (the round-up
+// method: with s = ceil(log2 d) and m = floor(2^32 (2^s - d) / d) + 1, n / d = (mulhi(n, m) + n) >> s).
+struct FastDiv {
+    unsigned m;
+    int s;
+};
+static FastDiv fast_div(unsigned d) {
+    int s = 0;
+    while ((1ull << s) < d) ++s;
+    return FastDiv{(unsigned)((((1ull << s) - d) << 32) / d + 1), s};
+}
+__device__ __forceinline__ unsigned div_by(unsigned n, FastDiv d) { return (__umulhi(n, d.m) + n) >> d.s; }
+
+typedef unsigned u32x4v __attribute__((ext_vector_type(4)));
+
+// im2col in 16-byte pieces for the common case (channel rows that are multiples of 16 bytes, fewer than 2^31
+// patch rows).  A workgroup owns `rows_per_block` consecutive patch rows, i.e. one contiguous stretch of col,
+// and walks it 256 pieces at a time, four stretches per round: four image reads in flight per thread, then
+// four stores.  All index arithmetic is 32-bit, with the divisions by runtime constants done by multiplication
+// (the 64-bit divisions of the generic kernel above cost more than the copy).  The patch matrix is written once
+// and not read again by this kernel, so its stores are streamed past the cache, which stays with the image
+// (every pixel is read FH * FW times).
+struct Im2colVec {
+    int CV, K16;  // 16-byte pieces per tap and per patch row
+    FastDiv by_K16, by_CV, by_FW, by_OW, by_OH;
+    long rows;
+    int rows_per_block;
+};
+
+__global__ __launch_bounds__(256) void im2col_vec_kernel(const u32x4v *__restrict__ im, u32x4v *__restrict__ col,
+                                                         MapGeom g, Im2colVec q) {
+    // workgroup ids congruent modulo 8 run on the same XCD: each XCD takes one contiguous eighth of the patch
+    // rows, so its L2 fetches one eighth of the image (plus a halo) instead of most of it
+    const unsigned chunk = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const long row0 = (long)chunk * q.rows_per_block;
+    const long left = q.rows - row0;
+    if (left <= 0) return;
+    const unsigned nrows = (unsigned)(left < q.rows_per_block ? left : q.rows_per_block);
+    const unsigned span = nrows * (unsigned)q.K16;
+    u32x4v *out = col + row0 * q.K16;
+    constexpr int U = 4;
+    for (unsigned base = threadIdx.x; base < span; base += 256 * U) {
+        u32x4v v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned l = base + 256 * u;
+            v[u] = u32x4v{0u, 0u, 0u, 0u};
+            if (l < span) {
+                const unsigned rl = div_by(l, q.by_K16), piece = l - rl * q.K16;
+                const unsigned tap = div_by(piece, q.by_CV), cv = piece - tap * q.CV;
+                const unsigned fy = div_by(tap, q.by_FW), fx = tap - fy * g.FW;
+                const unsigned r = (unsigned)row0 + rl;
+                const unsigned t = div_by(r, q.by_OW), ox = r - t * g.OW;
+                const unsigned b = div_by(t, q.by_OH), oy = t - b * g.OH;
+                const int iy = (int)oy * g.sy + (int)fy * g.dy - g.pt;
+                const int ix = (int)ox * g.sx + (int)fx * g.dx - g.pl;
+                if (iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW)
+                    v[u] = im[(((long)b * g.IH + iy) * g.IW + ix) * q.CV + cv];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned l = base + 256 * u;
+            if (l < span) __builtin_nontemporal_store(v[u], out + l);
+        }
+    }
+}
+
 // The same with rows padded to `pitch` elements (a patch row whose own length cannot be moved in 16-byte
 // pieces: 1- and 3-channel images); the padding is written as zeros.  A thread gathers the NV elements of one
 // 16-byte piece of a row (the pitch is a multiple of that) and stores them at once.
@@ -286,7 +354,22 @@ int launch_im2col(int dtype, const void *im, void *col, const MapGeom &g, hipStr
     }
     const long elems = (long)g.B * g.OH * g.OW * g.FH * g.FW * g.C;
     const size_t row_bytes = (size_t)g.C * es;
-    if (row_bytes % 16 == 0 && aligned16(im) && aligned16(col)) {
+    const long rows = (long)g.B * g.OH * g.OW;
+    if (row_bytes % 16 == 0 && aligned16(im) && aligned16(col) && rows < (1L << 31) && (long)g.FH * g.FW * row_bytes / 16 < (1L << 20)) {
+        Im2colVec q;
+        q.CV = (int)(row_bytes / 16);
+        q.K16 = g.FH * g.FW * q.CV;
+        q.rows = rows;
+        // about 32 workgroups per CU, whole patch rows each, a stretch of fewer than 2^31 pieces
+        long per = (rows + (long)cu_count() * 32 - 1) / ((long)cu_count() * 32);
+        per = (per + 3) & ~3L;
+        while (per > 4 && per * q.K16 >= (1L << 31)) per /= 2;
+        q.rows_per_block = (int)per;
+        q.by_K16 = fast_div(q.K16), q.by_CV = fast_div(q.CV), q.by_FW = fast_div(g.FW), q.by_OW = fast_div(g.OW), q.by_OH = fast_div(g.OH);
+        const unsigned blocks = ((unsigned)((rows + per - 1) / per) + 7u) & ~7u;  // a multiple of 8 (see the kernel)
+        hipLaunchKernelGGL(im2col_vec_kernel, dim3(blocks), dim3(256), 0, s,
+                           (const u32x4v *)im, (u32x4v *)col, g, q);
+    } else if (row_bytes % 16 == 0 && aligned16(im) && aligned16(col)) {
         const int CV = (int)(row_bytes / 16);
         const long total = elems / (16 / es);
         hipLaunchKernelGGL((im2col_kernel<uint4>), dim3(grid_for(total, 256)), dim3(256), 0, s,

@@ -526,24 +526,11 @@ size_t d8_gemm_workspace_bytes(int dtype, int transA, int transB, int M, int N, 
     return splits > 1 ? (size_t)splits * outs * M * N * sizeof(float) : 0;
 }
 
-int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
-            const void *A, int lda, long strideA,
-            const void *B, int ldb, long strideB,
-            float beta, void *C, int ldc, long strideC, int batch,
-            void *workspace, size_t workspace_bytes, void *stream) {
-    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
-        return fail(D8_ERR_DTYPE, "d8_gemm: element type %d is not supported", dtype);
-    D8_REQUIRE(!(transA && transB), "d8_gemm: transA and transB together are not supported");
-    D8_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "d8_gemm: negative size");
-    D8_REQUIRE(beta == 0.f || beta == 1.f, "d8_gemm: beta must be 0 or 1");
-    if (M == 0 || N == 0 || batch == 0) return 0;
-    D8_REQUIRE(A && B && C, "d8_gemm: null operand");
-    D8_REQUIRE(lda >= (transA ? M : K), "d8_gemm: lda %d too small", lda);
-    D8_REQUIRE(ldb >= (transB ? K : N), "d8_gemm: ldb %d too small", ldb);
-    D8_REQUIRE(ldc >= N, "d8_gemm: ldc %d too small", ldc);
-    D8_REQUIRE(strideA >= 0 && strideB >= 0 && strideC >= 0, "d8_gemm: negative stride");
-    D8_REQUIRE((long)ceil_div(M, 128) < 65536 && (long)batch * 128 < 65536, "d8_gemm: grid too large");
-
+// One product whose grid fits the launch limits (at most MAX_BATCH independent outputs, at most MAX_ROWS rows).
+static int gemm_one(int dtype, int transA, int transB, int M, int N, int K,
+                    const void *A, int lda, long strideA, const void *B, int ldb, long strideB,
+                    float beta, void *C, int ldc, long strideC, int batch,
+                    void *workspace, size_t workspace_bytes, void *stream) {
     GemmArgs g;
     memset(&g, 0, sizeof(g));
     g.A = A;
@@ -576,6 +563,49 @@ int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
     }
     return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, tiled, as_stream(stream))
                                : launch<float>(g, transA, transB, tiled, as_stream(stream));
+}
+
+int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,
+            const void *A, int lda, long strideA,
+            const void *B, int ldb, long strideB,
+            float beta, void *C, int ldc, long strideC, int batch,
+            void *workspace, size_t workspace_bytes, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
+        return fail(D8_ERR_DTYPE, "d8_gemm: element type %d is not supported", dtype);
+    D8_REQUIRE(!(transA && transB), "d8_gemm: transA and transB together are not supported");
+    D8_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "d8_gemm: negative size");
+    D8_REQUIRE(beta == 0.f || beta == 1.f, "d8_gemm: beta must be 0 or 1");
+    if (M == 0 || N == 0 || batch == 0) return 0;
+    D8_REQUIRE(A && B && C, "d8_gemm: null operand");
+    D8_REQUIRE(lda >= (transA ? M : K), "d8_gemm: lda %d too small", lda);
+    D8_REQUIRE(ldb >= (transB ? K : N), "d8_gemm: ldb %d too small", ldb);
+    D8_REQUIRE(ldc >= N, "d8_gemm: ldc %d too small", ldc);
+    D8_REQUIRE(strideA >= 0 && strideB >= 0 && strideC >= 0, "d8_gemm: negative stride");
+    D8_REQUIRE(dtype != D8_FLOAT64 || (long)ceil_div(N, 64) < 65536, "d8_gemm: N = %d is beyond the %d columns a Float64 launch covers", N, 65535 * 64);
+
+    // A launch covers at most 65535 workgroups along its second and third axes.  A longer batch of independent
+    // products and a taller matrix are walked in slices, each an ordinary product on advanced pointers (the
+    // slices run one after the other on the stream, so they may share the workspace).
+    constexpr int MAX_BATCH = 448;            // independent outputs per launch (the tiled kernels take fewer than 512)
+    constexpr int MAX_ROWS = 65535 * 128;     // rows of C per launch
+    const size_t es = dtype_bytes(dtype);
+    const bool summed = strideC == 0 && batch > 1;
+    const int nb = summed ? 1 : ceil_div(batch, MAX_BATCH), per_b = summed ? batch : ceil_div(batch, nb);
+    const int nm = ceil_div(M, MAX_ROWS);
+    const int per_m = nm > 1 ? (ceil_div(ceil_div(M, nm), 128) * 128) : M;
+    for (int b0 = 0; b0 < batch; b0 += per_b) {
+        const int bn = batch - b0 < per_b ? batch - b0 : per_b;
+        for (int m0 = 0; m0 < M; m0 += per_m) {
+            const int mn = M - m0 < per_m ? M - m0 : per_m;
+            const char *a = (const char *)A + ((size_t)b0 * strideA + (transA ? (size_t)m0 : (size_t)m0 * lda)) * es;
+            const char *b = (const char *)B + (size_t)b0 * strideB * es;
+            char *c = (char *)C + ((size_t)b0 * strideC + (size_t)m0 * ldc) * es;
+            if (int rc = gemm_one(dtype, transA, transB, mn, N, K, a, lda, strideA, b, ldb, strideB, beta, c, ldc, strideC, bn,
+                                  workspace, workspace_bytes, stream))
+                return rc;
+        }
+    }
+    return 0;
 }
 
 }  // extern "C"

@@ -78,6 +78,9 @@ int d8_event_elapsed_ms(void *start, void *stop, float *ms);  /* synchronises on
  * D8_FLOAT64 operands accumulate in fp64 (the cublasDgemm twins of the call sites below); a split
  * reduction keeps its partial sums in fp64 too.
  *
+ * Sizes: any batch and any M (a batch of more than 448 independent products and a matrix of more than
+ * 8 388 480 rows are run as several launches on slices); Float64 takes at most 4 194 240 columns.
+ *
  * `workspace` (may be NULL) lets the kernel split the reduction (long K / summed batch, small
  * M x N) over more workgroups; d8_gemm_workspace_bytes says how much it can use.  It must be
  * 16-byte aligned (a misaligned workspace is ignored).

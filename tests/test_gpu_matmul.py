@@ -186,3 +186,32 @@ def test_matmul_step_replayed_from_a_hip_graph(oracle_port):
         capi.sync()
     check(lib.d8_graph_destroy(graph))
     check(lib.d8_stream_destroy(side))
+
+
+# Batches longer than one launch's third grid axis takes: cublas*gemmStridedBatched has no such limit
+# (deep8/src/math/MatrixMultiply.cu:115-134), so neither may d8_gemm.  600 and 1000 are walked in slices.
+LONG_BATCH = [
+    ((600, 24, 16), (600, 16, 40)),     # F3/X3/Y3: both batched, any-shape kernel
+    ((1000, 128, 32), (1000, 32, 128)),  # the same on the tiled kernel (128 x 128 outputs)
+    ((1, 24, 16), (600, 16, 40)),       # x broadcast: dX is summed over the 600 products
+    ((600, 24, 16), (1, 16, 40)),       # collapsed batch (one product of 14 400 rows)
+]
+
+
+@pytest.mark.parametrize("xs,ys", LONG_BATCH)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.float64])
+def test_matmul_batch_beyond_one_launch(oracle, oracle_port, xs, ys, dtype):
+    from deep8_amd import ops
+    r = rng(sum(xs) + sum(ys) + 5)
+    hi = 2 if dtype == np.float16 else 10
+    x, y = ints(r, xs, hi), ints(r, ys, hi)
+    if dtype == np.float16:  # keep every sum below 2048
+        x, y = x * (r.random(xs) < 0.1), y * (r.random(ys) < 0.1)
+    dz = ints(r, oracle_port.matmul(x, y).shape, hi)
+    dx0, dy0 = ints(r, xs, hi), ints(r, ys, hi)
+    c = lambda a: a.astype(dtype)
+    want = (oracle_port.matmul(x, y), oracle_port.matmul_grad_x(x, y, dz, dx0), oracle_port.matmul_grad_y(x, y, dz, dy0))
+    assert dtype != np.float16 or max(np.abs(w).max() for w in want) < 2048
+    assert np.array_equal(f(ops.matmul(c(x), c(y))), want[0])
+    assert np.array_equal(f(ops.matmul_grad_x(c(x), c(y), c(dz), c(dx0))), want[1])
+    assert np.array_equal(f(ops.matmul_grad_y(c(x), c(y), c(dz), c(dy0))), want[2])
