@@ -801,6 +801,61 @@ def graph_replay_ms(wl, steps, warmup):
         lib.d8_stream_destroy(side)
 
 
+WIDE_DIAGNOSTICS = {"same_k": "D8_WIDE_DIAG_SAME_K", "barrier_clocks": "D8_WIDE_DIAG_BARRIER_CLOCKS",
+                    "no_store": "D8_WIDE_DIAG_NO_STORE", "direct_store": "D8_WIDE_DIAG_DIRECT_STORE"}
+
+
+def build_wide_diagnostic(name):
+    """compiles deep8_amd/csrc/gemm_wide.hip with one of its diagnostic switches and links it with the objects of
+    the shipped library (deep8_amd/csrc/obj, left by __graft_entry__.build()) into a scratch library; returns its path"""
+    import subprocess
+    import tempfile
+    import __graft_entry__ as ge
+    csrc = os.path.join(ROOT, "deep8_amd", "csrc")
+    tmp = tempfile.mkdtemp(prefix="d8_wide_diag_")
+    obj, lib = os.path.join(tmp, "gemm_wide.o"), os.path.join(tmp, "libdeep8_hip_%s.so" % name)
+    subprocess.check_call([ge.HIPCC] + ge.HIP_FLAGS + ["-D" + WIDE_DIAGNOSTICS[name], "-c", os.path.join(csrc, "gemm_wide.hip"), "-o", obj],
+                          stderr=subprocess.DEVNULL)
+    # the other sources: their objects from the shipped build where present, else compiled here (all at once)
+    objs, jobs = [obj], []
+    for src in sorted(f for f in os.listdir(csrc) if f.endswith(".hip") and f != "gemm_wide.hip"):
+        have = os.path.join(csrc, "obj", src[:-4] + ".o")
+        if os.path.exists(have):
+            objs.append(have)
+        else:
+            o = os.path.join(tmp, src[:-4] + ".o")
+            jobs.append(subprocess.Popen([ge.HIPCC] + ge.HIP_FLAGS + ["-c", os.path.join(csrc, src), "-o", o], stderr=subprocess.DEVNULL))
+            objs.append(o)
+    for j in jobs:
+        if j.wait() != 0:
+            raise SystemExit("bench.py: compiling the library's sources for the diagnostic build failed")
+    subprocess.check_call([ge.HIPCC] + ge.HIP_FLAGS + ["-shared", "-o", lib] + objs, stderr=subprocess.DEVNULL)
+    return lib
+
+
+def barrier_clock_record():
+    """phase record of the D8_WIDE_DIAG_BARRIER_CLOCKS build: cycles per K step spent in the wait for the step's
+    own loads and in its barrier (each figure includes one clock read; the first column is that cost alone)"""
+    from deep8_amd import capi
+    lib = capi.init()
+    wl = make_workload("c3")
+    n = 4096
+    out = capi.DeviceArray((n, n), np.float16)
+    rec = capi.DeviceArray((256 * 6,), np.uint64, zero=True)
+    for name, ta, tb, A, B in (("forward NN", 0, 0, wl.x, wl.y), ("dX NT", 0, 1, wl.dz, wl.y), ("dY TN", 1, 0, wl.x, wl.dz)):
+        def launch():
+            capi.check(lib.d8_gemm(wl.dt, ta, tb, n, n, n, A.ptr, n, 0, B.ptr, n, 0, 0.0, out.ptr, n, 0, 1, rec.ptr, 256 * 6 * 8, None))
+        _settle(launch)
+        for _ in range(10):
+            launch()
+        capi.sync()
+        r = rec.numpy().astype(np.int64).reshape(256, 6)
+        st = n // 64
+        print("%s: cycles per K step (mean over the 256 workgroups): two clock reads back to back %.0f, wait for the "
+              "step's own loads %.0f, barrier %.0f; whole loop %.0f (with the four clock reads in it)" % (
+                  name, r[:, 0].mean() / st, r[:, 1].mean() / st, r[:, 2].mean() / st, (r[:, 5] - r[:, 4]).mean() / st), flush=True)
+
+
 def phase_record(launches=12):
     """The fp16 4096^3 launches of workload c3 with the kernel's own phase record switched on (D8_GEMM_STAMPS):
     every workgroup notes the wall clock (100 MHz, common to the chip) at its start, after its prologue, after
@@ -868,6 +923,9 @@ def main():
                          "(0: start from an idle device)")
     ap.add_argument("--phases", action="store_true",
                     help="only print the phase record of workload c3's three products (see phase_record)")
+    ap.add_argument("--wide-diagnostic", choices=sorted(WIDE_DIAGNOSTICS), default=None,
+                    help="with --phases: compile the fp16 kernel with one of its diagnostic switches into a scratch "
+                         "library and print that build's phase record (see the header of deep8_amd/csrc/gemm_wide.hip)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
@@ -882,7 +940,14 @@ def main():
     if a.phases:
         os.environ["D8_GEMM_STAMPS"] = "1"  # read by the library at its first launch
     from deep8_amd import capi
+    if a.wide_diagnostic:
+        if not a.phases:
+            raise SystemExit("--wide-diagnostic goes with --phases")
+        capi.LIB_PATH = build_wide_diagnostic(a.wide_diagnostic)
+        print("diagnostic build of gemm_wide.hip: -D%s" % WIDE_DIAGNOSTICS[a.wide_diagnostic], flush=True)
     capi.init()
+    if a.phases and a.wide_diagnostic == "barrier_clocks":
+        return barrier_clock_record()
     if a.calibrate_copy:
         return calibrate_copy(a.calibrate_copy)
     if a.phases:

@@ -28,6 +28,19 @@
 // The MFMAs are volatile asm statements (accumulators pinned to AGPRs, updated in place); the
 // compiler keeps memory instructions between the two MFMAs they were written between, so the
 // issue order is the program order.
+//
+// Diagnostic builds (never defined in the shipped library; `python bench.py --phases --wide-diagnostic NAME`
+// compiles this file with one of them into a scratch copy of the library and prints the kernel's phase
+// record).  Each answers one question about where a launch's time goes; SAME_K and NO_STORE give wrong results:
+//   D8_WIDE_DIAG_SAME_K          every K step fetches the tile's first step again, so all loads after the first
+//                                hit in cache: what the loop costs when no load ever waits for HBM
+//   D8_WIDE_DIAG_BARRIER_CLOCKS  reads the shader clock around the step's wait for its own loads and around its
+//                                barrier; the record's first three fields become the summed cycles of a pair of
+//                                back-to-back clock reads, of the wait and of the barrier
+//   D8_WIDE_DIAG_NO_STORE        the epilogue does everything but the stores to C: its cost without HBM writes
+//   D8_WIDE_DIAG_DIRECT_STORE    accumulates the blocks transposed (MFMA operands exchanged) so that a lane owns
+//                                four consecutive columns, and stores them straight from registers, 8 bytes per
+//                                lane, without the LDS patch (correct results)
 #include <type_traits>
 
 #include "gemm_args.h"
@@ -124,7 +137,11 @@ struct Operand {
 };
 
 __device__ __forceinline__ void mfma(f32x4 &acc, const f16x8 &a, const f16x8 &b) {
+#ifdef D8_WIDE_DIAG_DIRECT_STORE
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %2, %1, %0" : "+a"(acc) : "v"(a), "v"(b));
+#else
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+#endif
 }
 
 }  // namespace wide
@@ -165,8 +182,13 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
     oa.init(g.lda, wave, lane, wm * 128);
     ob.init(g.ldb, wave, lane, wn * 128);
     // uniform byte offset of the tile at step 0, and from one step to the next
-    const unsigned a_org = 2u * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0), a_step = A_KC ? 128u : 2u * BK * g.lda;
-    const unsigned b_org = 2u * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0), b_step = B_KC ? 128u : 2u * BK * g.ldb;
+    const unsigned a_org = 2u * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0), a_step_ = A_KC ? 128u : 2u * BK * g.lda;
+    const unsigned b_org = 2u * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0), b_step_ = B_KC ? 128u : 2u * BK * g.ldb;
+#ifndef D8_WIDE_DIAG_SAME_K
+    const unsigned a_step = a_step_, b_step = b_step_;
+#else
+    const unsigned a_step = 0u * a_step_, b_step = 0u * b_step_;
+#endif
     const int nsteps = g.K / BK;
 
     f32x4 acc[8][8];
@@ -178,6 +200,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
             asm volatile("" : "+a"(acc[i][j]));  // from here on the value lives in AGPRs
         }
     f16x8 fa[2][8], fb[2][8];
+#ifdef D8_WIDE_DIAG_BARRIER_CLOCKS
+    unsigned long long bar_cal = 0, bar_vm = 0, bar_sync = 0;
+#endif
 
     // ---- prologue: steps 0 and 1 into the two stages, fragments of step 0's k group 0
 #pragma unroll
@@ -219,8 +244,23 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
             }
         }
         // half 1
+#ifdef D8_WIDE_DIAG_BARRIER_CLOCKS
+        const unsigned long long tb0 = __builtin_readcyclecounter();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const unsigned long long tb1 = __builtin_readcyclecounter();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#endif
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): my pieces of the next step have landed
+#ifdef D8_WIDE_DIAG_BARRIER_CLOCKS
+        const unsigned long long tb2 = __builtin_readcyclecounter();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#endif
         __syncthreads();
+#ifdef D8_WIDE_DIAG_BARRIER_CLOCKS
+        const unsigned long long tb3 = __builtin_readcyclecounter();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        bar_cal += tb1 - tb0, bar_vm += tb2 - tb1, bar_sync += tb3 - tb2;
+#endif
 #pragma unroll
         for (int m = 0; m < 64; ++m) {
             if ((m & 3) == 0) {
@@ -253,6 +293,35 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
     // ---- epilogue: 16 rows of the wave's 128 x 128 at a time through a patch of LDS, so that C
     // is read (beta = 1) and written 16 bytes per lane, 256 contiguous bytes per 16 lanes
     if (g.stamps) wall[2] = wall_clock64(), clk[1] = __builtin_readcyclecounter();
+#ifdef D8_WIDE_DIAG_DIRECT_STORE
+    {
+        // the blocks were accumulated transposed (operands exchanged): lane holds C[i*16 + (lane & 15)][j*16 + 4*(lane >> 4) + 0..3]
+        f16 *C = (f16 *)g.C + (long)b * g.sC;
+        const int l15 = lane & 15, l4 = lane >> 4;
+        typedef __fp16 h4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int m = m0 + wm * 128 + i * 16 + l15;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int n = n0 + wn * 128 + j * 16 + 4 * l4;
+                if (m >= m_own && n >= n_own) {
+                    f16 *c = C + (long)m * g.ldc + n;
+                    h4 out;
+                    if (g.beta != 0.f) {
+                        const h4 old = *(const h4 *)c;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) out[e] = (__fp16)(acc[i][j][e] + (float)old[e]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) out[e] = (__fp16)acc[i][j][e];
+                    }
+                    __builtin_nontemporal_store(out, (h4 *)c);
+                }
+            }
+        }
+    }
+#else
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();  // no load is still on its way into LDS, every wave is past its last read
     float *patch = (float *)lds + wave * (16 * PATCH_LD);
@@ -271,7 +340,11 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
             float v[8];
             *(f32x4 *)&v[0] = *(const f32x4 *)(patch + row * PATCH_LD + cc);
             *(f32x4 *)&v[4] = *(const f32x4 *)(patch + row * PATCH_LD + cc + 4);
+#ifdef D8_WIDE_DIAG_NO_STORE
+            if (m >= m_own && n >= n_own && g.K < 0) {
+#else
             if (m >= m_own && n >= n_own) {
+#endif
                 f16 *c = C + (long)m * g.ldc + n;
                 f16x8 out;
                 if (g.beta != 0.f) {
@@ -288,12 +361,16 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
             }
         }
     }
+#endif
     if (g.stamps) {
         __builtin_amdgcn_s_waitcnt(0x0f70);  // this wave's stores have been acknowledged
         wall[3] = wall_clock64();
         if (tid == 0) {
             unsigned long long *rec = (unsigned long long *)g.ws + 6 * (blockIdx.x + gridDim.x * blockIdx.z);
             rec[0] = wall[0], rec[1] = wall[1], rec[2] = wall[2], rec[3] = wall[3], rec[4] = clk[0], rec[5] = clk[1];
+#ifdef D8_WIDE_DIAG_BARRIER_CLOCKS
+            rec[0] = bar_cal, rec[1] = bar_vm, rec[2] = bar_sync;
+#endif
         }
     }
 }
