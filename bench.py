@@ -392,6 +392,51 @@ class ConvWorkload:
                 "frac": round(ach / PEAK[dtype], 4), "launch_us": round(ms * 1e3, 2), **_traffic_fields(self.key)}
 
 
+class ConvBiasReluWorkload(ConvWorkload):
+    """Configuration 4's layer as it sits in a network: Conv2d -> Add (per-channel bias) -> ReLu, forward and backward.
+    fused:   d8_conv2d_bias_relu | d8_bias_relu_grad, d8_conv2d_grad_x, d8_conv2d_grad_y          (4 calls)
+    unfused: d8_conv2d, d8_add, d8_relu | d8_relu_grad, d8_add_grad, d8_conv2d_grad_x, d8_conv2d_grad_y   (7 calls, the
+             reference's sequence: deep8/src/math/Add.cu:21-52, ReLu.cu:20-116)"""
+
+    def __init__(self, name, dtype, B, IH, IW, IC, OC, FH, FW, seed, fused):
+        import ctypes
+        from deep8_amd import capi
+        ConvWorkload.__init__(self, name, dtype, False, B, IH, IW, IC, OC, FH, FW, True, 1, 1, seed)
+        self.fused = fused
+        r = np.random.default_rng(seed + 100)
+        self.bias = _dev(r.standard_normal((OC,)).astype(np.float32).astype(dtype))
+        zs = self.z.shape
+        self.pre, self.sum, self.dpre = capi.DeviceArray(zs, dtype), capi.DeviceArray(zs, dtype), capi.DeviceArray(zs, dtype)
+        self.gb = capi.DeviceArray((OC,), dtype)
+        self.rows, self.OC = int(np.prod(zs[:-1])), OC
+        I5 = ctypes.c_int * 5
+        self.zd, self.bd = I5(zs[0], 1, zs[1], zs[2], OC), I5(1, 1, 1, 1, OC)
+        self.rs_bytes = max(self.lib.d8_add_grad_scratch_bytes(self.dt, self.bd, self.zd),
+                            self.lib.d8_bias_relu_grad_scratch_bytes(self.dt, self.rows, OC))
+        self.rs = capi.DeviceArray((max(self.rs_bytes, 16),), np.uint8)
+        nz = self.rows * OC * self.dtype.itemsize
+        self.bytes += 4 * nz if fused else 9 * nz   # fused: z written by the product anyway; r z, r dz, w dpre (+ dpre read by the products)
+
+    def step(self):
+        from deep8_amd.capi import check
+        L, n = self.lib, self.rows * self.OC
+        B, IH, IW, IC = self.xd
+        OC, FH, FW, _ = self.wd
+        if self.fused:
+            check(L.d8_conv2d_bias_relu(self.dt, self.x.ptr, B, IH, IW, IC, self.w.ptr, OC, FH, FW, self.bias.ptr, 1, self.z.ptr,
+                                        *self.geo, self.ws.ptr, self.ws_bytes, None))
+            check(L.d8_bias_relu_grad(self.dt, self.z.ptr, self.gz.ptr, self.dpre.ptr, self.gb.ptr, self.rows, OC, 0,
+                                      self.rs.ptr, self.rs_bytes, None))
+        else:
+            self._call(L.d8_conv2d, self.x.ptr, self.w.ptr, self.pre.ptr)
+            check(L.d8_add(self.dt, self.pre.ptr, self.zd, self.bias.ptr, self.bd, self.sum.ptr, self.zd, None))
+            check(L.d8_relu(self.dt, self.sum.ptr, self.z.ptr, n, None))
+            check(L.d8_relu_grad_overwrite(self.dt, self.sum.ptr, self.dpre.ptr, self.gz.ptr, n, None))
+            check(L.d8_add_grad_overwrite(self.dt, self.gb.ptr, self.bd, self.dpre.ptr, self.zd, self.rs.ptr, self.rs_bytes, None))
+        self._call(L.d8_conv2d_grad_x_overwrite, self.gx.ptr, self.w.ptr, self.dpre.ptr)
+        self._call(L.d8_conv2d_grad_y_overwrite, self.x.ptr, self.gw.ptr, self.dpre.ptr)
+
+
 class DeconvLiteralWorkload:
     """Benchmark configuration 5 at its literal geometry (28 -> 56, PyTorch's ConvTranspose2d(k=4, s=2, p=1)),
     which Deep8's DeConv2d does not admit (deep8/src/nodes/DeConv2d.cpp:36-52 allows 58 or 55): kernel level only,
@@ -633,6 +678,10 @@ def make_workload(key):
         return ConvWorkload("c4x: Conv2d fwd+dX+dW fp32 B32 56x56x64 3x3x64->64 s1 same, the reference's lowering "
                             "(im2col -> GEMM, GEMM -> col2im, 231 MB interim matrix)", np.float32, False,
                             32, 56, 56, 64, 64, 3, 3, True, 1, 1, 5, explicit=True)
+    if key in ("c4e", "c4e_unfused"):
+        return ConvBiasReluWorkload("%s: Conv2d + bias Add + ReLu fwd+bwd fp32 B32 56x56x64 3x3x64->64, %s" % (
+            key, "bias and ReLu in the product's store, ReLuGrad + bias gradient in one pass" if key == "c4e" else
+            "every operator a call of its own (the reference's sequence)"), np.float32, 32, 56, 56, 64, 64, 3, 3, 5, key == "c4e")
     if key == "i4":
         return GatherMapsWorkload("i4: d8_im2col + d8_col2im alone at config 4's size, fp32 B32 56x56x64 3x3 s1 pad 1",
                                   np.float32, 32, 56, 56, 64, 3, 11)
@@ -707,10 +756,10 @@ def cpu_baseline(key, seconds=12.0):
         n, dt = _repeat_for(one, seconds)
         return {"value": n * B / dt, "unit": "images/s", "cores": port.threads(), "kind": "port",
                 "sample": "im2col + col2im on %d images x %d repeats (fp32, C restatement), %.1f s" % (B, n, dt)}
-    if key in ("c4", "c4x", "c5"):
+    if key in ("c4", "c4x", "c4e", "c4e_unfused", "c5"):
         # the reference runs Conv2d/DeConv2d on Eigen's thread pool: all host cores
         B = 8
-        if key in ("c4", "c4x"):
+        if key != "c5":
             x, w = r.standard_normal((B, 56, 56, 64)).astype(np.float32), r.standard_normal((64, 3, 3, 64)).astype(np.float32)
             args, f3 = (True, 1, 1, 1, 1), (src.conv2d, src.conv2d_grad_x, src.conv2d_grad_y)
         else:
@@ -1037,7 +1086,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4x", "i4", "c5", "c5l", "e4", "p4", "d3"):
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4e", "c4e_unfused", "c4x", "i4", "c5", "c5l", "e4", "p4", "d3"):
             if key == a.workload:
                 continue
             del wl

@@ -192,6 +192,91 @@ __global__ __launch_bounds__(256) void column_sum_finish_kernel(const float *__r
     }
 }
 
+// ReLuGrad and the bias gradient in one pass over a [R][C] gradient: dpre = z > 0 ? dz : 0 is written out and its
+// column sums are taken on the way, with column_sum_kernel's chunks, row order and LDS meeting order, so the sums
+// are bit for bit those of d8_add_grad run on dpre afterwards.  z is the layer's output relu(pre): z > 0 exactly
+// where pre > 0 (deep8/src/math/ReLu.cu:61-116 gates on pre; Add.cu:64-133 sums).  dpre may be dz (in place).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void relu_gate_column_sum_kernel(const T *__restrict__ z, const T *dz, T *dpre,
+                                                                   T *__restrict__ g, float *__restrict__ partial, int R, int C,
+                                                                   int TX, int rows_per_chunk, int chunks, float keep) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    __shared__ float part[256][VEC];
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX, lanes = 256 / TX;
+    const int cv = blockIdx.x * TX + tx;
+    const int chunk = blockIdx.y;
+    const bool live = (long)cv * VEC < C;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    if (live) {
+        const int r1 = min(R, (chunk + 1) * rows_per_chunk);
+        const long col = (long)cv * VEC;
+        int r = chunk * rows_per_chunk + ty;
+        for (; r + 3 * lanes < r1; r += 4 * lanes) {
+            VT a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a[u] = *(const VT *)(z + (long)(r + u * lanes) * C + col);
+                b[u] = *(const VT *)(dz + (long)(r + u * lanes) * C + col);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    if (!(ew_f32(a[u][e]) > 0.f)) b[u][e] = (T)0.f;
+                    acc[e] += ew_f32(b[u][e]);
+                }
+                *(VT *)(dpre + (long)(r + u * lanes) * C + col) = b[u];
+            }
+        }
+        for (; r < r1; r += lanes) {
+            const VT a = *(const VT *)(z + (long)r * C + col);
+            VT b = *(const VT *)(dz + (long)r * C + col);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if (!(ew_f32(a[e]) > 0.f)) b[e] = (T)0.f;
+                acc[e] += ew_f32(b[e]);
+            }
+            *(VT *)(dpre + (long)r * C + col) = b;
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) part[threadIdx.x][e] = acc[e];
+    __syncthreads();
+    if (ty == 0 && live) {
+        for (int k = 1; k < lanes; ++k)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += part[k * TX + tx][e];
+        if (chunks == 1) {
+            T *o = g + (long)cv * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = (T)((keep != 0.f ? ew_f32(o[e]) : 0.f) + acc[e]);
+        } else {
+            float *o = partial + (long)chunk * C + (long)cv * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = acc[e];
+        }
+    }
+}
+
+// z[r][c] = relu?(z[r][c] + bias[c]) in place: the one-pass fallback of the fused GEMM store.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bias_relu_kernel(T *z, const T *__restrict__ bias, long nvec, int CV, int relu) {
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < nvec; idx += (long)gridDim.x * blockDim.x) {
+        VT v = *(const VT *)(z + idx * VEC);
+        const int c = (int)(idx % CV) * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float f = ew_f32(v[e]);
+            if (bias) f = ew_f32((T)(f + ew_f32(bias[c + e])));  // rounded as the separate Add pass rounds it
+            v[e] = (T)(relu && !(f > 0.f) ? 0.f : f);
+        }
+        *(VT *)(z + idx * VEC) = v;
+    }
+}
+
 // Any other pattern of kept and summed axes: a thread per element of g walks the summed index
 // space in memory order (the order of the reference kernel, GPUBinaryElementWise.h:42-95).
 struct ReduceGeom {
@@ -491,11 +576,75 @@ static int check_norm(const char *who, int dtype, const void *x, const void *y, 
     return 0;
 }
 
+template <typename T, int WIDE>
+static int bias_relu_t(T *z, const T *bias, long rows, int cols, int relu, hipStream_t s) {
+    const long n = rows * cols;
+    if (cols % WIDE == 0 && al16(z) && al16(bias))
+        hipLaunchKernelGGL((bias_relu_kernel<T, WIDE>), dim3(ew_grid(n / WIDE, 256)), dim3(256), 0, s, z, bias, n / WIDE, cols / WIDE, relu);
+    else
+        hipLaunchKernelGGL((bias_relu_kernel<T, 1>), dim3(ew_grid(n, 256)), dim3(256), 0, s, z, bias, n, cols, relu);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_bias_relu(int dtype, void *z, const void *bias, long rows, int cols, int relu, hipStream_t stream) {
+    if (rows <= 0 || cols <= 0 || (!bias && !relu)) return 0;
+    if (dtype == D8_FLOAT32) return bias_relu_t<float, 4>((float *)z, (const float *)bias, rows, cols, relu, stream);
+    if (dtype == D8_FLOAT16) return bias_relu_t<f16, 8>((f16 *)z, (const f16 *)bias, rows, cols, relu, stream);
+    return fail(D8_ERR_DTYPE, "bias / ReLu store: element type %d is not supported", dtype);
+}
+
+// dpre = z > 0 ? dz : 0;  g = keep * g + column sums of dpre.  Same plan as reduce_t on a [R][C] tensor.
+template <typename T, int WIDE>
+static int relu_gate_sum_t(const T *z, const T *dz, T *dpre, T *g, long rows, int cols, void *scratch, size_t scratch_bytes,
+                           float keep, hipStream_t s) {
+    const int gd[5] = {1, 1, 1, 1, cols}, zd[5] = {1, 1, 1, (int)rows, cols};
+    const ReducePlan p = plan_reduce(gd, zd);
+    // (a single row has nothing to sum: one chunk, the sums are the row itself)
+    int chunks = p.kind == 1 ? p.chunks : 1, rpc = p.kind == 1 ? p.rows_per_chunk : (int)rows;
+    const size_t need = (size_t)chunks * cols * sizeof(float);
+    if (chunks > 1 && (!scratch || scratch_bytes < need || !al16(scratch))) chunks = 1, rpc = (int)rows;
+    const bool wide = cols % WIDE == 0 && al16(g) && al16(dz) && al16(z) && al16(dpre);
+    const long cvs = cols / (wide ? WIDE : 1);
+    int TX = 1;
+    while (TX < 32 && TX < cvs) TX *= 2;
+    dim3 grid((unsigned)((cvs + TX - 1) / TX), (unsigned)chunks, 1);
+    if (wide)
+        hipLaunchKernelGGL((relu_gate_column_sum_kernel<T, WIDE>), grid, dim3(256), 0, s, z, dz, dpre, g, (float *)scratch, (int)rows, cols, TX, rpc, chunks, keep);
+    else
+        hipLaunchKernelGGL((relu_gate_column_sum_kernel<T, 1>), grid, dim3(256), 0, s, z, dz, dpre, g, (float *)scratch, (int)rows, cols, TX, rpc, chunks, keep);
+    D8_LAUNCH_CHECK();
+    if (chunks > 1) {
+        hipLaunchKernelGGL((column_sum_finish_kernel<T>), dim3((unsigned)((cols + 15) / 16)), dim3(256), 0, s,
+                           (const float *)scratch, g, cols, chunks, (long)cols, 1.f, keep);
+        D8_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
 }  // namespace d8
 
 using namespace d8;
 
 extern "C" {
+
+size_t d8_bias_relu_grad_scratch_bytes(int dtype, long rows, int cols) {
+    if (rows < 1 || cols < 1 || rows >= (1L << 31)) return 0;
+    const int gd[5] = {1, 1, 1, 1, cols}, zd[5] = {1, 1, 1, (int)rows, cols};
+    return d8_add_grad_scratch_bytes(dtype, gd, zd);
+}
+
+int d8_bias_relu_grad(int dtype, const void *z, const void *dz, void *dpre, void *dbias, long rows, int cols,
+                      int accumulate_bias, void *scratch, size_t scratch_bytes, void *stream) {
+    if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32)
+        return fail(D8_ERR_DTYPE, "d8_bias_relu_grad: element type %d is not supported", dtype);
+    D8_REQUIRE(z && dz && dpre && dbias, "d8_bias_relu_grad: null tensor");
+    D8_REQUIRE(rows > 0 && cols > 0 && rows < (1L << 31), "d8_bias_relu_grad: %ld rows x %d columns", rows, cols);
+    const float keep = accumulate_bias ? 1.f : 0.f;
+    return dtype == D8_FLOAT32
+               ? relu_gate_sum_t<float, 4>((const float *)z, (const float *)dz, (float *)dpre, (float *)dbias, rows, cols, scratch, scratch_bytes, keep, as_stream(stream))
+               : relu_gate_sum_t<f16, 8>((const f16 *)z, (const f16 *)dz, (f16 *)dpre, (f16 *)dbias, rows, cols, scratch, scratch_bytes, keep, as_stream(stream));
+}
 
 int d8_add(int dtype, const void *x, const int *xdims, const void *y, const int *ydims, void *z, const int *zdims,
            void *stream) {

@@ -329,7 +329,8 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(GemmArgs g) {
             T *c = c0 + c_index(g, m, n + k);
             float o = v[k];
             if (g.beta != 0.f) o += to_f32(*c);
-            *c = (T)o;
+            if (g.bias) o += to_f32(((const T *)g.bias)[n + k]);
+            *c = (T)(g.relu && !(o > 0.f) ? 0.f : o);
         }
     }
 }
@@ -366,7 +367,8 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_scalar_kernel(GemmArgs 
         const int m = (int)(e / g.N), n = (int)(e - (long)m * g.N);
         T *c = (T *)g.C + (long)b * g.sC + c_index(g, m, n);
         if (g.beta != 0.f) v += to_f32(*c);
-        *c = (T)v;
+        if (g.bias) v += to_f32(((const T *)g.bias)[n]);
+        *c = (T)(g.relu && !(v > 0.f) ? 0.f : v);
     }
 }
 
@@ -498,6 +500,16 @@ int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspa
         return gemm_tiled_run_whole(dtype, g, transA, transB, workspace, workspace_bytes, stream);
     if (int rc = gemm_tiled_run_whole(dtype, first, transA, transB, nullptr, 0, stream)) return rc;
     return gemm_tiled_run_whole(dtype, second, transA, transB, workspace, workspace_bytes, stream);
+}
+
+bool gemm_fuses_store(int dtype, const GemmArgs &g, int transA, int transB) {
+    if (dtype == D8_FLOAT64 || g.K < 1 || g.beta != 0.f || g.red != 1 || g.batch > 448) return false;
+    if (g.virt == VIRT_NONE && gemm_is_small(g.M, g.N, g.K, g.batch, g.red)) return false;  // gemm_small_kernel has no fused store
+    return gemm_tiled_eligible(dtype, g, transA, transB);
+}
+
+int gemm_run_fused(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    return gemm_tiled_run(dtype, g, transA, transB, workspace, workspace_bytes, stream);
 }
 
 }  // namespace d8

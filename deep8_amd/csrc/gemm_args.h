@@ -71,7 +71,21 @@ struct GemmArgs {
     // is given): every workgroup records when its prologue, K loop and epilogue ended into ws
     int stamps;
     size_t ws_bytes;  // size of ws as d8_gemm received it (0 where a planner filled the block in)
+    // Fused store (the tiled kernels, the large-output fp16 kernel and the split reduction): after the product
+    // (and beta * C), column n of the result gets bias[n] added (bias: N elements of C's type, may be null),
+    // then negative values become 0 when relu is set.  What Add (a per-column bias broadcast over the rows) and
+    // ReLu do as separate passes over C in the reference (deep8/src/math/Add.cu:21-52, ReLu.cu:20-59).
+    const void *bias;
+    int relu;
 };
+
+// Whether a product with these arguments would run on a kernel that applies GemmArgs::bias / relu in its store
+// (else the caller runs the plain product and launch_bias_relu).
+bool gemm_fuses_store(int dtype, const GemmArgs &g, int transA, int transB);
+// The product of d8_gemm (beta = 0, no summed batch) with the fused store; the shape must pass gemm_fuses_store.
+int gemm_run_fused(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes, hipStream_t stream);
+// z[r][c] = relu?(z[r][c] + bias[c]) in place, one pass (bias may be null): the fallback for shapes the fused store does not take.
+int launch_bias_relu(int dtype, void *z, const void *bias, long rows, int cols, int relu, hipStream_t stream);
 
 // Tiled kernels (fp16 and fp32) for shapes whose operands can be moved in 16-byte pieces.
 int gemm_tiled_k_step(int dtype);  // K elements per step: 64 (fp16) or 32 (fp32)

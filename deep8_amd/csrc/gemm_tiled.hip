@@ -260,13 +260,14 @@ struct RowMap {
 
 template <typename T, typename O>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *lds0, float *lds1, O *C, int ldc, float beta,
-                                           bool aligned, int N, const Origin &o, const RowMap &crow) {
+                                           bool aligned, int N, const Origin &o, const RowMap &crow,
+                                           const O *bias = nullptr, bool relu = false) {
     constexpr int TM = T::TM, TN = T::TN, OPV = 16 / sizeof(O);
     typedef O OV __attribute__((ext_vector_type(OPV)));
     constexpr int HALF_WAVES = T::NT / 128;
     static_assert((size_t)T::PATCH_SZ * T::ES >= (size_t)HALF_WAVES * 32 * 36 * sizeof(float), "patch space");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lhi = lane >> 5;
-    if (aligned && N % 8 == 0 && !crow.perm_OC) {
+    if (aligned && N % 8 == 0 && !crow.perm_OC && ((size_t)bias & 15) == 0) {
         float *patch = (wave < HALF_WAVES ? lds0 + wave * (32 * 36) : lds1 + (wave - HALF_WAVES) * (32 * 36));
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -289,11 +290,15 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
                             if (beta != 0.f) {
                                 const OV old = *(const OV *)(c + h * OPV);
 #pragma unroll
-                                for (int e = 0; e < OPV; ++e) out[e] = (O)(v[h * OPV + e] + as_f32(old[e]));
-                            } else {
-#pragma unroll
-                                for (int e = 0; e < OPV; ++e) out[e] = (O)v[h * OPV + e];
+                                for (int e = 0; e < OPV; ++e) v[h * OPV + e] += as_f32(old[e]);
                             }
+                            if (bias) {
+                                const OV bv = *(const OV *)(bias + n + h * OPV);
+#pragma unroll
+                                for (int e = 0; e < OPV; ++e) v[h * OPV + e] += as_f32(bv[e]);
+                            }
+#pragma unroll
+                            for (int e = 0; e < OPV; ++e) out[e] = (O)(relu && !(v[h * OPV + e] > 0.f) ? 0.f : v[h * OPV + e]);
                             *(OV *)(c + h * OPV) = out;
                         }
                     }
@@ -313,7 +318,8 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
                     O *c = C + crow.at(m, n, ldc);
                     float v = acc[i][j][r];
                     if (beta != 0.f) v += as_f32(*c);
-                    *c = (O)v;
+                    if (bias) v += as_f32(bias[n]);
+                    *c = (O)(relu && !(v > 0.f) ? 0.f : v);
                 }
             }
         }
@@ -579,7 +585,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o, plain);
     else
         store_tile<T, E>(acc, patches, patches1, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
-                         g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o, crow);
+                         g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o, crow, (const E *)g.bias, g.relu != 0);
 }
 
 template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int VIRT>

@@ -350,11 +350,15 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
                 if (g.beta != 0.f) {
                     const f16x8 old = *(const f16x8 *)c;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) out[e] = (f16)(v[e] + (float)old[e]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) out[e] = (f16)v[e];
+                    for (int e = 0; e < 8; ++e) v[e] += (float)old[e];
                 }
+                if (g.bias) {  // fused store: per-column bias, then ReLu (see GemmArgs::bias)
+                    const f16x8 bv = *(const f16x8 *)((const f16 *)g.bias + n);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] += (float)bv[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) out[e] = (f16)(g.relu && !(v[e] > 0.f) ? 0.f : v[e]);
                 // streamed past the L2: the whole output leaves the chip during the kernel's last microseconds
                 // either way, and lines left dirty in L2 are written back only after the last wave has ended
                 __builtin_nontemporal_store(out, (f16x8 *)c);
@@ -380,7 +384,7 @@ bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB) {
     if (g.M < 256 || g.N < 256 || g.K < 64 || g.K % 64) return false;
     if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || g.sA % 8 || g.sB % 8 || g.sC % 8 || g.N % 8) return false;
     if (transA && g.M % 8) return false;
-    if (((size_t)g.A | (size_t)g.B | (size_t)g.C) & 15) return false;
+    if (((size_t)g.A | (size_t)g.B | (size_t)g.C | (size_t)g.bias) & 15) return false;
     if (2L * (transA ? g.K : g.M) * g.lda >= (1L << 31) || 2L * (transB ? g.N : g.K) * g.ldb >= (1L << 31)) return false;
     if ((long)ceil_div(g.M, 256) * ceil_div(g.N, 256) > 0x7fffffffL || g.batch > 65535) return false;
     return true;

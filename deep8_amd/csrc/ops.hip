@@ -36,6 +36,34 @@ static int run(int dtype, const Gemm &g, void *ws, size_t ws_bytes, void *stream
                    g.C, g.ldc, g.sC, g.batch, ws, ws_bytes, stream);
 }
 
+// The same product as a GemmArgs block (what d8_gemm builds from its arguments), for the planners that take one.
+static GemmArgs to_args(const Gemm &p) {
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.A = p.A, g.B = p.B, g.C = p.C;
+    g.M = p.M, g.N = p.N, g.K = p.K;
+    g.lda = p.lda, g.ldb = p.ldb, g.ldc = p.ldc;
+    g.sA = p.sA, g.sB = p.sB, g.sC = p.sC;
+    g.beta = p.beta;
+    g.red = (p.sC == 0 && p.batch > 1) ? p.batch : 1;
+    g.batch = g.red > 1 ? 1 : p.batch;
+    g.splits = 1;
+    g.virt = VIRT_NONE;
+    return g;
+}
+
+// A forward product followed by Add (bias[n] onto column n) and ReLu: in the product's own store where the kernel
+// that runs it has one, else the product and one in-place pass over its result.
+static int run_bias_relu(int dtype, const Gemm &p, const void *bias, int relu, void *ws, size_t ws_bytes, void *stream) {
+    if (bias || relu) {
+        GemmArgs g = to_args(p);
+        g.bias = bias, g.relu = relu;
+        if (gemm_fuses_store(dtype, g, p.ta, p.tb)) return gemm_run_fused(dtype, g, p.ta, p.tb, ws, ws_bytes, as_stream(stream));
+    }
+    if (int rc = run(dtype, p, ws, ws_bytes, stream)) return rc;
+    return launch_bias_relu(dtype, p.C, bias, (long)p.M * p.batch, p.N, relu, as_stream(stream));
+}
+
 static int check_mm(const char *who, int dtype, int xb, int xr, int xc, int yb, int yr, int yc) {
     if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
@@ -192,6 +220,14 @@ int d8_matmul(int dtype, const void *x, int xb, int xr, int xc, const void *y, i
     return run(dtype, mm_plan(0, x, xb, xr, xc, y, yb, yr, yc, z), scratch, scratch_bytes, stream);
 }
 
+int d8_matmul_bias_relu(int dtype, const void *x, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
+                        const void *bias, int relu, void *z, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_mm("d8_matmul_bias_relu", dtype, xb, xr, xc, yb, yr, yc)) return rc;
+    if (dtype == D8_FLOAT64) return fail(D8_ERR_DTYPE, "d8_matmul_bias_relu: element type %d is not supported", dtype);
+    D8_REQUIRE(x && y && z, "d8_matmul_bias_relu: null tensor");
+    return run_bias_relu(dtype, mm_plan(0, x, xb, xr, xc, y, yb, yr, yc, z), bias, relu, scratch, scratch_bytes, stream);
+}
+
 int d8_matmul_grad_x(int dtype, void *dx, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
                      const void *dz, void *scratch, size_t scratch_bytes, void *stream) {
     if (int rc = check_mm("d8_matmul_grad_x", dtype, xb, xr, xc, yb, yr, yc)) return rc;
@@ -315,10 +351,10 @@ size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int 
     return plain;
 }
 
-int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
-              const void *w, int OC, int FH, int FW, void *z,
-              int covered, int sy, int sx, int dy, int dx,
-              void *scratch, size_t scratch_bytes, void *stream) {
+static int conv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
+                       const void *w, int OC, int FH, int FW, void *z,
+                       int covered, int sy, int sx, int dy, int dx,
+                       void *scratch, size_t scratch_bytes, void *stream, const void *bias, int relu) {
     int g[4];
     if (int rc = check_conv("d8_conv2d", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return rc;
     if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
@@ -329,8 +365,10 @@ int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
         const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
         GemmArgs ga;
         int ta, tb;
-        if (conv_implicit_plan(dtype, 0, cs, x, w, z, ga, ta, tb))
+        if (conv_implicit_plan(dtype, 0, cs, x, w, z, ga, ta, tb)) {
+            ga.bias = bias, ga.relu = relu;  // applied in the tile store (and in the remainder band's reduction)
             return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+        }
     }
     D8_REQUIRE(scratch, "d8_conv2d: null scratch");
     D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d: scratch too small");
@@ -342,13 +380,28 @@ int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
             if (int rc = launch_im2col(dtype, x, colp, mg, as_stream(stream))) return rc;
             if (int rc = launch_pad_rows(dtype, w, wp, OC, K, pitch, as_stream(stream))) return rc;
             Gemm plan = conv_plan(0, M, pitch, OC, colp, wp, z);  // z = xcol W^T over K = pitch
-            return run(dtype, plan, ws, scratch_bytes - ps.col - ps.filt, stream);
+            return run_bias_relu(dtype, plan, bias, relu, ws, scratch_bytes - ps.col - ps.filt, stream);
         }
     }
     if (int rc = d8_im2col(dtype, x, scratch, B, IH, IW, IC, g[0], g[1], FH, FW, sy, sx, dy, dx, g[2], g[3], stream))
         return rc;
     const size_t ws = scratch_bytes > col ? scratch_bytes - col : 0;
-    return run(dtype, conv_plan(0, M, K, OC, scratch, w, z), ws ? (char *)scratch + col : nullptr, ws, stream);
+    return run_bias_relu(dtype, conv_plan(0, M, K, OC, scratch, w, z), bias, relu, ws ? (char *)scratch + col : nullptr, ws, stream);
+}
+
+int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
+              const void *w, int OC, int FH, int FW, void *z,
+              int covered, int sy, int sx, int dy, int dx,
+              void *scratch, size_t scratch_bytes, void *stream) {
+    return conv2d_impl(dtype, x, B, IH, IW, IC, w, OC, FH, FW, z, covered, sy, sx, dy, dx, scratch, scratch_bytes, stream, nullptr, 0);
+}
+
+int d8_conv2d_bias_relu(int dtype, const void *x, int B, int IH, int IW, int IC,
+                        const void *w, int OC, int FH, int FW, const void *bias, int relu, void *z,
+                        int covered, int sy, int sx, int dy, int dx,
+                        void *scratch, size_t scratch_bytes, void *stream) {
+    if (dtype == D8_FLOAT64) return fail(D8_ERR_DTYPE, "d8_conv2d_bias_relu: element type %d is not supported", dtype);
+    return conv2d_impl(dtype, x, B, IH, IW, IC, w, OC, FH, FW, z, covered, sy, sx, dy, dx, scratch, scratch_bytes, stream, bias, relu);
 }
 
 static int d8_conv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int IC,

@@ -140,6 +140,58 @@ def conv2d(x, w, covered=True, sy=1, sx=1, dy=1, dx=1):
     return dz_.numpy()
 
 
+def conv2d_bias_relu(x, w, bias, relu=True, covered=True, sy=1, sx=1, dy=1, dx=1):
+    """relu?(conv2d(x, w) + bias) from one call (bias: OC values or None)"""
+    lib = capi.init()
+    x, w = np.ascontiguousarray(x), _filt(w)
+    dt = _same_dtype(x, w)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = w.shape
+    OH, OW, _, _ = conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx)
+    dx_, dw_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w)
+    db = DeviceArray.from_numpy(np.ascontiguousarray(bias, dtype=x.dtype).reshape(OC)) if bias is not None else None
+    dz_ = DeviceArray((B, OH, OW, OC), x.dtype)
+    nb = lib.d8_conv2d_scratch_bytes(dt, 0, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx)
+    ws = _scratch(nb)
+    check(lib.d8_conv2d_bias_relu(dt, dx_.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, db.ptr if db else None, int(relu), dz_.ptr,
+                                  int(covered), sy, sx, dy, dx, ws.ptr, nb, None))
+    return dz_.numpy()
+
+
+def matmul_bias_relu(x, y, bias, relu=True):
+    """relu?(matmul(x, y) + bias) from one call (bias: one value per column of the result, or None)"""
+    lib = capi.init()
+    x, y = np.ascontiguousarray(x), np.ascontiguousarray(y)
+    dt = _same_dtype(x, y)
+    zs = matmul_out_shape(x, y)
+    xb, xr, xc = _mat(x)
+    yb, yr, yc = _mat(y)
+    dx_, dy_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray(zs, x.dtype)
+    db = DeviceArray.from_numpy(np.ascontiguousarray(bias, dtype=x.dtype).reshape(zs[-1])) if bias is not None else None
+    nb = lib.d8_matmul_scratch_bytes(dt, 0, xb, xr, xc, yb, yr, yc)
+    ws = _scratch(nb) if nb else None
+    check(lib.d8_matmul_bias_relu(dt, dx_.ptr, xb, xr, xc, dy_.ptr, yb, yr, yc, db.ptr if db else None, int(relu), dz_.ptr,
+                                  ws.ptr if ws else None, nb, None))
+    return dz_.numpy()
+
+
+def bias_relu_grad(z, dz, dbias=None, use_scratch=True, in_place=False):
+    """returns (dpre, dbias): dpre = dz where z > 0 else 0; dbias (+)= column sums of dpre over all leading axes"""
+    lib = capi.init()
+    z, dz = np.ascontiguousarray(z), np.ascontiguousarray(dz)
+    dt = _same_dtype(z, dz)
+    cols = z.shape[-1]
+    rows = z.size // cols
+    dz_, dg_ = DeviceArray.from_numpy(z), DeviceArray.from_numpy(dz)
+    dp_ = dg_ if in_place else DeviceArray(z.shape, z.dtype)
+    acc = dbias is not None
+    db_ = DeviceArray.from_numpy(np.ascontiguousarray(dbias, dtype=z.dtype).reshape(cols)) if acc else DeviceArray.from_numpy(np.full(cols, np.nan, z.dtype))
+    nb = lib.d8_bias_relu_grad_scratch_bytes(dt, rows, cols) if use_scratch else 0
+    ws = _scratch(nb)
+    check(lib.d8_bias_relu_grad(dt, dz_.ptr, dg_.ptr, dp_.ptr, db_.ptr, rows, cols, int(acc), ws.ptr if nb else None, nb, None))
+    return dp_.numpy(), db_.numpy()
+
+
 def conv2d_grad_x(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None, overwrite=False):
     lib = capi.init()
     w, gz = _filt(w), np.ascontiguousarray(gz)

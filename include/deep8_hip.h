@@ -256,6 +256,36 @@ int d8_add_grad_overwrite(int dtype, void *g, const int *gdims, const void *dz, 
                           void *scratch, size_t scratch_bytes, void *stream);
 int d8_relu_grad_overwrite(int dtype, const void *x, void *dx, const void *dy, long n, void *stream);
 
+/* ---- bias and activation folded into the contraction --------------------------------------------------
+ * In a network Add (a per-channel bias broadcast over the rows) and ReLu follow every MatrixMultiply / Conv2d as
+ * passes of their own over the result (Math::AddGPU, deep8/src/math/Add.cu:21-52; Math::ReLuGPU,
+ * deep8/src/math/ReLu.cu:20-59).  These entry points give the result of the three-call sequence from one call:
+ *
+ * d8_matmul_bias_relu   z = relu?(x * y + bias): d8_matmul, then bias[n] added to column n of z (the last axis;
+ *                       bias: that many elements of the tensors' type, or NULL), then ReLu when relu != 0.
+ * d8_conv2d_bias_relu   the same after d8_conv2d (bias: OC elements).
+ *     Both apply bias and ReLu in the store of the product's kernel (before the one rounding to the element type)
+ *     wherever that kernel is one of the tiled ones, and otherwise run the product followed by ONE in-place pass.
+ *     Float32: bit for bit the result of d8_matmul / d8_conv2d, d8_add, d8_relu.  Float16: the fused store rounds
+ *     once instead of three times.  scratch as for d8_matmul / d8_conv2d.  Float64 is rejected.
+ * d8_bias_relu_grad     the way back in one pass over the [rows][cols] gradient of z: dpre = z > 0 ? dz : 0 is
+ *                       written (dpre may be dz), and dbias (cols elements) receives its column sums, added to
+ *                       what it holds when accumulate_bias != 0, else written.  z is the layer's output (it is
+ *                       positive exactly where the pre-activation was).  Replaces Math::ReLuGradGPU
+ *                       (ReLu.cu:61-116) + Math::AddGradYGPU (Add.cu:99-133); the sums are bit for bit those of
+ *                       d8_add_grad on dpre.  scratch (may be NULL): d8_bias_relu_grad_scratch_bytes, 16-byte aligned.
+ *                       dpre then feeds d8_matmul_grad_* / d8_conv2d_grad_* as dz.                                  */
+int d8_matmul_bias_relu(int dtype, const void *x, int xb, int xr, int xc,
+                        const void *y, int yb, int yr, int yc, const void *bias, int relu, void *z,
+                        void *scratch, size_t scratch_bytes, void *stream);
+int d8_conv2d_bias_relu(int dtype, const void *x, int B, int IH, int IW, int IC,
+                        const void *w, int OC, int FH, int FW, const void *bias, int relu, void *z,
+                        int covered, int sy, int sx, int dy, int dx,
+                        void *scratch, size_t scratch_bytes, void *stream);
+size_t d8_bias_relu_grad_scratch_bytes(int dtype, long rows, int cols);
+int d8_bias_relu_grad(int dtype, const void *z, const void *dz, void *dpre, void *dbias, long rows, int cols,
+                      int accumulate_bias, void *scratch, size_t scratch_bytes, void *stream);
+
 /* ---- Minus, L1Norm / L2Norm, ReduceMean, AXPBY ------------------------------------------------
  * What a loss and a trainer step need on top of the operators above.  Shapes as for d8_add.
  * Reductions take an optional two-pass `scratch` (16-byte aligned; size from
