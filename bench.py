@@ -438,13 +438,10 @@ class ConvBiasReluWorkload(ConvWorkload):
 
 
 class DeconvLiteralWorkload:
-    """Benchmark configuration 5 at its literal geometry (28 -> 56, PyTorch's ConvTranspose2d(k=4, s=2, p=1)),
-    which Deep8's DeConv2d does not admit (deep8/src/nodes/DeConv2d.cpp:36-52 allows 58 or 55): kernel level only,
-    through the explicit pads of the gather maps, the route the reference's GPU path takes
-    (deep8/src/math/DeConv2d.cu:251-308, 557-622, 826-891):
-      forward  zmat = X W^T (one GEMM)  ->  d8_deconv_col2im (padTop = padLeft = 2)
-      dX       d8_deconv_im2col(dz)     ->  dX = dzmat W
-      dW       d8_deconv_im2col(dz)     ->  dW = dzmat^T X"""
+    """Benchmark configuration 5 at its literal geometry (28 -> 56, PyTorch's ConvTranspose2d(k=4, s=2, p=1)), which
+    Deep8's DeConv2d does not admit (deep8/src/nodes/DeConv2d.cpp:36-52 allows 58 or 55): the operators' explicit-geometry
+    entry points d8_deconv2d_ex / _grad_x_ex / _grad_y_ex with OH = OW = 56, padTop = padLeft = 2 -- the same three
+    launches as the operator at Deep8's own geometries (workload c5)."""
 
     def __init__(self, name, seed):
         from deep8_amd import capi
@@ -453,48 +450,52 @@ class DeconvLiteralWorkload:
         self.dt = capi.dtype_id(self.dtype)
         r = np.random.default_rng(seed)
         B, IH, IC, OC, F, S, OH, P = 16, 28, 128, 64, 4, 2, 56, 2
-        self.B, self.geo = B, (B, IH, IH, OH, OH, OC, F, F, S, S, P, P)
-        self.M, self.N, self.K = B * IH * IH, OC * F * F, IC
+        self.B = B
+        self.shape = (B, IH, IH, IC)
+        self.filt = (OC, F, F)
+        self.geo = (OH, OH, P, P, S, S)
         h = lambda a: _dev(a.astype(np.float32).astype(np.float16))
-        self.x = h(r.standard_normal((self.M, IC)))
-        self.w = h(r.standard_normal((self.N, IC)) * np.sqrt(2.0 / (F * F * IC)))
+        self.x = h(r.standard_normal((B, IH, IH, IC)))
+        self.w = h(r.standard_normal((OC, F, F, IC)) * np.sqrt(2.0 / (F * F * IC)))
         self.dz = h(r.standard_normal((B, OH, OH, OC)))
-        self.zmat = capi.DeviceArray((self.M, self.N), np.float16)
         self.z = capi.DeviceArray((B, OH, OH, OC), np.float16)
-        self.dx = capi.DeviceArray((self.M, IC), np.float16)
-        self.dw = capi.DeviceArray((self.N, IC), np.float16)
-        self.ws_bytes = max(self.lib.d8_gemm_workspace_bytes(self.dt, ta, tb, m, n, k, 1, 0) for ta, tb, m, n, k in
-                            ((0, 1, self.M, self.N, self.K), (0, 0, self.M, self.K, self.N), (1, 0, self.N, self.K, self.M)))
+        self.dx = capi.DeviceArray((B, IH, IH, IC), np.float16)
+        self.dw = capi.DeviceArray((OC, F, F, IC), np.float16)
+        self.ws_bytes = max(self.lib.d8_deconv2d_scratch_bytes_ex(self.dt, wch, *self.shape, *self.filt, OH, OH, P, P, S, S) for wch in range(3))
         self.ws = capi.DeviceArray((max(self.ws_bytes, 16),), np.uint8)
-        self.flops = 3 * 2.0 * self.M * self.N * self.K
-        nx, nw, nz, nm = self.M * IC, self.N * IC, B * OH * OH * OC, self.M * self.N
-        # GEMM operands and results once, the interim matrix written and read once per pass
-        self.bytes = 2 * ((nx + nw + 2 * nm + nz) + (nz + 2 * nm + nw + nx) + (nz + 2 * nm + nx + nw))
-
-    def _gemm(self, ta, tb, m, n, k, a, lda, b, ldb, c, ldc):
-        from deep8_amd.capi import check
-        check(self.lib.d8_gemm(self.dt, ta, tb, m, n, k, a.ptr, lda, 0, b.ptr, ldb, 0, 0.0, c.ptr, ldc, 0, 1,
-                               self.ws.ptr, self.ws_bytes, None))
+        M, N = B * IH * IH, OC * F * F
+        self.flops = 3 * 2.0 * M * N * IC
+        nx, nw, nz = M * IC, N * IC, B * OH * OH * OC
+        self.bytes = 2 * ((nx + nw + nz) + (nz + nw + nx) + (nx + nz + nw))  # overwrite forms: each pass reads two tensors, writes one
 
     def fwd(self):
         from deep8_amd.capi import check
-        self._gemm(0, 1, self.M, self.N, self.K, self.x, self.K, self.w, self.K, self.zmat, self.N)
-        check(self.lib.d8_deconv_col2im(self.dt, self.zmat.ptr, self.z.ptr, *self.geo, None))
+        check(self.lib.d8_deconv2d_ex(self.dt, self.x.ptr, *self.shape, self.w.ptr, *self.filt, self.z.ptr, *self.geo,
+                                      self.ws.ptr, self.ws_bytes, None))
 
     def grad_x(self):
         from deep8_amd.capi import check
-        check(self.lib.d8_deconv_im2col(self.dt, self.dz.ptr, self.zmat.ptr, *self.geo, None))
-        self._gemm(0, 0, self.M, self.K, self.N, self.zmat, self.N, self.w, self.K, self.dx, self.K)
+        check(self.lib.d8_deconv2d_grad_x_ex(self.dt, self.dx.ptr, *self.shape, self.w.ptr, *self.filt, self.dz.ptr, *self.geo,
+                                             0 if EAGER_ZERO else 1, self.ws.ptr, self.ws_bytes, None))
 
     def grad_y(self):
         from deep8_amd.capi import check
-        check(self.lib.d8_deconv_im2col(self.dt, self.dz.ptr, self.zmat.ptr, *self.geo, None))
-        self._gemm(1, 0, self.N, self.K, self.M, self.zmat, self.N, self.x, self.K, self.dw, self.K)
+        check(self.lib.d8_deconv2d_grad_y_ex(self.dt, self.x.ptr, *self.shape, self.dw.ptr, *self.filt, self.dz.ptr, *self.geo,
+                                             0 if EAGER_ZERO else 1, self.ws.ptr, self.ws_bytes, None))
 
     def step(self):
         self.fwd()
+        if EAGER_ZERO:
+            self.dx.zero_()
+            self.dw.zero_()
         self.grad_x()
         self.grad_y()
+
+    kernel = "gemm_tiled_kernel<f16> (one launch each for forward, dX, dW; patch rows read by the tile loader)"
+
+    def parts(self):
+        f = self.flops / 3
+        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
 
 
 class GatherMapsWorkload:
@@ -689,8 +690,8 @@ def make_workload(key):
         return ConvWorkload("c5: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 58x58x64 (Deep8 covered=false)",
                             np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
     if key == "c5l":
-        return DeconvLiteralWorkload("c5l: DeConv2d half B16 28x28x128 4x4 s2 -> 56x56x64 (the literal geometry of configuration 5; "
-                                     "kernel level: GEMM + gather maps with explicit pads)", 9)
+        return DeconvLiteralWorkload("c5l: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 56x56x64 (configuration 5 as written, "
+                                     "through the explicit-geometry operator entry points)", 9)
     if key == "d3":
         return MatMulWorkload("d3: MatrixMultiply fwd+dX+dY double [2048x2048]x[2048x2048]", np.float64,
                               (1, 2048, 2048), (1, 2048, 2048), U, 10)

@@ -58,6 +58,10 @@ SIGNATURES = {
     "d8_matmul": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_x": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_y": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "d8_deconv2d_scratch_bytes_ex": (_Z, [_I] * 15),
+    "d8_deconv2d_ex": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P] + [_I] * 6 + [_P, _Z, _P]),
+    "d8_deconv2d_grad_x_ex": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P] + [_I] * 7 + [_P, _Z, _P]),
+    "d8_deconv2d_grad_y_ex": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P] + [_I] * 7 + [_P, _Z, _P]),
     "d8_matmul_bias_relu": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _P, _Z, _P]),
     "d8_conv2d_bias_relu": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P] + [_I] * 5 + [_P, _Z, _P]),
     "d8_bias_relu_grad_scratch_bytes": (_Z, [_I, _L, _I]),

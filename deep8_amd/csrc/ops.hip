@@ -590,11 +590,14 @@ static bool deconv_implicit_grad_y(int dtype, int B, int IH, int IW, int IC, int
     return gemm_tiled_eligible(dtype, g, 1, 0);
 }
 
-size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
-                                 int OC, int FH, int FW, int covered, int sy, int sx) {
-    int geo[4];
-    if (check_conv("d8_deconv2d_scratch_bytes", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return 0;
-    if (d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, geo)) return 0;
+// geo = {OH, OW, padTop, padLeft}: Deep8's own (from `covered`) or the caller's (the _ex entry points)
+static int check_deconv_geo(const char *who, const int *geo) {
+    D8_REQUIRE(geo[0] > 0 && geo[1] > 0 && geo[2] >= 0 && geo[3] >= 0, "%s: output %d x %d, pads %d / %d", who, geo[0], geo[1], geo[2], geo[3]);
+    return 0;
+}
+
+static size_t deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
+                                     int OC, int FH, int FW, const int *geo, int sy, int sx) {
     const int M = B * IH * IW, T = FH * FW;
     GemmArgs ga;
     if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
@@ -606,13 +609,25 @@ size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, in
     return mat + gemm_ws(dtype, deconv_plan(which, M, T, OC, IC, nullptr, nullptr, nullptr));
 }
 
-int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
-                const void *w, int OC, int FH, int FW, void *z,
-                int covered, int sy, int sx,
-                void *scratch, size_t scratch_bytes, void *stream) {
-    int g[4];
-    if (int rc = check_conv("d8_deconv2d", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
-    if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+size_t d8_deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
+                                 int OC, int FH, int FW, int covered, int sy, int sx) {
+    int geo[4];
+    if (check_conv("d8_deconv2d_scratch_bytes", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return 0;
+    if (d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, geo)) return 0;
+    return deconv2d_scratch_bytes(dtype, which, B, IH, IW, IC, OC, FH, FW, geo, sy, sx);
+}
+
+size_t d8_deconv2d_scratch_bytes_ex(int dtype, int which, int B, int IH, int IW, int IC,
+                                    int OC, int FH, int FW, int OH, int OW, int padTop, int padLeft, int sy, int sx) {
+    const int geo[4] = {OH, OW, padTop, padLeft};
+    if (check_conv("d8_deconv2d_scratch_bytes_ex", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return 0;
+    if (check_deconv_geo("d8_deconv2d_scratch_bytes_ex", geo)) return 0;
+    return deconv2d_scratch_bytes(dtype, which, B, IH, IW, IC, OC, FH, FW, geo, sy, sx);
+}
+
+static int deconv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
+                         const void *w, int OC, int FH, int FW, void *z, const int *g, int sy, int sx,
+                         void *scratch, size_t scratch_bytes, void *stream) {
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(x && w && z, "d8_deconv2d: null tensor");
@@ -629,13 +644,30 @@ int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
     return launch_col2im(dtype, scratch, z, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), false, as_stream(stream));
 }
 
-static int d8_deconv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int IC,
-                       const void *w, int OC, int FH, int FW, const void *gz,
-                       int covered, int sy, int sx,
-                       void *scratch, size_t scratch_bytes, void *stream, float beta) {
+int d8_deconv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
+                const void *w, int OC, int FH, int FW, void *z,
+                int covered, int sy, int sx,
+                void *scratch, size_t scratch_bytes, void *stream) {
     int g[4];
-    if (int rc = check_conv("d8_deconv2d_grad_x", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = check_conv("d8_deconv2d", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+    return deconv2d_impl(dtype, x, B, IH, IW, IC, w, OC, FH, FW, z, g, sy, sx, scratch, scratch_bytes, stream);
+}
+
+int d8_deconv2d_ex(int dtype, const void *x, int B, int IH, int IW, int IC,
+                   const void *w, int OC, int FH, int FW, void *z,
+                   int OH, int OW, int padTop, int padLeft, int sy, int sx,
+                   void *scratch, size_t scratch_bytes, void *stream) {
+    const int g[4] = {OH, OW, padTop, padLeft};
+    if (int rc = check_conv("d8_deconv2d_ex", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = check_deconv_geo("d8_deconv2d_ex", g)) return rc;
+    return deconv2d_impl(dtype, x, B, IH, IW, IC, w, OC, FH, FW, z, g, sy, sx, scratch, scratch_bytes, stream);
+}
+
+static int deconv2d_grad_x_geo(int dtype, void *gx, int B, int IH, int IW, int IC,
+                       const void *w, int OC, int FH, int FW, const void *gz,
+                       const int *g, int sy, int sx,
+                       void *scratch, size_t scratch_bytes, void *stream, float beta) {
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(gx && w && gz, "d8_deconv2d_grad_x: null tensor");
@@ -656,13 +688,30 @@ static int d8_deconv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, i
     return run(dtype, plan, ws ? (char *)scratch + mat : nullptr, ws, stream);
 }
 
-static int d8_deconv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
-                       void *gw, int OC, int FH, int FW, const void *gz,
+static int d8_deconv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int IC,
+                       const void *w, int OC, int FH, int FW, const void *gz,
                        int covered, int sy, int sx,
                        void *scratch, size_t scratch_bytes, void *stream, float beta) {
     int g[4];
-    if (int rc = check_conv("d8_deconv2d_grad_y", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = check_conv("d8_deconv2d_grad_x", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
     if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+    return deconv2d_grad_x_geo(dtype, gx, B, IH, IW, IC, w, OC, FH, FW, gz, g, sy, sx, scratch, scratch_bytes, stream, beta);
+}
+
+int d8_deconv2d_grad_x_ex(int dtype, void *gx, int B, int IH, int IW, int IC,
+                          const void *w, int OC, int FH, int FW, const void *gz,
+                          int OH, int OW, int padTop, int padLeft, int sy, int sx, int overwrite,
+                          void *scratch, size_t scratch_bytes, void *stream) {
+    const int g[4] = {OH, OW, padTop, padLeft};
+    if (int rc = check_conv("d8_deconv2d_grad_x_ex", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = check_deconv_geo("d8_deconv2d_grad_x_ex", g)) return rc;
+    return deconv2d_grad_x_geo(dtype, gx, B, IH, IW, IC, w, OC, FH, FW, gz, g, sy, sx, scratch, scratch_bytes, stream, overwrite ? 0.f : 1.f);
+}
+
+static int deconv2d_grad_y_geo(int dtype, const void *x, int B, int IH, int IW, int IC,
+                       void *gw, int OC, int FH, int FW, const void *gz,
+                       const int *g, int sy, int sx,
+                       void *scratch, size_t scratch_bytes, void *stream, float beta) {
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(x && gw && gz, "d8_deconv2d_grad_y: null tensor");
@@ -681,6 +730,26 @@ static int d8_deconv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int 
     Gemm plan = deconv_plan(2, M, T, OC, IC, scratch, gw, x);
     plan.beta = beta;
     return run(dtype, plan, ws ? (char *)scratch + mat : nullptr, ws, stream);
+}
+
+static int d8_deconv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
+                       void *gw, int OC, int FH, int FW, const void *gz,
+                       int covered, int sy, int sx,
+                       void *scratch, size_t scratch_bytes, void *stream, float beta) {
+    int g[4];
+    if (int rc = check_conv("d8_deconv2d_grad_y", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+    return deconv2d_grad_y_geo(dtype, x, B, IH, IW, IC, gw, OC, FH, FW, gz, g, sy, sx, scratch, scratch_bytes, stream, beta);
+}
+
+int d8_deconv2d_grad_y_ex(int dtype, const void *x, int B, int IH, int IW, int IC,
+                          void *gw, int OC, int FH, int FW, const void *gz,
+                          int OH, int OW, int padTop, int padLeft, int sy, int sx, int overwrite,
+                          void *scratch, size_t scratch_bytes, void *stream) {
+    const int g[4] = {OH, OW, padTop, padLeft};
+    if (int rc = check_conv("d8_deconv2d_grad_y_ex", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = check_deconv_geo("d8_deconv2d_grad_y_ex", g)) return rc;
+    return deconv2d_grad_y_geo(dtype, x, B, IH, IW, IC, gw, OC, FH, FW, gz, g, sy, sx, scratch, scratch_bytes, stream, overwrite ? 0.f : 1.f);
 }
 
 #define D8_CONV_GRAD_PAIR(name, first, grad)                                                                      \

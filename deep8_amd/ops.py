@@ -270,6 +270,34 @@ def deconv2d_grad_y(x, w, gz, covered=False, sy=1, sx=1, gw=None, overwrite=Fals
 
 
 # ---- the four maps ---------------------------------------------------------------------------------------
+def deconv2d_ex(which, x, w, gz, OH, OW, padTop, padLeft, sy, sx, acc=None, overwrite=False):
+    """DeConv2d at an explicit geometry: which 0 forward (gz unused), 1 gradient of x, 2 gradient of w; gradients are
+    added to `acc` (zeros by default) unless overwrite"""
+    lib = capi.init()
+    x, w = np.ascontiguousarray(x), _filt(w)
+    dt = _same_dtype(x, w)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = w.shape
+    nb = lib.d8_deconv2d_scratch_bytes_ex(dt, which, B, IH, IW, IC, OC, FH, FW, OH, OW, padTop, padLeft, sy, sx)
+    ws = _scratch(nb)
+    dx_, dw_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w)
+    if which == 0:
+        dz_ = DeviceArray((B, OH, OW, OC), x.dtype)
+        check(lib.d8_deconv2d_ex(dt, dx_.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dz_.ptr, OH, OW, padTop, padLeft, sy, sx,
+                                 ws.ptr, nb, None))
+        return dz_.numpy()
+    dgz = DeviceArray.from_numpy(np.ascontiguousarray(gz))
+    like = x if which == 1 else w
+    out = DeviceArray.from_numpy(np.zeros_like(like) if acc is None else np.ascontiguousarray(acc, dtype=like.dtype))
+    if which == 1:
+        check(lib.d8_deconv2d_grad_x_ex(dt, out.ptr, B, IH, IW, IC, dw_.ptr, OC, FH, FW, dgz.ptr, OH, OW, padTop, padLeft, sy, sx,
+                                        int(overwrite), ws.ptr, nb, None))
+    else:
+        check(lib.d8_deconv2d_grad_y_ex(dt, dx_.ptr, B, IH, IW, IC, out.ptr, OC, FH, FW, dgz.ptr, OH, OW, padTop, padLeft, sy, sx,
+                                        int(overwrite), ws.ptr, nb, None))
+    return out.numpy()
+
+
 def im2col(im, OH, OW, FH, FW, sy, sx, dy, dx, padTop, padLeft):
     lib = capi.init()
     im = np.ascontiguousarray(im)

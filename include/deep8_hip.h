@@ -209,6 +209,28 @@ int d8_deconv2d_grad_y(int dtype, const void *x, int B, int IH, int IW, int IC,
                        int covered, int sy, int sx,
                        void *scratch, size_t scratch_bytes, void *stream);
 
+/* DeConv2d with the geometry given outright instead of derived from `covered`: the output is OH x OW and
+ * z[b,oy,ox,:] sums the taps (fy,fx) with iy*sy == oy - padTop + fy, ix*sx == ox - padLeft + fx inside the input
+ * (padTop, padLeft >= 0: the pads of the stride-1 correlation over the zero-inflated input, as returned by
+ * d8_deconv2d_geometry).  Math::DeConv2d admits only two output sizes per input (deep8/src/nodes/DeConv2d.cpp:36-52,
+ * pads deep8/src/math/DeConv2d.cpp:295-301); these entry points run the same kernels on any other, e.g. PyTorch's
+ * ConvTranspose2d(k, s, p) = OH (IH-1)*s + k - 2p, padTop = k - 1 - p.  The gradients accumulate unless
+ * overwrite != 0.  scratch from d8_deconv2d_scratch_bytes_ex.                                                  */
+size_t d8_deconv2d_scratch_bytes_ex(int dtype, int which, int B, int IH, int IW, int IC,
+                                    int OC, int FH, int FW, int OH, int OW, int padTop, int padLeft, int sy, int sx);
+int d8_deconv2d_ex(int dtype, const void *x, int B, int IH, int IW, int IC,
+                   const void *w, int OC, int FH, int FW, void *z,
+                   int OH, int OW, int padTop, int padLeft, int sy, int sx,
+                   void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_x_ex(int dtype, void *gx, int B, int IH, int IW, int IC,
+                          const void *w, int OC, int FH, int FW, const void *gz,
+                          int OH, int OW, int padTop, int padLeft, int sy, int sx, int overwrite,
+                          void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_y_ex(int dtype, const void *x, int B, int IH, int IW, int IC,
+                          void *gw, int OC, int FH, int FW, const void *gz,
+                          int OH, int OW, int padTop, int padLeft, int sy, int sx, int overwrite,
+                          void *scratch, size_t scratch_bytes, void *stream);
+
 /* Overwrite forms of the four convolution gradients: the destination's old contents are ignored
  * (what "zero the gradient, then accumulate" leaves, without the fill and the read-back).      */
 int d8_conv2d_grad_x_overwrite(int dtype, void *gx, int B, int IH, int IW, int IC,

@@ -501,3 +501,76 @@ def test_conv2d_first_layers_padded_patch_rows(oracle_port, cfg, dtype):
     assert rel_fro(f(ops.conv2d(xr, wr, *a)), oracle_port.conv2d(f(xr), f(wr), *a)) <= tol
     assert rel_fro(f(ops.conv2d_grad_x(xr, wr, gzr, *a)), oracle_port.conv2d_grad_x(f(xr), f(wr), f(gzr), *a)) <= tol
     assert rel_fro(f(ops.conv2d_grad_y(xr, wr, gzr, *a)), oracle_port.conv2d_grad_y(f(xr), f(wr), f(gzr), *a)) <= tol
+
+
+# ---- DeConv2d at an explicit geometry (d8_deconv2d*_ex) ------------------------------------------------------------
+def _torch_deconv(x, w, gz, S, P, OH):
+    """torch's conv_transpose2d and its autograd gradients in Deep8's layout and filter convention (flipped kernel,
+    padding = F - 1 - padTop), float64"""
+    import torch
+    F = w.shape[1]
+    tx = torch.tensor(f(x), dtype=torch.float64).permute(0, 3, 1, 2).clone().requires_grad_(True)
+    tw = torch.tensor(f(w), dtype=torch.float64).requires_grad_(True)
+    wt = torch.flip(tw, (1, 2)).permute(3, 0, 1, 2)
+    tz = torch.nn.functional.conv_transpose2d(tx, wt, stride=S, padding=F - 1 - P)
+    assert tuple(tz.shape[2:]) == (OH, OH)
+    tz.backward(torch.tensor(f(gz), dtype=torch.float64).permute(0, 3, 1, 2))
+    return tz.detach().permute(0, 2, 3, 1).numpy(), tx.grad.permute(0, 2, 3, 1).numpy(), tw.grad.numpy()
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_config5_as_written_at_operator_level(dtype):
+    """Benchmark configuration 5 literally: B16 28x28x128 -> 56x56x64, 4x4, stride 2, PyTorch's pad 1 (padTop = 2 here),
+    forward and both gradients through d8_deconv2d*_ex at full size, against torch's conv_transpose2d in float64."""
+    pytest.importorskip("torch")
+    from deep8_amd import ops
+    r = rng(556)
+    B, IH, IC, OC, F, S, OH, P = 16, 28, 128, 64, 4, 2, 56, 2
+    c = (lambda a: h(a)) if dtype == np.float16 else (lambda a: a)
+    tol = FP16_TOL if dtype == np.float16 else FP32_TOL
+    x, w = c(nrm(r, (B, IH, IH, IC))), c(nrm(r, (OC, F, F, IC), np.sqrt(2.0 / 2048)))
+    gz = c(nrm(r, (B, OH, OH, OC)))
+    tz, tgx, tgw = _torch_deconv(x, w, gz, S, P, OH)
+    z = ops.deconv2d_ex(0, x, w, None, OH, OH, P, P, S, S)
+    assert z.shape == (B, OH, OH, OC) and rel_fro(f(z), tz) <= tol
+    assert rel_fro(f(ops.deconv2d_ex(1, x, w, gz, OH, OH, P, P, S, S)), tgx) <= tol
+    assert rel_fro(f(ops.deconv2d_ex(2, x, w, gz, OH, OH, P, P, S, S)), tgw) <= tol
+    # accumulate and overwrite forms
+    junk = c(nrm(r, x.shape))
+    got = ops.deconv2d_ex(1, x, w, gz, OH, OH, P, P, S, S, acc=junk, overwrite=True)
+    assert rel_fro(f(got), tgx) <= tol
+    got = ops.deconv2d_ex(1, x, w, gz, OH, OH, P, P, S, S, acc=junk)
+    assert rel_fro(f(got), tgx + f(junk)) <= tol
+
+
+@pytest.mark.parametrize("cfg", [
+    # B, IH, IC, OC, F, S, OH, P  (square; OH and P free)
+    (2, 7, 16, 8, 4, 2, 14, 2),     # k4 s2 p1 at a size that takes the im2col / col2im route
+    (2, 6, 64, 64, 3, 2, 12, 1),    # ConvTranspose2d(k3, s2, p1, output_padding 1): OH = 2 IH
+    (1, 5, 3, 2, 5, 3, 13, 3),
+    (2, 9, 64, 64, 4, 2, 18, 2),    # implicit route
+    (3, 8, 32, 64, 2, 2, 16, 1),    # filter = stride: no overlaps (p0 -> padTop = k - 1)
+])
+def test_deconv2d_ex_integer_exact(oracle_port, cfg):
+    """Small explicit geometries, integers, bit for bit against the kernel-level route through the oracle:
+    zmat = X W^T, then the oracle's deconv_col2im with the same pads; gradients via the oracle's deconv_im2col."""
+    from deep8_amd import ops
+    B, IH, IC, OC, F, S, OH, P = cfg
+    r = rng(sum(cfg))
+    x, w = ints(r, (B, IH, IH, IC), 4), ints(r, (OC, F, F, IC), 4)
+    gz = ints(r, (B, OH, OH, OC), 4)
+    zmat = x.reshape(-1, IC) @ w.reshape(OC * F * F, IC).T
+    want_z = oracle_port.deconv_col2im(zmat, B, IH, IH, OH, OH, OC, F, F, S, S, P, P)
+    dzmat = oracle_port.deconv_im2col(gz, IH, IH, F, F, S, S, P, P)
+    want_gx = (dzmat @ w.reshape(OC * F * F, IC)).reshape(x.shape)
+    want_gw = (dzmat.T @ x.reshape(-1, IC)).reshape(w.shape)
+    for dtype in (np.float32, np.float16):
+        if dtype == np.float16 and max(np.abs(want_z).max(), np.abs(want_gx).max(), np.abs(want_gw).max()) >= 2048:
+            continue
+        c = lambda a: a.astype(dtype)
+        assert np.array_equal(f(ops.deconv2d_ex(0, c(x), c(w), None, OH, OH, P, P, S, S)), want_z)
+        assert np.array_equal(f(ops.deconv2d_ex(1, c(x), c(w), c(gz), OH, OH, P, P, S, S)), want_gx)
+        assert np.array_equal(f(ops.deconv2d_ex(2, c(x), c(w), c(gz), OH, OH, P, P, S, S)), want_gw)
+    # Deep8's own geometry through the _ex entry points is the operator itself
+    OHd, OWd, pt, pl = ops.deconv2d_geometry(IH, IH, F, F, False, S, S)
+    assert np.array_equal(ops.deconv2d_ex(0, x, w, None, OHd, OWd, pt, pl, S, S), ops.deconv2d(x, w, False, S, S))
