@@ -34,7 +34,17 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(GemmArgs g) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    // Which tile: workgroups are dispatched x-fastest and ids congruent mod 8 share an XCD (and its L2).  Each XCD
+    // takes a contiguous run of tiles laid out in bands of 4 tile rows walked column by column, so the A and B
+    // panels it re-reads are few (2048^2: 4 + 8 panels per XCD instead of 2 + 16).
+    const int tilesM = gridDim.x, tilesN = gridDim.y, total = tilesM * tilesN;
+    int id = blockIdx.x + tilesM * blockIdx.y;
+    if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    constexpr int GM = 4;
+    const int band = id / (GM * tilesN), first = band * GM;
+    const int rows_in_band = min(GM, tilesM - first);
+    const int in_band = id - band * GM * tilesN;
+    const int m0 = (first + in_band % rows_in_band) * BM, n0 = (in_band / rows_in_band) * BN;
     const int b = blockIdx.z / g.splits, piece = blockIdx.z - b * g.splits;
 
     const int ktiles = (g.K + BK - 1) / BK;

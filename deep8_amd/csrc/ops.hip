@@ -64,6 +64,16 @@ static int run_bias_relu(int dtype, const Gemm &p, const void *bias, int relu, v
     return launch_bias_relu(dtype, p.C, bias, (long)p.M * p.batch, p.N, relu, as_stream(stream));
 }
 
+// The staged (im2col / col2im) route needs its interim matrix.  The size query plans with aligned tensors, so a
+// tensor that is not 16-byte aligned (a view at an odd offset) can land here with a scratch sized for the route
+// that stages nothing: the message says so.
+static int need_scratch(const char *who, const void *scratch, size_t have, size_t need, const void *a, const void *b, const void *c) {
+    if (scratch && have >= need) return 0;
+    const bool odd = (((size_t)a | (size_t)b | (size_t)c) & 15) != 0;
+    return fail(D8_ERR_ARGUMENT, "%s: the interim matrix needs %zu bytes of scratch, %zu given%s", who, need, scratch ? have : (size_t)0,
+                odd ? " (a tensor is not 16-byte aligned: it cannot be read by the tile loader, which the size query assumed)" : "");
+}
+
 static int check_mm(const char *who, int dtype, int xb, int xr, int xc, int yb, int yr, int yc) {
     if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
@@ -370,8 +380,7 @@ static int conv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
             return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
         }
     }
-    D8_REQUIRE(scratch, "d8_conv2d: null scratch");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d: scratch too small");
+    if (int rc = need_scratch("d8_conv2d", scratch, scratch_bytes, (size_t)M * K * dtype_bytes(dtype), x, w, z)) return rc;
     if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
         const PaddedScratch ps = conv_padded_scratch(dtype, 0, M, OC, pitch);
         if (scratch_bytes >= ps.total && ((size_t)scratch & 15) == 0) {  // a smaller scratch still serves the plain route
@@ -427,8 +436,7 @@ static int d8_conv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int
             return gemm_tiled_launch(dtype, ga, 0, 0, as_stream(stream));
         }
     }
-    D8_REQUIRE(scratch, "d8_conv2d_grad_x: null scratch");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_x: scratch too small");
+    if (int rc = need_scratch("d8_conv2d_grad_x", scratch, scratch_bytes, (size_t)M * K * dtype_bytes(dtype), gx, w, gz)) return rc;
     if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
         const PaddedScratch ps = conv_padded_scratch(dtype, 1, M, OC, pitch);
         if (scratch_bytes >= ps.total && ((size_t)scratch & 15) == 0) {
@@ -469,8 +477,7 @@ static int d8_conv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int IW
             return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
         }
     }
-    D8_REQUIRE(scratch, "d8_conv2d_grad_y: null scratch");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * K * dtype_bytes(dtype), "d8_conv2d_grad_y: scratch too small");
+    if (int rc = need_scratch("d8_conv2d_grad_y", scratch, scratch_bytes, (size_t)M * K * dtype_bytes(dtype), x, gw, gz)) return rc;
     if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
         const PaddedScratch ps = conv_padded_scratch(dtype, 2, M, OC, pitch);
         if (scratch_bytes >= ps.total && ((size_t)scratch & 15) == 0) {
@@ -636,8 +643,7 @@ static int deconv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC
         if (deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, w, z, ga))
             return gemm_tiled_launch(dtype, ga, 0, 1, as_stream(stream));
     }
-    D8_REQUIRE(scratch, "d8_deconv2d: null scratch");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d: scratch too small");
+    if (int rc = need_scratch("d8_deconv2d", scratch, scratch_bytes, (size_t)M * T * OC * dtype_bytes(dtype), x, w, z)) return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
     if (int rc = run(dtype, deconv_plan(0, M, T, OC, IC, scratch, w, x), ws ? (char *)scratch + mat : nullptr, ws, stream))
         return rc;
@@ -678,8 +684,7 @@ static int deconv2d_grad_x_geo(int dtype, void *gx, int B, int IH, int IW, int I
             return gemm_tiled_run(dtype, ga, 0, 0, scratch, scratch_bytes, as_stream(stream));
         }
     }
-    D8_REQUIRE(scratch, "d8_deconv2d_grad_x: null scratch");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d_grad_x: scratch too small");
+    if (int rc = need_scratch("d8_deconv2d_grad_x", scratch, scratch_bytes, (size_t)M * T * OC * dtype_bytes(dtype), gx, w, gz)) return rc;
     if (int rc = launch_im2col(dtype, gz, scratch, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), as_stream(stream)))
         return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
@@ -722,8 +727,7 @@ static int deconv2d_grad_y_geo(int dtype, const void *x, int B, int IH, int IW, 
             return gemm_tiled_run(dtype, ga, 1, 0, scratch, scratch_bytes, as_stream(stream));
         }
     }
-    D8_REQUIRE(scratch, "d8_deconv2d_grad_y: null scratch");
-    D8_REQUIRE(scratch_bytes >= (size_t)M * T * OC * dtype_bytes(dtype), "d8_deconv2d_grad_y: scratch too small");
+    if (int rc = need_scratch("d8_deconv2d_grad_y", scratch, scratch_bytes, (size_t)M * T * OC * dtype_bytes(dtype), x, gw, gz)) return rc;
     if (int rc = launch_im2col(dtype, gz, scratch, deconv_mirror(B, IH, IW, OC, FH, FW, sy, sx, g), as_stream(stream)))
         return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;

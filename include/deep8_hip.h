@@ -138,7 +138,11 @@ int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
  * function, which already includes any split-reduction workspace).  Where that function
  * returns 0 the operator stages nothing (its patch matrix is read by the GEMM's tile loader)
  * and `scratch` may be NULL; a scratch smaller than asked for is an error only when the
- * operator has to stage.                                                                     */
+ * operator has to stage.  The size functions assume tensors that are 16-byte aligned (every
+ * allocation of d8_malloc and of Deep8's pools is): a Conv2d / DeConv2d tensor at an address that
+ * is not can only take the staged route, whose interim matrix is sizeof(T)*B*OH*OW*FH*FW*IC
+ * (Conv2d) or sizeof(T)*B*IH*IW*OC*FH*FW (DeConv2d) bytes plus d8_gemm_workspace_bytes; with
+ * less the call fails with D8_ERR_ARGUMENT and says so.                                       */
 size_t d8_matmul_scratch_bytes(int dtype, int which /*0 fwd, 1 gradX, 2 gradY*/,
                                int xb, int xr, int xc, int yb, int yr, int yc);
 int d8_matmul(int dtype, const void *x, int xb, int xr, int xc,

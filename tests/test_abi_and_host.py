@@ -57,3 +57,16 @@ def test_host_layer_device_free_tests():
 def test_bench_refuses_more_than_one_gpu():
     out = subprocess.run(["python", os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert out.returncode != 0 and "ONE GPU" in out.stderr
+
+
+def test_cpu_pieces_run_clean_under_the_sanitizers():
+    """The oracle's C restatement and the host layer's device-free tests under AddressSanitizer +
+    UndefinedBehaviorSanitizer (`make asan` in oracle/ and deep8_amd/host/): any report aborts the run."""
+    import shutil
+    import subprocess
+    if not shutil.which("make") or not shutil.which("gcc") or not shutil.which("g++"):
+        pytest.skip("no host toolchain")
+    for where in ("oracle", os.path.join("deep8_amd", "host")):
+        r = subprocess.run(["make", "-s", "-C", os.path.join(ROOT, where), "asan"], capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0, (where, r.stdout[-2000:], r.stderr[-2000:])
+        assert "runtime error" not in r.stderr and "AddressSanitizer" not in r.stderr, (where, r.stderr[-2000:])

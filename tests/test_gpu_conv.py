@@ -574,3 +574,35 @@ def test_deconv2d_ex_integer_exact(oracle_port, cfg):
     # Deep8's own geometry through the _ex entry points is the operator itself
     OHd, OWd, pt, pl = ops.deconv2d_geometry(IH, IH, F, F, False, S, S)
     assert np.array_equal(ops.deconv2d_ex(0, x, w, None, OHd, OWd, pt, pl, S, S), ops.deconv2d(x, w, False, S, S))
+
+
+def test_conv2d_tensor_view_at_an_odd_offset(oracle_port):
+    """A tensor that is not 16-byte aligned cannot be read by the tile loader: the operator takes the staged route.
+    With the staged route's scratch the result is the same; with the scratch the size query names (it plans for
+    aligned tensors) the call fails and says why."""
+    from deep8_amd import capi
+    from deep8_amd.capi import DeviceArray, check
+    lib = capi.init()
+    r = rng(77)
+    B, IH, IC, OC, F = 2, 12, 64, 64, 3
+    x, w = ints(r, (B, IH, IH, IC), 5), ints(r, (OC, F, F, IC), 5)
+    gz = ints(r, (B, IH, IH, OC), 5)
+    want = (oracle_port.conv2d(x, w), oracle_port.conv2d_grad_x(x, w, gz), oracle_port.conv2d_grad_y(x, w, gz))
+    args = (1, 1, 1, 1, 1)
+    asked = lib.d8_conv2d_scratch_bytes(capi.FLOAT32, 0, B, IH, IH, IC, OC, F, F, *args)
+    assert asked < 4 * B * IH * IH * F * F * IC           # the query plans for the route that stages nothing
+    small = DeviceArray((max(asked, 16),), np.uint8)
+    raw = DeviceArray((x.size + 1,), np.float32)          # x lives 4 bytes into this allocation
+    check(lib.d8_memcpy_h2d(raw.ptr + 4, x.ctypes.data, x.nbytes))
+    dw, dgz = DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
+    z, gx_raw, gw = DeviceArray(gz.shape, np.float32), DeviceArray((x.size + 1,), np.float32, zero=True), DeviceArray(w.shape, np.float32, zero=True)
+    rc = lib.d8_conv2d(capi.FLOAT32, raw.ptr + 4, B, IH, IH, IC, dw.ptr, OC, F, F, z.ptr, *args, small.ptr, asked, None)
+    assert rc == 10001 and b"not 16-byte aligned" in lib.d8_last_error()
+    nb = 4 * B * IH * IH * F * F * IC + (32 << 20)        # the interim matrix + room for any split workspace
+    ws = DeviceArray((nb,), np.uint8)
+    check(lib.d8_conv2d(capi.FLOAT32, raw.ptr + 4, B, IH, IH, IC, dw.ptr, OC, F, F, z.ptr, *args, ws.ptr, nb, None))
+    assert np.array_equal(z.numpy(), want[0])
+    check(lib.d8_conv2d_grad_x(capi.FLOAT32, gx_raw.ptr + 4, B, IH, IH, IC, dw.ptr, OC, F, F, dgz.ptr, *args, ws.ptr, nb, None))
+    assert np.array_equal(gx_raw.numpy()[1:].reshape(x.shape), want[1])
+    check(lib.d8_conv2d_grad_y(capi.FLOAT32, raw.ptr + 4, B, IH, IH, IC, gw.ptr, OC, F, F, dgz.ptr, *args, ws.ptr, nb, None))
+    assert np.array_equal(gw.numpy(), want[2])
