@@ -282,6 +282,7 @@ class ConvWorkload:
         # explicit: the reference's own lowering (im2col -> GEMM, GEMM -> col2im through the interim matrix);
         # the library reads D8_CONV_EXPLICIT at every call
         self.explicit = explicit
+        self.stream = None  # a hipStream_t as an integer, or None for the default stream
         if explicit:
             os.environ["D8_CONV_EXPLICIT"] = "1"
         self.key = name.split(":")[0]
@@ -326,7 +327,7 @@ class ConvWorkload:
         if self.explicit:
             os.environ["D8_CONV_EXPLICIT"] = "1"
         try:
-            check(fn(self.dt, a, B, IH, IW, IC, b, OC, FH, FW, c, *self.geo, self.ws.ptr, self.ws_bytes, None))
+            check(fn(self.dt, a, B, IH, IW, IC, b, OC, FH, FW, c, *self.geo, self.ws.ptr, self.ws_bytes, self.stream))
         finally:
             if self.explicit:
                 os.environ.pop("D8_CONV_EXPLICIT", None)
@@ -1102,7 +1103,7 @@ def main():
                     pms = _time_events(fn, 100)
                     o[pname] = {"launch_us": round(pms * 1e3, 2), "algorithmic_GBps": round(amount / (pms * 1e-3) / 1e9, 1),
                                 "frac_of_hbm_peak": round(amount / (pms * 1e-3) / 1e9 / HBM_PEAK, 4), **_traffic_fields(key, pname)}
-            if key == "c1":  # launch-latency bound: the same three launches replayed from a HIP graph
+            if key in ("c1", "c5") and not EAGER_ZERO:  # launch-latency bound steps: the same launches replayed from a HIP graph
                 o["ms_per_step_graph_replay"] = round(graph_replay_ms(wl, 50, 5), 4)
             others[key] = o
         out["others"] = others

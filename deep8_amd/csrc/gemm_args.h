@@ -77,6 +77,11 @@ struct GemmArgs {
     // ReLu do as separate passes over C in the reference (deep8/src/math/Add.cu:21-52, ReLu.cu:20-59).
     const void *bias;
     int relu;
+    // Remainder band in the same launch (tail_splits > 0; unsplit, unbatched products only): rows tail_m0 .. M - 1
+    // are not tiled by the launch's first tiles(tail_m0) x tiles(N) workgroups but by further ones, tail_splits per
+    // tile, each walking tail_tps K steps and writing fp32 partial sums to ws[piece][row - tail_m0][n].  They start
+    // as the first workgroups retire, so the band costs a fraction of a tile's time instead of a launch of its own.
+    int tail_m0, tail_splits, tail_tps;
 };
 
 // Whether a product with these arguments would run on a kernel that applies GemmArgs::bias / relu in its store

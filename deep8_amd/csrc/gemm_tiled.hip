@@ -370,7 +370,15 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const int total = tilesM * tilesN;
     int b = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z / g.splits;
     int split = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z - b * g.splits;
-    {
+    // a workgroup past the product's own tiles works on the remainder band (GemmArgs::tail_m0)
+    const bool in_tail = VIRT != VIRT_A_CLASSES && g.tail_splits > 0 && id >= total;
+    int tps = g.tiles_per_split;
+    if (in_tail) {
+        const int t = id - total;
+        split = t % g.tail_splits;
+        id = t / g.tail_splits;  // tile of the band, column by column
+        tps = g.tail_tps;
+    } else {
         // an unsplit batched product is dealt out the same way over its batch index: one XCD takes all
         // tiles of a batch element, whose A and B it then reads once
         const bool by_batch = g.splits == 1;
@@ -389,12 +397,14 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     }
     constexpr int GM = 4;
     const int band = id / (GM * tilesN), first = band * GM;
-    const int rows_in_band = min(GM, tilesM - first);
+    const int rows_in_band = max(1, min(GM, tilesM - first));
     const int in_band = id - band * GM * tilesN;
-    const int tm = first + in_band % rows_in_band, tn = in_band / rows_in_band;
+    const int tail_tilesM = in_tail ? (M - g.tail_m0 + BM - 1) / BM : 1;
+    const int tm = in_tail ? id % tail_tilesM : first + in_band % rows_in_band;
+    const int tn = in_tail ? id / tail_tilesM : in_band / rows_in_band;
     // A tile that would stick out of the matrix is moved back inside; the rows / columns it then
     // shares with its neighbour are computed twice but stored only by the neighbour.
-    const int m_own = tm * BM, n_own = tn * BN;
+    const int m_own = (in_tail ? g.tail_m0 : 0) + tm * BM, n_own = tn * BN;
     // (a matrix with fewer rows or columns than the tile: the tile starts at 0 and reaches past it; what the loads
     // bring in from there -- zeros past the end of the buffer, otherwise whatever follows -- only ever enters
     // results of rows / columns past the matrix, which are not stored)
@@ -473,7 +483,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const int ktiles = (g.K + BK - 1) / BK, tail_len = g.K % BK;
     const unsigned av_plain = (unsigned)ES * ((unsigned)a_r * (unsigned)g.lda + a_c * EPV);
     const unsigned bv_plain = (unsigned)ES * ((unsigned)b_r * (unsigned)g.ldb + b_c * EPV);
-    const int x0 = split * g.tiles_per_split, nsteps = min(red * ktiles, x0 + g.tiles_per_split) - x0;
+    const int x0 = split * tps, nsteps = min(red * ktiles, x0 + tps) - x0;
     const unsigned a_prod = (unsigned)ES * (unsigned)g.sA, b_prod = (unsigned)ES * (unsigned)g.sB;
     const unsigned b_prod_row = (unsigned)ES * (unsigned)g.sB_row, b_first = (unsigned)ES * b_cls;
     auto step_a = [&](int i) -> unsigned {
@@ -581,7 +591,11 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     __syncthreads();  // every wave is past the last step: the operand areas are free
     const Origin o = {m0, n0, m_own, n_own, M, g.N, (wm * TM) * 32, (wn * TN) * 32};
     float *patches = (float *)(T::PATCH_IN_A ? As0 : Bs0), *patches1 = (float *)(T::PATCH_IN_A ? As1 : Bs1);
-    if (g.splits > 1)
+    if (in_tail) {  // partial sums of the band, rows counted from its first
+        const int tail_M = M - g.tail_m0;
+        const Origin ot = {m0 - g.tail_m0, n0, m_own - g.tail_m0, n_own, tail_M, g.N, (wm * TM) * 32, (wn * TN) * 32};
+        store_tile<T, float>(acc, patches, patches1, g.ws + ((long)split * tail_M) * g.N, g.N, 0.f, true, g.N, ot, plain);
+    } else if (g.splits > 1)
         store_tile<T, float>(acc, patches, patches1, g.ws + ((long)(b * g.splits + split) * g.M) * g.N, g.N, 0.f, true, g.N, o, plain);
     else
         store_tile<T, E>(acc, patches, patches1, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
@@ -591,7 +605,9 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
 template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int VIRT>
 static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
     typedef Tile<E, BM, BN, WGM, WGN, A_KC, B_KC, VIRT> T;
-    const int tilesM = ceil_div(g.M, BM), tilesN = ceil_div(g.N, BN);
+    const bool tail = g.tail_splits > 0;  // (gemm_tiled_run sets it only for 128-row tiles and a tail_m0 that is a multiple of them)
+    const int tilesM = ceil_div(tail ? g.tail_m0 : g.M, BM), tilesN = ceil_div(g.N, BN);
+    const int extra = tail ? ceil_div(g.M - g.tail_m0, BM) * tilesN * g.tail_splits : 0;
     // A launch of at most two workgroups per CU is spread evenly only if a CU cannot take a third:
     // where the tile's own LDS would let three in, unused dynamic LDS is requested on top.
     constexpr long lds = 2L * (T::A_SZ + T::B_SZ) * T::ES, third = 160 * 1024 / 3;
@@ -599,9 +615,9 @@ static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
     const long wgs = (long)tilesM * tilesN * layers, cus = cu_count();
     const unsigned pad = (lds <= third && wgs > cus && wgs <= 2 * cus) ? (unsigned)(third + 512 - lds) : 0u;
     if (VIRT == VIRT_NONE && g.K % T::BK)
-        hipLaunchKernelGGL((gemm_tiled_kernel<T, VIRT == VIRT_NONE>), dim3(tilesM * tilesN, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
+        hipLaunchKernelGGL((gemm_tiled_kernel<T, VIRT == VIRT_NONE>), dim3(tilesM * tilesN + extra, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
     else
-        hipLaunchKernelGGL((gemm_tiled_kernel<T, false>), dim3(tilesM * tilesN, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
+        hipLaunchKernelGGL((gemm_tiled_kernel<T, false>), dim3(tilesM * tilesN + extra, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
     D8_LAUNCH_CHECK();
     return 0;
 }
