@@ -45,7 +45,7 @@ EAGER_ZERO = False
 # of that row per launch; a list of alternatives is averaged).  None where the summary or a row is missing.
 TRAFFIC_ROWS = {
     "c3": ("gemm_wide_f16_matmul_4096_half.txt", [("gemm_wide_kernel", 1.0 / 3)]),           # NN, NT, TN averaged
-    "c4": ("conv2d_fp32_b32_56x56x64_3x3.txt", [("NT, A = patch rows", 2), ("gemm_split_reduce", 1)]),  # forward: rows cut in two + the band's reduction
+    XX
     "c5": ("deconv2d_half_b16_28x28x128_4x4s2.txt", [("one class of output pixels", 1)]),    # forward: one launch over the classes
     "d3": ("gemm_f64_matmul_2048_double.txt", [("gemm_f64_kernel", 1.0 / 3)]),
     "e4": ("elementwise_bias_relu_b32_56x56x64.txt", {"add (bias broadcast)": [("add_kernel", 1)], "relu": [("relu_kernel", 1)],

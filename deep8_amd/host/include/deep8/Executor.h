@@ -90,6 +90,8 @@ Variable &deConv2d(Variable &x, Variable &filter, bool covered = false, int stri
 Variable &operator+(Variable &x, Variable &y);  // Add, with broadcasting
 Variable &add(Variable &x, Variable &y);
 Variable &relu(Variable &x);
+Variable &matrixMultiplyBiasReLu(Variable &x, Variable &y, Variable &bias);  // relu(x * y + bias) as one node
+Variable &conv2dBiasReLu(Variable &x, Variable &filter, Variable &bias, bool covered = true, int strideY = 1, int strideX = 1, int dilationY = 1, int dilationX = 1);
 Variable &operator-(Variable &x, Variable &y);  // Minus, with broadcasting
 Variable &minus(Variable &x, Variable &y);
 Variable &l1Norm(Variable &x);

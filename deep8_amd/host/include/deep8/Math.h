@@ -113,6 +113,16 @@ Shape Pooling2dShape(const Shape &x, bool covered, int filterHeight, int filterW
 void AdamUpdate(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps);
 void AdamUpdateGPU(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float beta1, float beta2, float epsilon, float learningRate, float weightDecay, int64_t steps);
 
+// Add (a bias with one value per element of the last axis) and ReLu folded into the contraction before them; no
+// counterpart in the reference, which runs MatrixMultiplyGPU / Conv2dGPU, AddGPU (deep8/src/math/Add.cu:21-52) and
+// ReLuGPU (deep8/src/math/ReLu.cu:20-59) one after the other.  Same checks as the operators they combine.
+void MatrixMultiplyBiasReLu(const Tensor &x, const Tensor &y, const Tensor &bias, Tensor &z, bool relu = true);
+void Conv2dBiasReLu(const Tensor &x, const Tensor &y, const Tensor &bias, Tensor &z, bool covered, int strideY, int strideX,
+                    int dilationY, int dilationX, void *interimPtr, bool relu = true);
+// The way back through ReLu and the bias in one pass: dpre = dz where z > 0, else 0 (dpre may be dz); dbias += its sums
+// over every axis but the last.  Replaces ReLuGradGPU (ReLu.cu:61-116) followed by AddGradYGPU (Add.cu:99-133).
+void BiasReLuGrad(const Tensor &z, const Tensor &dz, Tensor &dpre, Tensor &dbias);
+
 }  // namespace Math
 }  // namespace Deep8
 

@@ -94,6 +94,10 @@ public:
     // the element-wise steps that follow them
     Variable &add(Variable &y);
     Variable &relu();
+    // ... and the three as one node: relu(this * y + bias), relu(conv2d(this, filter) + bias); bias has one value per
+    // element of the result's last dimension
+    Variable &matrixMultiplyBiasReLu(Variable &y, Variable &bias);
+    Variable &conv2dBiasReLu(Variable &filter, Variable &bias, bool covered = true, int strideY = 1, int strideX = 1, int dilationY = 1, int dilationX = 1);
     // what a loss needs (deep8/src/nodes/Variable.cpp:342-346,461-465,521-535)
     Variable &minus(Variable &y);
     Variable &l1Norm();
@@ -109,7 +113,8 @@ public:
     Variable &avgPooling2d(bool covered = false, int filterHeight = 1, int filterWidth = 1, int strideY = 1, int strideX = 1);
 };
 
-enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply, Add, ReLu, Minus, L1Norm, L2Norm, ReduceMean, MaxPooling2d, AvgPooling2d };
+enum class FunctionType { Unkown = 0, Conv2d, DeConv2d, MatrixMultiply, Add, ReLu, Minus, L1Norm, L2Norm, ReduceMean, MaxPooling2d, AvgPooling2d,
+                          MatrixMultiplyBiasReLu, Conv2dBiasReLu };
 
 class Function : public Node {
 protected:
@@ -130,7 +135,7 @@ public:
 
 class MatrixMultiply : public Function {
 public:
-    explicit MatrixMultiply(std::vector<Node *> &inputs);
+    explicit MatrixMultiply(std::vector<Node *> &inputs, size_t inputCount = 2);
     Shape checkShape(std::vector<Shape> &inputShapes) override;
     ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
@@ -144,7 +149,7 @@ public:
     int strideY, strideX, dilationY, dilationX;
 
     explicit Conv2d(std::vector<Node *> &inputs, bool covered = true, int strideY = 1, int strideX = 1,
-                    int dilationY = 1, int dilationX = 1);
+                    int dilationY = 1, int dilationX = 1, size_t inputCount = 2);
     Shape checkShape(std::vector<Shape> &inputShapes) override;
     ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
@@ -185,6 +190,38 @@ public:
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
     void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
                   size_t index, Tensor *iGradient) override;
+};
+
+// relu(x * y + bias) and relu(conv2d(x, filter) + bias) as ONE node each (inputs: x, y / filter, bias): the forward
+// pass is one call whose product kernel adds the bias and cuts at zero in its own store; the backward pass gates
+// the output gradient and sums the bias gradient in one pass, then runs the contraction's two gradient products on
+// the gated gradient.  Same values as the chain MatrixMultiply / Conv2d -> Add -> ReLu of separate nodes
+// (deep8/src/nodes/MatrixMultiply.cpp, Conv2d.cpp, Add.cpp, ReLu.cpp); no counterpart in the reference, whose
+// eager executor runs every node as it is created.
+class MatrixMultiplyBiasReLu : public MatrixMultiply {
+public:
+    explicit MatrixMultiplyBiasReLu(std::vector<Node *> &inputs);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    // one input at a time (gates the output gradient anew on every call)
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+    using Function::forward;
+    void backward() override;  // all inputs that want a gradient, gating once
+};
+
+class Conv2dBiasReLu : public Conv2d {
+public:
+    explicit Conv2dBiasReLu(std::vector<Node *> &inputs, bool covered = true, int strideY = 1, int strideX = 1,
+                            int dilationY = 1, int dilationX = 1);
+    Shape checkShape(std::vector<Shape> &inputShapes) override;
+    ElementType checkElementType(std::vector<ElementType> &inputTypes) override;
+    void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
+    void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
+                  size_t index, Tensor *iGradient) override;
+    using Function::forward;
+    void backward() override;
 };
 
 // z = x - y under the same broadcasting rule (deep8/include/nodes/Minus.h, deep8/src/nodes/Minus.cpp:6-39)

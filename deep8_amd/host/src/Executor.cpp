@@ -251,5 +251,9 @@ Variable &reduceMean(Variable &x, std::vector<int> axis, bool keepDims) { return
 Variable &l1NormLoss(Variable &x) { return x.l1NormLoss(); }
 Variable &l2NormLoss(Variable &x) { return x.l2NormLoss(); }
 Variable &relu(Variable &x) { return x.relu(); }
+Variable &matrixMultiplyBiasReLu(Variable &x, Variable &y, Variable &bias) { return x.matrixMultiplyBiasReLu(y, bias); }
+Variable &conv2dBiasReLu(Variable &x, Variable &filter, Variable &bias, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
+    return x.conv2dBiasReLu(filter, bias, covered, strideY, strideX, dilationY, dilationX);
+}
 
 }  // namespace Deep8

@@ -703,5 +703,52 @@ void AdamUpdateGPU(Tensor &value, Tensor &gradient, Tensor &m, Tensor &v, float 
                             (long)steps, (long)value.shape.size(), nullptr));
 }
 
+// ---- bias and ReLu folded into the contraction ----------------------------------------------------------------------------
+namespace {
+void checkBias(const Tensor &bias, const Tensor &z) {
+    DEEP8_ARGUMENT_CHECK(bias.deviceType() == z.deviceType(), "the device type must be same");
+    DEEP8_ARGUMENT_CHECK(bias.elementType == z.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(1 == bias.shape.batch && 1 == bias.shape.nDims && bias.shape.dim(0) == z.shape.dim(z.shape.nDims - 1),
+                         "the bias must have one value per element of the output's last dimension");
+}
+}  // namespace
+
+void MatrixMultiplyBiasReLu(const Tensor &x, const Tensor &y, const Tensor &bias, Tensor &z, bool relu) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == y.deviceType() && x.deviceType() == z.deviceType(), "the device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == y.elementType && x.elementType == z.elementType, "the data type must be same");
+    checkMatrixMultiplyShapes(x, y, z);
+    checkBias(bias, z);
+    requireGPU(x);
+    const MM d = mmDims(x, y);
+    const int dt = dtypeOf(x);
+    PoolScratch ws(x.device(), d8_matmul_scratch_bytes(dt, 0, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
+    D8_CHECK(d8_matmul_bias_relu(dt, x.raw(), d.xb, d.xr, d.xc, y.raw(), d.yb, d.yr, d.yc, bias.raw(), relu ? 1 : 0, z.raw(),
+                                 ws.ptr, ws.bytes, nullptr));
+}
+
+void Conv2dBiasReLu(const Tensor &x, const Tensor &y, const Tensor &bias, Tensor &z, bool covered, int strideY, int strideX,
+                    int dilationY, int dilationX, void *interimPtr, bool relu) {
+    const ConvDims d = checkConv(x, y, z, covered, strideY, strideX, dilationY, dilationX);
+    checkBias(bias, z);
+    requireGPU(x);
+    const int dt = dtypeOf(x);
+    const size_t bytes = d8_conv2d_scratch_bytes(dt, 0, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, covered, strideY, strideX, dilationY, dilationX);
+    D8_CHECK(d8_conv2d_bias_relu(dt, x.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), d.OC, d.FH, d.FW, bias.raw(), relu ? 1 : 0, z.raw(),
+                                 covered, strideY, strideX, dilationY, dilationX, interimPtr, bytes, nullptr));
+}
+
+void BiasReLuGrad(const Tensor &z, const Tensor &dz, Tensor &dpre, Tensor &dbias) {
+    DEEP8_ARGUMENT_CHECK(z.deviceType() == dz.deviceType() && z.deviceType() == dpre.deviceType(), "the device type must be same");
+    DEEP8_ARGUMENT_CHECK(z.elementType == dz.elementType && z.elementType == dpre.elementType, "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(z.shape == dz.shape && z.shape == dpre.shape, "the shape must be same");
+    checkBias(dbias, z);
+    requireGPU(z);
+    const int dt = dtypeOf(z), cols = (int)dbias.shape.dim(0);
+    const long rows = (long)(z.shape.size() / (size_t)cols);
+    PoolScratch ws(z.device(), d8_bias_relu_grad_scratch_bytes(dt, rows, cols));
+    const bool fresh = dbias.takeZero();  // deferred zero fill: write instead of add
+    D8_CHECK(d8_bias_relu_grad(dt, z.raw(), dz.raw(), dpre.raw(), dbias.raw(), rows, cols, fresh ? 0 : 1, ws.ptr, ws.bytes, nullptr));
+}
+
 }  // namespace Math
 }  // namespace Deep8

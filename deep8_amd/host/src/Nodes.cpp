@@ -172,6 +172,18 @@ Variable &Variable::relu() {
     return *executor->addFunction(new ReLu(in));
 }
 
+Variable &Variable::matrixMultiplyBiasReLu(Variable &y, Variable &bias) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this, &y, &bias};
+    return *executor->addFunction(new MatrixMultiplyBiasReLu(in));
+}
+
+Variable &Variable::conv2dBiasReLu(Variable &filter, Variable &bias, bool covered, int strideY, int strideX, int dilationY, int dilationX) {
+    DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
+    std::vector<Node *> in = {this, &filter, &bias};
+    return *executor->addFunction(new Conv2dBiasReLu(in, covered, strideY, strideX, dilationY, dilationX));
+}
+
 Variable &Variable::minus(Variable &y) {
     DEEP8_ARGUMENT_CHECK(nullptr != executor, "the Variable does not belong to an Executor");
     std::vector<Node *> in = {this, &y};
@@ -285,8 +297,8 @@ void Function::backward() {
 }
 
 // ---- MatrixMultiply ---------------------------------------------------------------------------------------------------
-MatrixMultiply::MatrixMultiply(std::vector<Node *> &in) : Function(in) {
-    DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the MatrixMultiply Function needs 2 input");
+MatrixMultiply::MatrixMultiply(std::vector<Node *> &in, size_t count) : Function(in) {
+    DEEP8_ARGUMENT_CHECK(count == inputs.size(), "the MatrixMultiply Function needs 2 input (3 with a bias)");
 }
 
 Shape MatrixMultiply::checkShape(std::vector<Shape> &inputShapes) {
@@ -337,9 +349,9 @@ void checkConvInputs(std::vector<Shape> &inputShapes) {
 }
 }  // namespace
 
-Conv2d::Conv2d(std::vector<Node *> &in, bool cov, int sy, int sx, int dy, int dx)
+Conv2d::Conv2d(std::vector<Node *> &in, bool cov, int sy, int sx, int dy, int dx, size_t count)
     : Function(in), covered(cov), strideY(sy), strideX(sx), dilationY(dy), dilationX(dx) {
-    DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the Conv2d Function needs 2 input");
+    DEEP8_ARGUMENT_CHECK(count == inputs.size(), "the Conv2d Function needs 2 input (3 with a bias)");
     DEEP8_ARGUMENT_CHECK(strideY >= 1 && strideX >= 1, "the stride can not smaller than 1");
     DEEP8_ARGUMENT_CHECK(dilationY >= 1 && dilationX >= 1, "the dilation can not smaller than 1");
 }
@@ -428,6 +440,124 @@ void DeConv2d::backward(const std::vector<const Tensor *> &in, const Tensor *out
     } else {
         DEEP8_RUNTIME_ERROR("the index of DeConv2d backward is error");
     }
+}
+
+// ---- contraction + bias + ReLu as one node ---------------------------------------------------------------------------
+namespace {
+// a tensor of t's shape and type from t's device pool (released with its last copy)
+Tensor tensorLike(const Tensor &t) {
+    Device *dev = t.device();
+    const size_t bytes = t.byteCount();
+    void *ptr = dev->malloc(bytes);
+    size_t *ref = (size_t *)dev->mallocCPU(sizeof(size_t));
+    TensorStorage storage(ptr, ref, bytes, dev);
+    Shape shape = t.shape;
+    return Tensor(storage, 0, shape, t.elementType);
+}
+
+void checkBiasShape(const Shape &bias, const Shape &out) {
+    DEEP8_ARGUMENT_CHECK(1 == bias.batch && 1 == bias.nDims && bias.dim(0) == out.dim(out.nDims - 1),
+                         "the bias needs one value per element of the output's last dimension");
+}
+
+// The backward pass shared by the two fused nodes: gate once, then the products `grads` asks for.
+template <typename Products>
+void fusedBackward(Function *f, const std::vector<const Tensor *> &values, Variable *out, const Products &products) {
+    Variable *bias = (Variable *)f->inputs[2];
+    Tensor dpre = tensorLike(out->gradient);
+    if (bias->updateGradient) {
+        Math::BiasReLuGrad(out->value, out->gradient, dpre, bias->gradient);
+    } else {
+        Tensor unused = tensorLike(bias->value);
+        Math::BiasReLuGrad(out->value, out->gradient, dpre, unused);
+    }
+    for (size_t i = 0; i < 2; ++i) {
+        Variable *in = (Variable *)f->inputs[i];
+        if (in->updateGradient) products(values, &out->value, &dpre, i, &in->gradient);
+    }
+}
+}  // namespace
+
+MatrixMultiplyBiasReLu::MatrixMultiplyBiasReLu(std::vector<Node *> &in) : MatrixMultiply(in, 3) {}
+
+Shape MatrixMultiplyBiasReLu::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(3 == inputShapes.size(), "the input count must be 3");
+    std::vector<Shape> two(inputShapes.begin(), inputShapes.begin() + 2);
+    const Shape out = MatrixMultiply::checkShape(two);
+    checkBiasShape(inputShapes[2], out);
+    return out;
+}
+
+ElementType MatrixMultiplyBiasReLu::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(3 == inputTypes.size(), "the input count must be 3");
+    return Function::checkElementType(inputTypes);
+}
+
+void MatrixMultiplyBiasReLu::forward(const std::vector<const Tensor *> &in, Tensor *output) {
+    Math::MatrixMultiplyBiasReLu(*in[0], *in[1], *in[2], *output);
+}
+
+void MatrixMultiplyBiasReLu::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient,
+                                      size_t index, Tensor *iGradient) {
+    DEEP8_ARGUMENT_CHECK(index < 3, "the index is error");
+    Tensor dpre = tensorLike(*outputGradient);
+    if (2 == index) {
+        Math::BiasReLuGrad(*output, *outputGradient, dpre, *iGradient);
+        return;
+    }
+    Tensor unused = tensorLike(*in[2]);
+    Math::BiasReLuGrad(*output, *outputGradient, dpre, unused);
+    MatrixMultiply::backward(in, output, &dpre, index, iGradient);
+}
+
+void MatrixMultiplyBiasReLu::backward() {
+    Variable *out = nullptr;
+    std::vector<const Tensor *> values = gatherInputs(this, out);
+    fusedBackward(this, values, out, [this](const std::vector<const Tensor *> &v, const Tensor *z, const Tensor *dz, size_t i, Tensor *g) {
+        MatrixMultiply::backward(v, z, dz, i, g);
+    });
+}
+
+Conv2dBiasReLu::Conv2dBiasReLu(std::vector<Node *> &in, bool cov, int sy, int sx, int dy, int dx) : Conv2d(in, cov, sy, sx, dy, dx, 3) {}
+
+Shape Conv2dBiasReLu::checkShape(std::vector<Shape> &inputShapes) {
+    DEEP8_ARGUMENT_CHECK(3 == inputShapes.size(), "the input count must be 3");
+    std::vector<Shape> two(inputShapes.begin(), inputShapes.begin() + 2);
+    const Shape out = Conv2d::checkShape(two);
+    checkBiasShape(inputShapes[2], out);
+    return out;
+}
+
+ElementType Conv2dBiasReLu::checkElementType(std::vector<ElementType> &inputTypes) {
+    DEEP8_ARGUMENT_CHECK(3 == inputTypes.size(), "the input count must be 3");
+    return Function::checkElementType(inputTypes);
+}
+
+void Conv2dBiasReLu::forward(const std::vector<const Tensor *> &in, Tensor *output) {
+    Interim buf(output->device(),
+                Math::Conv2dInterimSize(*in[0], *in[1], *output, covered, strideY, strideX, dilationY, dilationX));
+    Math::Conv2dBiasReLu(*in[0], *in[1], *in[2], *output, covered, strideY, strideX, dilationY, dilationX, buf.ptr);
+}
+
+void Conv2dBiasReLu::backward(const std::vector<const Tensor *> &in, const Tensor *output, const Tensor *outputGradient,
+                              size_t index, Tensor *iGradient) {
+    DEEP8_ARGUMENT_CHECK(index < 3, "the index is error");
+    Tensor dpre = tensorLike(*outputGradient);
+    if (2 == index) {
+        Math::BiasReLuGrad(*output, *outputGradient, dpre, *iGradient);
+        return;
+    }
+    Tensor unused = tensorLike(*in[2]);
+    Math::BiasReLuGrad(*output, *outputGradient, dpre, unused);
+    Conv2d::backward(in, output, &dpre, index, iGradient);
+}
+
+void Conv2dBiasReLu::backward() {
+    Variable *out = nullptr;
+    std::vector<const Tensor *> values = gatherInputs(this, out);
+    fusedBackward(this, values, out, [this](const std::vector<const Tensor *> &v, const Tensor *z, const Tensor *dz, size_t i, Tensor *g) {
+        Conv2d::backward(v, z, dz, i, g);
+    });
 }
 
 // ---- Add / ReLu -------------------------------------------------------------------------------------------------

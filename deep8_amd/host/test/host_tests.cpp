@@ -902,6 +902,61 @@ TEST_GPU(two_layer_convnet_trains_with_sgd) {
     EXPECT(executor.trainableParameters().size() == 3);
 }
 
+TEST_GPU(fused_bias_relu_nodes_match_the_chain_of_nodes) {
+    // relu(conv2d(x, w) + b) and relu(x2 * y + c) as chains of three nodes and as one fused node each: the same
+    // values and, after backward(l2NormLoss), the same gradients of every input (Float32: bit for bit for the
+    // forward values; the gradients pass through the same kernels in the same order).
+    std::mt19937 gen(11);
+    std::normal_distribution<float> nd(0.f, 1.f);
+    auto grad = [&](Variable &v) {
+        std::vector<float> h(v.shape().size());
+        gpu().copyFromGPUToCPU(v.gradient.raw(), h.data(), h.size() * 4);
+        return h;
+    };
+    auto value = [&](Variable &v) {
+        std::vector<float> h(v.shape().size());
+        v.fetch(h.data());
+        return h;
+    };
+    std::vector<std::vector<float>> results[2];
+    for (int fused = 0; fused < 2; ++fused) {
+        EagerExecutor executor;
+        gen.seed(11);
+        auto fill = [&](Variable &v, float scale) {
+            std::vector<float> h(v.shape().size());
+            for (float &f : h) f = nd(gen) * scale;
+            v.feed(h.data());
+        };
+        Variable &x = parameter(&executor, 4, {12, 12, 64}), &w = parameter(&executor, {64, 3, 3, 64}), &b = parameter(&executor, {64});
+        Variable &x2 = parameter(&executor, 5, {40, 96}), &y = parameter(&executor, {96, 136}), &c = parameter(&executor, {136});
+        fill(x, 1.f), fill(w, 0.1f), fill(b, 0.5f), fill(x2, 1.f), fill(y, 0.1f), fill(c, 0.5f);
+        Variable &z = fused ? conv2dBiasReLu(x, w, b) : relu(conv2d(x, w) + b);
+        Variable &z2 = fused ? matrixMultiplyBiasReLu(x2, y, c) : relu(x2 * y + c);
+        EXPECT(z.shape() == Shape(4, {12, 12, 64}) && z2.shape() == Shape(5, {40, 136}));
+        results[fused].push_back(value(z));
+        results[fused].push_back(value(z2));
+        backward(z.l2NormLoss() + z2.l2NormLoss());  // (one pass: the executor drops the graph after it)
+        for (Variable *v : {&x, &w, &b, &x2, &y, &c}) results[fused].push_back(grad(*v));
+    }
+    EXPECT(results[0].size() == 8 && results[1].size() == 8);
+    for (size_t k = 0; k < results[0].size(); ++k) {
+        const std::vector<float> &a = results[0][k], &f = results[1][k];
+        EXPECT(a.size() == f.size());
+        double num = 0, den = 0;
+        bool zeros = false, positives = false;
+        for (size_t i = 0; i < a.size(); ++i) {
+            num += (double)(a[i] - f[i]) * (a[i] - f[i]), den += (double)a[i] * a[i];
+            zeros |= a[i] == 0.f, positives |= a[i] > 0.f;
+        }
+        if (k < 2) EXPECT(zeros && positives);  // the ReLu cut something and kept something
+        EXPECT(den > 0 && std::sqrt(num / den) <= (k < 2 ? 0.0 : 1e-6));
+    }
+    // shape checks of the fused nodes
+    EagerExecutor executor;
+    Variable &x = parameter(&executor, 2, {8, 8, 4}), &w = parameter(&executor, {8, 3, 3, 4}), &bad = parameter(&executor, {7});
+    EXPECT(throws<std::invalid_argument>([&] { conv2dBiasReLu(x, w, bad); }));
+}
+
 }  // namespace
 
 // Node-level step times at the three large configurations: forward + both gradients through Function::forward /
