@@ -45,7 +45,7 @@ EAGER_ZERO = False
 # of that row per launch; a list of alternatives is averaged).  None where the summary or a row is missing.
 TRAFFIC_ROWS = {
     "c3": ("gemm_wide_f16_matmul_4096_half.txt", [("gemm_wide_kernel", 1.0 / 3)]),           # NN, NT, TN averaged
-    XX
+    "c4": ("conv2d_fp32_b32_56x56x64_3x3.txt", [("NT, A = patch rows", 1), ("gemm_split_reduce", 1)]),  # forward: one launch (remainder band included) + the band's reduction
     "c5": ("deconv2d_half_b16_28x28x128_4x4s2.txt", [("one class of output pixels", 1)]),    # forward: one launch over the classes
     "d3": ("gemm_f64_matmul_2048_double.txt", [("gemm_f64_kernel", 1.0 / 3)]),
     "e4": ("elementwise_bias_relu_b32_56x56x64.txt", {"add (bias broadcast)": [("add_kernel", 1)], "relu": [("relu_kernel", 1)],
@@ -363,8 +363,8 @@ class ConvWorkload:
     def gemm_roofline(self, reps):
         """The pass-forward GEMM launch, timed alone with HIP events, against the MFMA peak of its
         element type.  Conv2d forward runs the tiled kernel (its tile loader reads the patch matrix
-        straight from the image) over the rows that fill whole rounds of the chip, then over the
-        remaining band of rows with the reduction split, then the band's reduction: all three are
+        straight from the image) over the rows that fill whole rounds of the chip and, in the same launch,
+        over the remaining band of rows with the reduction split, then the band's reduction: both are
         inside the timed call; DeConv2d forward's GEMM (one product per filter tap,
         a single batched launch) is issued here through d8_gemm with the operator's own arguments."""
         from deep8_amd import capi
@@ -386,7 +386,7 @@ class ConvWorkload:
             name = "gemm_tiled_kernel<%s> (DeConv2d forward: %d per-tap products [%dx%d]x[%dx%d]^T, one launch)" % (dtype, T, M, IC, OC, IC)
         else:
             fn = self.fwd
-            name = "gemm_tiled_kernel<%s> (Conv2d forward, patch matrix read by the tile loader: whole rounds + split remainder band + its reduction, timed together)" % dtype
+            name = "gemm_tiled_kernel<%s> (Conv2d forward, patch matrix read by the tile loader: one launch over whole rounds and the split remainder band, + the band's reduction, timed together)" % dtype
         ms = _time_events(fn, reps)
         ach = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "kernel": name, "achieved": round(ach, 2), "peak": PEAK[dtype], "unit": "TFLOP/s",
