@@ -70,3 +70,17 @@ def test_cpu_pieces_run_clean_under_the_sanitizers():
         r = subprocess.run(["make", "-s", "-C", os.path.join(ROOT, where), "asan"], capture_output=True, text=True, timeout=600)
         assert r.returncode == 0, (where, r.stdout[-2000:], r.stderr[-2000:])
         assert "runtime error" not in r.stderr and "AddressSanitizer" not in r.stderr, (where, r.stderr[-2000:])
+
+
+def test_bench_reads_its_traffic_figures_from_the_committed_profiles():
+    """bench.py must import without a GPU, and every workload that reports `traffic` must find its rows in the
+    rocprofv3 summary under profiles/ (a renamed kernel or a regenerated summary would otherwise turn it into null)."""
+    import bench
+    for key, (fname, rows) in bench.TRAFFIC_ROWS.items():
+        assert os.path.exists(os.path.join(ROOT, "profiles", fname)), fname
+        parts = list(rows) if isinstance(rows, dict) else [None]
+        for part in parts:
+            t = bench.profile_traffic(key, part)
+            assert t is not None and t["bytes"] > 0, (key, part)
+    # the algorithmic bytes of the im2col launch at configuration 4's size are what the counters saw
+    assert abs(bench.profile_traffic("i4", "im2col")["bytes"] - 256.9e6) < 2e6
