@@ -676,6 +676,9 @@ def make_workload(key):
     if key == "c4":
         return ConvWorkload("c4: Conv2d fwd+dX+dW fp32 B32 56x56x64 3x3x64->64 s1 same", np.float32, False,
                             32, 56, 56, 64, 64, 3, 3, True, 1, 1, 5)
+    if key == "c4h":
+        return ConvWorkload("c4h: Conv2d fwd+dX+dW half B32 56x56x64 3x3x64->64 s1 same (configuration 4's layer in half precision)",
+                            np.float16, False, 32, 56, 56, 64, 64, 3, 3, True, 1, 1, 5)
     if key == "c4x":
         return ConvWorkload("c4x: Conv2d fwd+dX+dW fp32 B32 56x56x64 3x3x64->64 s1 same, the reference's lowering "
                             "(im2col -> GEMM, GEMM -> col2im, 231 MB interim matrix)", np.float32, False,
@@ -758,7 +761,7 @@ def cpu_baseline(key, seconds=12.0):
         n, dt = _repeat_for(one, seconds)
         return {"value": n * B / dt, "unit": "images/s", "cores": port.threads(), "kind": "port",
                 "sample": "im2col + col2im on %d images x %d repeats (fp32, C restatement), %.1f s" % (B, n, dt)}
-    if key in ("c4", "c4x", "c4e", "c4e_unfused", "c5"):
+    if key in ("c4", "c4h", "c4x", "c4e", "c4e_unfused", "c5"):
         # the reference runs Conv2d/DeConv2d on Eigen's thread pool: all host cores
         B = 8
         if key != "c5":
@@ -1088,7 +1091,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4e", "c4e_unfused", "c4x", "i4", "c5", "c5l", "e4", "p4", "d3"):
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4h", "c4e", "c4e_unfused", "c4x", "i4", "c5", "c5l", "e4", "p4", "d3"):
             if key == a.workload:
                 continue
             del wl
