@@ -327,8 +327,20 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
     float *patch = (float *)lds + wave * (16 * PATCH_LD);
     f16 *C = (f16 *)g.C + (long)b * g.sC;
     const int l15 = lane & 15, l4 = lane >> 4;
+    // beta = 1: the old C of a 16-row slab is fetched while the slab before it goes through the patch, so that
+    // only the first slab's read is waited for
+    f16x8 oldc[2][4];
+    auto fetch_old = [&](int i, f16x8(&dst)[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int m = m0 + wm * 128 + i * 16 + t * 4 + l4, n = n0 + wn * 128 + l15 * 8;
+            if (m >= m_own && n >= n_own) dst[t] = *(const f16x8 *)(C + (long)m * g.ldc + n);
+        }
+    };
+    if (g.beta != 0.f) fetch_old(0, oldc[0]);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
+        if (g.beta != 0.f && i + 1 < 8) fetch_old(i + 1, oldc[(i + 1) & 1]);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
 #pragma unroll
@@ -348,7 +360,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
                 f16 *c = C + (long)m * g.ldc + n;
                 f16x8 out;
                 if (g.beta != 0.f) {
-                    const f16x8 old = *(const f16x8 *)c;
+                    const f16x8 old = oldc[i & 1][t];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) v[e] += (float)old[e];
                 }
