@@ -381,8 +381,9 @@ bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps) {
 // How many pieces to cut the reduction into, for a kernel whose K step is BK.  Splitting is only
 // worth a second pass when the output alone gives the 256 CUs too few tiles; the long reductions
 // this catches are also the ones whose single fp32 accumulation chain would be longest.
-static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t workspace_bytes, int *tiles_per_split) {
-    const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
+static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t workspace_bytes, int *tiles_per_split, int virt = VIRT_NONE) {
+    const bool t64 = gemm_tiled_krows_64(virt, M, N);  // 64 x 64 tiles, 37 KB of LDS each
+    const long tiles = t64 ? (long)ceil_div(M, 64) * ceil_div(N, 64) * batch : (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
     const long total = (long)red * ceil_div(K, BK);
     if (gemm_is_small(M, N, K, batch, red)) {  // runs whole on gemm_small_kernel
         *tiles_per_split = (int)total;
@@ -391,6 +392,7 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     const int cus = cu_count();
     long splits = 1;
     if (tiles < cus) splits = 2L * cus / tiles;  // at most two workgroups per CU: a third one would run alone, after the rest
+    if (tiles < cus && t64) splits = 3L * cus / tiles;  // three of the small tiles per CU (56 / 85 / 113 / 140 pieces on C4's dW: 75.6 / 73.8 / 75.0 / 78.5 us)
     // 128 x 128 tiles over a long reduction: one workgroup per CU with pieces of 32 K steps or more runs as fast as two
     // with half as many, and halves the partial sums (C2b's dY, 512 x 512 over 16 384: 72.8 -> 70.6 us)
     if (tiles < cus && M >= 128 && N >= 128 && total / (cus / tiles) >= 32) splits = cus / tiles;
@@ -472,14 +474,14 @@ static int balanced_rows(const GemmArgs &g) {
     return (int)((tiles - rest) * 128);
 }
 
-size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red) {
+size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red, int virt) {
     int tps = 0;
     GemmArgs probe;
     memset(&probe, 0, sizeof(probe));
     probe.M = M, probe.N = N, probe.K = K, probe.batch = 1, probe.red = red;
     const int head = balanced_rows(probe);
     const int rows = head ? M - head : M;  // with a cut, only the second part is split
-    const int splits = plan_splits(gemm_tiled_k_step(dtype), rows, N, K, 1, red, (size_t)-1, &tps);
+    const int splits = plan_splits(gemm_tiled_k_step(dtype), rows, N, K, 1, red, (size_t)-1, &tps, virt);
     return splits > 1 ? (size_t)splits * rows * N * sizeof(float) : 0;
 }
 
@@ -487,7 +489,7 @@ static int gemm_tiled_run_whole(int dtype, GemmArgs &g, int transA, int transB, 
                                 hipStream_t stream) {
     g.ws = (float *)workspace;
     g.splits = plan_splits(gemm_tiled_k_step(dtype), g.M, g.N, g.K, g.batch, g.red, (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0,
-                           &g.tiles_per_split);
+                           &g.tiles_per_split, g.virt);
     return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, true, stream) : launch<float>(g, transA, transB, true, stream);
 }
 

@@ -119,7 +119,10 @@ bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps);
 int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
                    hipStream_t stream);
 // Workspace gemm_tiled_run may use for this shape.
-size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red);
+size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red, int virt = VIRT_NONE);
+// Whether a product whose B is a patch matrix (VIRT_B_KROWS) runs on 64 x 64 tiles: fewer than 128 rows, and the last
+// 128-column tile would be half empty or emptier (a 3 x 3 x 64 filter gradient: N = 576 = 4.5 x 128).
+inline bool gemm_tiled_krows_64(int virt, int M, int N) { return virt == VIRT_B_KROWS && M < 128 && N % 128 != 0 && N % 128 <= 64; }
 
 }  // namespace d8
 

@@ -638,6 +638,11 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     }
     // a 64-wide side gets a tile of that width (im2col products with 64 output channels)
     if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+    // a patch-matrix product whose last 128-column tile would be at most half full: 64 x 64 tiles, no padding
+    // multiplied (C4's filter gradient, N = 576: 83.7 -> 73.8 us)
+    if constexpr (VIRT == VIRT_B_KROWS) {
+        if (gemm_tiled_krows_64(VIRT, g.M, g.N)) return launch_tiled<E, 64, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+    }
     if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
     if (g.splits == 1 && gemm_tiled_half_tiles(g.M, g.N, g.batch, (long)g.red * ceil_div(g.K, 128 / (int)sizeof(E))))
         return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);

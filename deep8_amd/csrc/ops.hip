@@ -350,7 +350,7 @@ size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int 
     GemmArgs ga;
     int ta, tb;
     if (conv_implicit_plan(dtype, which, cs, nullptr, nullptr, nullptr, ga, ta, tb))
-        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
+        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red, ga.virt);
     if (which == 1 && conv_classes_grad_x(dtype, cs, nullptr, nullptr, nullptr, ga)) return 0;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
     const size_t plain = col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
@@ -608,10 +608,10 @@ static size_t deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW
     const int M = B * IH * IW, T = FH * FW;
     GemmArgs ga;
     if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
-        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
+        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red, ga.virt);
     if (which == 0 && deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga)) return 0;
     if (which == 2 && deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
-        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red);
+        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red, ga.virt);
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     return mat + gemm_ws(dtype, deconv_plan(which, M, T, OC, IC, nullptr, nullptr, nullptr));
 }
