@@ -538,6 +538,43 @@ class GatherMapsWorkload:
         return {"im2col": (self.im2col, self.im_bytes + self.col_bytes), "col2im": (self.col2im, self.col_bytes + 2 * self.im_bytes)}
 
 
+class DeconvMapsWorkload:
+    """d8_deconv_col2im and d8_deconv_im2col alone at configuration 5's literal size (half, B16 28x28 -> 56x56x64, 4x4,
+    stride 2, pads 2): the gather maps of the reference's DeConv2d lowering in the reference's own matrix layout
+    (deep8/src/math/DeConv2d.cu:11-58, 310-351).  HBM-bound: each reads or writes the 25.7 MB matrix once."""
+
+    def __init__(self, name, seed):
+        from deep8_amd import capi
+        self.name, self.dtype, self.key = name, np.dtype(np.float16), name.split(":")[0]
+        self.lib = capi.init()
+        self.dt = capi.dtype_id(self.dtype)
+        r = np.random.default_rng(seed)
+        B, IH, OC, F, S, OH, P = 16, 28, 64, 4, 2, 56, 2
+        self.B, self.geo = B, (B, IH, IH, OH, OH, OC, F, F, S, S, P, P)
+        self.dz = _dev(r.standard_normal((B, OH, OH, OC)).astype(np.float32).astype(np.float16))
+        self.mat = capi.DeviceArray((B * IH * IH, OC * F * F), np.float16, zero=True)
+        self.z = capi.DeviceArray((B, OH, OH, OC), np.float16)
+        self.mat_bytes, self.im_bytes = 2 * B * IH * IH * OC * F * F, 2 * B * OH * OH * OC
+        self.flops = float(B * IH * IH * OC * F * F)
+        self.bytes = 2 * (self.mat_bytes + self.im_bytes)
+
+    def im2col(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_deconv_im2col(self.dt, self.dz.ptr, self.mat.ptr, *self.geo, None))
+
+    def col2im(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_deconv_col2im(self.dt, self.mat.ptr, self.z.ptr, *self.geo, None))
+
+    def step(self):
+        self.im2col()
+        self.col2im()
+
+    def parts(self):
+        """name -> (call, algorithmic bytes)"""
+        return {"deconv_im2col": (self.im2col, self.mat_bytes + self.im_bytes), "deconv_col2im": (self.col2im, self.mat_bytes + self.im_bytes)}
+
+
 class BiasReluWorkload:
     """The element-wise steps after a convolution: Add (per-channel bias, broadcast) -> ReLu, and back:
     ReLuGrad -> AddGradY (bias gradient: a sum over batch, rows and columns).  HBM-bound."""
@@ -690,6 +727,8 @@ def make_workload(key):
     if key == "i4":
         return GatherMapsWorkload("i4: d8_im2col + d8_col2im alone at config 4's size, fp32 B32 56x56x64 3x3 s1 pad 1",
                                   np.float32, 32, 56, 56, 64, 3, 11)
+    if key == "k5":
+        return DeconvMapsWorkload("k5: d8_deconv_im2col + d8_deconv_col2im alone at config 5's literal size, half B16 28x28 -> 56x56x64 4x4 s2", 12)
     if key == "c5":
         return ConvWorkload("c5: DeConv2d fwd+dX+dW half B16 28x28x128 4x4 s2 -> 58x58x64 (Deep8 covered=false)",
                             np.float16, True, 16, 28, 28, 128, 64, 4, 4, False, 2, 2, 6)
@@ -747,6 +786,17 @@ def cpu_baseline(key, seconds=12.0):
         return {"value": n * B / dt, "unit": "images/s", "cores": src.threads(), "kind": kind,
                 "sample": "%s fwd+bwd on %d images x %d repeats (fp32 CPU path, host-side array copies included), %.1f s"
                           % (key, B, n, dt)}
+    if key == "k5":
+        port = oracle.port
+        B = 4
+        dz = r.standard_normal((B, 56, 56, 64)).astype(np.float32)
+
+        def one():
+            m = port.deconv_im2col(dz, 28, 28, 4, 4, 2, 2, 2, 2)
+            port.deconv_col2im(m, B, 28, 28, 56, 56, 64, 4, 4, 2, 2, 2, 2)
+        n, dt = _repeat_for(one, seconds)
+        return {"value": n * B / dt, "unit": "images/s", "cores": port.threads(), "kind": "port",
+                "sample": "deconv_im2col + deconv_col2im on %d images x %d repeats (fp32, C restatement), %.1f s" % (B, n, dt)}
     if key == "i4":
         # the reference's CPU path never materialises the patch matrix (it is a lazy Eigen expression), so the
         # two maps are timed on the C restatement of the reference's GPU kernels' index maps
@@ -1012,7 +1062,7 @@ def main():
     dtype = {2: "f16", 4: "f32", 8: "f64"}[wl.dtype.itemsize]
     is_conv = isinstance(wl, ConvWorkload)
     is_mm = isinstance(wl, MatMulWorkload)
-    is_stream = isinstance(wl, (BiasReluWorkload, PoolWorkload, GatherMapsWorkload))  # HBM-bound kernels
+    is_stream = isinstance(wl, (BiasReluWorkload, PoolWorkload, GatherMapsWorkload, DeconvMapsWorkload))  # HBM-bound kernels
     tflops = wl.flops / (ms * 1e-3) / 1e12
 
     def time_parts(table):
@@ -1091,7 +1141,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4h", "c4e", "c4e_unfused", "c4x", "i4", "c5", "c5l", "e4", "p4", "d3"):
+        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4h", "c4e", "c4e_unfused", "c4x", "i4", "k5", "c5", "c5l", "e4", "p4", "d3"):
             if key == a.workload:
                 continue
             del wl
@@ -1099,9 +1149,9 @@ def main():
             oms, _ = _time_steps(wl.step, 20, 3, reps=3)
             o = {"ms_per_step": round(oms, 4), "tflops": round(wl.flops / (oms * 1e-3) / 1e12, 2),
                  "algorithmic_GBps": round(wl.bytes / (oms * 1e-3) / 1e9, 1)}
-            if isinstance(wl, (ConvWorkload, DeconvLiteralWorkload, BiasReluWorkload, PoolWorkload, GatherMapsWorkload)):
+            if isinstance(wl, (ConvWorkload, DeconvLiteralWorkload, BiasReluWorkload, PoolWorkload, GatherMapsWorkload, DeconvMapsWorkload)):
                 o["images_per_s"] = round(wl.B / (oms * 1e-3), 1)
-            if isinstance(wl, GatherMapsWorkload):  # the two kernels alone, against the HBM peak
+            if isinstance(wl, (GatherMapsWorkload, DeconvMapsWorkload)):  # the two kernels alone, against the HBM peak
                 for pname, (fn, amount) in wl.parts().items():
                     pms = _time_events(fn, 100)
                     o[pname] = {"launch_us": round(pms * 1e3, 2), "algorithmic_GBps": round(amount / (pms * 1e-3) / 1e9, 1),

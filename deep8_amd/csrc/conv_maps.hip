@@ -293,6 +293,132 @@ __global__ __launch_bounds__(256) void deconv_im2col_kernel(const T *__restrict_
     }
 }
 
+// ---- the two DeConv2d maps staged through LDS ------------------------------------------------------------------
+// The reference's matrix layout [B*IH*IW][OC][FH*FW] puts the channels of one tap FH*FW elements apart, so a thread
+// per element (the kernels above) moves 2 or 4 bytes at a time.  These forms move 16 bytes per lane on the matrix
+// side and on the image side and turn the layout around in LDS.
+//
+// col2im: a workgroup owns one output row (b, oy).  For each filter row fy that reaches it (ascending, then fx
+// ascending inside: the reference's addition order, so sums round identically) the slab
+// zmat[(b, iy, ix)][oc][fy][0 .. FW) of all ix, oc is copied into LDS as [ix][fx][oc]; a thread then owns VEC
+// channels of one output pixel, adds its taps from LDS into fp32 registers and, after the last fy, writes once.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restrict__ zmat, T *__restrict__ z, MapGeom g) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char deconv_lds[];
+    T *slab = (T *)deconv_lds;  // [IW][FW][C]
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    const int oy = blockIdx.x % g.OH, b = blockIdx.x / g.OH;
+    const int taps = g.FH * g.FW, C = g.C, CV = C / VEC;
+    const long N = (long)C * taps;
+    const int pairs = g.IW * C;      // (ix, oc) pairs staged per filter row
+    const int outs = g.OW * CV;      // (ox, channel vector) outputs of this row
+    // each thread keeps the sums of up to MAXO of the row's outputs (outs <= 256 * MAXO is checked by the launcher)
+    constexpr int MAXO = 4;
+    float acc[MAXO][VEC];
+#pragma unroll
+    for (int o = 0; o < MAXO; ++o)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[o][e] = 0.f;
+    for (int fy = 0; fy < g.FH; ++fy) {
+        const int ty = oy - g.pt + fy;
+        if (ty < 0 || ty % g.sy) continue;  // (uniform over the workgroup)
+        const int iy = ty / g.sy;
+        if (iy >= g.IH) continue;
+        __syncthreads();  // the previous slab has been consumed
+        const T *src = zmat + ((long)b * g.IH + iy) * g.IW * N + (long)fy * g.FW;
+        // a filter row of a channel is FW contiguous elements: fetched as one 8- or 16-byte piece where it is one
+        const bool row8 = g.FW * sizeof(T) == 8 && (taps * sizeof(T)) % 8 == 0 && ((size_t)zmat & 7) == 0;
+        const bool row16 = g.FW * sizeof(T) == 16 && (taps * sizeof(T)) % 16 == 0 && ((size_t)zmat & 15) == 0;
+        for (int q = threadIdx.x; q < pairs; q += 256) {
+            const int ix = q / C, oc = q - ix * C;
+            const T *p = src + (long)ix * N + (long)oc * taps;
+            T *d = slab + ix * g.FW * C + oc;
+            if (row8) {
+                typedef T V8 __attribute__((ext_vector_type(8 / sizeof(T))));
+                const V8 v = *(const V8 *)p;
+#pragma unroll
+                for (int fx = 0; fx < (int)(8 / sizeof(T)); ++fx) d[fx * C] = v[fx];
+            } else if (row16) {
+                typedef T V16 __attribute__((ext_vector_type(16 / sizeof(T))));
+                const V16 v = *(const V16 *)p;
+#pragma unroll
+                for (int fx = 0; fx < (int)(16 / sizeof(T)); ++fx) d[fx * C] = v[fx];
+            } else {
+                for (int fx = 0; fx < g.FW; ++fx) d[fx * C] = p[fx];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int o = 0; o < MAXO; ++o) {
+            const int q = threadIdx.x + 256 * o;
+            if (q < outs) {
+                const int ox = q / CV, cv = q - ox * CV;
+                for (int fx = 0; fx < g.FW; ++fx) {
+                    const int tx = ox - g.pl + fx;
+                    if (tx < 0 || tx % g.sx) continue;
+                    const int ix = tx / g.sx;
+                    if (ix >= g.IW) continue;
+                    const VT v = *(const VT *)(slab + (ix * g.FW + fx) * C + cv * VEC);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[o][e] += (float)v[e];
+                }
+            }
+        }
+    }
+    T *row = z + ((long)b * g.OH + oy) * g.OW * C;
+#pragma unroll
+    for (int o = 0; o < MAXO; ++o) {
+        const int q = threadIdx.x + 256 * o;
+        if (q < outs) {
+            VT out;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out[e] = (T)acc[o][e];
+            *(VT *)(row + (long)q * VEC) = out;
+        }
+    }
+}
+
+// im2col: a workgroup owns one input row (b, iy).  The FH rows of dz its taps read are copied into LDS as
+// [fy][ox][oc] (zeros where the row lies outside the image); a thread then assembles VEC consecutive columns
+// (oc, fy, fx) of a matrix row from LDS and stores them at once.  A pure copy: bit-exact.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void deconv_im2col_lds_kernel(const T *__restrict__ dz, T *__restrict__ dzmat, MapGeom g,
+                                                                FastDiv by_T, FastDiv by_FW, FastDiv by_NV) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char deconv_lds[];
+    T *rows = (T *)deconv_lds;  // [FH][OW][C]
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    const int iy = blockIdx.x % g.IH, b = blockIdx.x / g.IH;
+    const int taps = g.FH * g.FW, C = g.C;
+    const int N = C * taps, NV = N / VEC, rowlen = g.OW * C;
+    for (int fy = 0; fy < g.FH; ++fy) {
+        const int oy = iy * g.sy + g.pt - fy;
+        const bool inside = oy >= 0 && oy < g.OH;
+        const T *src = dz + ((long)b * g.OH + (inside ? oy : 0)) * rowlen;
+        for (int q = threadIdx.x * VEC; q < rowlen; q += 256 * VEC) {  // rowlen is a multiple of VEC (C is)
+            VT v;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = (T)0;
+            if (inside) v = *(const VT *)(src + q);
+            *(VT *)(rows + (long)fy * rowlen + q) = v;
+        }
+    }
+    __syncthreads();
+    T *out = dzmat + ((long)b * g.IH + iy) * g.IW * N;
+    const int chunks = g.IW * NV;
+    for (int q = threadIdx.x; q < chunks; q += 256) {
+        const unsigned ix = div_by((unsigned)q, by_NV), c0 = ((unsigned)q - ix * NV) * VEC;
+        VT v;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const unsigned col = c0 + e, oc = div_by(col, by_T), tap = col - oc * taps;
+            const unsigned fy = div_by(tap, by_FW), fx = tap - fy * g.FW;
+            const int ox = (int)ix * g.sx + g.pl - (int)fx;
+            v[e] = (ox >= 0 && ox < g.OW) ? rows[((long)fy * g.OW + ox) * C + oc] : (T)0;
+        }
+        *(VT *)(out + (long)q * VEC) = v;
+    }
+}
+
 static int check_geom(const char *who, int dtype, const void *a, const void *b, const MapGeom &g) {
     if (dtype != D8_FLOAT16 && dtype != D8_FLOAT32 && dtype != D8_FLOAT64)
         return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
@@ -446,6 +572,17 @@ int d8_deconv_col2im(int dtype, const void *zmat, void *z,
     if (B == 0) return 0;
     const long elems = (long)B * OH * OW * OC;
     hipStream_t s = as_stream(stream);
+    {   // the LDS-staged form: 16-byte channel vectors, a slab of one filter row in LDS, at most 1024 outputs per row
+        const size_t es = dtype_bytes(dtype), vec = 16 / es, lds = (size_t)IW * FW * OC * es;
+        if (es <= 4 && OC % vec == 0 && aligned16(z) && lds <= 60 * 1024 && (long)OW * (OC / vec) <= 1024 && (long)B * OH < (1L << 31)) {
+            if (es == 4)
+                hipLaunchKernelGGL((deconv_col2im_lds_kernel<float, 4>), dim3(B * OH), dim3(256), lds, s, (const float *)zmat, (float *)z, g);
+            else
+                hipLaunchKernelGGL((deconv_col2im_lds_kernel<f16, 8>), dim3(B * OH), dim3(256), lds, s, (const f16 *)zmat, (f16 *)z, g);
+            D8_LAUNCH_CHECK();
+            return 0;
+        }
+    }
     if (dtype == D8_FLOAT64)
         hipLaunchKernelGGL((deconv_col2im_kernel<double>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
                            (const double *)zmat, (double *)z, g, elems);
@@ -467,6 +604,20 @@ int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
     if (B == 0) return 0;
     const long elems = (long)B * IH * IW * OC * FH * FW;
     hipStream_t s = as_stream(stream);
+    {   // the LDS-staged form: the FH rows of dz an input row reads in LDS, 16-byte pieces of the matrix rows written
+        const size_t es = dtype_bytes(dtype), vec = 16 / es, lds = (size_t)FH * OW * OC * es;
+        const long N = (long)OC * FH * FW;
+        if (es <= 4 && OC % vec == 0 && N % vec == 0 && aligned16(dz) && aligned16(dzmat) && lds <= 60 * 1024 && N < (1L << 24) &&
+            (long)IW * N < (1L << 31) && (long)B * IH < (1L << 31)) {
+            const FastDiv by_T = fast_div((unsigned)(FH * FW)), by_FW = fast_div((unsigned)FW), by_NV = fast_div((unsigned)(N / vec));
+            if (es == 4)
+                hipLaunchKernelGGL((deconv_im2col_lds_kernel<unsigned, 4>), dim3(B * IH), dim3(256), lds, s, (const unsigned *)dz, (unsigned *)dzmat, g, by_T, by_FW, by_NV);
+            else
+                hipLaunchKernelGGL((deconv_im2col_lds_kernel<unsigned short, 8>), dim3(B * IH), dim3(256), lds, s, (const unsigned short *)dz, (unsigned short *)dzmat, g, by_T, by_FW, by_NV);
+            D8_LAUNCH_CHECK();
+            return 0;
+        }
+    }
     if (dtype == D8_FLOAT64)
         hipLaunchKernelGGL((deconv_im2col_kernel<unsigned long long>), dim3(grid_for(elems, 256)), dim3(256), 0, s,
                            (const unsigned long long *)dz, (unsigned long long *)dzmat, g, elems);
