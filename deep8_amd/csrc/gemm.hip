@@ -509,7 +509,7 @@ int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspa
         return gemm_tiled_run_whole(dtype, g, transA, transB, workspace, workspace_bytes, stream);
     // The band's pieces ride in the first part's launch (GemmArgs::tail_m0) when it is split at all and is at least
     // one tile high; only its reduction is a launch of its own.
-    static const bool two_launches = getenv("D8_GEMM_BAND_LAUNCH") != nullptr;  // tuning and test aid
+    const bool two_launches = getenv("D8_GEMM_BAND_LAUNCH") != nullptr;  // tuning and test aid (read at every call)
     second.ws = (float *)workspace;
     second.splits = plan_splits(gemm_tiled_k_step(dtype), second.M, second.N, second.K, 1, second.red,
                                 (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0, &second.tiles_per_split);
@@ -559,7 +559,9 @@ size_t d8_gemm_workspace_bytes(int dtype, int transA, int transB, int M, int N, 
     const int a = plan_splits(gemm_tiled_k_step(dtype), M, N, K, outs, red, (size_t)-1, &tps);
     const int b = plan_splits(dtype == D8_FLOAT16 ? Tile<f16>::BK : Tile<float>::BK, M, N, K, outs, red, (size_t)-1, &tps);
     const int splits = a > b ? a : b;
-    return splits > 1 ? (size_t)splits * outs * M * N * sizeof(float) : 0;
+    const size_t whole = splits > 1 ? (size_t)splits * outs * M * N * sizeof(float) : 0;
+    const size_t band = outs == 1 ? gemm_tiled_workspace(dtype, M, N, K, red) : 0;  // a tall product's remainder band, split
+    return whole > band ? whole : band;
 }
 
 // One product whose grid fits the launch limits (at most MAX_BATCH independent outputs, at most MAX_ROWS rows).
@@ -593,6 +595,8 @@ static int gemm_one(int dtype, int transA, int transB, int M, int N, int K,
     memset(&g.pg, 0, sizeof(g.pg));
     if (dtype == D8_FLOAT64) return gemm_f64_launch(g, transA, transB, as_stream(stream));
     const bool tiled = K > 0 && gemm_tiled_eligible(dtype, g, transA, transB);
+    // the tiled kernels' own driver plans the split and cuts a tall product's remainder band
+    if (tiled && !gemm_is_small(M, N, K, g.batch, g.red)) return gemm_tiled_run(dtype, g, transA, transB, workspace, workspace_bytes, as_stream(stream));
     if (K > 0) {  // K == 0 is the empty reduction: C = beta * C
         const int BK = tiled ? gemm_tiled_k_step(dtype) : (dtype == D8_FLOAT16 ? Tile<f16>::BK : Tile<float>::BK);
         g.splits = plan_splits(BK, M, N, K, g.batch, g.red, (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0, &g.tiles_per_split);

@@ -261,3 +261,29 @@ def test_gemm_reduction_not_a_multiple_of_the_k_step(ta, tb, M, N, K, dtype):
         capi.check(lib.d8_gemm(dt, ta, tb, M, N, K, dA.ptr, Ap.shape[2], Ap.shape[1] * Ap.shape[2], dB.ptr, Bp.shape[2],
                                Bp.shape[1] * Bp.shape[2], 0.0, dC.ptr, N, 0, batch, ws.ptr, wsb, None))
         assert np.array_equal(dC.numpy().astype(np.float64), want), (ta, tb, M, N, K, batch)
+
+
+@pytest.mark.parametrize("ta,tb,M,N,K", [
+    (0, 0, 99304, 64, 96),     # 776 tiles of 128 rows on 256 CUs: 768 in whole rounds, a ragged band of 1000 rows
+    (0, 1, 98304 + 128, 64, 64),  # a band of exactly one tile
+    (0, 1, 98304 + 100, 96, 64),  # a band shorter than a tile: runs as a product of its own
+    (0, 0, 131072 + 2048, 64, 32),
+])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_gemm_tall_product_with_a_remainder_band(ta, tb, M, N, K, dtype, monkeypatch):
+    """A tall product whose tile count is not a multiple of the chip's rounds: the remainder band's split pieces
+    ride in the main launch (or, forced, run as a second launch); both forms, beta 0 and 1, against numpy on
+    integers (exact)."""
+    from deep8_amd import ops
+    r = rng(M + N + K)
+    c = (lambda a: h(a)) if dtype == np.float16 else (lambda a: a)
+    A, B = _ab(r, ta, tb, M, N, K, lambda r, s: ints(r, s, 3))
+    C0 = ints(r, (M, N), 3)
+    prod = (A.T if ta else A) @ (B.T if tb else B)
+    assert prod.max() < 2048
+    for band_launch in (False, True):
+        if band_launch:
+            monkeypatch.setenv("D8_GEMM_BAND_LAUNCH", "1")  # read once per process: only effective if set before the first such call
+        for beta, C in ((0.0, None), (1.0, C0)):
+            got = ops.gemm(ta, tb, c(A), c(B), None if C is None else c(C), beta)
+            assert np.array_equal(f(got), prod + (0 if C is None else C)), (band_launch, beta)
