@@ -307,7 +307,11 @@ __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restr
     extern __shared__ __attribute__((aligned(16))) unsigned char deconv_lds[];
     T *slab = (T *)deconv_lds;  // [IW][FW][C]
     typedef T VT __attribute__((ext_vector_type(VEC)));
-    const int oy = blockIdx.x % g.OH, b = blockIdx.x / g.OH;
+    // (workgroup ids congruent mod 8 share an XCD: each XCD takes a contiguous eighth of the rows, so neighbouring
+    // output rows, which read the same matrix rows, meet in one L2)
+    const unsigned line = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    if (line >= (unsigned)(g.B * g.OH)) return;
+    const int oy = line % g.OH, b = line / g.OH;
     const int taps = g.FH * g.FW, C = g.C, CV = C / VEC;
     const long N = (long)C * taps;
     const int pairs = g.IW * C;      // (ix, oc) pairs staged per filter row
@@ -387,7 +391,9 @@ __global__ __launch_bounds__(256) void deconv_im2col_lds_kernel(const T *__restr
     extern __shared__ __attribute__((aligned(16))) unsigned char deconv_lds[];
     T *rows = (T *)deconv_lds;  // [FH][OW][C]
     typedef T VT __attribute__((ext_vector_type(VEC)));
-    const int iy = blockIdx.x % g.IH, b = blockIdx.x / g.IH;
+    const unsigned line = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);  // contiguous rows per XCD, as above
+    if (line >= (unsigned)(g.B * g.IH)) return;
+    const int iy = line % g.IH, b = line / g.IH;
     const int taps = g.FH * g.FW, C = g.C;
     const int N = C * taps, NV = N / VEC, rowlen = g.OW * C;
     for (int fy = 0; fy < g.FH; ++fy) {
@@ -576,9 +582,9 @@ int d8_deconv_col2im(int dtype, const void *zmat, void *z,
         const size_t es = dtype_bytes(dtype), vec = 16 / es, lds = (size_t)IW * FW * OC * es;
         if (es <= 4 && OC % vec == 0 && aligned16(z) && lds <= 60 * 1024 && (long)OW * (OC / vec) <= 1024 && (long)B * OH < (1L << 31)) {
             if (es == 4)
-                hipLaunchKernelGGL((deconv_col2im_lds_kernel<float, 4>), dim3(B * OH), dim3(256), lds, s, (const float *)zmat, (float *)z, g);
+                hipLaunchKernelGGL((deconv_col2im_lds_kernel<float, 4>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const float *)zmat, (float *)z, g);
             else
-                hipLaunchKernelGGL((deconv_col2im_lds_kernel<f16, 8>), dim3(B * OH), dim3(256), lds, s, (const f16 *)zmat, (f16 *)z, g);
+                hipLaunchKernelGGL((deconv_col2im_lds_kernel<f16, 8>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const f16 *)zmat, (f16 *)z, g);
             D8_LAUNCH_CHECK();
             return 0;
         }
@@ -611,9 +617,9 @@ int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
             (long)IW * N < (1L << 31) && (long)B * IH < (1L << 31)) {
             const FastDiv by_T = fast_div((unsigned)(FH * FW)), by_FW = fast_div((unsigned)FW), by_NV = fast_div((unsigned)(N / vec));
             if (es == 4)
-                hipLaunchKernelGGL((deconv_im2col_lds_kernel<unsigned, 4>), dim3(B * IH), dim3(256), lds, s, (const unsigned *)dz, (unsigned *)dzmat, g, by_T, by_FW, by_NV);
+                hipLaunchKernelGGL((deconv_im2col_lds_kernel<unsigned, 4>), dim3((B * IH + 7) & ~7), dim3(256), lds, s, (const unsigned *)dz, (unsigned *)dzmat, g, by_T, by_FW, by_NV);
             else
-                hipLaunchKernelGGL((deconv_im2col_lds_kernel<unsigned short, 8>), dim3(B * IH), dim3(256), lds, s, (const unsigned short *)dz, (unsigned short *)dzmat, g, by_T, by_FW, by_NV);
+                hipLaunchKernelGGL((deconv_im2col_lds_kernel<unsigned short, 8>), dim3((B * IH + 7) & ~7), dim3(256), lds, s, (const unsigned short *)dz, (unsigned short *)dzmat, g, by_T, by_FW, by_NV);
             D8_LAUNCH_CHECK();
             return 0;
         }

@@ -196,6 +196,24 @@ TEST_CPU(node_shape_inference) {
     EXPECT(upCovered.checkShape(s) == Shape(16, {55, 55, 64}));
     s = {Shape(16, {28, 28, 128}), Shape(1, {64, 4, 4, 100})};
     EXPECT(throws<std::invalid_argument>([&] { up.checkShape(s); }));
+
+    // the fused nodes take a third input, one bias value per element of the output's last dimension
+    Probe c;
+    std::vector<Node *> in3 = {&a, &b, &c};
+    Conv2dBiasReLu fusedConv(in3, true, 1, 1, 1, 1);
+    s = {Shape(32, {56, 56, 64}), Shape(1, {64, 3, 3, 64}), Shape(1, {64})};
+    EXPECT(fusedConv.checkShape(s) == Shape(32, {56, 56, 64}));
+    s[2] = Shape(1, {63});
+    EXPECT(throws<std::invalid_argument>([&] { fusedConv.checkShape(s); }));
+    s[2] = Shape(2, {64});
+    EXPECT(throws<std::invalid_argument>([&] { fusedConv.checkShape(s); }));
+    MatrixMultiplyBiasReLu fusedMm(in3);
+    s = {Shape(10, {400, 200}), Shape(1, {200, 300}), Shape(1, {300})};
+    EXPECT(fusedMm.checkShape(s) == Shape(10, {400, 300}));
+    s = {Shape(1, {300, 100}), Shape(10, {100}), Shape(1, {300})};  // a batch of vectors: the last dimension is x's rows
+    EXPECT(fusedMm.checkShape(s) == Shape(10, {300}));
+    EXPECT(throws<std::invalid_argument>([&] { Conv2dBiasReLu two(in, true, 1, 1, 1, 1); }));
+    EXPECT(throws<std::invalid_argument>([&] { MatrixMultiply three(in3); }));
 }
 
 TEST_GPU(memory_pool) {
