@@ -1007,6 +1007,62 @@ def phase_record(launches=12):
             (r[:, 5] - r[:, 4]).mean() / (n // 64)))
 
 
+def tiled_phase_record(key, launches=8):
+    """The calls of a workload that run gemm_tiled_kernel (the fp32 products, the convolutions) with the kernel's
+    per-workgroup phase record switched on (d8_gemm_phase_record): for each part of the step, when its workgroups
+    started, how long their prologue, K loop and epilogue took, at which shader clock the loop ran, how many tiles
+    a CU worked on and when they ended, and the same for the workgroups of a remainder band riding in the launch.
+    A diagnostic: it shows what a launch's time is made of (the matrix pipe's own share is printed beside it)."""
+    from deep8_amd import capi
+    lib = capi.init()
+    wl = make_workload(key)
+    nrec = 1 << 14
+    bufs = [capi.DeviceArray((nrec * 8,), np.uint64, zero=True) for _ in range(launches)]
+    peak_per_cu_cycle = {2: 2048.0, 4: 256.0}[wl.dtype.itemsize]  # flops per CU and cycle of the dense MFMA peak
+    for name, (fn, flops) in wl.parts().items():
+        capi.check(lib.d8_gemm_phase_record(None, 0))
+        for b in bufs:  # (records of the previous part)
+            b.zero_()
+        _settle(fn)
+        for b in bufs:  # (each launch writes its records from index 0: one buffer per launch)
+            capi.check(lib.d8_gemm_phase_record(b.ptr, nrec * 64))
+            fn()
+        capi.sync()
+        capi.check(lib.d8_gemm_phase_record(None, 0))
+        r = bufs[-1].numpy().astype(np.int64).reshape(nrec, 8)
+        r = r[r[:, 3] != 0]
+        if not len(r):
+            print("%s: no records (the call does not run gemm_tiled_kernel, or its grid exceeds %d workgroups)" % (name, nrec), flush=True)
+            continue
+        us = lambda v: v / 100.0
+        t0 = r[:, 0].min()
+        start, end = us(r[:, 0] - t0), us(r[:, 3] - t0)
+        pro, loop, epi = us(r[:, 1] - r[:, 0]), us(r[:, 2] - r[:, 1]), us(r[:, 3] - r[:, 2])
+        band = r[:, 7] == 1
+        key_cu = ((r[:, 6] >> 32) & 0xf) * 65536 + (r[:, 6] & 0xff00)  # XCD, and the SE / SH / CU bits of HW_ID
+        cus = len(np.unique(key_cu))
+        ghz = ((r[:, 5] - r[:, 4]) / np.maximum(loop * 1e3, 1e-9))[~band].mean()
+        pipe_us = flops / (cus * peak_per_cu_cycle * ghz * 1e9) * 1e6
+        print("%s: %d workgroups on %d CUs (%d of them on the remainder band); first start to last store acknowledged "
+              "%.1f us; the matrix pipe alone at the loop's own clock (%.2f GHz) would need %.1f us" % (
+                  name, len(r), cus, band.sum(), end.max(), ghz, pipe_us), flush=True)
+        for label, m in (("tiles", ~band), ("band pieces", band)):
+            if not m.any():
+                continue
+            print("  %s: start %.1f-%.1f us; prologue %.1f-%.1f (mean %.1f); K loop %.1f-%.1f (mean %.1f); epilogue "
+                  "%.1f-%.1f (mean %.1f); end %.1f-%.1f" % (label, start[m].min(), start[m].max(), pro[m].min(), pro[m].max(),
+                                                          pro[m].mean(), loop[m].min(), loop[m].max(), loop[m].mean(),
+                                                          epi[m].min(), epi[m].max(), epi[m].mean(), end[m].min(), end[m].max()))
+        _, per_cu = np.unique(key_cu[~band], return_counts=True)
+        print("  tiles per CU: " + ", ".join("%d CUs x %d" % (c, n) for n, c in zip(*np.unique(per_cu, return_counts=True))))
+        edges = np.arange(0, min(end.max(), 1000.0) + 5, 5)
+        hist, _ = np.histogram(end[~band], bins=edges)
+        print("  tiles ending in each 5 us: " + " ".join("%d" % h for h in hist))
+        one = np.where(key_cu == key_cu[np.argmin(start)])[0]
+        print("  one CU: " + "; ".join("%s start %.1f prologue %.1f loop %.1f epilogue %.1f end %.1f" % (
+            "band piece" if band[i] else "tile", start[i], pro[i], loop[i], epi[i], end[i]) for i in one[np.argsort(start[one])]))
+
+
 def main():
     global ZERO_OPERANDS, EAGER_ZERO, SETTLE_MS, REPS
     ap = argparse.ArgumentParser()
@@ -1028,7 +1084,8 @@ def main():
                     help="untimed work issued before every measurement so that it runs at the sustained clock "
                          "(0: start from an idle device)")
     ap.add_argument("--phases", action="store_true",
-                    help="only print the phase record of workload c3's three products (see phase_record)")
+                    help="only print the kernels' own phase record: of workload c3's three products (see phase_record), or, with "
+                         "--workload, of another workload's tiled launches (see tiled_phase_record)")
     ap.add_argument("--wide-diagnostic", choices=sorted(WIDE_DIAGNOSTICS), default=None,
                     help="with --phases: compile the fp16 kernel with one of its diagnostic switches into a scratch "
                          "library and print that build's phase record (see the header of deep8_amd/csrc/gemm_wide.hip)")
@@ -1057,7 +1114,7 @@ def main():
     if a.calibrate_copy:
         return calibrate_copy(a.calibrate_copy)
     if a.phases:
-        return phase_record()
+        return phase_record() if a.workload == "c3" else tiled_phase_record(a.workload)
 
     wl = make_workload(a.workload)
     ms, samples = _time_steps(wl.step, a.steps, a.warmup)

@@ -106,6 +106,7 @@ SIGNATURES = {
     "d8_avgpool2d_grad": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
     "d8_avgpool2d_grad_overwrite": (_I, [_I, _P, _P] + [_I] * 9 + [_P]),
     "d8_adam_update": (_I, [_I, _P, _P, _P, _P, _F, _F, _F, _F, _F, ctypes.c_long, ctypes.c_long, _P]),
+    "d8_gemm_phase_record": (_I, [_P, _Z]),
     "d8_mfma_stream_out_bytes": (_Z, []),
     "d8_mfma_stream": (_I, [_I, _P, _Z, _P, _I, ctypes.POINTER(ctypes.c_double), _P]),
 }

@@ -474,6 +474,24 @@ static int balanced_rows(const GemmArgs &g) {
     return (int)((tiles - rest) * 128);
 }
 
+// Pieces of a remainder band whose workgroups ride in the launch of the rows before it: they start as that launch's
+// first tiles retire and cost neither a launch nor a tile's prologue on an idle chip, so they may be short -- about one
+// piece per CU, two K steps at least (C4's band of 16 tiles over 18 steps: 4 / 6 / 9 pieces per tile gave
+// 0.2105 / 0.2065 / 0.2060 ms per Conv2d step, 18 pieces 0.2147).  0: the band does not ride along.
+static int plan_band_pieces(int BK, int rows, int N, int K, int red, size_t workspace_bytes, int *tiles_per_split) {
+    if (rows < 128) return 0;
+    const long total = (long)red * ceil_div(K, BK), tiles = (long)ceil_div(rows, 128) * ceil_div(N, 128);
+    long tps = ceil_div(total, (long)ceil_div((long)cu_count(), tiles));
+    if (tps < 2) tps = 2;
+    long splits = ceil_div(total, tps);
+    const long fit = (long)(workspace_bytes / ((size_t)rows * N * sizeof(float)));
+    if (splits > fit) splits = fit;
+    if (splits < 2) return 0;
+    tps = ceil_div(total, splits);
+    *tiles_per_split = (int)tps;
+    return (int)ceil_div(total, tps);
+}
+
 size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red, int virt) {
     int tps = 0;
     GemmArgs probe;
@@ -481,7 +499,11 @@ size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red, int virt) {
     probe.M = M, probe.N = N, probe.K = K, probe.batch = 1, probe.red = red;
     const int head = balanced_rows(probe);
     const int rows = head ? M - head : M;  // with a cut, only the second part is split
-    const int splits = plan_splits(gemm_tiled_k_step(dtype), rows, N, K, 1, red, (size_t)-1, &tps, virt);
+    int splits = plan_splits(gemm_tiled_k_step(dtype), rows, N, K, 1, red, (size_t)-1, &tps, virt);
+    if (head) {  // (the band may run either way: as pieces of the first part's launch or as a launch of its own)
+        const int riding = plan_band_pieces(gemm_tiled_k_step(dtype), rows, N, K, red, (size_t)-1, &tps);
+        if (riding > splits) splits = riding;
+    }
     return splits > 1 ? (size_t)splits * rows * N * sizeof(float) : 0;
 }
 
@@ -511,9 +533,10 @@ int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspa
     // one tile high; only its reduction is a launch of its own.
     const bool two_launches = getenv("D8_GEMM_BAND_LAUNCH") != nullptr;  // tuning and test aid (read at every call)
     second.ws = (float *)workspace;
-    second.splits = plan_splits(gemm_tiled_k_step(dtype), second.M, second.N, second.K, 1, second.red,
-                                (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0, &second.tiles_per_split);
-    if (!two_launches && second.splits > 1 && second.M >= 128 && g.splits == 1 && g.perm_OC == 0) {
+    second.splits = (two_launches || g.splits != 1 || g.perm_OC != 0) ? 0
+                    : plan_band_pieces(gemm_tiled_k_step(dtype), second.M, second.N, second.K, second.red,
+                                       (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0, &second.tiles_per_split);
+    if (second.splits > 1) {
         GemmArgs both = g;
         both.ws = second.ws;
         both.splits = 1;
@@ -603,6 +626,12 @@ static int gemm_one(int dtype, int transA, int transB, int M, int N, int K,
     }
     return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, tiled, as_stream(stream))
                                : launch<float>(g, transA, transB, tiled, as_stream(stream));
+}
+
+int d8_gemm_phase_record(void *records, size_t bytes) {
+    D8_REQUIRE(((size_t)records & 7) == 0, "d8_gemm_phase_record: the record buffer is not 8-byte aligned");
+    gemm_tiled_phase_record(records, bytes);
+    return 0;
 }
 
 int d8_gemm(int dtype, int transA, int transB, int M, int N, int K,

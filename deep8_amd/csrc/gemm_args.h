@@ -82,6 +82,11 @@ struct GemmArgs {
     // tile, each walking tail_tps K steps and writing fp32 partial sums to ws[piece][row - tail_m0][n].  They start
     // as the first workgroups retire, so the band costs a fraction of a tile's time instead of a launch of its own.
     int tail_m0, tail_splits, tail_tps;
+    // measurement aid of the tiled kernels (d8_gemm_phase_record): when set, every workgroup writes eight 64-bit words
+    // at index blockIdx.x + gridDim.x * blockIdx.z -- the chip's 100 MHz wall clock at its start, after its prologue,
+    // after its K loop and after its last store was acknowledged, the shader clock at both ends of the loop, its
+    // placement (XCC_ID << 32 | HW_ID) and whether it worked on the remainder band
+    unsigned long long *phase_rec;
 };
 
 // Whether a product with these arguments would run on a kernel that applies GemmArgs::bias / relu in its store
@@ -98,6 +103,8 @@ int gemm_tiled_k_step(int dtype);  // K elements per step: 64 (fp16) or 32 (fp32
 bool gemm_tiled_eligible(int dtype, const GemmArgs &g, int transA, int transB);
 // Launch; with g.splits > 1 the fp32 partial sums go to g.ws for the caller to reduce.
 int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipStream_t stream);
+// Where the next launches write their per-workgroup phase records (GemmArgs::phase_rec); null switches them off.
+void gemm_tiled_phase_record(void *records, size_t bytes);
 
 // fp16 kernel for large outputs (256 x 256 tiles, v_mfma_f32_16x16x32_f16, loads straight into
 // LDS): unsplit, unsummed products of real matrices with M, N >= 256 and K a multiple of 64.

@@ -343,6 +343,8 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / T::WGN, wn = wave % T::WGN;
+    unsigned long long st_w[4] = {0, 0, 0, 0}, st_c[2] = {0, 0};  // phase record (GemmArgs::phase_rec), a measurement aid
+    if (g.phase_rec) st_w[0] = wall_clock64();
 
     // ---- which tile: ids of one XCD (same id mod 8) form a contiguous run, runs are laid out in
     // bands of GM tile rows walked column by column
@@ -573,6 +575,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     for (int j = 0; j < TN; ++j)
         fb[0][j] = B_KC ? EL::read_kc(Bs0 + b_frag + j * T::B_BLK) : EL::read_tr(Bs0 + b_frag + j * 32, B_LD);
 
+    if (g.phase_rec) st_w[1] = wall_clock64(), st_c[0] = __builtin_readcyclecounter();
     // ---- main loop, two steps per trip so that the LDS half of every access is known statically;
     for (int i = 0; i < nsteps; i += 2) {
         {
@@ -587,6 +590,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         }
     }
 
+    if (g.phase_rec) st_w[2] = wall_clock64(), st_c[1] = __builtin_readcyclecounter();
     // ---- epilogue: the result itself, or this piece's fp32 partial sums when the reduction is split
     __syncthreads();  // every wave is past the last step: the operand areas are free
     const Origin o = {m0, n0, m_own, n_own, M, g.N, (wm * TM) * 32, (wn * TN) * 32};
@@ -600,10 +604,31 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     else
         store_tile<T, E>(acc, patches, patches1, (E *)g.C + (long)b * g.sC, g.ldc, g.beta,
                          g.ldc % EPV == 0 && g.sC % EPV == 0 && ((size_t)g.C & 15) == 0, g.N, o, crow, (const E *)g.bias, g.relu != 0);
+    if (g.phase_rec) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // this wave's stores have been acknowledged
+        st_w[3] = wall_clock64();
+        if (tid == 0) {
+            unsigned long long *rec = g.phase_rec + 8 * (blockIdx.x + (unsigned long long)gridDim.x * blockIdx.z);
+            rec[0] = st_w[0], rec[1] = st_w[1], rec[2] = st_w[2], rec[3] = st_w[3], rec[4] = st_c[0], rec[5] = st_c[1];
+            // s_getreg_b32 of all 32 bits of hardware registers 20 (XCC_ID) and 4 (HW_ID: wave, SIMD, CU, SH, SE)
+            rec[6] = ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
+            rec[7] = in_tail ? 1 : 0;
+        }
+    }
+}
+
+// where d8_gemm_phase_record asked the next launches to write their records (process-wide; null: no records)
+static unsigned long long *phase_rec_buf = nullptr;
+static size_t phase_rec_bytes = 0;
+
+void gemm_tiled_phase_record(void *records, size_t bytes) {
+    phase_rec_buf = (unsigned long long *)records;
+    phase_rec_bytes = records ? bytes : 0;
 }
 
 template <typename E, int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int VIRT>
-static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
+static int launch_tiled(const GemmArgs &g0, hipStream_t stream) {
+    GemmArgs g = g0;
     typedef Tile<E, BM, BN, WGM, WGN, A_KC, B_KC, VIRT> T;
     const bool tail = g.tail_splits > 0;  // (gemm_tiled_run sets it only for 128-row tiles and a tail_m0 that is a multiple of them)
     const int tilesM = ceil_div(tail ? g.tail_m0 : g.M, BM), tilesN = ceil_div(g.N, BN);
@@ -614,6 +639,8 @@ static int launch_tiled(const GemmArgs &g, hipStream_t stream) {
     const int layers = VIRT == VIRT_A_CLASSES ? g.ncls : g.batch * g.splits;  // for classes g.M is the largest one's
     const long wgs = (long)tilesM * tilesN * layers, cus = cu_count();
     const unsigned pad = (lds <= third && wgs > cus && wgs <= 2 * cus) ? (unsigned)(third + 512 - lds) : 0u;
+    // a launch whose records would not fit the caller's buffer writes none
+    g.phase_rec = (size_t)(tilesM * tilesN + extra) * layers * 64 <= phase_rec_bytes ? phase_rec_buf : nullptr;
     if (VIRT == VIRT_NONE && g.K % T::BK)
         hipLaunchKernelGGL((gemm_tiled_kernel<T, VIRT == VIRT_NONE>), dim3(tilesM * tilesN + extra, 1, layers), dim3(T::NT), pad, stream, g, tilesM, tilesN);
     else

@@ -392,6 +392,13 @@ int d8_avgpool2d_grad_overwrite(int dtype, void *dx, const void *dy, int B, int 
  * 48 bytes per 256 x 256 tile of C leaves there, per workgroup, six 64-bit values: the chip's 100 MHz wall
  * clock at its start, after its prologue, after its K loop and after its last store was acknowledged, and
  * the shader clock before and after the loop.                                                          */
+/* A third one, for the tiled kernels (fp16 / fp32 products and the convolutions they carry): after
+ * d8_gemm_phase_record(records, bytes) every tiled launch whose records fit leaves 64 bytes per workgroup in
+ * `records` (a device buffer, 8-byte aligned; index = workgroup id x + grid size x * id z): the same four wall
+ * clock values and two shader clock values, then (XCC_ID << 32 | HW_ID) of the wave that wrote them and 1 if the
+ * workgroup worked on a remainder band.  Each launch writes from index 0, so read the buffer between launches.
+ * records = null switches the records off again.  Process-wide and not thread-safe: a tool for one measuring thread. */
+int d8_gemm_phase_record(void *records, size_t bytes);
 size_t d8_mfma_stream_out_bytes(void);
 int d8_mfma_stream(int dtype, const void *operands, size_t operand_bytes, void *out, int iters,
                    double *flops, void *stream);

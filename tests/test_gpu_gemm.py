@@ -268,6 +268,7 @@ def test_gemm_reduction_not_a_multiple_of_the_k_step(ta, tb, M, N, K, dtype):
     (0, 1, 98304 + 128, 64, 64),  # a band of exactly one tile
     (0, 1, 98304 + 100, 96, 64),  # a band shorter than a tile: runs as a product of its own
     (0, 0, 131072 + 2048, 64, 32),
+    (0, 1, 100352, 64, 576),   # 16 band tiles over 18 (fp32) / 9 (fp16) K steps: nine / five pieces per tile ride along
 ])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_gemm_tall_product_with_a_remainder_band(ta, tb, M, N, K, dtype, monkeypatch):
@@ -287,3 +288,37 @@ def test_gemm_tall_product_with_a_remainder_band(ta, tb, M, N, K, dtype, monkeyp
         for beta, C in ((0.0, None), (1.0, C0)):
             got = ops.gemm(ta, tb, c(A), c(B), None if C is None else c(C), beta)
             assert np.array_equal(f(got), prod + (0 if C is None else C)), (band_launch, beta)
+
+
+@pytest.mark.gpu
+def test_gemm_phase_record_of_the_tiled_kernels():
+    """d8_gemm_phase_record: a tiled launch leaves one record per workgroup (clock values in order, band pieces
+    marked), the product is the same with and without it, a buffer that is too small stays untouched, and null
+    switches the records off."""
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    r = rng(77)
+    M, N, K = 98304 + 2048, 64, 256
+    A, B = ints(r, (M, K), 3), ints(r, (K, N), 3)
+    want = A @ B
+    nrec = 1024
+    rec = capi.DeviceArray((nrec * 8,), np.uint64, zero=True)
+    try:
+        capi.check(lib.d8_gemm_phase_record(rec.ptr, nrec * 64))
+        got = ops.gemm(0, 0, A, B)
+        v = rec.numpy().astype(np.int64).reshape(nrec, 8)
+        done = v[v[:, 3] != 0]
+        band = done[:, 7] == 1
+        assert len(done) == 768 + band.sum() and band.sum() >= 32, (len(done), band.sum())
+        assert (done[:, 0] <= done[:, 1]).all() and (done[:, 1] <= done[:, 2]).all() and (done[:, 2] <= done[:, 3]).all()
+        assert (done[:, 5] > done[:, 4]).all()
+        assert np.array_equal(got, want)
+        small = capi.DeviceArray((64,), np.uint64, zero=True)
+        capi.check(lib.d8_gemm_phase_record(small.ptr, 64 * 8))  # 8 records: the launch has more workgroups
+        assert np.array_equal(ops.gemm(0, 0, A, B), want)
+        assert not small.numpy().any()
+    finally:
+        capi.check(lib.d8_gemm_phase_record(None, 0))
+    rec.zero_()
+    assert np.array_equal(ops.gemm(0, 0, A, B), want)
+    assert not rec.numpy().any()
