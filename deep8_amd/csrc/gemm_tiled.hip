@@ -133,10 +133,14 @@ struct Tile {
     // 16-byte pieces each thread moves per K step, and the rows one pass of all threads covers
     static constexpr int A_IT = BM * 8 / NT, B_IT = BN * 8 / NT, NP = A_IT + B_IT;
     static constexpr int A_ROWS = A_KC ? NT / 8 : NT / (BM / EPV);
-    static constexpr int B_ROWS = B_KC ? NT / 8 : NT / (BN / EPV);
+    // Patch k-rows as B, fp32: the threads' passes walk the tile's columns instead of its rows -- a pass is all BK k-rows
+    // x 32 columns, so a thread keeps ONE patch row per K step, decoded once, and its pieces differ by tap and channel
+    // (an add and a bounds check each).  Decoding a row per piece cost Conv2d C4's filter gradient 11 of its 74 us.
+    static constexpr bool B_COLS = VIRT == VIRT_B_KROWS && ES == 4 && NT / 8 == BK;
+    static constexpr int B_ROWS = B_COLS ? BK : B_KC ? NT / 8 : NT / (BN / EPV);
     static_assert(A_ROWS % 2 == 0 && B_ROWS % 2 == 0, "a pass of all threads starts on an even row");
     // elements between the pieces two consecutive passes write, and between a wave's 32-row blocks
-    static constexpr int A_PASS = A_KC ? kc_row(A_ROWS) : A_ROWS * A_LD, B_PASS = B_KC ? kc_row(B_ROWS) : B_ROWS * B_LD;
+    static constexpr int A_PASS = A_KC ? kc_row(A_ROWS) : A_ROWS * A_LD, B_PASS = B_COLS ? 8 * EPV : B_KC ? kc_row(B_ROWS) : B_ROWS * B_LD;
     static constexpr int A_BLK = A_KC ? KC_BLK : 32, B_BLK = B_KC ? KC_BLK : 32;
     static constexpr int A_RD = A_KC ? 1 : EL::TR_READS, B_RD = B_KC ? 1 : EL::TR_READS;
     // the epilogue's transposing patches reuse the two halves of the larger operand area: the first
@@ -428,7 +432,7 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     const unsigned Au = (unsigned)ES * (A_KC ? (unsigned)m0 * g.lda : (unsigned)m0);
     const unsigned Bu = (unsigned)ES * (B_KC ? (unsigned)n0 * g.ldb : (unsigned)n0);
     const int a_r = A_KC ? tid >> 3 : tid / (BM / EPV), a_c = A_KC ? tid & 7 : tid % (BM / EPV);
-    const int b_r = B_KC ? tid >> 3 : tid / (BN / EPV), b_c = B_KC ? tid & 7 : tid % (BN / EPV);
+    const int b_r = (B_KC || T::B_COLS) ? tid >> 3 : tid / (BN / EPV), b_c = (B_KC || T::B_COLS) ? tid & 7 : tid % (BN / EPV);
     const int a_dst = (A_KC ? T::kc_row(a_r) : a_r * A_LD) + a_c * EPV, b_dst = (B_KC ? T::kc_row(b_r) : b_r * B_LD) + b_c * EPV;
     const unsigned a_pass = VA ? 0u : (unsigned)ES * T::A_ROWS * g.lda;  // bytes
     const unsigned b_pass = VIRT == VIRT_B_KROWS ? 0u : (unsigned)ES * T::B_ROWS * g.ldb;
@@ -456,8 +460,18 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         }
     }
     // patch k-rows as B: this thread's tap and channel never change; a step selects the rows
+    // (with column passes, Tile::B_COLS: this thread's k-row within the step never changes; piece p has its own tap and channel)
     int vb_dy = 0, vb_dx = 0, vb_c = 0;
-    if constexpr (VIRT == VIRT_B_KROWS) {
+    int vb_ty[B_IT], vb_tx[B_IT], vb_off[B_IT];
+    if constexpr (T::B_COLS) {
+#pragma unroll
+        for (int p = 0; p < B_IT; ++p) {
+            const int n = n0 + p * T::B_PASS + b_c * EPV, t = n / pg.C, fy = t / pg.FW, fx = t - fy * pg.FW;
+            vb_ty[p] = fy * pg.dy;
+            vb_tx[p] = fx * pg.dx;
+            vb_off[p] = ((vb_ty[p] * pg.W + vb_tx[p]) * pg.C + (n - t * pg.C)) * ES;
+        }
+    } else if constexpr (VIRT == VIRT_B_KROWS) {
         const int n = n0 + b_c * EPV, t = n / pg.C, fy = t / pg.FW, fx = t - fy * pg.FW;
         vb_c = n - t * pg.C;
         vb_dy = fy * pg.dy - pg.pt;
@@ -516,7 +530,21 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     };
     auto step_b = [&](int i) -> unsigned {
         const int x = x0 + min(i, nsteps - 1), r = x / ktiles;
-        if constexpr (VIRT == VIRT_B_KROWS) {
+        if constexpr (T::B_COLS) {
+            const unsigned plane = pg.OH * pg.OW, m = (unsigned)x * BK + b_r;
+            unsigned img = __umulhi(m, pg.mg_plane), rem = m - img * plane;
+            if (rem >= plane) ++img, rem -= plane;
+            unsigned oy = __umulhi(rem, pg.mg_ow), ox = rem - oy * pg.OW;
+            if (ox >= (unsigned)pg.OW) ++oy, ox -= pg.OW;
+            const int iy0 = (int)oy * pg.sy - pg.pt, ix0 = (int)ox * pg.sx - pg.pl;
+            const int base = (((int)img * pg.H + iy0) * pg.W + ix0) * pg.C * ES;
+#pragma unroll
+            for (int p = 0; p < B_IT; ++p) {
+                const bool inside = (unsigned)(iy0 + vb_ty[p]) < (unsigned)pg.H && (unsigned)(ix0 + vb_tx[p]) < (unsigned)pg.W;
+                bv[p] = inside ? (unsigned)(base + vb_off[p]) : OUTSIDE;
+            }
+            return 0u;
+        } else if constexpr (VIRT == VIRT_B_KROWS) {
             const unsigned plane = pg.OH * pg.OW;
 #pragma unroll
             for (int p = 0; p < B_IT; ++p) {
