@@ -136,6 +136,12 @@ struct Operand {
     }
 };
 
+// Order of a k group's 64 MFMAs over the wave's 8 x 8 blocks: row by row, every other row backwards, so that each MFMA
+// differs from the one before it in ONE operand (the A fragment stays for a row, the B fragment at a row's end).  The
+// kernel is power-limited, and the order is measurable: forward 4096^3 102.3 us row by row, 101.6 this way, 105.0
+// with both operands changing every time.  (Each block still sums its k values in the same order.)
+#define BI(m) ((m) >> 3)
+#define BJ(m) ((((m) >> 3) & 1) ? 7 - ((m) & 7) : ((m) & 7))
 __device__ __forceinline__ void mfma(f32x4 &acc, const f16x8 &a, const f16x8 &b) {
 #ifdef D8_WIDE_DIAG_DIRECT_STORE
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %2, %1, %0" : "+a"(acc) : "v"(a), "v"(b));
@@ -236,7 +242,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
         // half 0
 #pragma unroll
         for (int m = 0; m < 64; ++m) {
-            mfma(acc[m >> 3][m & 7], fa[0][m >> 3], fb[0][m & 7]);
+            mfma(acc[BI(m)][BJ(m)], fa[0][BI(m)], fb[0][BJ(m)]);
             if (m % 3 == 0 && m < 48) {
                 const int e = m / 3;  // 16 reads: the B fragments first (all needed by the first row)
                 if (e < 8) fb[1][e] = ob.read(Bs, 1, e);
@@ -267,7 +273,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
                 if ((m >> 2) < 8) oa.aim_round(As, wave, m >> 2);
                 else ob.aim_round(Bs, wave, (m >> 2) - 8);
             }
-            mfma(acc[m >> 3][m & 7], fa[1][m >> 3], fb[1][m & 7]);
+            mfma(acc[BI(m)][BJ(m)], fa[1][BI(m)], fb[1][BJ(m)]);
             if ((m & 3) == 0) {
                 // 16 loads into the stage every wave has finished with, one per 4 MFMAs: a load
                 // keeps the CU's address path busy for 16 cycles, as long as an MFMA runs, and all
