@@ -263,6 +263,35 @@ IMPLICIT = [
 ]
 
 
+@pytest.mark.parametrize("IC,FH,FW,dil", [(4, 7, 7, 1), (8, 5, 5, 1), (12, 5, 3, 2), (20, 3, 3, 1), (40, 2, 2, 1), (96, 3, 3, 1)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_conv2d_filter_gradient_with_few_input_channels(oracle_port, monkeypatch, IC, FH, FW, dil, dtype):
+    """The filter gradient's patch loader where one 32-column pass of a tile spans several taps (fewer than 32
+    input channels) or straddles a tap's end (40, 96): bit for bit against the oracle on integers, accumulate and
+    overwrite forms, on the route that stages nothing."""
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    B, IH, IW, OC = 2, 16, 16, 64
+    a = (True, 1, 1, dil, dil)
+    OH, OW, _, _ = ops.conv2d_geometry(IH, IW, FH, FW, *a)
+    if IC % (16 // np.dtype(dtype).itemsize) == 0:  # the channels of a tap move in 16-byte pieces
+        q = lambda: lib.d8_conv2d_scratch_bytes(capi.dtype_id(np.dtype(dtype)), 2, B, IH, IW, IC, OC, FH, FW, 1, 1, 1, dil, dil)
+        monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+        explicit = q()
+        monkeypatch.delenv("D8_CONV_EXPLICIT")
+        assert q() < explicit, (q(), explicit)
+    r = rng(IC + FH)
+    c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
+    hi = 3 if dtype == np.float16 else 20
+    x, w, gz = ints(r, (B, IH, IW, IC), hi), ints(r, (OC, FH, FW, IC), hi), ints(r, (B, OH, OW, OC), hi)
+    if dtype == np.float16:
+        x, gz = x * (r.random(x.shape) < 0.3), gz * (r.random(gz.shape) < 0.1)
+    want = oracle_port.conv2d_grad_y(x, w, gz, *a, w)
+    assert dtype == np.float32 or np.abs(want).max() < 2048
+    assert np.array_equal(f(ops.conv2d_grad_y(c(x), c(w), c(gz), *a, c(w))), want)
+    assert np.array_equal(f(ops.conv2d_grad_y(c(x), c(w), c(gz), *a, c(w), overwrite=True)), want - w)
+
+
 @pytest.mark.parametrize("cfg,imp32,imp16", IMPLICIT)
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_conv2d_implicit_route(oracle_port, monkeypatch, cfg, imp32, imp16, dtype):
