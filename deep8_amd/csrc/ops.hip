@@ -80,6 +80,8 @@ static int check_mm(const char *who, int dtype, int xb, int xr, int xc, int yb, 
     D8_REQUIRE(xb > 0 && xr > 0 && xc > 0 && yb > 0 && yr > 0 && yc > 0, "%s: sizes must be positive", who);
     D8_REQUIRE(xb == yb || xb == 1 || yb == 1, "%s: batch %d vs %d", who, xb, yb);
     D8_REQUIRE(xc == yr, "%s: inner dimensions %d vs %d", who, xc, yr);
+    // (a shared y collapses x's batch into the rows of one product, whose row count is an int)
+    D8_REQUIRE((long)xb * xr < (1L << 31), "%s: %d x %d rows of x exceed 2^31 - 1", who, xb, xr);
     return 0;
 }
 
@@ -112,6 +114,10 @@ static int check_conv(const char *who, int dtype, int B, int IH, int IW, int IC,
         return fail(D8_ERR_DTYPE, "%s: element type %d is not supported", who, dtype);
     D8_REQUIRE(B > 0 && IH > 0 && IW > 0 && IC > 0 && OC > 0 && FH > 0 && FW > 0, "%s: sizes must be positive", who);
     D8_REQUIRE(sy >= 1 && sx >= 1 && dy >= 1 && dx >= 1, "%s: the stride and dilation must >= 1", who);
+    // row and column counts of the products are ints: pixels of the batch, elements of a patch row / of a filter's taps
+    D8_REQUIRE((long)B * IH * IW < (1L << 31) && (long)FH * FW * IC < (1L << 31) && (long)FH * FW * OC < (1L << 31),
+               "%s: %d x %d x %d pixels or a %d x %d filter over %d -> %d channels exceed 2^31 - 1 rows or columns", who, B, IH, IW, FH,
+               FW, IC, OC);
     return 0;
 }
 
@@ -602,9 +608,15 @@ static int check_deconv_geo(const char *who, const int *geo) {
     D8_REQUIRE(geo[0] > 0 && geo[1] > 0 && geo[2] >= 0 && geo[3] >= 0, "%s: output %d x %d, pads %d / %d", who, geo[0], geo[1], geo[2], geo[3]);
     return 0;
 }
+// ... and the output's pixel count is an int as well
+static int check_deconv_out(const char *who, int B, const int *geo) {
+    D8_REQUIRE((long)B * geo[0] * geo[1] < (1L << 31), "%s: %d x %d x %d output pixels exceed 2^31 - 1", who, B, geo[0], geo[1]);
+    return 0;
+}
 
 static size_t deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                      int OC, int FH, int FW, const int *geo, int sy, int sx) {
+    if (check_deconv_out("d8_deconv2d_scratch_bytes", B, geo)) return 0;
     const int M = B * IH * IW, T = FH * FW;
     GemmArgs ga;
     if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
@@ -638,6 +650,7 @@ static int deconv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(x && w && z, "d8_deconv2d: null tensor");
+    if (int rc = check_deconv_out("d8_deconv2d", B, g)) return rc;
     {
         GemmArgs ga;
         if (deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, w, z, ga))
@@ -677,6 +690,7 @@ static int deconv2d_grad_x_geo(int dtype, void *gx, int B, int IH, int IW, int I
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(gx && w && gz, "d8_deconv2d_grad_x: null tensor");
+    if (int rc = check_deconv_out("d8_deconv2d_grad_x", B, g)) return rc;
     {
         GemmArgs ga;
         if (deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, gx, w, gz, ga)) {
@@ -720,6 +734,7 @@ static int deconv2d_grad_y_geo(int dtype, const void *x, int B, int IH, int IW, 
     const int M = B * IH * IW, T = FH * FW;
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     D8_REQUIRE(x && gw && gz, "d8_deconv2d_grad_y: null tensor");
+    if (int rc = check_deconv_out("d8_deconv2d_grad_y", B, g)) return rc;
     {
         GemmArgs ga;
         if (deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, gw, gz, ga)) {

@@ -635,3 +635,19 @@ def test_conv2d_tensor_view_at_an_odd_offset(oracle_port):
     assert np.array_equal(gx_raw.numpy()[1:].reshape(x.shape), want[1])
     check(lib.d8_conv2d_grad_y(capi.FLOAT32, raw.ptr + 4, B, IH, IH, IC, gw.ptr, OC, F, F, dgz.ptr, *args, ws.ptr, nb, None))
     assert np.array_equal(gw.numpy(), want[2])
+
+
+def test_conv_sizes_beyond_int_range_are_refused():
+    """Pixel and patch-row counts are ints inside the library: a geometry whose products pass 2^31 - 1 is refused
+    with a message (no launch), by the operators and by their scratch queries alike."""
+    from deep8_amd import capi
+    lib = capi.init()
+    a = capi.DeviceArray((64,), np.float32, zero=True)
+    big = (capi.FLOAT32, a.ptr, 40000, 300, 300, 4, a.ptr, 4, 3, 3, a.ptr)  # 3.6e9 pixels
+    assert lib.d8_conv2d(*big, 1, 1, 1, 1, 1, None, 0, None) == 10001 and b"exceed" in lib.d8_last_error()
+    assert lib.d8_conv2d_scratch_bytes(capi.FLOAT32, 0, 40000, 300, 300, 4, 4, 3, 3, 1, 1, 1, 1, 1) == 0
+    assert lib.d8_deconv2d(*big, 0, 2, 2, None, 0, None) == 10001 and b"exceed" in lib.d8_last_error()
+    # a DeConv2d whose input fits but whose output does not: 2e9 input pixels x stride 2 x 2
+    assert lib.d8_deconv2d(capi.FLOAT32, a.ptr, 20000, 300, 300, 4, a.ptr, 4, 2, 2, a.ptr, 0, 2, 2, None, 0, None) == 10001
+    assert b"output pixels" in lib.d8_last_error()
+    assert lib.d8_deconv2d_scratch_bytes(capi.FLOAT32, 0, 20000, 300, 300, 4, 4, 2, 2, 0, 2, 2) == 0
