@@ -372,10 +372,15 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_scalar_kernel(GemmArgs 
     }
 }
 
-bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps) {
+bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps, int BK) {
     if (M < 128 || N < 128) return false;
     const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch, cus = cu_count();
-    return tiles < cus && 4 * tiles >= cus && k_steps <= 32;
+    if (tiles >= cus || 4 * tiles < cus) return false;
+    if (k_steps <= 32) return true;
+    // fp32 (K steps of 32), twice as long a reduction, when the half tiles still give every CU one: 1024 x 2048 x 2048
+    // 77.4 -> 64.9 us, 1280 x 1280 x 2048 74.4 -> 64.2, 1024 x 2048 x 1536 64.2 -> 50.5 (with fewer half tiles than
+    // CUs splitting the reduction stays better: 1024 x 1024 x 2048 46.9 us against 63.4)
+    return BK == 32 && 2 * tiles >= cus && k_steps <= 64;
 }
 
 // How many pieces to cut the reduction into, for a kernel whose K step is BK.  Splitting is only
@@ -399,7 +404,7 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     // A short reduction over an output that half-height tiles spread over most of the chip is better
     // left whole: the tiled kernel then takes 64 x 128 tiles (gemm_tiled_half_tiles) and the fp32
     // partial sums, their round trip through memory and the second launch are saved.
-    if (gemm_tiled_half_tiles(M, N, batch, total)) splits = 1;
+    if (gemm_tiled_half_tiles(M, N, batch, total, BK)) splits = 1;
     static const char *force = getenv("D8_GEMM_SPLITS");  // tuning aid
     if (force && splits > 1) splits = atoi(force);
     // Every piece costs a tile's prologue, a tile of fp32 partial sums written and read back: at least 8 K steps
@@ -409,6 +414,29 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     if (max_by_len < 1) max_by_len = 1;
     if (splits > max_by_len) splits = max_by_len;
     if (splits > 512) splits = 512;
+    // The rules above aim at a workgroup or two per CU; how the pieces then fall into rounds matters as much.  A CU's
+    // share is ceil(tiles * s / CUs) pieces of ceil(total / s) steps (+ a prologue and an epilogue each), and the
+    // second pass costs a launch plus the s partial sums read back: 98 tiles over 72 steps (Conv2d 14 x 14 x 256,
+    // fp32) take 36 / 48 / 36 / 30 / 36 steps per CU for s = 2 .. 6 and ran 83.9 / 103.3 / 82.9 / 72.8 / 86.9 us; 52
+    // tiles over 144 steps (7 x 7 x 512) 146 / 102 / 80.7 / 116 / 100 us for s = 2 .. 6.  Among the piece counts the
+    // length rule admits, take the cheapest by that count, the rules' own choice on a tie.  In units of a K step
+    // (about 2 us of a CU's time in fp32, 0.5 us in half): prologue + epilogue 2.5 / 7 steps, the second launch 2 / 6,
+    // a partial sum read back at some 4 TB/s.
+    if (!t64 && !force && splits > 1 && tiles < cus) {
+        const bool half = BK == 64;
+        const double ends = half ? 7.0 : 2.5, second = half ? 6.0 : 2.0, per_split = (double)M * N * batch / (half ? 0.5e6 : 2e6);
+        auto cost = [&](long s) {
+            const long rounds = (tiles * s + cus - 1) / cus, len = (total + s - 1) / s;
+            // (a workgroup alone on its CU walks its steps about a tenth slower than two that share one)
+            return rounds * (len * (rounds == 1 ? 1.1 : 1.0) + ends) + second + s * per_split;
+        };
+        long best = splits;
+        double best_cost = cost(splits) * 0.97;
+        const long top = max_by_len < 512 ? max_by_len : 512;
+        for (long c = 2; c <= top; ++c)
+            if (cost(c) < best_cost) best = c, best_cost = cost(c);
+        splits = best;
+    }
     // no more pieces than the caller's workspace holds
     const size_t per_split = (size_t)batch * M * N * sizeof(float);
     const long fit = (long)(workspace_bytes / per_split);

@@ -120,7 +120,7 @@ int gemm_f64_splits(int M, int N, int K, int batch, int red, size_t workspace_by
 // Whether an unsplit product of this shape should run on 64 x 128 tiles: too few 128 x 128 tiles
 // for the chip, enough half-height ones, and a reduction (k_steps K steps in all) too short to
 // be worth splitting.
-bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps);
+bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps, int BK);
 
 // Plan the split of the reduction, launch the tiled kernel (which must be eligible) and reduce.
 int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,

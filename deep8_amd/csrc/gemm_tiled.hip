@@ -699,7 +699,7 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
         if (gemm_tiled_krows_64(VIRT, g.M, g.N)) return launch_tiled<E, 64, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
     }
     if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
-    if (g.splits == 1 && gemm_tiled_half_tiles(g.M, g.N, g.batch, (long)g.red * ceil_div(g.K, 128 / (int)sizeof(E))))
+    if (g.splits == 1 && gemm_tiled_half_tiles(g.M, g.N, g.batch, (long)g.red * ceil_div(g.K, 128 / (int)sizeof(E)), 128 / (int)sizeof(E)))
         return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
     return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
 }
