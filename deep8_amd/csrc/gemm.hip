@@ -372,15 +372,70 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_scalar_kernel(GemmArgs 
     }
 }
 
+// ---- planning a product whose 128 x 128 tiles are fewer than the CUs -----------------------------------------
+// Three ways to spread it: cut the reduction into s pieces per tile (a second pass adds them up), run it whole on
+// 64 x 128 tiles (twice as many workgroups, no second pass), or leave it.  Rules of thumb give a first choice --
+// a workgroup or two per CU, pieces of at least 8 K steps -- and a count of steps per CU decides among the
+// admitted alternatives, because how the workgroups fall into rounds matters as much as how many there are: a
+// CU's share is ceil(workgroups / CUs) pieces of ceil(total / s) steps plus a prologue and an epilogue each, a
+// workgroup alone on its CU walks its steps about a tenth slower than two that share one, a half tile's step is
+// half a step (0.65 in half precision), and the second pass costs a launch plus the s partial sums read back (at some 4 TB/s).  In units
+// of a K step (about 2 us of a CU's time in fp32, 0.5 us in half): prologue + epilogue 2.5 / 7, second pass 2 / 14.
+// Measured against it: Conv2d 14 x 14 x 256 fp32, 98 tiles over 72 steps, 36 / 48 / 36 / 30 / 36 steps per CU for
+// s = 2 .. 6, ran 83.9 / 103.3 / 82.9 / 72.8 / 86.9 us; 7 x 7 x 512, 52 tiles over 144 steps, 146 / 102 / 80.7 / 116 /
+// 100 us for s = 2 .. 6; 1024 x 2048 x 2048 fp32 64.9 us on half tiles against 77.4 in two pieces, 1024 x 1024 x 2048
+// 63.4 us on (128) half tiles against 43.9 in four pieces.
+struct FewTiles {
+    long splits;  // pieces per tile (1: unsplit)
+    bool half;    // unsplit on 64 x 128 tiles
+};
+
+static long piece_limit(long tiles, long total, int cus) {
+    // Every piece costs a tile's prologue, a tile of fp32 partial sums written and read back: at least 8 K steps
+    // per piece, or 4 where 8 would leave more than half of the CUs without a workgroup.
+    long most = total / 8;
+    if (most * tiles < cus / 2) most = total / 4;
+    if (most > 512) most = 512;
+    return most < 1 ? 1 : most;
+}
+
+static FewTiles plan_few_tiles(int BK, int M, int N, int batch, long total) {
+    const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch, cus = cu_count();
+    // the rules' choice: at most two workgroups per CU (a third one would run alone, after the rest) ...
+    long rule = 2L * cus / tiles;
+    // ... one per CU where its pieces are then still 32 K steps or longer: as fast, and half the partial sums (C2b's
+    // dY, 512 x 512 over 16 384: 72.8 -> 70.6 us)
+    if (M >= 128 && N >= 128 && total / (cus / tiles) >= 32) rule = cus / tiles;
+    const long most = piece_limit(tiles, total, (int)cus);
+    if (rule > most) rule = most;
+    if (rule < 1) rule = 1;
+    const bool half_elems = BK == 64;
+    const double ends = half_elems ? 7.0 : 2.5, second = half_elems ? 14.0 : 2.0;
+    const double per_split = (double)M * N * batch / (half_elems ? 0.5e6 : 2e6);
+    auto cost = [&](long s) {
+        const long rounds = (tiles * s + cus - 1) / cus, len = (total + s - 1) / s;
+        return rounds * (len * (rounds == 1 ? 1.1 : 1.0) + ends) + (s > 1 ? second + s * per_split : 0.0);
+    };
+    FewTiles best = {rule, false};
+    double best_cost = cost(rule) * 0.97;  // the rules' own choice on a tie
+    for (long c = 1; c <= most; ++c)
+        if (cost(c) < best_cost) best.splits = c, best_cost = cost(c);
+    // half tiles: a short reduction over an output that they spread over most of the chip saves the fp32 partial
+    // sums, their round trip through memory and the second launch (C5's dX, 98 tiles over 16 steps: 16.8 + 10.9 us
+    // in four pieces, 11.3 us whole on 196 half tiles)
+    if (M >= 128 && N >= 128 && 4 * tiles >= cus) {
+        const long rounds = (2 * tiles + cus - 1) / cus;
+        // (a 64 x 128 tile's step against a 128 x 128 tile's: half the MFMAs; 0.65 in half, where the rest of the step weighs more)
+        const double c = rounds * ((half_elems ? 0.65 : 0.5) * total * (rounds == 1 ? 1.1 : 1.0) + ends);
+        if (c < best_cost) best = {1, true};
+    }
+    return best;
+}
+
 bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps, int BK) {
     if (M < 128 || N < 128) return false;
-    const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch, cus = cu_count();
-    if (tiles >= cus || 4 * tiles < cus) return false;
-    if (k_steps <= 32) return true;
-    // fp32 (K steps of 32), twice as long a reduction, when the half tiles still give every CU one: 1024 x 2048 x 2048
-    // 77.4 -> 64.9 us, 1280 x 1280 x 2048 74.4 -> 64.2, 1024 x 2048 x 1536 64.2 -> 50.5 (with fewer half tiles than
-    // CUs splitting the reduction stays better: 1024 x 1024 x 2048 46.9 us against 63.4)
-    return BK == 32 && 2 * tiles >= cus && k_steps <= 64;
+    const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
+    return tiles < cu_count() && plan_few_tiles(BK, M, N, batch, k_steps).half;
 }
 
 // How many pieces to cut the reduction into, for a kernel whose K step is BK.  Splitting is only
@@ -396,46 +451,18 @@ static int plan_splits(int BK, int M, int N, int K, int batch, int red, size_t w
     }
     const int cus = cu_count();
     long splits = 1;
-    if (tiles < cus) splits = 2L * cus / tiles;  // at most two workgroups per CU: a third one would run alone, after the rest
-    if (tiles < cus && t64) splits = 3L * cus / tiles;  // three of the small tiles per CU (56 / 85 / 113 / 140 pieces on C4's dW: 75.6 / 73.8 / 75.0 / 78.5 us)
-    // 128 x 128 tiles over a long reduction: one workgroup per CU with pieces of 32 K steps or more runs as fast as two
-    // with half as many, and halves the partial sums (C2b's dY, 512 x 512 over 16 384: 72.8 -> 70.6 us)
-    if (tiles < cus && M >= 128 && N >= 128 && total / (cus / tiles) >= 32) splits = cus / tiles;
-    // A short reduction over an output that half-height tiles spread over most of the chip is better
-    // left whole: the tiled kernel then takes 64 x 128 tiles (gemm_tiled_half_tiles) and the fp32
-    // partial sums, their round trip through memory and the second launch are saved.
-    if (gemm_tiled_half_tiles(M, N, batch, total, BK)) splits = 1;
-    static const char *force = getenv("D8_GEMM_SPLITS");  // tuning aid
-    if (force && splits > 1) splits = atoi(force);
-    // Every piece costs a tile's prologue, a tile of fp32 partial sums written and read back: at least 8 K steps
-    // per piece, or 4 where 8 would leave more than half of the CUs without a workgroup.
-    long max_by_len = total / 8;
-    if (max_by_len * tiles < cus / 2) max_by_len = total / 4;
-    if (max_by_len < 1) max_by_len = 1;
-    if (splits > max_by_len) splits = max_by_len;
-    if (splits > 512) splits = 512;
-    // The rules above aim at a workgroup or two per CU; how the pieces then fall into rounds matters as much.  A CU's
-    // share is ceil(tiles * s / CUs) pieces of ceil(total / s) steps (+ a prologue and an epilogue each), and the
-    // second pass costs a launch plus the s partial sums read back: 98 tiles over 72 steps (Conv2d 14 x 14 x 256,
-    // fp32) take 36 / 48 / 36 / 30 / 36 steps per CU for s = 2 .. 6 and ran 83.9 / 103.3 / 82.9 / 72.8 / 86.9 us; 52
-    // tiles over 144 steps (7 x 7 x 512) 146 / 102 / 80.7 / 116 / 100 us for s = 2 .. 6.  Among the piece counts the
-    // length rule admits, take the cheapest by that count, the rules' own choice on a tie.  In units of a K step
-    // (about 2 us of a CU's time in fp32, 0.5 us in half): prologue + epilogue 2.5 / 7 steps, the second launch 2 / 6,
-    // a partial sum read back at some 4 TB/s.
-    if (!t64 && !force && splits > 1 && tiles < cus) {
-        const bool half = BK == 64;
-        const double ends = half ? 7.0 : 2.5, second = half ? 6.0 : 2.0, per_split = (double)M * N * batch / (half ? 0.5e6 : 2e6);
-        auto cost = [&](long s) {
-            const long rounds = (tiles * s + cus - 1) / cus, len = (total + s - 1) / s;
-            // (a workgroup alone on its CU walks its steps about a tenth slower than two that share one)
-            return rounds * (len * (rounds == 1 ? 1.1 : 1.0) + ends) + second + s * per_split;
-        };
-        long best = splits;
-        double best_cost = cost(splits) * 0.97;
-        const long top = max_by_len < 512 ? max_by_len : 512;
-        for (long c = 2; c <= top; ++c)
-            if (cost(c) < best_cost) best = c, best_cost = cost(c);
-        splits = best;
+    if (tiles < cus) {
+        if (t64) {
+            // three of the small tiles per CU (56 / 85 / 113 / 140 pieces on C4's dW: 75.6 / 73.8 / 75.0 / 78.5 us)
+            splits = 3L * cus / tiles;
+            const long most = piece_limit(tiles, total, cus);
+            if (splits > most) splits = most;
+        } else {
+            const FewTiles plan = plan_few_tiles(BK, M, N, batch, total);
+            splits = plan.half ? 1 : plan.splits;  // (half: the tiled kernel asks gemm_tiled_half_tiles itself)
+        }
+        static const char *force = getenv("D8_GEMM_SPLITS");  // tuning aid
+        if (force && splits > 1) splits = atoi(force);
     }
     // no more pieces than the caller's workspace holds
     const size_t per_split = (size_t)batch * M * N * sizeof(float);
