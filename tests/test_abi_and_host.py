@@ -84,3 +84,31 @@ def test_bench_reads_its_traffic_figures_from_the_committed_profiles():
             assert t is not None and t["bytes"] > 0, (key, part)
     # the algorithmic bytes of the im2col launch at configuration 4's size are what the counters saw
     assert abs(bench.profile_traffic("i4", "im2col")["bytes"] - 256.9e6) < 2e6
+
+
+def test_planner_keeps_the_plans_of_the_baseline_configs():
+    """The split planner's choices for the BASELINE configurations, read off the scratch queries (host code only; with
+    no device the planner assumes the MI355X's 256 CUs): a change of its rules or constants that moves one of them
+    shows up here before it shows up in a benchmark."""
+    import ctypes
+    from deep8_amd import capi
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    for name, (res, args) in capi.SIGNATURES.items():
+        if name.endswith("scratch_bytes") or name == "d8_gemm_workspace_bytes":
+            getattr(lib, name).restype, getattr(lib, name).argtypes = res, args
+    F16, F32 = capi.FLOAT16, capi.FLOAT32
+    # C2b's dY: 512 x 512 over 16 384 in 16 pieces
+    assert lib.d8_matmul_scratch_bytes(F32, 2, 32, 512, 512, 1, 512, 512) == 16 * 512 * 512 * 4
+    # C2a and C3: whole
+    assert lib.d8_matmul_scratch_bytes(F32, 2, 32, 512, 512, 32, 512, 512) == 0
+    assert lib.d8_matmul_scratch_bytes(F16, 2, 1, 4096, 4096, 1, 4096, 4096) == 0
+    # C4: the remainder band of 2048 rows in nine pieces (forward, dX), dW on 64 x 64 tiles in 85 pieces
+    c4 = (32, 56, 56, 64, 64, 3, 3, 1, 1, 1, 1, 1)
+    assert lib.d8_conv2d_scratch_bytes(F32, 0, *c4) == 9 * 2048 * 64 * 4
+    assert lib.d8_conv2d_scratch_bytes(F32, 1, *c4) == 9 * 2048 * 64 * 4
+    assert lib.d8_conv2d_scratch_bytes(F32, 2, *c4) == 85 * 64 * 576 * 4
+    # C5: forward by classes and dX on half tiles stage nothing, dW in 22 pieces
+    c5 = (16, 28, 28, 128, 64, 4, 4, 0, 2, 2)
+    assert lib.d8_deconv2d_scratch_bytes(F16, 0, *c5) == 0
+    assert lib.d8_deconv2d_scratch_bytes(F16, 1, *c5) == 0
+    assert lib.d8_deconv2d_scratch_bytes(F16, 2, *c5) == 22 * 1024 * 128 * 4
