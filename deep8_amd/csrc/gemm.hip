@@ -406,7 +406,10 @@ static FewTiles plan_few_tiles(int BK, int M, int N, int batch, long total) {
     // ... one per CU where its pieces are then still 32 K steps or longer: as fast, and half the partial sums (C2b's
     // dY, 512 x 512 over 16 384: 72.8 -> 70.6 us)
     if (M >= 128 && N >= 128 && total / (cus / tiles) >= 32) rule = cus / tiles;
-    const long most = piece_limit(tiles, total, (int)cus);
+    // (never more than two pieces per CU in all: a long reduction would otherwise be cut ever finer for an ever
+    // smaller gain, and the partial sums -- at most 2 x CUs tiles of fp32, 32 MiB -- would grow with it)
+    long most = piece_limit(tiles, total, (int)cus);
+    if (most > 2 * cus / tiles) most = 2 * cus / tiles;
     if (rule > most) rule = most;
     if (rule < 1) rule = 1;
     const bool half_elems = BK == 64;
