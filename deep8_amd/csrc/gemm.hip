@@ -386,8 +386,9 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_scalar_kernel(GemmArgs 
 // 100 us for s = 2 .. 6; 1024 x 2048 x 2048 fp32 64.9 us on half tiles against 77.4 in two pieces, 1024 x 1024 x 2048
 // 63.4 us on (128) half tiles against 43.9 in four pieces.
 struct FewTiles {
-    long splits;  // pieces per tile (1: unsplit)
-    bool half;    // unsplit on 64 x 128 tiles
+    long splits;         // pieces per tile (1: unsplit)
+    bool half;           // unsplit on 64 x 128 tiles
+    bool half_if_whole;  // were it to run unsplit (no workspace for the pieces, say): on 64 x 128 tiles rather than 128 x 128
 };
 
 static long piece_limit(long tiles, long total, int cus) {
@@ -419,7 +420,7 @@ static FewTiles plan_few_tiles(int BK, int M, int N, int batch, long total) {
         const long rounds = (tiles * s + cus - 1) / cus, len = (total + s - 1) / s;
         return rounds * (len * (rounds == 1 ? 1.1 : 1.0) + ends) + (s > 1 ? second + s * per_split : 0.0);
     };
-    FewTiles best = {rule, false};
+    FewTiles best = {rule, false, false};
     double best_cost = cost(rule) * 0.97;  // the rules' own choice on a tie
     for (long c = 1; c <= most; ++c)
         if (cost(c) < best_cost) best.splits = c, best_cost = cost(c);
@@ -430,7 +431,8 @@ static FewTiles plan_few_tiles(int BK, int M, int N, int batch, long total) {
         const long rounds = (2 * tiles + cus - 1) / cus;
         // (a 64 x 128 tile's step against a 128 x 128 tile's: half the MFMAs; 0.65 in half, where the rest of the step weighs more)
         const double c = rounds * ((half_elems ? 0.65 : 0.5) * total * (rounds == 1 ? 1.1 : 1.0) + ends);
-        if (c < best_cost) best = {1, true};
+        best.half_if_whole = c < cost(1);
+        if (c < best_cost) best.splits = 1, best.half = true;
     }
     return best;
 }
@@ -438,7 +440,7 @@ static FewTiles plan_few_tiles(int BK, int M, int N, int batch, long total) {
 bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps, int BK) {
     if (M < 128 || N < 128) return false;
     const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
-    return tiles < cu_count() && plan_few_tiles(BK, M, N, batch, k_steps).half;
+    return tiles < cu_count() && plan_few_tiles(BK, M, N, batch, k_steps).half_if_whole;  // (asked of an unsplit product)
 }
 
 // How many pieces to cut the reduction into, for a kernel whose K step is BK.  Splitting is only
