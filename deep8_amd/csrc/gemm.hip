@@ -379,8 +379,9 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_scalar_kernel(GemmArgs 
 // admitted alternatives, because how the workgroups fall into rounds matters as much as how many there are: a
 // CU's share is ceil(workgroups / CUs) pieces of ceil(total / s) steps plus a prologue and an epilogue each, a
 // workgroup alone on its CU walks its steps about a tenth slower than two that share one, a half tile's step is
-// half a step (0.65 in half precision), and the second pass costs a launch plus the s partial sums read back (at some 4 TB/s).  In units
-// of a K step (about 2 us of a CU's time in fp32, 0.5 us in half): prologue + epilogue 2.5 / 7, second pass 2 / 14.
+// half a step (0.65 in half precision), and the second pass costs a launch plus the s partial sums read back (at
+// some 4 TB/s).  In units of a K step (about 2 us of a CU's time in fp32, 0.5 us in half): prologue + epilogue
+// 2.5 / 7, second pass 2 / 14.
 // Measured against it: Conv2d 14 x 14 x 256 fp32, 98 tiles over 72 steps, 36 / 48 / 36 / 30 / 36 steps per CU for
 // s = 2 .. 6, ran 83.9 / 103.3 / 82.9 / 72.8 / 86.9 us; 7 x 7 x 512, 52 tiles over 144 steps, 146 / 102 / 80.7 / 116 /
 // 100 us for s = 2 .. 6; 1024 x 2048 x 2048 fp32 64.9 us on half tiles against 77.4 in two pieces, 1024 x 1024 x 2048
