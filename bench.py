@@ -907,8 +907,11 @@ def graph_replay_ms(wl, steps, warmup):
         lib.d8_stream_destroy(side)
 
 
-WIDE_DIAGNOSTICS = {"same_k": "D8_WIDE_DIAG_SAME_K", "barrier_clocks": "D8_WIDE_DIAG_BARRIER_CLOCKS",
-                    "no_store": "D8_WIDE_DIAG_NO_STORE", "direct_store": "D8_WIDE_DIAG_DIRECT_STORE"}
+WIDE_DIAGNOSTICS = {"same_k": ["D8_WIDE_DIAG_SAME_K"], "barrier_clocks": ["D8_WIDE_DIAG_BARRIER_CLOCKS"],
+                    "no_store": ["D8_WIDE_DIAG_NO_STORE"], "direct_store": ["D8_WIDE_DIAG_DIRECT_STORE"],
+                    "no_fragment_reads": ["D8_WIDE_DIAG_NO_FRAGMENT_READS"], "no_loads": ["D8_WIDE_DIAG_NO_LOADS"],
+                    "no_barrier": ["D8_WIDE_DIAG_NO_BARRIER"],
+                    "mfma_only": ["D8_WIDE_DIAG_NO_FRAGMENT_READS", "D8_WIDE_DIAG_NO_LOADS", "D8_WIDE_DIAG_NO_BARRIER"]}
 
 
 def build_wide_diagnostic(name):
@@ -920,7 +923,7 @@ def build_wide_diagnostic(name):
     csrc = os.path.join(ROOT, "deep8_amd", "csrc")
     tmp = tempfile.mkdtemp(prefix="d8_wide_diag_")
     obj, lib = os.path.join(tmp, "gemm_wide.o"), os.path.join(tmp, "libdeep8_hip_%s.so" % name)
-    subprocess.check_call([ge.HIPCC] + ge.HIP_FLAGS + ["-D" + WIDE_DIAGNOSTICS[name], "-c", os.path.join(csrc, "gemm_wide.hip"), "-o", obj],
+    subprocess.check_call([ge.HIPCC] + ge.HIP_FLAGS + ["-D" + d for d in WIDE_DIAGNOSTICS[name]] + ["-c", os.path.join(csrc, "gemm_wide.hip"), "-o", obj],
                           stderr=subprocess.DEVNULL)
     # the other sources: their objects from the shipped build where present, else compiled here (all at once)
     objs, jobs = [obj], []
@@ -1107,7 +1110,7 @@ def main():
         if not a.phases:
             raise SystemExit("--wide-diagnostic goes with --phases")
         capi.LIB_PATH = build_wide_diagnostic(a.wide_diagnostic)
-        print("diagnostic build of gemm_wide.hip: -D%s" % WIDE_DIAGNOSTICS[a.wide_diagnostic], flush=True)
+        print("diagnostic build of gemm_wide.hip: " + " ".join("-D" + d for d in WIDE_DIAGNOSTICS[a.wide_diagnostic]), flush=True)
     capi.init()
     if a.phases and a.wide_diagnostic == "barrier_clocks":
         return barrier_clock_record()

@@ -31,13 +31,19 @@
 //
 // Diagnostic builds (never defined in the shipped library; `python bench.py --phases --wide-diagnostic NAME`
 // compiles this file with one of them into a scratch copy of the library and prints the kernel's phase
-// record).  Each answers one question about where a launch's time goes; SAME_K and NO_STORE give wrong results:
+// record).  Each answers one question about where a launch's time goes; all but BARRIER_CLOCKS and DIRECT_STORE give
+// wrong results (none of them reads or writes outside the operands):
 //   D8_WIDE_DIAG_SAME_K          every K step fetches the tile's first step again, so all loads after the first
 //                                hit in cache: what the loop costs when no load ever waits for HBM
 //   D8_WIDE_DIAG_BARRIER_CLOCKS  reads the shader clock around the step's wait for its own loads and around its
 //                                barrier; the record's first three fields become the summed cycles of a pair of
 //                                back-to-back clock reads, of the wait and of the barrier
 //   D8_WIDE_DIAG_NO_STORE        the epilogue does everything but the stores to C: its cost without HBM writes
+//   D8_WIDE_DIAG_NO_FRAGMENT_READS  the K loop without its LDS reads (the MFMAs keep the first fragments)
+//   D8_WIDE_DIAG_NO_LOADS        ... without its global -> LDS loads (the MFMAs see the first two steps again and again)
+//   D8_WIDE_DIAG_NO_BARRIER      ... without its barrier
+//                                (the three combine: what each part of the loop costs in cycles -- on all-zero operands,
+//                                `--operands zeros` -- and in energy, i.e. in clock, on the config's data)
 //   D8_WIDE_DIAG_DIRECT_STORE    accumulates the blocks transposed (MFMA operands exchanged) so that a lane owns
 //                                four consecutive columns, and stores them straight from registers, 8 bytes per
 //                                lane, without the LDS patch (correct results)
@@ -243,11 +249,13 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
 #pragma unroll
         for (int m = 0; m < 64; ++m) {
             mfma(acc[BI(m)][BJ(m)], fa[0][BI(m)], fb[0][BJ(m)]);
+#ifndef D8_WIDE_DIAG_NO_FRAGMENT_READS
             if (m % 3 == 0 && m < 48) {
                 const int e = m / 3;  // 16 reads: the B fragments first (all needed by the first row)
                 if (e < 8) fb[1][e] = ob.read(Bs, 1, e);
                 else fa[1][e - 8] = oa.read(As, 1, e - 8);
             }
+#endif
         }
         // half 1
 #ifdef D8_WIDE_DIAG_BARRIER_CLOCKS
@@ -261,7 +269,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
         const unsigned long long tb2 = __builtin_readcyclecounter();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #endif
+#ifndef D8_WIDE_DIAG_NO_BARRIER
         __syncthreads();
+#endif
 #ifdef D8_WIDE_DIAG_BARRIER_CLOCKS
         const unsigned long long tb3 = __builtin_readcyclecounter();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -269,25 +279,31 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
 #endif
 #pragma unroll
         for (int m = 0; m < 64; ++m) {
+#ifndef D8_WIDE_DIAG_NO_LOADS
             if ((m & 3) == 0) {
                 if ((m >> 2) < 8) oa.aim_round(As, wave, m >> 2);
                 else ob.aim_round(Bs, wave, (m >> 2) - 8);
             }
+#endif
             mfma(acc[BI(m)][BJ(m)], fa[1][BI(m)], fb[1][BJ(m)]);
             if ((m & 3) == 0) {
                 // 16 loads into the stage every wave has finished with, one per 4 MFMAs: a load
                 // keeps the CU's address path busy for 16 cycles, as long as an MFMA runs, and all
                 // four waves issue theirs in the same window; issued closer together they hold up
                 // instruction issue (2600 cycles per step at one per 2 MFMAs, 2330 at one per 4)
+#ifndef D8_WIDE_DIAG_NO_LOADS
                 const int d = m >> 2;
                 if (d < 8) oa.fetch_round(ra, a_src, d);
                 else ob.fetch_round(rb, b_src, d - 8);
+#endif
             }
+#ifndef D8_WIDE_DIAG_NO_FRAGMENT_READS
             if (m % 3 == 1 && m < 48) {
                 const int e = m / 3;  // fragments of the next step's k group 0
                 if (e < 8) fb[0][e] = ob.read(Bn, 0, e);
                 else fa[0][e - 8] = oa.read(An, 0, e - 8);
             }
+#endif
         }
     };
 
