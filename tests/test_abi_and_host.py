@@ -86,8 +86,8 @@ def test_bench_reads_its_traffic_figures_from_the_committed_profiles():
     assert abs(bench.profile_traffic("i4", "im2col")["bytes"] - 256.9e6) < 2e6
 
 
-def test_planner_keeps_the_plans_of_the_baseline_configs():
-    """The split planner's choices for the BASELINE configurations, read off the scratch queries (host code only; with
+def test_planner_keeps_the_plans_of_the_benchmark_configs():
+    """The split planner's choices for the benchmark configurations (bench.py workloads c2a, c2b, c3, c4, c5), read off the scratch queries (host code only; with
     no device the planner assumes the MI355X's 256 CUs): a change of its rules or constants that moves one of them
     shows up here before it shows up in a benchmark."""
     import ctypes
