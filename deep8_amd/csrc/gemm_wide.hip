@@ -230,7 +230,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(GemmArgs g, int tilesM, 
             ob.fetch_round(rb, b_org + step * b_step, t);
         }
     }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces are in LDS
+    // vmcnt(16): this wave's pieces of the first stage are in LDS (the 16 loads of the second stage may still be on
+    // their way: the first step's own wait, before its barrier, covers them)
+    __builtin_amdgcn_s_waitcnt(0x4f70);
     __syncthreads();
     if (g.stamps) wall[1] = wall_clock64(), clk[0] = __builtin_readcyclecounter();
 #pragma unroll
