@@ -14,10 +14,13 @@ starts on an idle device and times 20 steps after 3 warm-up steps measures the r
 loop sees (MatrixMultiply half 4096^3: about 1185 TFLOP/s from idle, about 1425 sustained, same box, same
 binary).  --settle-ms 0 gives the from-idle number; the JSON line reports the value used as "settle_ms".
 
-  value          whole-step throughput: algorithmic FLOPs of fwd + dX + dY / wall time of a step
-                 (gradient destinations are zeroed inside the step, as Deep8's executor does)
-  roofline       flops of one GEMM launch / the average duration of the step's launches, each timed alone
-                 with HIP events on the stream it runs on, against the dense MFMA peak of the element type
+  value          whole-step throughput: algorithmic FLOPs of fwd + dX + dY / wall time of a step.  A step is what this
+                 build's executor issues: the forward product, then both gradient products in their overwrite form
+                 (the executor's zero fill of a gradient is deferred until something reads it; --eager-zero times
+                 the reference executor's literal fill + accumulate instead, and the line always carries it beside
+                 the headline as "eager_zero")
+  roofline       flops of one product / the average duration per product of the step's launches, each launch timed
+                 alone with HIP events on the stream it runs on, against the dense MFMA peak of the element type
                  (element-wise and pooling workloads: the longest kernel's bytes / its duration, against HBM)
   cpu_baseline   Deep8's own CPU (Eigen) path from oracle/_ref -- or the C restatement when that was
                  not built -- on a bounded sample of the same workload, on this host's cores
@@ -187,11 +190,12 @@ class MatMulWorkload:
         self.flops = 3 * 2.0 * zb * m * k * n
         wide = self.dtype == np.float16 and m >= 256 and n >= 256 and k % 64 == 0 and zb * (-(-m // 256)) * (-(-n // 256)) >= 192
         small = zb * (-(-m // 128)) * (-(-n // 128)) <= 4 and max(m, n, k) * (zb if 1 in (xs[0], ys[0]) else 1) <= 512
-        self.kernel = "%s (one launch each for fwd, dX, dY)" % (
+        self.kernel = "%s (%s)" % (
             "gemm_f64_kernel (%s tiles, v_mfma_f64_16x16x4_f64)" % ("128x128" if zb * (-(-m // 128)) * (-(-n // 128)) >= 192 else "64x64")
             if self.dtype == np.float64 else
             "gemm_wide_kernel (fp16, 256x256 tiles)" if wide else
-            "gemm_%s_kernel<%s>" % ("small" if small else "tiled", "f16" if self.dtype == np.float16 else "f32"))
+            "gemm_%s_kernel<%s>" % ("small" if small else "tiled", "f16" if self.dtype == np.float16 else "f32"),
+            "one launch for fwd, one for dX and dY together" if wide else "one launch each for fwd, dX, dY")
         es = self.dtype.itemsize
         nx, ny, nz = np.prod(xs), np.prod(ys), np.prod(self.zs)
         # fwd reads x,y writes z; dX reads dz,y and read-modify-writes dx; dY likewise
@@ -222,16 +226,27 @@ class MatMulWorkload:
         check(self.lib.d8_matmul_grad_y_overwrite(self.dt, self.x.ptr, *self.xs, self.dy.ptr, *self.ys, self.dz.ptr,
                                                   self.ws.ptr, self.ws_bytes, self.stream))
 
+    def grad_xy(self, overwrite):
+        """both gradients from one call, as MatrixMultiply::backward() of the host layer issues them"""
+        from deep8_amd.capi import check
+        check(self.lib.d8_matmul_grad_xy(self.dt, self.x.ptr, self.dx.ptr, *self.xs, self.y.ptr, self.dy.ptr, *self.ys,
+                                         self.dz.ptr, 3 if overwrite else 0, self.ws.ptr, self.ws_bytes, self.stream))
+
+    def grad_xy_first(self):
+        self.grad_xy(True)
+
+    def grad_xy_accumulate(self):
+        self.grad_xy(False)
+
     def step(self):
         """One forward + backward of a MatrixMultiply node as this build's executor issues it: forward, then the
-        two gradient products.  The executor's zeroGradient() before a backward pass is deferred
+        two gradient products from one call.  The executor's zeroGradient() before a backward pass is deferred
         (Device::zeroLater), so the first product into each gradient is the overwrite form: same
         result as fill + accumulate, without the fill and without reading the zeros back."""
         if EAGER_ZERO:
             return self.step_eager_zero()
         self.fwd()
-        self.grad_x_first()
-        self.grad_y_first()
+        self.grad_xy(True)
 
     def step_eager_zero(self):
         """The reference executor's literal sequence (deep8/src/model/EagerExecutor.cpp:51-65, then
@@ -239,19 +254,21 @@ class MatMulWorkload:
         self.fwd()
         self.dx.zero_()
         self.dy.zero_()
-        self.grad_x()
-        self.grad_y()
+        self.grad_xy(False)
 
     def parts(self):
+        """the calls of a step, each alone: the forward product, and both gradients from one call (for large Float16
+        products one launch); beside them each gradient product as a call of its own"""
         f = self.flops / 3
         if EAGER_ZERO:
-            return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
-        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x_first, f), "grad_y": (self.grad_y_first, f)}
+            return {"fwd": (self.fwd, f), "grad_xy": (self.grad_xy_accumulate, 2 * f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
+        return {"fwd": (self.fwd, f), "grad_xy": (self.grad_xy_first, 2 * f), "grad_x": (self.grad_x_first, f), "grad_y": (self.grad_y_first, f)}
 
     def parts_accumulate(self):
-        """the two gradient launches in their beta = 1 form (read the destination, add, write)"""
+        """the gradient launches in their beta = 1 form (read the destination, add, write)"""
         f = self.flops / 3
-        return {"grad_x_accumulate": (self.grad_x, f), "grad_y_accumulate": (self.grad_y, f)}
+        return {"grad_xy_accumulate": (self.grad_xy_accumulate, 2 * f), "grad_x_accumulate": (self.grad_x, f),
+                "grad_y_accumulate": (self.grad_y, f)}
 
 
 def mfma_stream_ceiling(wl, dtype_name):
@@ -907,25 +924,24 @@ def graph_replay_ms(wl, steps, warmup):
         lib.d8_stream_destroy(side)
 
 
-WIDE_DIAGNOSTICS = {"same_k": ["D8_WIDE_DIAG_SAME_K"], "barrier_clocks": ["D8_WIDE_DIAG_BARRIER_CLOCKS"],
-                    "no_store": ["D8_WIDE_DIAG_NO_STORE"], "direct_store": ["D8_WIDE_DIAG_DIRECT_STORE"],
-                    "no_fragment_reads": ["D8_WIDE_DIAG_NO_FRAGMENT_READS"], "no_loads": ["D8_WIDE_DIAG_NO_LOADS"],
-                    "no_barrier": ["D8_WIDE_DIAG_NO_BARRIER"],
-                    "mfma_only": ["D8_WIDE_DIAG_NO_FRAGMENT_READS", "D8_WIDE_DIAG_NO_LOADS", "D8_WIDE_DIAG_NO_BARRIER"]}
+WIDE_DIAGNOSTICS = {"same_k": ["D8_DIAG_SAME_K"], "no_stores": ["D8_DIAG_NO_STORES"],
+                    "no_fragment_reads": ["D8_DIAG_NO_FRAGMENT_READS"], "no_loads": ["D8_DIAG_NO_LOADS"],
+                    "no_barrier": ["D8_DIAG_NO_BARRIER"],
+                    "mfma_only": ["D8_DIAG_NO_FRAGMENT_READS", "D8_DIAG_NO_LOADS", "D8_DIAG_NO_BARRIER"]}
 
 
 def build_wide_diagnostic(name):
-    """compiles deep8_amd/csrc/gemm_wide.hip with one of its diagnostic switches and links it with the objects of
-    the shipped library (deep8_amd/csrc/obj, left by __graft_entry__.build()) into a scratch library; returns its path"""
+    """compiles deep8_amd/csrc/diag/gemm_wide_diag.hip (the fp16 kernel with one of its parts left out) and links it,
+    in place of gemm_wide.hip's object, with the library's other objects (deep8_amd/csrc/obj, left by
+    __graft_entry__.build(); compiled here where absent) into a scratch library; returns its path"""
     import subprocess
     import tempfile
     import __graft_entry__ as ge
     csrc = os.path.join(ROOT, "deep8_amd", "csrc")
     tmp = tempfile.mkdtemp(prefix="d8_wide_diag_")
     obj, lib = os.path.join(tmp, "gemm_wide.o"), os.path.join(tmp, "libdeep8_hip_%s.so" % name)
-    subprocess.check_call([ge.HIPCC] + ge.HIP_FLAGS + ["-D" + d for d in WIDE_DIAGNOSTICS[name]] + ["-c", os.path.join(csrc, "gemm_wide.hip"), "-o", obj],
-                          stderr=subprocess.DEVNULL)
-    # the other sources: their objects from the shipped build where present, else compiled here (all at once)
+    subprocess.check_call([ge.HIPCC] + ge.HIP_FLAGS + ["-D" + d for d in WIDE_DIAGNOSTICS[name]] +
+                          ["-c", os.path.join(csrc, "diag", "gemm_wide_diag.hip"), "-o", obj], stderr=subprocess.DEVNULL)
     objs, jobs = [obj], []
     for src in sorted(f for f in os.listdir(csrc) if f.endswith(".hip") and f != "gemm_wide.hip"):
         have = os.path.join(csrc, "obj", src[:-4] + ".o")
@@ -940,29 +956,6 @@ def build_wide_diagnostic(name):
             raise SystemExit("bench.py: compiling the library's sources for the diagnostic build failed")
     subprocess.check_call([ge.HIPCC] + ge.HIP_FLAGS + ["-shared", "-o", lib] + objs, stderr=subprocess.DEVNULL)
     return lib
-
-
-def barrier_clock_record():
-    """phase record of the D8_WIDE_DIAG_BARRIER_CLOCKS build: cycles per K step spent in the wait for the step's
-    own loads and in its barrier (each figure includes one clock read; the first column is that cost alone)"""
-    from deep8_amd import capi
-    lib = capi.init()
-    wl = make_workload("c3")
-    n = 4096
-    out = capi.DeviceArray((n, n), np.float16)
-    rec = capi.DeviceArray((256 * 6,), np.uint64, zero=True)
-    for name, ta, tb, A, B in (("forward NN", 0, 0, wl.x, wl.y), ("dX NT", 0, 1, wl.dz, wl.y), ("dY TN", 1, 0, wl.x, wl.dz)):
-        def launch():
-            capi.check(lib.d8_gemm(wl.dt, ta, tb, n, n, n, A.ptr, n, 0, B.ptr, n, 0, 0.0, out.ptr, n, 0, 1, rec.ptr, 256 * 6 * 8, None))
-        _settle(launch)
-        for _ in range(10):
-            launch()
-        capi.sync()
-        r = rec.numpy().astype(np.int64).reshape(256, 6)
-        st = n // 64
-        print("%s: cycles per K step (mean over the 256 workgroups): two clock reads back to back %.0f, wait for the "
-              "step's own loads %.0f, barrier %.0f; whole loop %.0f (with the four clock reads in it)" % (
-                  name, r[:, 0].mean() / st, r[:, 1].mean() / st, r[:, 2].mean() / st, (r[:, 5] - r[:, 4]).mean() / st), flush=True)
 
 
 def phase_record(launches=12):
@@ -1008,6 +1001,47 @@ def phase_record(launches=12):
         print("  shader clock during the loop, per XCD: " + ", ".join(
             "%.2f" % ghz[np.arange(256) % 8 == x].mean() for x in range(8)) + " GHz; cycles per K step %.0f" % (
             (r[:, 5] - r[:, 4]).mean() / (n // 64)))
+    pair_phase_record(wl, launches)
+
+
+def pair_phase_record(wl, launches=12):
+    """the same record for both gradients as ONE launch (d8_matmul_grad_xy): 256 workgroups, each a tile of dX and then
+    a tile of dY; what separates the two K loops of a workgroup is printed as its turn-around"""
+    from deep8_amd import capi
+    lib = capi.init()
+    n = 4096
+    recs = [capi.DeviceArray((512 * 6,), np.uint64, zero=True) for _ in range(launches)]
+
+    def launch(i):
+        capi.check(lib.d8_matmul_grad_xy(wl.dt, wl.x.ptr, wl.dx.ptr, 1, n, n, wl.y.ptr, wl.dy.ptr, 1, n, n, wl.dz.ptr, 3,
+                                         recs[i].ptr, 512 * 6 * 8, None))
+    _settle(lambda: launch(0))
+    for i in range(launches):
+        launch(i)
+    capi.sync()
+    t = capi.Timer(None)
+    t.start()
+    for i in range(launches):
+        launch(i)
+    ms = t.stop_ms() / launches
+    r = recs[-1].numpy().astype(np.int64).reshape(512, 6)
+    if not r[:, 3].all():
+        raise SystemExit("no phase record was written for the launch of two products")
+    us = lambda v: v / 100.0
+    first, second = r[:256], r[256:]
+    print("dX NT + dY TN as one launch: %.1f us per launch by HIP events over %d launches (%.0f TFLOP/s)" % (
+        ms * 1e3, launches, 4.0 * n**3 / ms / 1e9))
+    for name, q in (("dX tiles", first), ("dY tiles", second)):
+        loop = us(q[:, 2] - q[:, 1])
+        ghz = (q[:, 5] - q[:, 4]) / (loop * 1e3)
+        print("  %s: K loop %.1f-%.1f us (mean %.1f) at %.2f GHz, %.0f cycles per K step" % (
+            name, loop.min(), loop.max(), loop.mean(), ghz.mean(), (q[:, 5] - q[:, 4]).mean() / (n // 64)))
+    turn = us(second[:, 1] - first[:, 2])
+    print("  prologue %.1f us; from the end of a workgroup's first K loop to the start of its second (the next tile's first "
+          "loads issued, the epilogue, the wait for those loads) %.1f-%.1f us (mean %.1f); last epilogue until its stores "
+          "are acknowledged %.1f-%.1f us; last workgroup done %.1f us after the first started" % (
+              us(first[:, 1] - first[:, 0]).mean(), turn.min(), turn.max(), turn.mean(),
+              us(second[:, 3] - second[:, 2]).min(), us(second[:, 3] - second[:, 2]).max(), us(r[:, 3].max() - r[:, 0].min())))
 
 
 def tiled_phase_record(key, launches=8):
@@ -1112,8 +1146,6 @@ def main():
         capi.LIB_PATH = build_wide_diagnostic(a.wide_diagnostic)
         print("diagnostic build of gemm_wide.hip: " + " ".join("-D" + d for d in WIDE_DIAGNOSTICS[a.wide_diagnostic]), flush=True)
     capi.init()
-    if a.phases and a.wide_diagnostic == "barrier_clocks":
-        return barrier_clock_record()
     if a.calibrate_copy:
         return calibrate_copy(a.calibrate_copy)
     if a.phases:
@@ -1152,9 +1184,11 @@ def main():
         for k, v in parts.items():  # every kernel of the step against the HBM peak
             v["frac_of_hbm_peak"] = round(v["algorithmic_GBps"] / HBM_PEAK, 4)
     else:
-        # each of fwd / dX / dY is ONE launch of the same tiled GEMM kernel (its NN, NT and TN
-        # instances): flops per launch / average launch duration, HIP events on the launch stream
-        avg_ms = sum(p["ms"] for p in parts.values()) / len(parts)
+        # a MatrixMultiply step is the forward call and the call for both gradients (one launch of the large-output
+        # fp16 kernel each; one launch per product elsewhere): flops per product / duration per product of those
+        # calls, HIP events on the launch stream
+        avg_ms = ((parts["fwd"]["ms"] + parts["grad_xy"]["ms"]) / 3 if "grad_xy" in parts else
+                  sum(p["ms"] for p in parts.values()) / len(parts))
         ach = wl.flops / 3 / (avg_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "kernel": wl.kernel, "achieved": round(ach, 2), "peak": PEAK[dtype],
                 "unit": "TFLOP/s", "frac": round(ach / PEAK[dtype], 4), "launch_us": round(avg_ms * 1e3, 2),
@@ -1166,18 +1200,19 @@ def main():
             ems, esamples = _time_steps(wl.step_eager_zero, a.steps, a.warmup)
             acc = time_parts(wl.parts_accumulate())
             parts.update(acc)
-            eavg = (parts["fwd"]["ms"] + sum(p["ms"] for p in acc.values())) / 3
+            eavg = (parts["fwd"]["ms"] + acc["grad_xy_accumulate"]["ms"]) / 3
             et = wl.flops / (ems * 1e-3) / 1e12
-            eager = {"sequence": "forward, zero-fill dX and dY, dX += dZ.Y^T, dY += X^T.dZ (beta = 1): the reference "
-                                 "executor's literal calls",
+            eager = {"sequence": "forward, zero-fill dX and dY, then dX += dZ.Y^T and dY += X^T.dZ (beta = 1) from one call: "
+                                 "the reference executor's literal fill + accumulate",
                      "ms_per_step": round(ems, 4), "ms_per_step_samples": [round(v, 4) for v in esamples],
                      "tflops": round(et, 2), "pct_mfma_peak": round(100.0 * et / PEAK[dtype], 2),
                      "frac": round(wl.flops / 3 / (eavg * 1e-3) / 1e12 / PEAK[dtype], 4), "launch_us": round(eavg * 1e3, 2)}
 
-    form = ""
+    form, note = "", None
     if is_mm or is_conv:
-        form = ("; gradients: zero fill + accumulate (beta = 1), the reference executor's literal sequence" if EAGER_ZERO else
-                "; gradients: written by the overwrite form (beta = 0) that this build's executor issues while the zero fill "
+        form = ", fill + accumulate" if EAGER_ZERO else ", overwrite form"
+        note = ("gradients: zero fill + accumulate (beta = 1), the reference executor's literal sequence" if EAGER_ZERO else
+                "gradients: written by the overwrite form (beta = 0) that this build's executor issues while the zero fill "
                 "of a gradient is still deferred -- same flops, same result as fill + accumulate"
                 + (", which is reported beside it under eager_zero" if eager else ""))
     out = {
@@ -1190,7 +1225,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "ALL-ZERO OPERANDS (diagnostic run, not a benchmark value)" if ZERO_OPERANDS else
         "synthetic (seeded numpy generators, resident in HBM before timing)",
-        "config": {"workload": wl.name + form},
+        "config": {"workload": wl.name + form, **({"note": note} if note else {})},
         "pct_mfma_peak": None if is_stream else round(100.0 * tflops / PEAK[dtype], 2),
         "tflops": round(tflops, 2),
         "algorithmic_GBps": round(wl.bytes / (ms * 1e-3) / 1e9, 1),

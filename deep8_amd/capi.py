@@ -28,6 +28,7 @@ SIGNATURES = {
     "d8_device_init": (_I, [_I]),
     "d8_device_count": (_I, [ctypes.POINTER(_I)]),
     "d8_device_info": (_I, [ctypes.POINTER(_I), ctypes.POINTER(_I), ctypes.POINTER(_Z), ctypes.c_char_p, _I]),
+    "d8_mem_info": (_I, [ctypes.POINTER(_Z), ctypes.POINTER(_Z)]),
     "d8_malloc": (_I, [_PP, _Z]),
     "d8_free": (_I, [_P]),
     "d8_host_malloc": (_I, [_PP, _Z]),
@@ -69,6 +70,7 @@ SIGNATURES = {
     "d8_matmul_grad_y_static": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P]),
     "d8_matmul_grad_x_overwrite": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
     "d8_matmul_grad_y_overwrite": (_I, [_I, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P, _Z, _P]),
+    "d8_matmul_grad_xy": (_I, [_I, _P, _P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _I, _P, _Z, _P]),
     "d8_conv2d_geometry": (_I, [_I] * 9 + [ctypes.POINTER(_I)]),
     "d8_deconv2d_geometry": (_I, [_I] * 7 + [ctypes.POINTER(_I)]),
     "d8_conv2d_scratch_bytes": (_Z, [_I] * 14),

@@ -73,6 +73,14 @@ int d8_device_info(int *cus, int *clock_khz, size_t *hbm_bytes, char *name, int 
     return 0;
 }
 
+int d8_mem_info(size_t *free_bytes, size_t *total_bytes) {
+    size_t f = 0, t = 0;
+    D8_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return 0;
+}
+
 int d8_malloc(void **ptr, size_t bytes) {
     D8_REQUIRE(ptr, "ptr is null");
     D8_HIP(hipMalloc(ptr, bytes));

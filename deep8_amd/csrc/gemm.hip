@@ -611,7 +611,9 @@ int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspa
 }
 
 bool gemm_fuses_store(int dtype, const GemmArgs &g, int transA, int transB) {
-    if (dtype == D8_FLOAT64 || g.K < 1 || g.beta != 0.f || g.red != 1 || g.batch > 448) return false;
+    // (a product beyond one launch's limits -- more than 448 outputs, more than 65535 * 128 rows -- is cut into several
+    // by d8_gemm; the fused store stays out of that: the caller runs the product and one pass over its result)
+    if (dtype == D8_FLOAT64 || g.K < 1 || g.beta != 0.f || g.red != 1 || g.batch > 448 || g.M > 65535 * 128) return false;
     if (g.virt == VIRT_NONE && gemm_is_small(g.M, g.N, g.K, g.batch, g.red)) return false;  // gemm_small_kernel has no fused store
     return gemm_tiled_eligible(dtype, g, transA, transB);
 }

@@ -110,6 +110,12 @@ void gemm_tiled_phase_record(void *records, size_t bytes);
 // LDS): unsplit, unsummed products of real matrices with M, N >= 256 and K a multiple of 64.
 bool gemm_wide_eligible(const GemmArgs &g, int transA, int transB);
 int gemm_wide_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);
+// Two such products (each eligible) as ONE launch: a workgroup that has finished a tile of the first goes on to a
+// tile of the second without the kernel boundary in between (the end of one launch -- the write of the whole of
+// C, the wait for its acknowledgement, the gap -- and the start of the next, whose first operand bytes come from
+// memory).  Built for the two gradients of a MatrixMultiply, which are independent of each other.
+int gemm_wide_pair_launch(const GemmArgs &g0, int transA0, int transB0, const GemmArgs &g1, int transA1, int transB1,
+                          hipStream_t stream);
 
 // fp64 kernel (64 x 64 or 128 x 128 tiles, v_mfma_f64_16x16x4_f64): any shape; plans its own split of the
 // reduction from g.ws / g.ws_bytes (double partial sums) and reduces.

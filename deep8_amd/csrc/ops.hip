@@ -241,7 +241,14 @@ int d8_matmul_bias_relu(int dtype, const void *x, int xb, int xr, int xc, const 
     if (int rc = check_mm("d8_matmul_bias_relu", dtype, xb, xr, xc, yb, yr, yc)) return rc;
     if (dtype == D8_FLOAT64) return fail(D8_ERR_DTYPE, "d8_matmul_bias_relu: element type %d is not supported", dtype);
     D8_REQUIRE(x && y && z, "d8_matmul_bias_relu: null tensor");
-    return run_bias_relu(dtype, mm_plan(0, x, xb, xr, xc, y, yb, yr, yc, z), bias, relu, scratch, scratch_bytes, stream);
+    const Gemm p = mm_plan(0, x, xb, xr, xc, y, yb, yr, yc, z);
+    if (yc == 1 && !(xb == 1 && yb > 1) && (bias || relu)) {
+        // y is a vector (or a batch of vectors): z is [batch][xr] and its last axis -- the one the bias runs along -- is
+        // x's rows, which this plan puts on the product's M side.  The product, then one pass over z as [batch][xr].
+        if (int rc = run(dtype, p, scratch, scratch_bytes, stream)) return rc;
+        return launch_bias_relu(dtype, z, bias, (long)(xb > yb ? xb : yb), xr, relu, as_stream(stream));
+    }
+    return run_bias_relu(dtype, p, bias, relu, scratch, scratch_bytes, stream);
 }
 
 int d8_matmul_grad_x(int dtype, void *dx, int xb, int xr, int xc, const void *y, int yb, int yr, int yc,
@@ -270,6 +277,31 @@ int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc,
     if (int rc = check_mm("d8_matmul_grad_y_overwrite", dtype, xb, xr, xc, yb, yr, yc)) return rc;
     D8_REQUIRE(x && dy && dz, "d8_matmul_grad_y_overwrite: null tensor");
     return run(dtype, mm_plan(2, x, xb, xr, xc, dy, yb, yr, yc, dz, 0.f), scratch, scratch_bytes, stream);
+}
+
+int d8_matmul_grad_xy(int dtype, const void *x, void *dx, int xb, int xr, int xc, const void *y, void *dy, int yb, int yr,
+                      int yc, const void *dz, int overwrite, void *scratch, size_t scratch_bytes, void *stream) {
+    if (int rc = check_mm("d8_matmul_grad_xy", dtype, xb, xr, xc, yb, yr, yc)) return rc;
+    D8_REQUIRE(x && dx && y && dy && dz, "d8_matmul_grad_xy: null tensor");
+    D8_REQUIRE(dx != dy, "d8_matmul_grad_xy: dx and dy are the same tensor");
+    const Gemm px = mm_plan(1, dx, xb, xr, xc, y, yb, yr, yc, dz, (overwrite & 1) ? 0.f : 1.f);
+    const Gemm py = mm_plan(2, x, xb, xr, xc, dy, yb, yr, yc, dz, (overwrite & 2) ? 0.f : 1.f);
+    if (dtype == D8_FLOAT16) {
+        // both products large enough for the 256 x 256-tile kernel: one launch whose workgroups go from a tile of
+        // dX straight on to a tile of dY
+        static const char *wide = getenv("D8_GEMM_WIDE");  // tuning aid: 0 keeps the products apart
+        GemmArgs gx = to_args(px);
+        const GemmArgs gy = to_args(py);
+        gx.ws = (float *)scratch, gx.ws_bytes = scratch_bytes;  // (only ever used for the kernel's phase record, a measurement aid)
+        const long tx = (long)ceil_div(gx.M, 256) * ceil_div(gx.N, 256) * gx.batch;
+        const long ty = (long)ceil_div(gy.M, 256) * ceil_div(gy.N, 256) * gy.batch;
+        const long most = (long)cu_count() * 3 / 4;
+        if (!(wide && atoi(wide) == 0) && gx.red == 1 && gy.red == 1 && tx >= most && ty >= most && tx + ty < 0x3fffffffL &&
+            gemm_wide_eligible(gx, px.ta, px.tb) && gemm_wide_eligible(gy, py.ta, py.tb))
+            return gemm_wide_pair_launch(gx, px.ta, px.tb, gy, py.ta, py.tb, as_stream(stream));
+    }
+    if (int rc = run(dtype, px, scratch, scratch_bytes, stream)) return rc;
+    return run(dtype, py, scratch, scratch_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

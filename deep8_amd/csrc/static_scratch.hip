@@ -12,6 +12,8 @@
 // Every call on a device shares the device's array: calls that overlap on one device (two streams, two
 // host threads) race on the partial sums.  Nothing in it has to start at zero: every partial sum a call
 // reads was written by that call's own product kernel earlier on the same stream.
+#include <mutex>
+
 #include "common.h"
 
 namespace d8 {
@@ -25,12 +27,21 @@ int static_scratch_setup() {
     int dev = 0;
     D8_HIP(hipGetDevice(&dev));
     D8_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "static scratch: device %d beyond the %d this library tracks", dev, (int)MAX_DEVICES);
-    if (scratch_ptr[dev]) return 0;
-    void *p = nullptr;
-    D8_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-    D8_REQUIRE(p && ((size_t)p & 255) == 0, "static scratch: bad device address %p", p);
-    scratch_ptr[dev] = p;
-    return 0;
+    // one look-up per device, whichever host thread gets here first (the others wait for it)
+    static std::once_flag once[MAX_DEVICES];
+    static int status[MAX_DEVICES];
+    std::call_once(once[dev], [dev] {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            status[dev] = fail((int)e, "static scratch: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        } else if (!p || ((size_t)p & 255) != 0) {
+            status[dev] = fail(D8_ERR_ARGUMENT, "static scratch: bad device address %p", p);
+        } else {
+            scratch_ptr[dev] = p;
+        }
+    });
+    return status[dev];
 }
 
 }  // namespace d8

@@ -27,6 +27,9 @@ void MatrixMultiplyGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const 
 /** dy += x^T * dz */
 void MatrixMultiplyGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
 void MatrixMultiplyGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+// both at once (this build's addition: the executor calls it when both inputs take a gradient)
+void MatrixMultiplyGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
+void MatrixMultiplyGradXYGPU(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz);
 
 /** x [B,IH,IW,IC], y [OC,FH,FW,IC] (batch 1), z [B,OH,OW,OC]; the *InterimSize functions give
  *  the bytes of device scratch the caller must pass as the last argument. */

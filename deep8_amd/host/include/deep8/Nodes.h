@@ -141,6 +141,7 @@ public:
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
     void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
                   size_t index, Tensor *iGradient) override;
+    void backward() override;  // both gradients through one Math call when both inputs take one
 };
 
 class Conv2d : public Function {

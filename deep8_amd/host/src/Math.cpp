@@ -1,5 +1,6 @@
 // Math:: dispatchers (argument checks as in the reference) and their GPU bodies, which hand the
 // raw pointers and sizes to libdeep8_hip.so.  See deep8/Math.h for the reference line numbers.
+#include <algorithm>
 #include "deep8/Math.h"
 
 #include "deep8_hip.h"
@@ -166,6 +167,34 @@ void MatrixMultiplyGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const 
     const bool fresh = dy.takeZero();
     D8_CHECK((fresh ? d8_matmul_grad_y_overwrite : d8_matmul_grad_y)(dt, x.raw(), d.xb, d.xr, d.xc, dy.raw(), d.yb, d.yr, d.yc,
                                                                     dz.raw(), ws.ptr, ws.bytes, nullptr));
+}
+
+// Both gradients from one call (no counterpart in the reference, whose Function::backward runs once per input:
+// deep8/src/nodes/MatrixMultiply.cpp:31-52).  The two products are independent, so the library may run them as
+// one launch (d8_matmul_grad_xy); the results are those of MatrixMultiplyGradX followed by MatrixMultiplyGradY.
+void MatrixMultiplyGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz) {
+    DEEP8_ARGUMENT_CHECK(x.deviceType() == dx.deviceType() && x.deviceType() == y.deviceType() && x.deviceType() == dy.deviceType() &&
+                             x.deviceType() == z.deviceType() && x.deviceType() == dz.deviceType(),
+                         "the device type must be same");
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == dy.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    checkMatrixMultiplyShapes(x, y, z);
+    requireGPU(x);
+    MatrixMultiplyGradXYGPU(x, dx, y, dy, z, dz);
+}
+
+void MatrixMultiplyGradXYGPU(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &, const Tensor &dz) {
+    const MM d = mmDims(x, y);
+    const int dt = dtypeOf(x);
+    const size_t need = std::max(d8_matmul_scratch_bytes(dt, 1, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc),
+                                 d8_matmul_scratch_bytes(dt, 2, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
+    PoolScratch ws(x.device(), need);
+    // a gradient whose zero fill is still deferred is written, not added to
+    const int overwrite = (dx.takeZero() ? 1 : 0) | (dy.takeZero() ? 2 : 0);
+    D8_CHECK(d8_matmul_grad_xy(dt, x.raw(), dx.raw(), d.xb, d.xr, d.xc, y.raw(), dy.raw(), d.yb, d.yr, d.yc, dz.raw(), overwrite,
+                               ws.ptr, ws.bytes, nullptr));
 }
 
 // ---- Conv2d -------------------------------------------------------------------------------------------------------

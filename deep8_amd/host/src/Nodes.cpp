@@ -328,6 +328,17 @@ void MatrixMultiply::backward(const std::vector<const Tensor *> &in, const Tenso
     else DEEP8_RUNTIME_ERROR("the index is error");
 }
 
+// Both inputs take a gradient (the usual case): one Math call for the two products, which the library may run as one
+// launch.  The two gradients must be different tensors (x * x has one input twice: its two products add into the same
+// gradient, one after the other).
+void MatrixMultiply::backward() {
+    Variable *a = (Variable *)inputs[0], *b = (Variable *)inputs[1];
+    if (2 != inputs.size() || !a->updateGradient || !b->updateGradient || a == b) return Function::backward();
+    Variable *out = nullptr;
+    std::vector<const Tensor *> values = gatherInputs(this, out);
+    Math::MatrixMultiplyGradXY(*values[0], a->gradient, *values[1], b->gradient, out->value, out->gradient);
+}
+
 // ---- Conv2d / DeConv2d ---------------------------------------------------------------------------------------------------
 // An interim buffer from the device pool for one Math call; freed as soon as the call has
 // queued its kernels (single stream + a pool that never gives memory back while alive).

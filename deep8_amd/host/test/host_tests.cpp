@@ -310,6 +310,14 @@ void matmulCase(ElementType type, size_t xb, std::vector<size_t> xd, size_t yb, 
     EXPECT(z.host == wz);
     EXPECT(dx.host == wdx);
     EXPECT(dy.host == wdy);
+    // both gradients from one Math call, added to what the two calls left: twice the sums
+    Math::MatrixMultiplyGradXY(x.t, dx.t, y.t, dy.t, z.t, dz.t);
+    download(dx);
+    download(dy);
+    for (float &v : wdx) v *= 2;
+    for (float &v : wdy) v *= 2;
+    EXPECT(dx.host == wdx);
+    EXPECT(dy.host == wdy);
 }
 
 TEST_GPU(matrix_multiply_float_collapsed_batch) {  // MatrixMultiplyTest GPU1_float shape, reduced
@@ -947,16 +955,21 @@ TEST_GPU(fused_bias_relu_nodes_match_the_chain_of_nodes) {
         };
         Variable &x = parameter(&executor, 4, {12, 12, 64}), &w = parameter(&executor, {64, 3, 3, 64}), &b = parameter(&executor, {64});
         Variable &x2 = parameter(&executor, 5, {40, 96}), &y = parameter(&executor, {96, 136}), &c = parameter(&executor, {136});
+        // (a vector as y: z3 is [5][40] and the bias runs along x3's rows)
+        Variable &x3 = parameter(&executor, 5, {40, 96}), &v = parameter(&executor, {96}), &c3 = parameter(&executor, {40});
         fill(x, 1.f), fill(w, 0.1f), fill(b, 0.5f), fill(x2, 1.f), fill(y, 0.1f), fill(c, 0.5f);
+        fill(x3, 1.f), fill(v, 0.1f), fill(c3, 0.5f);
         Variable &z = fused ? conv2dBiasReLu(x, w, b) : relu(conv2d(x, w) + b);
         Variable &z2 = fused ? matrixMultiplyBiasReLu(x2, y, c) : relu(x2 * y + c);
-        EXPECT(z.shape() == Shape(4, {12, 12, 64}) && z2.shape() == Shape(5, {40, 136}));
+        Variable &z3 = fused ? matrixMultiplyBiasReLu(x3, v, c3) : relu(x3 * v + c3);
+        EXPECT(z.shape() == Shape(4, {12, 12, 64}) && z2.shape() == Shape(5, {40, 136}) && z3.shape() == Shape(5, {40}));
         results[fused].push_back(value(z));
         results[fused].push_back(value(z2));
-        backward(z.l2NormLoss() + z2.l2NormLoss());  // (one pass: the executor drops the graph after it)
-        for (Variable *v : {&x, &w, &b, &x2, &y, &c}) results[fused].push_back(grad(*v));
+        results[fused].push_back(value(z3));
+        backward(z.l2NormLoss() + z2.l2NormLoss() + z3.l2NormLoss());  // (one pass: the executor drops the graph after it)
+        for (Variable *p : {&x, &w, &b, &x2, &y, &c, &x3, &v, &c3}) results[fused].push_back(grad(*p));
     }
-    EXPECT(results[0].size() == 8 && results[1].size() == 8);
+    EXPECT(results[0].size() == 12 && results[1].size() == 12);
     for (size_t k = 0; k < results[0].size(); ++k) {
         const std::vector<float> &a = results[0][k], &f = results[1][k];
         EXPECT(a.size() == f.size());
@@ -966,8 +979,8 @@ TEST_GPU(fused_bias_relu_nodes_match_the_chain_of_nodes) {
             num += (double)(a[i] - f[i]) * (a[i] - f[i]), den += (double)a[i] * a[i];
             zeros |= a[i] == 0.f, positives |= a[i] > 0.f;
         }
-        if (k < 2) EXPECT(zeros && positives);  // the ReLu cut something and kept something
-        EXPECT(den > 0 && std::sqrt(num / den) <= (k < 2 ? 0.0 : 1e-6));
+        if (k < 3) EXPECT(zeros && positives);  // the ReLu cut something and kept something
+        EXPECT(den > 0 && std::sqrt(num / den) <= (k < 3 ? 0.0 : 1e-6));
     }
     // shape checks of the fused nodes
     EagerExecutor executor;

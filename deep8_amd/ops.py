@@ -105,6 +105,24 @@ def matmul_grad_y(x, y, dz, dy=None, overwrite=False):
     return _mm(2, x, dy, dz, overwrite)
 
 
+def matmul_grad_xy(x, y, dz, dx=None, dy=None, overwrite_x=False, overwrite_y=False):
+    """both gradients from one call (d8_matmul_grad_xy): returns (dx + dz * y^T, dy + x^T * dz)"""
+    lib = capi.init()
+    x, y, dz = np.ascontiguousarray(x), np.ascontiguousarray(y), np.ascontiguousarray(dz)
+    dx = np.zeros(x.shape, x.dtype) if dx is None else np.ascontiguousarray(dx)
+    dy = np.zeros(y.shape, y.dtype) if dy is None else np.ascontiguousarray(dy)
+    dt = _same_dtype(x, y, dz, dx, dy)
+    xb, xr, xc = _mat(x)
+    yb, yr, yc = _mat(y)
+    x_, y_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray.from_numpy(dz)
+    dx_, dy_ = DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
+    nb = max(lib.d8_matmul_scratch_bytes(dt, w, xb, xr, xc, yb, yr, yc) for w in (1, 2))
+    ws = _scratch(nb) if nb else None
+    check(lib.d8_matmul_grad_xy(dt, x_.ptr, dx_.ptr, xb, xr, xc, y_.ptr, dy_.ptr, yb, yr, yc, dz_.ptr,
+                                int(overwrite_x) | int(overwrite_y) << 1, ws.ptr if ws else None, nb, None))
+    return dx_.numpy(), dy_.numpy()
+
+
 # ---- geometry -------------------------------------------------------------------------------------
 def conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx):
     out = (ctypes.c_int * 4)()

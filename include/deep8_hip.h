@@ -37,6 +37,8 @@ const char *d8_last_error(void);
 int d8_device_init(int device_id);                /* hipSetDevice + arch check (gfx950)    */
 int d8_device_count(int *count);
 int d8_device_info(int *cu_count, int *clock_khz, size_t *hbm_bytes, char *name, int name_len);
+int d8_mem_info(size_t *free_bytes, size_t *total_bytes); /* device memory free / in all (no counterpart in
+                                                     the reference; lets a caller see that a call allocated nothing) */
 int d8_malloc(void **ptr, size_t bytes);          /* cudaMalloc      GPUMemoryAllocator.cu:17 */
 int d8_free(void *ptr);                           /* cudaFree        GPUMemoryAllocator.cu:27 */
 int d8_host_malloc(void **ptr, size_t bytes);     /* pinned host memory                    */
@@ -164,6 +166,16 @@ int d8_matmul_grad_x_overwrite(int dtype, void *dx, int xb, int xr, int xc,
 int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc,
                                void *dy, int yb, int yr, int yc, const void *dz,
                                void *scratch, size_t scratch_bytes, void *stream);
+/* Both gradients of one MatrixMultiply from one call: what Function::backward leaves after it has run for
+ * index 0 and for index 1 (deep8/src/nodes/MatrixMultiply.cpp:31-52 -> Math::MatrixMultiplyGradX, then
+ * Math::MatrixMultiplyGradY; deep8/src/math/MatrixMultiply.cu:193-363,381-551).  The two products are independent
+ * of each other, so large Float16 ones run as ONE launch in which a workgroup goes from a tile of dx straight on
+ * to a tile of dy; everything else is d8_matmul_grad_x followed by d8_matmul_grad_y.  The results are bit for bit
+ * those of the two calls.  overwrite: bit 0 -- dx is written instead of added to, bit 1 -- dy likewise (the
+ * _overwrite forms above).  scratch: the larger of d8_matmul_scratch_bytes(which = 1) and (which = 2).          */
+int d8_matmul_grad_xy(int dtype, const void *x, void *dx, int xb, int xr, int xc,
+                      const void *y, void *dy, int yb, int yr, int yc, const void *dz, int overwrite,
+                      void *scratch, size_t scratch_bytes, void *stream);
 
 /* d8_matmul_grad_y for callers that cannot allocate and have no scratch to pass.  No counterpart in the
  * reference: it is for code under HIP graph capture, tight serving loops and harnesses that forbid
@@ -287,8 +299,10 @@ int d8_relu_grad_overwrite(int dtype, const void *x, void *dx, const void *dy, l
  * passes of their own over the result (Math::AddGPU, deep8/src/math/Add.cu:21-52; Math::ReLuGPU,
  * deep8/src/math/ReLu.cu:20-59).  These entry points give the result of the three-call sequence from one call:
  *
- * d8_matmul_bias_relu   z = relu?(x * y + bias): d8_matmul, then bias[n] added to column n of z (the last axis;
- *                       bias: that many elements of the tensors' type, or NULL), then ReLu when relu != 0.
+ * d8_matmul_bias_relu   z = relu?(x * y + bias): d8_matmul, then bias[n] added along z's last axis (bias: that many
+ *                       elements of the tensors' type, or NULL), then ReLu when relu != 0.  z's last axis has yc
+ *                       elements when yc > 1; when y is a vector or a batch of vectors (yc == 1) z is [batch][xr]
+ *                       (deep8/src/nodes/MatrixMultiply.cpp:23-27) and the bias has xr elements.
  * d8_conv2d_bias_relu   the same after d8_conv2d (bias: OC elements).
  *     Both apply bias and ReLu in the store of the product's kernel (before the one rounding to the element type)
  *     wherever that kernel is one of the tiled ones, and otherwise run the product followed by ONE in-place pass.

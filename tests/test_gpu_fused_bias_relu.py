@@ -20,6 +20,9 @@ MM = [
     ((1, 1024, 512), (1, 512, 512)),   # 32 tiles over K = 512: split reduction, store in the reduce kernel
     ((1, 2048, 256), (1, 256, 2048)),  # 256 x 256 tiles (fp16: the large-output kernel)
     ((32, 8, 4096), (1, 4096, 200)),   # few rows against a wide layer
+    ((5, 40, 64), (1, 64)),            # a shared vector: z is [5][40], the bias runs along x's rows (40 values)
+    ((5, 40, 64), (5, 64)),            # a vector per batch element, x batched as well: likewise
+    ((1, 300, 128), (1, 128)),         # one matrix times one vector
 ]
 
 

@@ -284,7 +284,7 @@ def test_gemm_tall_product_with_a_remainder_band(ta, tb, M, N, K, dtype, monkeyp
     assert prod.max() < 2048
     for band_launch in (False, True):
         if band_launch:
-            monkeypatch.setenv("D8_GEMM_BAND_LAUNCH", "1")  # read once per process: only effective if set before the first such call
+            monkeypatch.setenv("D8_GEMM_BAND_LAUNCH", "1")  # (read at every call) the band as a second launch of its own
         for beta, C in ((0.0, None), (1.0, C0)):
             got = ops.gemm(ta, tb, c(A), c(B), None if C is None else c(C), beta)
             assert np.array_equal(f(got), prod + (0 if C is None else C)), (band_launch, beta)

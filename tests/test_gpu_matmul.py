@@ -97,6 +97,74 @@ def test_grad_accumulates_running_twice_doubles(oracle_port):
     assert np.array_equal(ops.matmul_grad_x(x, y, dz, once), 2 * once)
 
 
+@pytest.mark.parametrize("xs,ys", CASES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_matmul_both_gradients_from_one_call(oracle_port, xs, ys, dtype):
+    """d8_matmul_grad_xy leaves what d8_matmul_grad_x followed by d8_matmul_grad_y leave, in its accumulating and in
+    its overwriting form, for every shape case (small shapes: the two products run one after the other)."""
+    from deep8_amd import ops
+    r = rng(sum(xs) + 3 * sum(ys))
+    c = (lambda a: h(a)) if dtype == np.float16 else (lambda a: a)
+    hi = 2 if dtype == np.float16 else 20
+    x, y = ints(r, xs, hi), ints(r, ys, hi)
+    dz = ints(r, oracle_port.matmul(x, y).shape, hi)
+    dx0, dy0 = ints(r, xs, 3), ints(r, ys, 3)
+    want_dx, want_dy = oracle_port.matmul_grad_x(x, y, dz), oracle_port.matmul_grad_y(x, y, dz)
+    assert dtype == np.float32 or max(np.abs(want_dx).max(), np.abs(want_dy).max()) < 2040
+    gx, gy = ops.matmul_grad_xy(c(x), c(y), c(dz), c(dx0), c(dy0))
+    assert np.array_equal(f(gx), want_dx + dx0) and np.array_equal(f(gy), want_dy + dy0)
+    gx, gy = ops.matmul_grad_xy(c(x), c(y), c(dz), c(dx0 - 500), c(dy0 + 500), overwrite_x=True, overwrite_y=True)
+    assert np.array_equal(f(gx), want_dx) and np.array_equal(f(gy), want_dy)
+    gx, gy = ops.matmul_grad_xy(c(x), c(y), c(dz), c(dx0), c(dy0 + 500), overwrite_y=True)
+    assert np.array_equal(f(gx), want_dx + dx0) and np.array_equal(f(gy), want_dy)
+
+
+# (xr, xc, yc): both products large enough for the 256 x 256-tile kernel, so the call is ONE launch whose workgroups
+# walk tiles of dX, then tiles of dY
+PAIRS = [
+    (4096, 4096, 4096),   # configuration 3: 256 + 256 tiles on 256 compute units
+    (4096, 4360, 4096),   # tiles that stick out of C (moved back inside) in both products, 288 + 288 tiles
+    (3072, 4104, 4160),   # neither tile count divisible by eight: no XCD-contiguous runs
+    (4096, 3072, 8192),   # 192 + 384 tiles, reductions of 8192 and 4096
+]
+
+
+@pytest.mark.parametrize("xr,xc,yc", PAIRS)
+@pytest.mark.parametrize("overwrite", [True, False])
+def test_matmul_both_gradients_as_one_launch(xr, xc, yc, overwrite):
+    """integers, sparse enough that every sum stays below 2048: bit for bit against numpy in float32"""
+    from deep8_amd import ops
+    r = rng(xr + xc + yc)
+    keep = 300.0 / max(xr, xc, yc)
+    x = h(ints(r, (1, xr, xc), 3) * (r.random((1, xr, xc)) < keep))
+    y = h(ints(r, (1, xc, yc), 3))
+    dz = h(ints(r, (1, xr, yc), 3) * (r.random((1, xr, yc)) < keep))
+    dx0, dy0 = h(ints(r, x.shape, 3)), h(ints(r, y.shape, 3))
+    gx, gy = ops.matmul_grad_xy(x, y, dz, dx0, dy0, overwrite, overwrite)
+    wx = f(dz[0]) @ f(y[0]).T + (0 if overwrite else f(dx0[0]))
+    wy = f(x[0]).T @ f(dz[0]) + (0 if overwrite else f(dy0[0]))
+    assert wx.max() < 2048 and wy.max() < 2048
+    assert np.array_equal(f(gx[0]), wx) and np.array_equal(f(gy[0]), wy)
+    # and the two separate calls give the same bits
+    sx = ops.matmul_grad_x(x, y, dz, dx0, overwrite=overwrite)
+    sy = ops.matmul_grad_y(x, y, dz, dy0, overwrite=overwrite)
+    assert np.array_equal(gx.view(np.uint16), sx.view(np.uint16)) and np.array_equal(gy.view(np.uint16), sy.view(np.uint16))
+
+
+def test_matmul_both_gradients_as_one_launch_on_reals(oracle_port):
+    """configuration 3's data: the one-launch form against the two calls, bit for bit, and sampled rows against the oracle"""
+    from deep8_amd import ops
+    r = rng(77)
+    n = 4096
+    A, B, dC = h(nrm(r, (1, n, n), 1 / 64.0)), h(nrm(r, (1, n, n), 1 / 64.0)), h(nrm(r, (1, n, n), 1.0))
+    gx, gy = ops.matmul_grad_xy(A, B, dC, overwrite_x=True, overwrite_y=True)
+    assert np.array_equal(gx.view(np.uint16), ops.matmul_grad_x(A, B, dC, overwrite=True).view(np.uint16))
+    assert np.array_equal(gy.view(np.uint16), ops.matmul_grad_y(A, B, dC, overwrite=True).view(np.uint16))
+    rows = r.choice(n, 16, replace=False)
+    assert rel_fro(f(gx[0][rows]), oracle_port.gemm(0, 1, f(dC[0])[rows], f(B[0]))) <= FP16_TOL
+    assert rel_fro(f(gy[0][rows]), oracle_port.gemm(1, 0, np.ascontiguousarray(f(A[0])[:, rows]), f(dC[0]))) <= FP16_TOL
+
+
 def _against_reference_or_port(oracle_port, name, *args):
     import oracle
     src = oracle.ref if oracle.ref is not None else oracle_port

@@ -62,6 +62,32 @@ def test_two_calls_in_a_row_match_the_scratch_taking_entry_point(dtype, integers
 
 
 @pytest.mark.gpu
+def test_the_static_call_leaves_free_device_memory_unchanged():
+    """allocates and frees nothing: hipMemGetInfo's free bytes are the same before and after the call, the first
+    one on this device included (the look-up of the array's address allocates nothing either)"""
+    import ctypes
+    lib = capi.init()
+    rng = np.random.default_rng(9)
+    xb, xr, xc, yc = 16, 256, 256, 256
+    assert lib.d8_matmul_scratch_bytes(capi.FLOAT32, 2, xb, xr, xc, 1, xc, yc) > 0
+    x, dy0, dz = _case(rng, np.float32, xb, xr, xc, yc, True)
+    dx_, dy_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(dy0), DeviceArray.from_numpy(dz)
+
+    def free_bytes():
+        capi.sync()
+        f, t = ctypes.c_size_t(), ctypes.c_size_t()
+        check(lib.d8_mem_info(ctypes.byref(f), ctypes.byref(t)))
+        return f.value
+
+    before = free_bytes()
+    for _ in range(3):
+        check(lib.d8_matmul_grad_y_static(capi.FLOAT32, dx_.ptr, xb, xr, xc, dy_.ptr, 1, xc, yc, dz_.ptr, None))
+    assert free_bytes() == before
+    want = dy0 + 3 * np.einsum("brk,brn->kn", x.astype(np.float64), dz.astype(np.float64))[None]
+    assert np.array_equal(dy_.numpy().astype(np.float64), want)
+
+
+@pytest.mark.gpu
 def test_unsplit_shape_needs_no_scratch():
     rng = np.random.default_rng(8)
     x, dy0, dz = _case(rng, np.float32, 1, 64, 128, 256, True)
