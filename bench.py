@@ -1126,6 +1126,9 @@ def main():
     ap.add_argument("--wide-diagnostic", choices=sorted(WIDE_DIAGNOSTICS), default=None,
                     help="with --phases: compile the fp16 kernel with one of its diagnostic switches into a scratch "
                          "library and print that build's phase record (see the header of deep8_amd/csrc/gemm_wide.hip)")
+    ap.add_argument("--step-only", action="store_true",
+                    help="time the steps and print a short line: nothing else is launched (no per-call timings, no "
+                         "second sequence, no CPU baseline), so that a kernel trace of the run holds the step's kernels only")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain copy of this size (counter calibration under rocprofv3 --pmc)")
     a = ap.parse_args()
@@ -1154,6 +1157,11 @@ def main():
     wl = make_workload(a.workload)
     ms, samples = _time_steps(wl.step, a.steps, a.warmup)
     dtype = {2: "f16", 4: "f32", 8: "f64"}[wl.dtype.itemsize]
+    if a.step_only:
+        print(json.dumps({"workload": wl.name + (", fill + accumulate" if EAGER_ZERO else ""), "steps": a.steps, "warmup": a.warmup,
+                          "settle_ms": SETTLE_MS, "ms_per_step": round(ms, 4), "ms_per_step_samples": [round(v, 4) for v in samples],
+                          "tflops": round(wl.flops / (ms * 1e-3) / 1e12, 2), "dtype": dtype}), flush=True)
+        return
     is_conv = isinstance(wl, ConvWorkload)
     is_mm = isinstance(wl, MatMulWorkload)
     is_stream = isinstance(wl, (BiasReluWorkload, PoolWorkload, GatherMapsWorkload, DeconvMapsWorkload))  # HBM-bound kernels

@@ -382,6 +382,63 @@ __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restr
     }
 }
 
+// im2col where a thread writes whole filter windows: a workgroup owns one input row (b, iy).  The FH rows of dz its taps
+// read are copied into LDS as [fy][ox][oc] (zeros where the row lies outside the image; eight 16-byte pieces fetched per
+// thread before the first is written).  A thread then owns the FH * FW consecutive matrix columns of one (ix, oc): it
+// walks (fy, fx) with two counters, gathers VEC values at a time from LDS and stores them as one 16-byte piece (FH * FW
+// a multiple of VEC).  A pure copy: bit-exact.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void deconv_im2col_windows_kernel(const T *__restrict__ dz, T *__restrict__ dzmat, MapGeom g, FastDiv by_C,
+                                                                    FastDiv by_row) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char deconv_lds[];
+    T *rows = (T *)deconv_lds;  // [FH][OW][C]
+    typedef T VT __attribute__((ext_vector_type(VEC)));
+    const unsigned line = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);  // contiguous rows per XCD, as above
+    if (line >= (unsigned)(g.B * g.IH)) return;
+    const int iy = line % g.IH, b = line / g.IH;
+    const int taps = g.FH * g.FW, C = g.C;
+    const int N = C * taps, rowlen = g.OW * C, rowv = rowlen / VEC;  // rowlen is a multiple of VEC (C is)
+    constexpr int U = 8;
+    const int pieces = g.FH * rowv;
+    for (int p0 = threadIdx.x; p0 < pieces; p0 += 256 * U) {
+        VT v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned p = p0 + 256 * u;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[u][e] = (T)0;
+            if (p < (unsigned)pieces) {
+                const unsigned fy = div_by(p, by_row), q = p - fy * rowv;
+                const int oy = iy * g.sy + g.pt - (int)fy;
+                if (oy >= 0 && oy < g.OH) v[u] = *(const VT *)(dz + ((long)b * g.OH + oy) * rowlen + (long)q * VEC);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned p = p0 + 256 * u;
+            if (p < (unsigned)pieces) *(VT *)(rows + (long)p * VEC) = v[u];
+        }
+    }
+    __syncthreads();
+    T *out = dzmat + ((long)b * g.IH + iy) * g.IW * N;
+    const int cells = g.IW * C;
+    for (int p = threadIdx.x; p < cells; p += 256) {
+        const unsigned ix = div_by((unsigned)p, by_C), oc = (unsigned)p - ix * C;
+        T *dst = out + (long)ix * N + (long)oc * taps;
+        int fy = 0, fx = 0;
+        for (int t0 = 0; t0 < taps; t0 += VEC) {
+            VT v;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const int ox = (int)ix * g.sx + g.pl - fx;
+                v[e] = (ox >= 0 && ox < g.OW) ? rows[((long)fy * g.OW + ox) * C + oc] : (T)0;
+                if (++fx == g.FW) fx = 0, ++fy;
+            }
+            *(VT *)(dst + t0) = v;
+        }
+    }
+}
+
 // im2col: a workgroup owns one input row (b, iy).  The FH rows of dz its taps read are copied into LDS as
 // [fy][ox][oc] (zeros where the row lies outside the image); a thread then assembles VEC consecutive columns
 // (oc, fy, fx) of a matrix row from LDS and stores them at once.  A pure copy: bit-exact.
@@ -615,6 +672,15 @@ int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
         const long N = (long)OC * FH * FW;
         if (es <= 4 && OC % vec == 0 && N % vec == 0 && aligned16(dz) && aligned16(dzmat) && lds <= 60 * 1024 && N < (1L << 24) &&
             (long)IW * N < (1L << 31) && (long)B * IH < (1L << 31)) {
+            if ((FH * FW) % vec == 0 && (long)FH * OW * OC < (1L << 31)) {  // whole filter windows per thread
+                const FastDiv by_C = fast_div((unsigned)OC), by_row = fast_div((unsigned)(OW * OC / vec));
+                if (es == 4)
+                    hipLaunchKernelGGL((deconv_im2col_windows_kernel<unsigned, 4>), dim3((B * IH + 7) & ~7), dim3(256), lds, s, (const unsigned *)dz, (unsigned *)dzmat, g, by_C, by_row);
+                else
+                    hipLaunchKernelGGL((deconv_im2col_windows_kernel<unsigned short, 8>), dim3((B * IH + 7) & ~7), dim3(256), lds, s, (const unsigned short *)dz, (unsigned short *)dzmat, g, by_C, by_row);
+                D8_LAUNCH_CHECK();
+                return 0;
+            }
             const FastDiv by_T = fast_div((unsigned)(FH * FW)), by_FW = fast_div((unsigned)FW), by_NV = fast_div((unsigned)(N / vec));
             if (es == 4)
                 hipLaunchKernelGGL((deconv_im2col_lds_kernel<unsigned, 4>), dim3((B * IH + 7) & ~7), dim3(256), lds, s, (const unsigned *)dz, (unsigned *)dzmat, g, by_T, by_FW, by_NV);
