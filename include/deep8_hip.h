@@ -403,9 +403,11 @@ int d8_avgpool2d_grad_overwrite(int dtype, void *dx, const void *dy, int B, int 
  * d8_mfma_stream_out_bytes() bytes; *flops receives the flops one launch performs.             */
 /* A second aid needs no entry point: with D8_GEMM_STAMPS set in the environment before the first launch, a
  * d8_gemm call that runs the large-output fp16 kernel and is given an 8-byte aligned workspace of at least
- * 48 bytes per 256 x 256 tile of C leaves there, per workgroup, six 64-bit values: the chip's 100 MHz wall
- * clock at its start, after its prologue, after its K loop and after its last store was acknowledged, and
- * the shader clock before and after the loop.                                                          */
+ * 48 bytes per 256 x 256 tile of C leaves there, per tile, six 64-bit values: the chip's 100 MHz wall
+ * clock when its workgroup turned to the tile, when its K loop began and ended and when its epilogue was through
+ * (its stores acknowledged, for the workgroup's last tile), and the shader clock before and after the loop.
+ * d8_matmul_grad_xy does the same with its scratch when the two products run as one launch (the first product's
+ * tiles, then the second's).                                                                            */
 /* A third one, for the tiled kernels (fp16 / fp32 products and the convolutions they carry): after
  * d8_gemm_phase_record(records, bytes) every tiled launch whose records fit leaves 64 bytes per workgroup in
  * `records` (a device buffer, 8-byte aligned; index = workgroup id x + grid size x * id z): the same four wall
