@@ -303,7 +303,8 @@ __global__ __launch_bounds__(256) void deconv_im2col_kernel(const T *__restrict_
 // zmat[(b, iy, ix)][oc][fy][0 .. FW) of all ix, oc is copied into LDS as [ix][fx][oc]; a thread then owns VEC
 // channels of one output pixel, adds its taps from LDS into fp32 registers and, after the last fy, writes once.
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restrict__ zmat, T *__restrict__ z, MapGeom g) {
+__global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restrict__ zmat, T *__restrict__ z, MapGeom g, FastDiv by_C,
+                                                                FastDiv by_CV) {
     extern __shared__ __attribute__((aligned(16))) unsigned char deconv_lds[];
     T *slab = (T *)deconv_lds;  // [IW][FW][C]
     typedef T VT __attribute__((ext_vector_type(VEC)));
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restr
         const bool row8 = g.FW * sizeof(T) == 8 && (taps * sizeof(T)) % 8 == 0 && ((size_t)zmat & 7) == 0;
         const bool row16 = g.FW * sizeof(T) == 16 && (taps * sizeof(T)) % 16 == 0 && ((size_t)zmat & 15) == 0;
         for (int q = threadIdx.x; q < pairs; q += 256) {
-            const int ix = q / C, oc = q - ix * C;
+            const int ix = (int)div_by((unsigned)q, by_C), oc = q - ix * C;
             const T *p = src + (long)ix * N + (long)oc * taps;
             T *d = slab + ix * g.FW * C + oc;
             if (row8) {
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restr
         for (int o = 0; o < MAXO; ++o) {
             const int q = threadIdx.x + 256 * o;
             if (q < outs) {
-                const int ox = q / CV, cv = q - ox * CV;
+                const int ox = (int)div_by((unsigned)q, by_CV), cv = q - ox * CV;
                 for (int fx = 0; fx < g.FW; ++fx) {
                     const int tx = ox - g.pl + fx;
                     if (tx < 0 || tx % g.sx) continue;
@@ -639,9 +640,11 @@ int d8_deconv_col2im(int dtype, const void *zmat, void *z,
         const size_t es = dtype_bytes(dtype), vec = 16 / es, lds = (size_t)IW * FW * OC * es;
         if (es <= 4 && OC % vec == 0 && aligned16(z) && lds <= 60 * 1024 && (long)OW * (OC / vec) <= 1024 && (long)B * OH < (1L << 31)) {
             if (es == 4)
-                hipLaunchKernelGGL((deconv_col2im_lds_kernel<float, 4>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const float *)zmat, (float *)z, g);
+                hipLaunchKernelGGL((deconv_col2im_lds_kernel<float, 4>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const float *)zmat, (float *)z, g,
+                                   fast_div((unsigned)OC), fast_div((unsigned)(OC / vec)));
             else
-                hipLaunchKernelGGL((deconv_col2im_lds_kernel<f16, 8>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const f16 *)zmat, (f16 *)z, g);
+                hipLaunchKernelGGL((deconv_col2im_lds_kernel<f16, 8>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const f16 *)zmat, (f16 *)z, g,
+                                   fast_div((unsigned)OC), fast_div((unsigned)(OC / vec)));
             D8_LAUNCH_CHECK();
             return 0;
         }
