@@ -131,6 +131,36 @@ struct ConvShape {
 
 static unsigned magic_of(unsigned d) { return d <= 1 ? 0xFFFFFFFFu : (unsigned)((1ull << 32) / d); }
 
+// Whether a product with a patch-matrix operand can run: the tiled kernels have their alignment and size rules,
+// the fp64 kernel moves single elements and takes any shape.
+static bool implicit_eligible(int dtype, const GemmArgs &g, int ta, int tb) {
+    return dtype == D8_FLOAT64 ? true : gemm_tiled_eligible(dtype, g, ta, tb);
+}
+// Workspace such a product may use (the split of its reduction).
+static size_t implicit_workspace(int dtype, const GemmArgs &g) {
+    if (dtype == D8_FLOAT64) {
+        if (g.virt == VIRT_A_CLASSES) return 0;
+        int tps = 0;
+        const int pieces = gemm_f64_splits(g.M, g.N, g.K, g.batch, g.red, (size_t)-1, &tps);
+        return pieces > 1 ? (size_t)pieces * g.batch * g.M * g.N * sizeof(double) : 0;
+    }
+    return gemm_tiled_workspace(dtype, g.M, g.N, g.K, g.red, g.virt);
+}
+static int implicit_run(int dtype, GemmArgs &g, int ta, int tb, void *scratch, size_t scratch_bytes, hipStream_t stream) {
+    if (dtype == D8_FLOAT64) {
+        g.ws = (float *)scratch, g.ws_bytes = scratch ? scratch_bytes : 0;
+        return gemm_f64_launch(g, ta, tb, stream);
+    }
+    if (g.virt == VIRT_A_CLASSES) return gemm_tiled_launch(dtype, g, ta, tb, stream);
+    return gemm_tiled_run(dtype, g, ta, tb, scratch, scratch_bytes, stream);
+}
+
+// Float64 gradient of x: the product's N is the input channel count, and under 128 channels the fp64 kernel is
+// left with its 64 x 64 tiles, half the flops per operand byte of the 128 x 128 tiles that the staged product
+// ([patch rows] x [taps x channels]) runs on -- measured at B32 56x56x64 3x3: 0.53 ms against 0.42 ms staged,
+// col2im included.  From 128 channels on the patch product fills the large tiles too.
+static bool f64_grad_x_fills_tiles(int dtype, int IC) { return dtype != D8_FLOAT64 || IC >= 128; }
+
 static bool conv_implicit_plan(int dtype, int which, const ConvShape &c, const void *x, const void *w, const void *z,
                                GemmArgs &g, int &ta, int &tb) {
     const bool off = getenv("D8_CONV_EXPLICIT") != nullptr;  // tuning and test aid: force the im2col route
@@ -146,6 +176,7 @@ static bool conv_implicit_plan(int dtype, int which, const ConvShape &c, const v
     PatchGeom &pg = g.pg;
     if (which == 1) {  // dx[(b,iy,ix)][ic] += sum over taps of dz[b][iy + pt - fy*dy][ix + pl - fx*dx][:] . w[:][tap][ic]
         if (c.sy != 1 || c.sx != 1) return false;
+        if (!f64_grad_x_fills_tiles(dtype, c.IC)) return false;
         pg = {c.OH, c.OW, c.OC, c.IH, c.IW, c.FW, 1, 1, -c.dy, -c.dx, -c.pt, -c.pl, 0, 0, (unsigned)(M * c.OC * es)};
         g.virt = VIRT_A_ROWS;
         g.A = z, g.B = w, g.C = (void *)x;
@@ -171,7 +202,7 @@ static bool conv_implicit_plan(int dtype, int which, const ConvShape &c, const v
     }
     pg.mg_plane = magic_of((unsigned)pg.OH * pg.OW);
     pg.mg_ow = magic_of((unsigned)pg.OW);
-    return gemm_tiled_eligible(dtype, g, ta, tb);
+    return implicit_eligible(dtype, g, ta, tb);
 }
 
 // Conv2d's gradient of x for a stride above 1 (dilation 1), input pixel by input pixel: the pixels of dx with
@@ -182,9 +213,10 @@ static bool conv_classes_grad_x(int dtype, const ConvShape &c, const void *gx, c
     if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
     if ((c.sy == 1 && c.sx == 1) || c.dy != 1 || c.dx != 1 || c.sy * c.sx > MAX_CLASSES) return false;
     if (c.FH < c.sy || c.FW < c.sx || c.IH < c.sy || c.IW < c.sx) return false;  // every class needs a tap
+    if (!f64_grad_x_fills_tiles(dtype, c.IC)) return false;
     const long es = (long)dtype_bytes(dtype), T = (long)c.FH * c.FW;
     const long zbytes = (long)c.B * c.OH * c.OW * c.OC * es;
-    if (es == 8 || zbytes >= (1L << 31) || (long)c.B * c.IH * c.IW * c.IC * es >= (1L << 31) || T * c.IC * c.OC * es >= (1L << 31))
+    if (zbytes >= (1L << 31) || (long)c.B * c.IH * c.IW * c.IC * es >= (1L << 31) || T * c.IC * c.OC * es >= (1L << 31))
         return false;
     memset(&g, 0, sizeof(g));
     g.pg = {c.OH, c.OW, c.OC, 0, 0, 0, 1, 1, -1, -1, 0, 0, 0, 0, (unsigned)zbytes};
@@ -210,9 +242,9 @@ static bool conv_classes_grad_x(int dtype, const ConvShape &c, const void *gx, c
             smallest = k.M < smallest ? k.M : smallest;
             most_taps = k.red > most_taps ? k.red : most_taps;
         }
-    g.tiles_per_split = most_taps * (c.OC / gemm_tiled_k_step(dtype) + 1);
+    g.tiles_per_split = most_taps * (c.OC / (dtype == D8_FLOAT64 ? 16 : gemm_tiled_k_step(dtype)) + 1);
     g.M = smallest;
-    const bool ok = gemm_tiled_eligible(dtype, g, 0, 0);
+    const bool ok = implicit_eligible(dtype, g, 0, 0);
     g.M = largest;
     return ok;
 }
@@ -388,7 +420,7 @@ size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int 
     GemmArgs ga;
     int ta, tb;
     if (conv_implicit_plan(dtype, which, cs, nullptr, nullptr, nullptr, ga, ta, tb))
-        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red, ga.virt);
+        return implicit_workspace(dtype, ga);
     if (which == 1 && conv_classes_grad_x(dtype, cs, nullptr, nullptr, nullptr, ga)) return 0;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
     const size_t plain = col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
@@ -415,7 +447,7 @@ static int conv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC,
         int ta, tb;
         if (conv_implicit_plan(dtype, 0, cs, x, w, z, ga, ta, tb)) {
             ga.bias = bias, ga.relu = relu;  // applied in the tile store (and in the remainder band's reduction)
-            return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+            return implicit_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
         }
     }
     if (int rc = need_scratch("d8_conv2d", scratch, scratch_bytes, (size_t)M * K * dtype_bytes(dtype), x, w, z)) return rc;
@@ -467,11 +499,11 @@ static int d8_conv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int
         int ta, tb;
         if (conv_implicit_plan(dtype, 1, cs, gx, w, gz, ga, ta, tb)) {
             ga.beta = beta;
-            return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+            return implicit_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
         }
         if (conv_classes_grad_x(dtype, cs, gx, w, gz, ga)) {
             ga.beta = beta;
-            return gemm_tiled_launch(dtype, ga, 0, 0, as_stream(stream));
+            return implicit_run(dtype, ga, 0, 0, nullptr, 0, as_stream(stream));
         }
     }
     if (int rc = need_scratch("d8_conv2d_grad_x", scratch, scratch_bytes, (size_t)M * K * dtype_bytes(dtype), gx, w, gz)) return rc;
@@ -512,7 +544,7 @@ static int d8_conv2d_grad_y_impl(int dtype, const void *x, int B, int IH, int IW
         int ta, tb;
         if (conv_implicit_plan(dtype, 2, cs, x, gw, gz, ga, ta, tb)) {
             ga.beta = beta;
-            return gemm_tiled_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
+            return implicit_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
         }
     }
     if (int rc = need_scratch("d8_conv2d_grad_y", scratch, scratch_bytes, (size_t)M * K * dtype_bytes(dtype), x, gw, gz)) return rc;
@@ -568,7 +600,7 @@ static bool deconv_implicit_grad_x(int dtype, int B, int IH, int IW, int IC, int
     g.M = B * IH * IW, g.N = IC, g.K = OC;
     g.ldb = (int)(T * IC), g.sB = IC, g.ldc = IC;
     g.batch = 1, g.red = (int)T, g.splits = 1, g.beta = 1.f;
-    return gemm_tiled_eligible(dtype, g, 0, 0);
+    return implicit_eligible(dtype, g, 0, 0);
 }
 
 // z computed output pixel by output pixel: the sy * sx residue classes of output coordinates are each
@@ -579,7 +611,7 @@ static bool deconv_implicit_fwd(int dtype, int B, int IH, int IW, int IC, int OC
     if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
     const long es = (long)dtype_bytes(dtype), T = (long)FH * FW;
     const int OH = geo[0], OW = geo[1], pt = geo[2], pl = geo[3];
-    if (es == 8 || sy * sx > MAX_CLASSES || FH < sy || FW < sx || OH < sy || OW < sx) return false;
+    if (sy * sx > MAX_CLASSES || FH < sy || FW < sx || OH < sy || OW < sx) return false;
     const long xbytes = (long)B * IH * IW * IC * es;
     if (xbytes >= (1L << 31) || (long)B * OH * OW * OC * es >= (1L << 31) || T * IC * OC * es >= (1L << 31)) return false;
     memset(&g, 0, sizeof(g));
@@ -607,9 +639,9 @@ static bool deconv_implicit_fwd(int dtype, int B, int IH, int IW, int IC, int OC
             smallest = c.M < smallest ? c.M : smallest;
             most_taps = c.red > most_taps ? c.red : most_taps;
         }
-    g.tiles_per_split = most_taps * (IC / gemm_tiled_k_step(dtype) + 1);  // never the limit: a class walks all its taps
+    g.tiles_per_split = most_taps * (IC / (dtype == D8_FLOAT64 ? 16 : gemm_tiled_k_step(dtype)) + 1);  // never the limit: a class walks all its taps
     g.M = smallest;
-    const bool ok = gemm_tiled_eligible(dtype, g, 0, 1);
+    const bool ok = implicit_eligible(dtype, g, 0, 1);
     g.M = largest;
     return ok;
 }
@@ -622,7 +654,7 @@ static bool deconv_implicit_grad_y(int dtype, int B, int IH, int IW, int IC, int
     if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
     const long es = (long)dtype_bytes(dtype), T = (long)FH * FW;
     const long zbytes = (long)B * geo[0] * geo[1] * OC * es;
-    if (es == 8 || zbytes >= (1L << 31) || (long)B * IH * IW >= (1L << 31) || T * OC >= (1L << 31)) return false;
+    if (zbytes >= (1L << 31) || (long)B * IH * IW >= (1L << 31) || T * OC >= (1L << 31)) return false;
     memset(&g, 0, sizeof(g));
     g.pg = {geo[0], geo[1], OC, IH, IW, FW, sy, sx, -1, -1, -geo[2], -geo[3],
             magic_of((unsigned)IH * IW), magic_of((unsigned)IW), (unsigned)zbytes};
@@ -632,7 +664,7 @@ static bool deconv_implicit_grad_y(int dtype, int B, int IH, int IW, int IC, int
     g.lda = IC, g.ldc = IC;
     g.batch = 1, g.red = 1, g.splits = 1, g.beta = 1.f;
     g.perm_T = (int)T, g.perm_OC = OC;
-    return gemm_tiled_eligible(dtype, g, 1, 0);
+    return implicit_eligible(dtype, g, 1, 0);
 }
 
 // geo = {OH, OW, padTop, padLeft}: Deep8's own (from `covered`) or the caller's (the _ex entry points)
@@ -652,10 +684,10 @@ static size_t deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW
     const int M = B * IH * IW, T = FH * FW;
     GemmArgs ga;
     if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
-        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red, ga.virt);
+        return implicit_workspace(dtype, ga);
     if (which == 0 && deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga)) return 0;
     if (which == 2 && deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
-        return gemm_tiled_workspace(dtype, ga.M, ga.N, ga.K, ga.red, ga.virt);
+        return implicit_workspace(dtype, ga);
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
     return mat + gemm_ws(dtype, deconv_plan(which, M, T, OC, IC, nullptr, nullptr, nullptr));
 }
@@ -686,7 +718,7 @@ static int deconv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC
     {
         GemmArgs ga;
         if (deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, w, z, ga))
-            return gemm_tiled_launch(dtype, ga, 0, 1, as_stream(stream));
+            return implicit_run(dtype, ga, 0, 1, nullptr, 0, as_stream(stream));
     }
     if (int rc = need_scratch("d8_deconv2d", scratch, scratch_bytes, (size_t)M * T * OC * dtype_bytes(dtype), x, w, z)) return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;
@@ -727,7 +759,7 @@ static int deconv2d_grad_x_geo(int dtype, void *gx, int B, int IH, int IW, int I
         GemmArgs ga;
         if (deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, gx, w, gz, ga)) {
             ga.beta = beta;
-            return gemm_tiled_run(dtype, ga, 0, 0, scratch, scratch_bytes, as_stream(stream));
+            return implicit_run(dtype, ga, 0, 0, scratch, scratch_bytes, as_stream(stream));
         }
     }
     if (int rc = need_scratch("d8_deconv2d_grad_x", scratch, scratch_bytes, (size_t)M * T * OC * dtype_bytes(dtype), gx, w, gz)) return rc;
@@ -771,7 +803,7 @@ static int deconv2d_grad_y_geo(int dtype, const void *x, int B, int IH, int IW, 
         GemmArgs ga;
         if (deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, gw, gz, ga)) {
             ga.beta = beta;
-            return gemm_tiled_run(dtype, ga, 1, 0, scratch, scratch_bytes, as_stream(stream));
+            return implicit_run(dtype, ga, 1, 0, scratch, scratch_bytes, as_stream(stream));
         }
     }
     if (int rc = need_scratch("d8_deconv2d_grad_y", scratch, scratch_bytes, (size_t)M * T * OC * dtype_bytes(dtype), x, gw, gz)) return rc;

@@ -105,7 +105,17 @@ def test_matmul_f64(oracle, oracle_port, xs, ys):
         assert rel_fro(ops.matmul_grad_y(x, y, g), oracle_port.matmul_grad_y(x, y, g)) <= F64_TOL
 
 
-@pytest.mark.parametrize("cfg", CONV)
+# 128 input channels or more: the gradient of x reads its patch rows of dz inside the GEMM as well (stride 1:
+# one product per tap; stride 2: by residue classes of input pixels)
+CONV_WIDE = [
+    (2, 12, 12, 128, 24, 3, 3, True, 1, 1, 1, 1),
+    (1, 10, 10, 136, 8, 3, 3, False, 1, 1, 2, 2),
+    (2, 12, 12, 128, 16, 3, 3, True, 2, 2, 1, 1),
+    (1, 11, 9, 130, 5, 4, 3, False, 2, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", CONV + CONV_WIDE)
 def test_conv2d_f64(oracle, oracle_port, cfg):
     from deep8_amd import ops
     B, IH, IW, IC, OC, FH, FW = cfg[:7]
@@ -151,6 +161,78 @@ def test_deconv2d_f64(oracle, oracle_port, cfg):
         assert rel_fro(ops.deconv2d(x, w, *a), oracle_port.deconv2d(x, w, *a)) <= F64_TOL
         assert rel_fro(ops.deconv2d_grad_x(x, w, g, *a), oracle_port.deconv2d_grad_x(x, w, g, *a)) <= F64_TOL
         assert rel_fro(ops.deconv2d_grad_y(x, w, g, *a), oracle_port.deconv2d_grad_y(x, w, g, *a)) <= F64_TOL
+
+
+@pytest.mark.parametrize("cfg", CONV + CONV_WIDE)
+def test_conv2d_f64_stages_nothing_and_the_staged_route_agrees(oracle, oracle_port, monkeypatch, cfg):
+    """Float64 convolutions read their patch matrix from the image inside the GEMM (every shape: the fp64 kernel
+    moves single elements), so they ask for less scratch than the im2col matrix -- except the gradient of x under
+    128 input channels, or strided with a dilation or without a tap for every class of input pixels, which stays
+    staged; the staged route, forced through the same entry points, still gives the oracle's result."""
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx, dy, dx = cfg
+    a = cfg[7:]
+    OH, OW, _, _ = ops.conv2d_geometry(IH, IW, FH, FW, *a)
+    col = B * OH * OW * FH * FW * IC * 8
+    for which in range(3):
+        q = lambda: lib.d8_conv2d_scratch_bytes(capi.FLOAT64, which, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx, dy, dx)
+        staged = which == 1 and (IC < 128 or ((sy, sx) != (1, 1) and ((dy, dx) != (1, 1) or FH < sy or FW < sx or IH < sy or IW < sx)))
+        assert (q() < col) == (not staged), (which, q(), col)
+        monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+        assert q() >= col
+        monkeypatch.delenv("D8_CONV_EXPLICIT")
+    r = rng(B + IH + OC + 31)
+    xi, wi = d(ints(r, (B, IH, IW, IC))), d(ints(r, (OC, FH, FW, IC)))
+    gz = d(ints(r, (B, OH, OW, OC), 10))
+    monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+    with oracle.float64():
+        assert np.array_equal(ops.conv2d(xi, wi, *a), oracle_port.conv2d(xi, wi, *a))
+        assert np.array_equal(ops.conv2d_grad_x(xi, wi, gz, *a, xi), oracle_port.conv2d_grad_x(xi, wi, gz, *a, xi))
+        assert np.array_equal(ops.conv2d_grad_y(xi, wi, gz, *a, wi), oracle_port.conv2d_grad_y(xi, wi, gz, *a, wi))
+
+
+@pytest.mark.parametrize("cfg", DECONV)
+def test_deconv2d_f64_stages_nothing_and_the_staged_route_agrees(oracle, oracle_port, monkeypatch, cfg):
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    B, IH, IW, IC, OC, FH, FW, cov, sy, sx = cfg
+    a = cfg[7:]
+    OH, OW, _, _ = ops.deconv2d_geometry(IH, IW, FH, FW, *a)
+    interim = B * IH * IW * FH * FW * OC * 8
+    for which in range(3):
+        q = lambda: lib.d8_deconv2d_scratch_bytes(capi.FLOAT64, which, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx)
+        staged = which == 0 and (FH < sy or FW < sx or OH < sy or OW < sx or sy * sx > 16)  # a class of output pixels without a tap
+        assert (q() < interim) == (not staged), (which, q(), interim)
+        monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+        assert q() >= interim
+        monkeypatch.delenv("D8_CONV_EXPLICIT")
+    r = rng(B + IH + OC + 32)
+    xi, wi = d(ints(r, (B, IH, IW, IC), 10)), d(ints(r, (OC, FH, FW, IC), 10))
+    gz = d(ints(r, (B, OH, OW, OC), 10))
+    monkeypatch.setenv("D8_CONV_EXPLICIT", "1")
+    with oracle.float64():
+        assert np.array_equal(ops.deconv2d(xi, wi, *a), oracle_port.deconv2d(xi, wi, *a))
+        assert np.array_equal(ops.deconv2d_grad_x(xi, wi, gz, *a, xi), oracle_port.deconv2d_grad_x(xi, wi, gz, *a, xi))
+        assert np.array_equal(ops.deconv2d_grad_y(xi, wi, gz, *a, wi), oracle_port.deconv2d_grad_y(xi, wi, gz, *a, wi))
+
+
+def test_f64_convolutions_on_the_large_tiles(oracle, oracle_port):
+    """Shapes whose products fill the chip with 128 x 128 tiles: Conv2d forward (patch rows as A) and DeConv2d
+    forward (four classes of output pixels), integers bit for bit and reals to 1e-12."""
+    from deep8_amd import ops
+    r = rng(4242)
+    with oracle.float64():
+        xi, wi = d(ints(r, (8, 28, 28, 256), 4)), d(ints(r, (512, 3, 3, 256), 4))
+        a = (True, 1, 1, 1, 1)
+        assert np.array_equal(ops.conv2d(xi, wi, *a), oracle_port.conv2d(xi, wi, *a))
+        x, w = r.standard_normal(xi.shape), r.standard_normal(wi.shape)
+        assert rel_fro(ops.conv2d(x, w, *a), oracle_port.conv2d(x, w, *a)) <= F64_TOL
+        xi, wi = d(ints(r, (8, 14, 14, 256), 4)), d(ints(r, (512, 4, 4, 256), 4))
+        a = (True, 2, 2)
+        assert np.array_equal(ops.deconv2d(xi, wi, *a), oracle_port.deconv2d(xi, wi, *a))
+        x, w = r.standard_normal(xi.shape), r.standard_normal(wi.shape)
+        assert rel_fro(ops.deconv2d(x, w, *a), oracle_port.deconv2d(x, w, *a)) <= F64_TOL
 
 
 @pytest.mark.parametrize("cfg", CONV[:5])
