@@ -256,6 +256,50 @@ def test_matmul_step_replayed_from_a_hip_graph(oracle_port):
     check(lib.d8_stream_destroy(side))
 
 
+def test_half_step_with_both_gradients_in_one_launch_replayed_from_a_hip_graph():
+    """The same for the large half products: forward on the 256 x 256-tile kernel, d8_matmul_grad_xy as one launch of
+    workgroups that walk several tiles -- captured once, replayed three times with eager calls in between, every
+    replay bit for bit the eager result (3072 x 4104 x 4160: tile counts that fill neither the chip nor the XCDs
+    evenly)."""
+    import ctypes
+    from deep8_amd import capi
+    from deep8_amd.capi import DeviceArray, check
+    lib = capi.init()
+    r = rng(31)
+    xs, ys, zs = (1, 3072, 4104), (1, 4104, 4160), (1, 3072, 4160)
+    x, y, dz = h(nrm(r, xs, 1 / 64.0)), h(nrm(r, ys, 1 / 64.0)), h(nrm(r, zs, 1.0))
+    dx_, dy_, ddz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray.from_numpy(dz)
+    z_, gx_, gy_ = DeviceArray(zs, np.float16), DeviceArray(xs, np.float16), DeviceArray(ys, np.float16)
+    nb = max(lib.d8_matmul_scratch_bytes(capi.FLOAT16, w, *xs, *ys) for w in range(3))
+    ws = DeviceArray((max(nb, 16),), np.uint8)
+
+    def step(stream):
+        check(lib.d8_matmul(capi.FLOAT16, dx_.ptr, *xs, dy_.ptr, *ys, z_.ptr, ws.ptr, nb, stream))
+        gy_.zero_(stream)  # dY accumulates into a zeroed gradient, dX is written by the overwrite form
+        check(lib.d8_matmul_grad_xy(capi.FLOAT16, dx_.ptr, gx_.ptr, *xs, dy_.ptr, gy_.ptr, *ys, ddz.ptr, 1, ws.ptr, nb, stream))
+
+    step(None)
+    capi.sync()
+    want = [a.numpy().view(np.uint16).copy() for a in (z_, gx_, gy_)]
+    assert all(w_.any() for w_ in want)
+    side, graph = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib.d8_stream_create(ctypes.byref(side)))
+    check(lib.d8_graph_begin(side))
+    step(side)
+    check(lib.d8_graph_end(side, ctypes.byref(graph)))
+    for replay in range(3):
+        for out in (z_, gx_, gy_):
+            out.copy_from(np.full(out.shape, -7.0, np.float16))
+        check(lib.d8_graph_launch(graph, side))
+        capi.sync(side)
+        for out, w_ in zip((z_, gx_, gy_), want):
+            assert np.array_equal(out.numpy().view(np.uint16), w_), replay
+        step(None)  # eager work between the replays
+        capi.sync()
+    check(lib.d8_graph_destroy(graph))
+    check(lib.d8_stream_destroy(side))
+
+
 # Batches longer than one launch's third grid axis takes: cublas*gemmStridedBatched has no such limit
 # (deep8/src/math/MatrixMultiply.cu:115-134), so neither may d8_gemm.  600 and 1000 are walked in slices.
 LONG_BATCH = [
