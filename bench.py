@@ -364,6 +364,22 @@ class ConvWorkload:
         self._call(getattr(self.lib, ("d8_deconv2d_grad_y" if self.deconv else "d8_conv2d_grad_y") + first),
                    self.x.ptr, self.gw.ptr, self.gz.ptr)
 
+    def grad_xy(self):
+        """both gradients from one call (d8_conv2d_grad_xy / d8_deconv2d_grad_xy), as this build's Conv2d / DeConv2d
+        nodes issue them; on a layer whose products each leave compute units idle they share a launch"""
+        from deep8_amd.capi import check
+        B, IH, IW, IC = self.xd
+        OC, FH, FW, _ = self.wd
+        fn = self.lib.d8_deconv2d_grad_xy if self.deconv else self.lib.d8_conv2d_grad_xy
+        if self.explicit:
+            os.environ["D8_CONV_EXPLICIT"] = "1"
+        try:
+            check(fn(self.dt, self.x.ptr, self.gx.ptr, B, IH, IW, IC, self.w.ptr, self.gw.ptr, OC, FH, FW, self.gz.ptr, *self.geo,
+                     0 if EAGER_ZERO else 3, self.ws.ptr, self.ws_bytes, self.stream))
+        finally:
+            if self.explicit:
+                os.environ.pop("D8_CONV_EXPLICIT", None)
+
     def step(self):
         """forward + both gradients as the executor issues them: its zeroGradient() is deferred, so the
         first (here: only) product into each gradient is the overwrite form; --eager-zero fills and
@@ -372,12 +388,11 @@ class ConvWorkload:
         if EAGER_ZERO:
             self.gx.zero_()
             self.gw.zero_()
-        self.grad_x()
-        self.grad_y()
+        self.grad_xy()
 
     def parts(self):
         f = self.flops / 3
-        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
+        return {"fwd": (self.fwd, f), "grad_xy": (self.grad_xy, 2 * f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
 
     def gemm_roofline(self, reps):
         """The pass-forward GEMM launch, timed alone with HIP events, against the MFMA peak of its
@@ -503,19 +518,23 @@ class DeconvLiteralWorkload:
         check(self.lib.d8_deconv2d_grad_y_ex(self.dt, self.x.ptr, *self.shape, self.dw.ptr, *self.filt, self.dz.ptr, *self.geo,
                                              0 if EAGER_ZERO else 1, self.ws.ptr, self.ws_bytes, None))
 
+    def grad_xy(self):
+        from deep8_amd.capi import check
+        check(self.lib.d8_deconv2d_grad_xy_ex(self.dt, self.x.ptr, self.dx.ptr, *self.shape, self.w.ptr, self.dw.ptr, *self.filt, self.dz.ptr,
+                                              *self.geo, 0 if EAGER_ZERO else 3, self.ws.ptr, self.ws_bytes, None))
+
     def step(self):
         self.fwd()
         if EAGER_ZERO:
             self.dx.zero_()
             self.dw.zero_()
-        self.grad_x()
-        self.grad_y()
+        self.grad_xy()
 
-    kernel = "gemm_tiled_kernel<f16> (one launch each for forward, dX, dW; patch rows read by the tile loader)"
+    kernel = "gemm_tiled_kernel<f16> (one launch for forward, one for dX and dW together; patch rows read by the tile loader)"
 
     def parts(self):
         f = self.flops / 3
-        return {"fwd": (self.fwd, f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
+        return {"fwd": (self.fwd, f), "grad_xy": (self.grad_xy, 2 * f), "grad_x": (self.grad_x, f), "grad_y": (self.grad_y, f)}
 
 
 class GatherMapsWorkload:

@@ -75,6 +75,10 @@ SIGNATURES = {
     "d8_deconv2d_geometry": (_I, [_I] * 7 + [ctypes.POINTER(_I)]),
     "d8_conv2d_scratch_bytes": (_Z, [_I] * 14),
     "d8_conv2d": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
+    "d8_conv_grad_pair_launches": (ctypes.c_ulong, []),
+    "d8_conv2d_grad_xy": (_I, [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P] + [_I] * 6 + [_P, _Z, _P]),
+    "d8_deconv2d_grad_xy": (_I, [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P] + [_I] * 4 + [_P, _Z, _P]),
+    "d8_deconv2d_grad_xy_ex": (_I, [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P] + [_I] * 7 + [_P, _Z, _P]),
     "d8_conv2d_grad_x": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "d8_conv2d_grad_y": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "d8_conv2d_grad_x_overwrite": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),

@@ -12,6 +12,8 @@
 //   accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32]
 // Both LDS tiles are kept K-contiguous ([row][k]), so one 16-byte LDS read feeds an MFMA
 // operand; the transposed-operand cases differ only in how the tile loader walks global memory.
+#include <atomic>
+
 #include "gemm_args.h"
 
 namespace d8 {
@@ -610,6 +612,40 @@ int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspa
     return gemm_tiled_run_whole(dtype, second, transA, transB, workspace, workspace_bytes, stream);
 }
 
+static std::atomic<unsigned long> pair_launches{0};  // d8_conv_grad_pair_launches
+
+// Both gradients of a convolution as one launch (gemm_tiled_pair_launch) when that fills compute units the two
+// products would each leave idle: gx is not cut into a band and not split, the workgroups of both fit the chip
+// side by side (two per compute unit).  gy's reduction is split as it would be alone and reduced afterwards.
+// Returns false, with nothing launched, when the pair does not qualify; *rc is the launches' status otherwise.
+bool gemm_tiled_run_pair(int dtype, GemmArgs &gx, GemmArgs &gy, void *workspace, size_t workspace_bytes, hipStream_t stream, int *rc) {
+    const bool off = getenv("D8_CONV_GRADS_APART") != nullptr;  // tuning and test aid (read at every call)
+    if (off || dtype == D8_FLOAT64) return false;
+    if (gx.virt != VIRT_A_ROWS || gy.virt != VIRT_B_KROWS || gx.batch != 1 || gy.batch != 1) return false;
+    if (!gemm_tiled_eligible(dtype, gx, 0, 0) || !gemm_tiled_eligible(dtype, gy, 1, 0)) return false;
+    if (balanced_rows(gx)) return false;
+    const size_t usable = (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0;
+    const int BK = gemm_tiled_k_step(dtype);
+    int tps = 0;
+    // Alone, a gx of few tiles would be cut into pieces to fill the chip; beside gy's workgroups it runs whole when
+    // its reduction is short: up to 40 K steps in half, where a step waits longer than it multiplies (B16 14x14x256
+    // 4x4 s2 DeConv2d: 43.3 -> 30.1 us, 3x3 Conv2d of 256 channels at B16 14x14: 45.5 -> 37.4 us); never in fp32,
+    // whose steps are bound by the matrix pipe (36 steps whole: 49 -> 80 us).
+    const char *lim = getenv("D8_CONV_PAIR_STEPS");  // tuning and test aid (read at every call)
+    const long whole_steps = lim ? atol(lim) : (dtype == D8_FLOAT16 ? 40 : 0);
+    if (plan_splits(BK, gx.M, gx.N, gx.K, 1, gx.red, usable, &tps, gx.virt) != 1 && (long)gx.red * ceil_div(gx.K, BK) > whole_steps) return false;
+    gx.splits = 1, gx.tiles_per_split = gx.red * ceil_div(gx.K, BK);
+    gx.ws = nullptr, gx.tail_splits = 0;
+    gy.ws = (float *)workspace, gy.tail_splits = 0;
+    gy.splits = plan_splits(BK, gy.M, gy.N, gy.K, 1, gy.red, usable, &gy.tiles_per_split, gy.virt);
+    const long wgs = gemm_tiled_pair_workgroups(dtype, gx, gy);
+    if (wgs <= 0 || wgs > 2L * cu_count()) return false;
+    ++pair_launches;
+    *rc = gemm_tiled_pair_launch(dtype, gx, gy, stream);
+    if (*rc == 0 && gy.splits > 1) *rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(gy, stream) : launch_reduce<float>(gy, stream);
+    return true;
+}
+
 bool gemm_fuses_store(int dtype, const GemmArgs &g, int transA, int transB) {
     // (a product beyond one launch's limits -- more than 448 outputs, more than 65535 * 128 rows -- is cut into several
     // by d8_gemm; the fused store stays out of that: the caller runs the product and one pass over its result)
@@ -690,6 +726,8 @@ static int gemm_one(int dtype, int transA, int transB, int M, int N, int K,
     return dtype == D8_FLOAT16 ? launch<f16>(g, transA, transB, tiled, as_stream(stream))
                                : launch<float>(g, transA, transB, tiled, as_stream(stream));
 }
+
+unsigned long d8_conv_grad_pair_launches(void) { return pair_launches.load(); }
 
 int d8_gemm_phase_record(void *records, size_t bytes) {
     D8_REQUIRE(((size_t)records & 7) == 0, "d8_gemm_phase_record: the record buffer is not 8-byte aligned");

@@ -103,6 +103,12 @@ int gemm_tiled_k_step(int dtype);  // K elements per step: 64 (fp16) or 32 (fp32
 bool gemm_tiled_eligible(int dtype, const GemmArgs &g, int transA, int transB);
 // Launch; with g.splits > 1 the fp32 partial sums go to g.ws for the caller to reduce.
 int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipStream_t stream);
+// Two patch-matrix products as ONE launch: gx with patch rows as A (NN: a convolution's gradient of its input), gy with
+// patch k-rows as B (TN: its filter gradient; g.splits / tiles_per_split set, the caller reduces).  Workgroups of
+// both are resident side by side.  gemm_tiled_pair_workgroups: how many workgroups the launch would have, 0 when the
+// pair cannot run this way (the tiles the two products would choose have no common kernel, or one is cut into a band).
+long gemm_tiled_pair_workgroups(int dtype, const GemmArgs &gx, const GemmArgs &gy);
+int gemm_tiled_pair_launch(int dtype, const GemmArgs &gx, const GemmArgs &gy, hipStream_t stream);
 // Where the next launches write their per-workgroup phase records (GemmArgs::phase_rec); null switches them off.
 void gemm_tiled_phase_record(void *records, size_t bytes);
 
@@ -131,6 +137,10 @@ bool gemm_tiled_half_tiles(int M, int N, int batch, long k_steps, int BK);
 // Plan the split of the reduction, launch the tiled kernel (which must be eligible) and reduce.
 int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspace, size_t workspace_bytes,
                    hipStream_t stream);
+// The two gradients of a convolution (gx: patch rows as A, NN, into the input's gradient; gy: patch k-rows as B, TN,
+// into the filter's) as one launch where that pays; false, with nothing launched, where it does not (the caller then
+// runs them one after the other).  The workspace is gy's.
+bool gemm_tiled_run_pair(int dtype, GemmArgs &gx, GemmArgs &gy, void *workspace, size_t workspace_bytes, hipStream_t stream, int *rc);
 // Workspace gemm_tiled_run may use for this shape.
 size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red, int virt = VIRT_NONE);
 // Whether a product whose B is a patch matrix (VIRT_B_KROWS) runs on 64 x 64 tiles: fewer than 128 rows, and the last

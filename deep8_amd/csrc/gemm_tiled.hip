@@ -329,21 +329,17 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[T::TM][T::TN], float *l
         }
 }
 
-// TAIL: K is not a multiple of the K step (an instantiation of its own, so that the per-piece offsets of the
-// ordinary case stay constants)
-template <typename T, bool TAIL = false>
-__global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tilesM, int tilesN) {
+// The work of one workgroup: workgroup (bx, bz) of a grid of nbx x layers (the launch's own blockIdx / gridDim, or what a
+// launch of two products makes of them).  As0 .. Bs1: the two halves of both operand areas in LDS.
+template <typename T, bool TAIL>
+__device__ __forceinline__ void gemm_tiled_body(const GemmArgs &g, int tilesM, const int tilesN, const int bx, const int bz, const int nbx,
+                                                typename T::E *As0, typename T::E *As1, typename T::E *Bs0, typename T::E *Bs1) {
     typedef typename T::E E;
     typedef typename T::EL EL;
     typedef E EV __attribute__((ext_vector_type(T::EPV)));
     constexpr int BM = T::BM, BN = T::BN, BK = T::BK, TM = T::TM, TN = T::TN, A_LD = T::A_LD, B_LD = T::B_LD;
     constexpr int A_IT = T::A_IT, NP = T::NP, ES = T::ES, EPV = T::EPV;
     constexpr bool A_KC = T::A_KC, B_KC = T::B_KC;
-    // four separate arrays, so that reads of one half are known not to touch the other
-    __shared__ __attribute__((aligned(16))) E As0[T::A_SZ];
-    __shared__ __attribute__((aligned(16))) E As1[T::A_SZ];
-    __shared__ __attribute__((aligned(16))) E Bs0[T::B_SZ];
-    __shared__ __attribute__((aligned(16))) E Bs1[T::B_SZ];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / T::WGN, wn = wave % T::WGN;
@@ -365,17 +361,17 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
     RowMap crow = {0, 0, 0, 0, 0, 0, 0, 0, g.perm_T, g.perm_OC};
     const RowMap plain = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     if constexpr (VIRT == VIRT_A_CLASSES) {
-        const OutClass &c = g.cls[blockIdx.z];
+        const OutClass &c = g.cls[bz];
         M = c.M, red = c.red, b_cls = c.b_off;
         pg.OH = c.OH, pg.OW = c.OW, pg.FW = c.taps_w, pg.pt = c.pt, pg.pl = c.pl;
         crow = {c.OH * c.OW, c.OW, g.out_H, g.out_W, g.out_sy, g.out_sx, c.py, c.px, 0, 0};
         tilesM = (M + BM - 1) / BM;
-        if ((int)blockIdx.x >= tilesM * tilesN) return;  // the grid is sized for the largest class
+        if (bx >= tilesM * tilesN) return;  // the grid is sized for the largest class
     }
-    int id = blockIdx.x;
+    int id = bx;
     const int total = tilesM * tilesN;
-    int b = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z / g.splits;
-    int split = VIRT == VIRT_A_CLASSES ? 0 : blockIdx.z - b * g.splits;
+    int b = VIRT == VIRT_A_CLASSES ? 0 : bz / g.splits;
+    int split = VIRT == VIRT_A_CLASSES ? 0 : bz - b * g.splits;
     // a workgroup past the product's own tiles works on the remainder band (GemmArgs::tail_m0)
     const bool in_tail = VIRT != VIRT_A_CLASSES && g.tail_splits > 0 && id >= total;
     int tps = g.tiles_per_split;
@@ -636,12 +632,49 @@ __global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tiles
         __builtin_amdgcn_s_waitcnt(0x0f70);  // this wave's stores have been acknowledged
         st_w[3] = wall_clock64();
         if (tid == 0) {
-            unsigned long long *rec = g.phase_rec + 8 * (blockIdx.x + (unsigned long long)gridDim.x * blockIdx.z);
+            unsigned long long *rec = g.phase_rec + 8 * (bx + (unsigned long long)nbx * bz);
             rec[0] = st_w[0], rec[1] = st_w[1], rec[2] = st_w[2], rec[3] = st_w[3], rec[4] = st_c[0], rec[5] = st_c[1];
             // s_getreg_b32 of all 32 bits of hardware registers 20 (XCC_ID) and 4 (HW_ID: wave, SIMD, CU, SH, SE)
             rec[6] = ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
             rec[7] = in_tail ? 1 : 0;
         }
+    }
+}
+
+// TAIL: K is not a multiple of the K step (an instantiation of its own, so that the per-piece offsets of the
+// ordinary case stay constants)
+template <typename T, bool TAIL = false>
+__global__ __launch_bounds__(T::NT) void gemm_tiled_kernel(GemmArgs g, int tilesM, int tilesN) {
+    typedef typename T::E E;
+    // four separate arrays, so that reads of one half are known not to touch the other
+    __shared__ __attribute__((aligned(16))) E As0[T::A_SZ];
+    __shared__ __attribute__((aligned(16))) E As1[T::A_SZ];
+    __shared__ __attribute__((aligned(16))) E Bs0[T::B_SZ];
+    __shared__ __attribute__((aligned(16))) E Bs1[T::B_SZ];
+    gemm_tiled_body<T, TAIL>(g, tilesM, tilesN, (int)blockIdx.x, (int)blockIdx.z, (int)gridDim.x, As0, As1, Bs0, Bs1);
+}
+
+// Two products in one launch: the first nx0 * nz0 workgroups are the first product's grid (x fastest), the rest the
+// second's.  Built for the two gradients of a convolution on a small layer, which are independent of each other and
+// each leave the chip half empty: their workgroups are short (a dozen K steps between a prologue and an epilogue
+// that nothing hides when a compute unit holds one workgroup), and side by side on a compute unit one's waits are
+// the other's issue slots.  The operand areas are as large as the larger tile needs.
+template <typename T0, typename T1>
+__global__ __launch_bounds__(T0::NT) void gemm_tiled_pair_kernel(GemmArgs g0, GemmArgs g1, int tilesM0, int tilesN0, int nx0, int nz0,
+                                                                 int tilesM1, int tilesN1, int nx1) {
+    typedef typename T0::E E;
+    static_assert(T0::NT == T1::NT && sizeof(typename T0::E) == sizeof(typename T1::E), "one workgroup shape, one element type");
+    constexpr int A_SZ = T0::A_SZ > T1::A_SZ ? T0::A_SZ : T1::A_SZ, B_SZ = T0::B_SZ > T1::B_SZ ? T0::B_SZ : T1::B_SZ;
+    __shared__ __attribute__((aligned(16))) E As0[A_SZ];
+    __shared__ __attribute__((aligned(16))) E As1[A_SZ];
+    __shared__ __attribute__((aligned(16))) E Bs0[B_SZ];
+    __shared__ __attribute__((aligned(16))) E Bs1[B_SZ];
+    const int id = (int)blockIdx.x, first = nx0 * nz0;
+    if (id < first) {
+        gemm_tiled_body<T0, false>(g0, tilesM0, tilesN0, id % nx0, id / nx0, nx0, As0, As1, Bs0, Bs1);
+    } else {
+        const int j = id - first;
+        gemm_tiled_body<T1, false>(g1, tilesM1, tilesN1, j % nx1, j / nx1, nx1, As0, As1, Bs0, Bs1);
     }
 }
 
@@ -677,8 +710,11 @@ static int launch_tiled(const GemmArgs &g0, hipStream_t stream) {
     return 0;
 }
 
+// Which tile a product runs on.
+enum TileId { TILE_WIDE, TILE_256, TILE_128x64, TILE_64x64, TILE_64x128, TILE_128x128 };
+
 template <typename E, bool A_KC, bool B_KC, int VIRT = VIRT_NONE>
-static int pick_tile(const GemmArgs &g, hipStream_t stream) {
+static TileId choose_tile(const GemmArgs &g) {
     static const char *force = getenv("D8_GEMM_TILE");  // tuning aid
     const long big_tiles = (long)ceil_div(g.M, 256) * ceil_div(g.N, 256) * g.batch * g.splits;
     bool big = g.M >= 256 && g.N >= 256 && big_tiles >= (long)cu_count() * 3 / 4;
@@ -687,21 +723,97 @@ static int pick_tile(const GemmArgs &g, hipStream_t stream) {
     // keeps the matrix pipe fed, and the compiler cannot hold the 256 x 256 variant in registers
     if constexpr (sizeof(E) == 2) {
         static const char *wide = getenv("D8_GEMM_WIDE");  // tuning aid: 0 keeps the 32x32x16 kernel
-        if (big && VIRT == VIRT_NONE && !(wide && atoi(wide) == 0) && gemm_wide_eligible(g, !A_KC, B_KC))
-            return gemm_wide_launch(g, !A_KC, B_KC, stream);
-        if (big) return launch_tiled<E, 256, 256, 4, 2, A_KC, B_KC, VIRT>(g, stream);
+        if (big && VIRT == VIRT_NONE && !(wide && atoi(wide) == 0) && gemm_wide_eligible(g, !A_KC, B_KC)) return TILE_WIDE;
+        if (big) return TILE_256;
     }
     // a 64-wide side gets a tile of that width (im2col products with 64 output channels)
-    if (g.N < 128) return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+    if (g.N < 128) return TILE_128x64;
     // a patch-matrix product whose last 128-column tile would be at most half full: 64 x 64 tiles, no padding
     // multiplied (C4's filter gradient, N = 576: 83.7 -> 73.8 us)
-    if constexpr (VIRT == VIRT_B_KROWS) {
-        if (gemm_tiled_krows_64(VIRT, g.M, g.N)) return launch_tiled<E, 64, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
-    }
-    if (g.M < 128) return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+    if (gemm_tiled_krows_64(VIRT, g.M, g.N)) return TILE_64x64;
+    if (g.M < 128) return TILE_64x128;
     if (g.splits == 1 && gemm_tiled_half_tiles(g.M, g.N, g.batch, (long)g.red * ceil_div(g.K, 128 / (int)sizeof(E)), 128 / (int)sizeof(E)))
-        return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+        return TILE_64x128;
+    return TILE_128x128;
+}
+
+template <typename E, bool A_KC, bool B_KC, int VIRT = VIRT_NONE>
+static int pick_tile(const GemmArgs &g, hipStream_t stream) {
+    switch (choose_tile<E, A_KC, B_KC, VIRT>(g)) {
+        case TILE_WIDE: return gemm_wide_launch(g, !A_KC, B_KC, stream);
+        case TILE_256:
+            if constexpr (sizeof(E) == 2) return launch_tiled<E, 256, 256, 4, 2, A_KC, B_KC, VIRT>(g, stream);
+            break;
+        case TILE_128x64: return launch_tiled<E, 128, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+        case TILE_64x64:
+            if constexpr (VIRT == VIRT_B_KROWS) return launch_tiled<E, 64, 64, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+            break;
+        case TILE_64x128: return launch_tiled<E, 64, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+        default: break;
+    }
     return launch_tiled<E, 128, 128, 2, 2, A_KC, B_KC, VIRT>(g, stream);
+}
+
+// ---- two products in one launch (gemm_tiled_pair_kernel): gx has patch rows as A (NN), gy patch k-rows as B (TN) --
+// the gradients of a convolution's input and filter.  Neither is split into a remainder band; gy may be split along
+// its reduction (the caller reduces).
+static void grid_of(TileId t, const GemmArgs &g, int &tilesM, int &tilesN) {
+    const int bm = (t == TILE_64x64 || t == TILE_64x128) ? 64 : 128, bn = (t == TILE_64x64 || t == TILE_128x64) ? 64 : 128;
+    tilesM = ceil_div(g.M, bm), tilesN = ceil_div(g.N, bn);
+}
+
+template <typename TX, typename TY>
+static int launch_pair_tiles(const GemmArgs &gx0, const GemmArgs &gy0, hipStream_t stream) {
+    GemmArgs gx = gx0, gy = gy0;
+    gx.phase_rec = gy.phase_rec = nullptr;
+    const int tMx = ceil_div(gx.M, TX::BM), tNx = ceil_div(gx.N, TX::BN), tMy = ceil_div(gy.M, TY::BM), tNy = ceil_div(gy.N, TY::BN);
+    // the longer-running product first: gy's pieces, then gx's tiles
+    const int ny = tMy * tNy, nzy = gy.batch * gy.splits, nx = tMx * tNx;
+    hipLaunchKernelGGL((gemm_tiled_pair_kernel<TY, TX>), dim3(ny * nzy + nx), dim3(TX::NT), 0, stream, gy, gx, tMy, tNy, ny, nzy, tMx, tNx, nx);
+    D8_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename E>
+static bool pair_tiles(const GemmArgs &gx, const GemmArgs &gy, TileId &tx, TileId &ty) {
+    tx = choose_tile<E, true, false, VIRT_A_ROWS>(gx), ty = choose_tile<E, false, false, VIRT_B_KROWS>(gy);
+    const bool x_ok = tx == TILE_64x128 || tx == TILE_128x128 || tx == TILE_128x64;
+    const bool y_ok = ty == TILE_128x128 || ty == TILE_64x128 || ty == TILE_64x64;
+    return x_ok && y_ok;
+}
+
+template <typename E>
+static int launch_pair(const GemmArgs &gx, const GemmArgs &gy, hipStream_t stream) {
+    TileId tx, ty;
+    if (!pair_tiles<E>(gx, gy, tx, ty)) return fail(D8_ERR_ARGUMENT, "gemm_tiled_pair_launch: no kernel for this pair of tiles");
+#define D8_PAIR_Y(TXT)                                                                                                  \
+    switch (ty) {                                                                                                       \
+        case TILE_128x128: return launch_pair_tiles<TXT, Tile<E, 128, 128, 2, 2, false, false, VIRT_B_KROWS>>(gx, gy, stream); \
+        case TILE_64x128: return launch_pair_tiles<TXT, Tile<E, 64, 128, 2, 2, false, false, VIRT_B_KROWS>>(gx, gy, stream);   \
+        default: return launch_pair_tiles<TXT, Tile<E, 64, 64, 2, 2, false, false, VIRT_B_KROWS>>(gx, gy, stream);            \
+    }
+    typedef Tile<E, 64, 128, 2, 2, true, false, VIRT_A_ROWS> X0;
+    typedef Tile<E, 128, 128, 2, 2, true, false, VIRT_A_ROWS> X1;
+    typedef Tile<E, 128, 64, 2, 2, true, false, VIRT_A_ROWS> X2;
+    if (tx == TILE_64x128) { D8_PAIR_Y(X0) }
+    if (tx == TILE_128x128) { D8_PAIR_Y(X1) }
+    D8_PAIR_Y(X2)
+#undef D8_PAIR_Y
+}
+
+long gemm_tiled_pair_workgroups(int dtype, const GemmArgs &gx, const GemmArgs &gy) {
+    TileId tx, ty;
+    if (gx.virt != VIRT_A_ROWS || gy.virt != VIRT_B_KROWS || gx.tail_splits || gy.tail_splits || gx.splits != 1 || gx.batch != 1 || gy.batch != 1)
+        return 0;
+    if (!(dtype == D8_FLOAT16 ? pair_tiles<f16>(gx, gy, tx, ty) : pair_tiles<float>(gx, gy, tx, ty))) return 0;
+    int mx, nx, my, ny;
+    grid_of(tx, gx, mx, nx);
+    grid_of(ty, gy, my, ny);
+    return (long)mx * nx + (long)my * ny * gy.splits;
+}
+
+int gemm_tiled_pair_launch(int dtype, const GemmArgs &gx, const GemmArgs &gy, hipStream_t stream) {
+    return dtype == D8_FLOAT16 ? launch_pair<f16>(gx, gy, stream) : launch_pair<float>(gx, gy, stream);
 }
 
 template <typename E>

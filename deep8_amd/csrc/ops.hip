@@ -866,4 +866,72 @@ D8_CONV_GRAD_PAIR(d8_conv2d_grad_y, const void *a0, void *a1)
 D8_DECONV_GRAD_PAIR(d8_deconv2d_grad_x, void *a0, const void *a1)
 D8_DECONV_GRAD_PAIR(d8_deconv2d_grad_y, const void *a0, void *a1)
 
+// Both gradients of a convolution from one call: what the _grad_x call followed by the _grad_y call leave
+// (overwrite: bit 0 -- gx is written instead of added to, bit 1 -- gw likewise).  Where both gradients read their
+// patch matrices inside the GEMM and each would leave compute units idle, they run as ONE launch
+// (gemm_tiled_run_pair); otherwise one after the other.
+int d8_conv2d_grad_xy(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
+                      const void *w, void *gw, int OC, int FH, int FW, const void *gz,
+                      int covered, int sy, int sx, int dy, int dx, int overwrite,
+                      void *scratch, size_t scratch_bytes, void *stream) {
+    const float bx = (overwrite & 1) ? 0.f : 1.f, bw = (overwrite & 2) ? 0.f : 1.f;
+    int g[4];
+    if (int rc = check_conv("d8_conv2d_grad_xy", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return rc;
+    if (int rc = d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return rc;
+    D8_REQUIRE(x && gx && w && gw && gz, "d8_conv2d_grad_xy: null tensor");
+    {
+        const ConvShape cs = {B, IH, IW, IC, OC, FH, FW, g[0], g[1], sy, sx, dy, dx, g[2], g[3]};
+        GemmArgs px, pw;
+        int ta, tb;
+        if (conv_implicit_plan(dtype, 1, cs, gx, w, gz, px, ta, tb) && conv_implicit_plan(dtype, 2, cs, x, gw, gz, pw, ta, tb)) {
+            px.beta = bx, pw.beta = bw;
+            int rc = 0;
+            if (gemm_tiled_run_pair(dtype, px, pw, scratch, scratch_bytes, as_stream(stream), &rc)) return rc;
+        }
+    }
+    if (int rc = d8_conv2d_grad_x_impl(dtype, gx, B, IH, IW, IC, w, OC, FH, FW, gz, covered, sy, sx, dy, dx, scratch, scratch_bytes, stream, bx))
+        return rc;
+    return d8_conv2d_grad_y_impl(dtype, x, B, IH, IW, IC, gw, OC, FH, FW, gz, covered, sy, sx, dy, dx, scratch, scratch_bytes, stream, bw);
+}
+
+static int deconv2d_grad_xy_geo(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
+                                const void *w, void *gw, int OC, int FH, int FW, const void *gz,
+                                const int *g, int sy, int sx, int overwrite,
+                                void *scratch, size_t scratch_bytes, void *stream) {
+    const float bx = (overwrite & 1) ? 0.f : 1.f, bw = (overwrite & 2) ? 0.f : 1.f;
+    D8_REQUIRE(x && gx && w && gw && gz, "d8_deconv2d_grad_xy: null tensor");
+    if (int rc = check_deconv_out("d8_deconv2d_grad_xy", B, g)) return rc;
+    {
+        GemmArgs px, pw;
+        if (deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, gx, w, gz, px) &&
+            deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, gw, gz, pw)) {
+            px.beta = bx, pw.beta = bw;
+            int rc = 0;
+            if (gemm_tiled_run_pair(dtype, px, pw, scratch, scratch_bytes, as_stream(stream), &rc)) return rc;
+        }
+    }
+    if (int rc = deconv2d_grad_x_geo(dtype, gx, B, IH, IW, IC, w, OC, FH, FW, gz, g, sy, sx, scratch, scratch_bytes, stream, bx)) return rc;
+    return deconv2d_grad_y_geo(dtype, x, B, IH, IW, IC, gw, OC, FH, FW, gz, g, sy, sx, scratch, scratch_bytes, stream, bw);
+}
+
+int d8_deconv2d_grad_xy(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
+                        const void *w, void *gw, int OC, int FH, int FW, const void *gz,
+                        int covered, int sy, int sx, int overwrite,
+                        void *scratch, size_t scratch_bytes, void *stream) {
+    int g[4];
+    if (int rc = check_conv("d8_deconv2d_grad_xy", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = d8_deconv2d_geometry(IH, IW, FH, FW, covered, sy, sx, g)) return rc;
+    return deconv2d_grad_xy_geo(dtype, x, gx, B, IH, IW, IC, w, gw, OC, FH, FW, gz, g, sy, sx, overwrite, scratch, scratch_bytes, stream);
+}
+
+int d8_deconv2d_grad_xy_ex(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
+                           const void *w, void *gw, int OC, int FH, int FW, const void *gz,
+                           int OH, int OW, int padTop, int padLeft, int sy, int sx, int overwrite,
+                           void *scratch, size_t scratch_bytes, void *stream) {
+    const int g[4] = {OH, OW, padTop, padLeft};
+    if (int rc = check_conv("d8_deconv2d_grad_xy_ex", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, 1, 1)) return rc;
+    if (int rc = check_deconv_geo("d8_deconv2d_grad_xy_ex", g)) return rc;
+    return deconv2d_grad_xy_geo(dtype, x, gx, B, IH, IW, IC, w, gw, OC, FH, FW, gz, g, sy, sx, overwrite, scratch, scratch_bytes, stream);
+}
+
 }  // extern "C"

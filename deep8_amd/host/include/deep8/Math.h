@@ -44,6 +44,8 @@ void Conv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor &
 size_t Conv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX);
 void Conv2dGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *interimPtr);
 void Conv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX, void *xcol);
+// both gradients from one call; takes its scratch from the device pool itself
+void Conv2dGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, int dilationY, int dilationX);
 
 size_t DeConv2dInterimSize(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX);
 void DeConv2d(const Tensor &x, const Tensor &y, Tensor &z, bool covered, int strideY, int strideX, void *interimPtr);
@@ -56,6 +58,7 @@ void DeConv2dGradXGPU(const Tensor &x, Tensor &dx, const Tensor &y, const Tensor
 size_t DeConv2dGradYInterimSize(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX);
 void DeConv2dGradY(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
 void DeConv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX, void *interimPtr);
+void DeConv2dGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY, int strideX);
 
 // Add (broadcasting) and ReLu: deep8/include/math/Add.h:15-42 (checks deep8/src/math/Add.cpp:7-107),
 // deep8/include/math/ReLu.h:14-30 (checks deep8/src/math/ReLu.cpp:6-36).  Unlike the reference, whose

@@ -156,6 +156,7 @@ public:
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
     void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
                   size_t index, Tensor *iGradient) override;
+    void backward() override;  // both gradients through one Math call when both inputs take one
 };
 
 class DeConv2d : public Function {
@@ -169,6 +170,7 @@ public:
     void forward(const std::vector<const Tensor *> &inputs, Tensor *output) override;
     void backward(const std::vector<const Tensor *> &inputs, const Tensor *output, const Tensor *outputGradient,
                   size_t index, Tensor *iGradient) override;
+    void backward() override;  // both gradients through one Math call when both inputs take one
 };
 
 // z = x + y under numpy's broadcasting rule (deep8/include/nodes/Add.h:8-27, deep8/src/nodes/Add.cpp:6-45)

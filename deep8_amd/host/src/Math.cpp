@@ -269,6 +269,26 @@ void Conv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor &
     D8_CHECK((fresh ? d8_conv2d_grad_y_overwrite : d8_conv2d_grad_y)(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS, xcol, bytes, nullptr));
 }
 
+// Both gradients from one call (no counterpart in the reference, whose Conv2d::backward runs once per input:
+// deep8/src/nodes/Conv2d.cpp:85-151).  The products are independent; on a small layer the library runs them as one
+// launch (d8_conv2d_grad_xy).  The results are those of Conv2dGradX followed by Conv2dGradY.
+void Conv2dGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY,
+                  int strideX, int dilationY, int dilationX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == dy.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    const ConvDims d = checkConv(x, y, z, CONV_ARGS);
+    requireGPU(x);
+    const int dt = dtypeOf(x);
+    const size_t need = std::max(d8_conv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS),
+                                 d8_conv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS));
+    PoolScratch ws(x.device(), need);
+    const int overwrite = (dx.takeZero() ? 1 : 0) | (dy.takeZero() ? 2 : 0);  // deferred zero fills: write instead of add
+    D8_CHECK(d8_conv2d_grad_xy(dt, x.raw(), dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), dy.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS,
+                               overwrite, ws.ptr, ws.bytes, nullptr));
+}
+
 #undef CONV_ARGS
 
 // ---- DeConv2d -------------------------------------------------------------------------------------------------------
@@ -341,6 +361,24 @@ void DeConv2dGradYGPU(const Tensor &x, const Tensor &y, Tensor &dy, const Tensor
     const size_t bytes = d8_deconv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
     const bool fresh = dy.takeZero();  // deferred zero fill: write instead of add
     D8_CHECK((fresh ? d8_deconv2d_grad_y_overwrite : d8_deconv2d_grad_y)(dt, x.raw(), d.B, d.IH, d.IW, d.IC, dy.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS, interimPtr, bytes, nullptr));
+}
+
+// Both gradients from one call, as Conv2dGradXY (deep8/src/nodes/DeConv2d.cpp:74-126 runs them one per input).
+void DeConv2dGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &z, const Tensor &dz, bool covered, int strideY,
+                    int strideX) {
+    DEEP8_ARGUMENT_CHECK(x.elementType == dx.elementType && x.elementType == y.elementType && x.elementType == dy.elementType &&
+                             x.elementType == z.elementType && x.elementType == dz.elementType,
+                         "the data type must be same");
+    DEEP8_ARGUMENT_CHECK(x.shape == dx.shape && y.shape == dy.shape && z.shape == dz.shape, "the shape is error");
+    const ConvDims d = checkDeConv(x, y, z, DECONV_ARGS);
+    requireGPU(x);
+    const int dt = dtypeOf(x);
+    const size_t need = std::max(d8_deconv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS),
+                                 d8_deconv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS));
+    PoolScratch ws(x.device(), need);
+    const int overwrite = (dx.takeZero() ? 1 : 0) | (dy.takeZero() ? 2 : 0);
+    D8_CHECK(d8_deconv2d_grad_xy(dt, x.raw(), dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), dy.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS,
+                                 overwrite, ws.ptr, ws.bytes, nullptr));
 }
 
 #undef DECONV_ARGS

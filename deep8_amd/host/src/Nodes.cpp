@@ -408,6 +408,17 @@ void Conv2d::backward(const std::vector<const Tensor *> &in, const Tensor *outpu
     }
 }
 
+// Input and filter both take a gradient (the usual case inside a network): one Math call for the two products, which
+// the library runs as one launch on a small layer.  (Conv2dBiasReLu has its own backward().)
+void Conv2d::backward() {
+    Variable *a = (Variable *)inputs[0], *b = (Variable *)inputs[1];
+    if (2 != inputs.size() || !a->updateGradient || !b->updateGradient || a == b) return Function::backward();
+    Variable *out = nullptr;
+    std::vector<const Tensor *> values = gatherInputs(this, out);
+    Math::Conv2dGradXY(*values[0], a->gradient, *values[1], b->gradient, out->value, out->gradient, covered, strideY, strideX,
+                       dilationY, dilationX);
+}
+
 DeConv2d::DeConv2d(std::vector<Node *> &in, bool cov, int sy, int sx)
     : Function(in), forwardCovered(cov), forwardStrideY(sy), forwardStrideX(sx) {
     DEEP8_ARGUMENT_CHECK(2 == inputs.size(), "the DeConv2d Function needs 2 input");
@@ -451,6 +462,15 @@ void DeConv2d::backward(const std::vector<const Tensor *> &in, const Tensor *out
     } else {
         DEEP8_RUNTIME_ERROR("the index of DeConv2d backward is error");
     }
+}
+
+void DeConv2d::backward() {
+    Variable *a = (Variable *)inputs[0], *b = (Variable *)inputs[1];
+    if (2 != inputs.size() || !a->updateGradient || !b->updateGradient || a == b) return Function::backward();
+    Variable *out = nullptr;
+    std::vector<const Tensor *> values = gatherInputs(this, out);
+    Math::DeConv2dGradXY(*values[0], a->gradient, *values[1], b->gradient, out->value, out->gradient, forwardCovered, forwardStrideY,
+                         forwardStrideX);
 }
 
 // ---- contraction + bias + ReLu as one node ---------------------------------------------------------------------------

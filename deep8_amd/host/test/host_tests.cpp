@@ -416,6 +416,14 @@ void convCase(ElementType type, int B, int IH, int IW, int IC, int OC, int FH, i
     EXPECT(z.host == wz);
     EXPECT(gx.host == wgx);
     EXPECT(gw.host == wgw);
+    // both gradients from one Math call, added to what the two calls left: twice the sums
+    Math::Conv2dGradXY(x.t, gx.t, w.t, gw.t, z.t, gz.t, covered, sy, sx, dy, dx);
+    download(gx);
+    download(gw);
+    for (float &v : wgx) v *= 2;
+    for (float &v : wgw) v *= 2;
+    EXPECT(gx.host == wgx);
+    EXPECT(gw.host == wgw);
 }
 
 TEST_GPU(conv2d_float_covered_stride_dilation) {  // Conv2dTest forwardCPU_float geometry, smaller tensors
@@ -425,6 +433,9 @@ TEST_GPU(conv2d_float_covered_5x5) { convCase(ElementType::from<float>(), 2, 12,
 TEST_GPU(conv2d_float_not_covered) { convCase(ElementType::from<float>(), 2, 13, 11, 5, 3, 3, 3, false, 1, 1, 1, 1, 20); }
 TEST_GPU(conv2d_double) { convCase(ElementType::from<double>(), 2, 13, 11, 5, 3, 3, 3, true, 2, 2, 1, 1, 20); }
 TEST_GPU(conv2d_half) { convCase(ElementType::from<half>(), 2, 8, 8, 8, 8, 3, 3, true, 1, 1, 1, 1, 2); }
+// wide enough for the tiled kernels: in half the two gradient products of the one-call form share a launch
+TEST_GPU(conv2d_half_64_channels) { convCase(ElementType::from<half>(), 2, 16, 16, 64, 64, 3, 3, true, 1, 1, 1, 1, 1); }
+TEST_GPU(conv2d_float_64_channels) { convCase(ElementType::from<float>(), 2, 16, 16, 64, 64, 3, 3, true, 1, 1, 1, 1, 5); }
 
 // ---- DeConv2d -----------------------------------------------------------------------------------------------------
 void deconvCase(ElementType type, int B, int IH, int IW, int IC, int OC, int FH, int FW, bool covered, int sy, int sx, int hi) {
@@ -474,6 +485,13 @@ void deconvCase(ElementType type, int B, int IH, int IW, int IC, int OC, int FH,
     EXPECT(z.host == wz);
     EXPECT(gx.host == wgx);
     EXPECT(gw.host == wgw);
+    Math::DeConv2dGradXY(x.t, gx.t, w.t, gw.t, z.t, gz.t, covered, sy, sx);
+    download(gx);
+    download(gw);
+    for (float &v : wgx) v *= 2;
+    for (float &v : wgw) v *= 2;
+    EXPECT(gx.host == wgx);
+    EXPECT(gw.host == wgw);
 }
 
 TEST_GPU(deconv2d_float_not_covered_stride3) { deconvCase(ElementType::from<float>(), 2, 8, 8, 8, 4, 4, 4, false, 3, 3, 20); }
@@ -481,6 +499,8 @@ TEST_GPU(deconv2d_float_covered_stride3) { deconvCase(ElementType::from<float>()
 TEST_GPU(deconv2d_float_stride2) { deconvCase(ElementType::from<float>(), 2, 7, 6, 4, 6, 4, 4, false, 2, 2, 20); }
 TEST_GPU(deconv2d_double) { deconvCase(ElementType::from<double>(), 2, 7, 6, 4, 6, 4, 4, false, 2, 2, 20); }
 TEST_GPU(deconv2d_half) { deconvCase(ElementType::from<half>(), 2, 6, 6, 8, 8, 4, 4, false, 2, 2, 2); }
+TEST_GPU(deconv2d_half_64_channels) { deconvCase(ElementType::from<half>(), 2, 8, 8, 64, 64, 4, 4, false, 2, 2, 1); }
+TEST_GPU(deconv2d_float_64_channels) { deconvCase(ElementType::from<float>(), 2, 8, 8, 64, 64, 4, 4, false, 2, 2, 5); }
 
 TEST_GPU(conv2d_errors) {
     ElementType f32 = ElementType::from<float>();

@@ -287,6 +287,53 @@ def deconv2d_grad_y(x, w, gz, covered=False, sy=1, sx=1, gw=None, overwrite=Fals
     return dgw.numpy()
 
 
+def _both(overwrite_x, overwrite_w):
+    return (1 if overwrite_x else 0) | (2 if overwrite_w else 0)
+
+
+def conv2d_grad_xy(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None, gw=None, overwrite_x=False, overwrite_w=False):
+    """both gradients of Conv2d from one call (d8_conv2d_grad_xy): returns (gx, gw)"""
+    lib = capi.init()
+    x, w, gz = np.ascontiguousarray(x), _filt(w), np.ascontiguousarray(gz)
+    dt = _same_dtype(x, w, gz)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = w.shape
+    gx = np.zeros(x.shape, x.dtype) if gx is None else np.ascontiguousarray(gx)
+    gw = np.zeros(w.shape, x.dtype) if gw is None else _filt(gw)
+    dx_, dw_, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
+    dgx, dgw = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(gw)
+    nb = max(lib.d8_conv2d_scratch_bytes(dt, which, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx) for which in (1, 2))
+    ws = _scratch(nb)
+    check(lib.d8_conv2d_grad_xy(dt, dx_.ptr, dgx.ptr, B, IH, IW, IC, dw_.ptr, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
+                                sy, sx, dy, dx, _both(overwrite_x, overwrite_w), ws.ptr, nb, None))
+    return dgx.numpy(), dgw.numpy()
+
+
+def deconv2d_grad_xy(x, w, gz, covered=False, sy=1, sx=1, gx=None, gw=None, overwrite_x=False, overwrite_w=False, geometry=None):
+    """both gradients of DeConv2d from one call (d8_deconv2d_grad_xy, or d8_deconv2d_grad_xy_ex with
+    geometry = (OH, OW, padTop, padLeft)): returns (gx, gw)"""
+    lib = capi.init()
+    x, w, gz = np.ascontiguousarray(x), _filt(w), np.ascontiguousarray(gz)
+    dt = _same_dtype(x, w, gz)
+    B, IH, IW, IC = x.shape
+    OC, FH, FW, _ = w.shape
+    gx = np.zeros(x.shape, x.dtype) if gx is None else np.ascontiguousarray(gx)
+    gw = np.zeros(w.shape, x.dtype) if gw is None else _filt(gw)
+    dx_, dw_, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
+    dgx, dgw = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(gw)
+    if geometry is None:
+        nb = max(lib.d8_deconv2d_scratch_bytes(dt, which, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx) for which in (1, 2))
+        ws = _scratch(nb)
+        check(lib.d8_deconv2d_grad_xy(dt, dx_.ptr, dgx.ptr, B, IH, IW, IC, dw_.ptr, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
+                                      sy, sx, _both(overwrite_x, overwrite_w), ws.ptr, nb, None))
+    else:
+        nb = max(lib.d8_deconv2d_scratch_bytes_ex(dt, which, B, IH, IW, IC, OC, FH, FW, *geometry, sy, sx) for which in (1, 2))
+        ws = _scratch(nb)
+        check(lib.d8_deconv2d_grad_xy_ex(dt, dx_.ptr, dgx.ptr, B, IH, IW, IC, dw_.ptr, dgw.ptr, OC, FH, FW, dgz.ptr, *geometry,
+                                         sy, sx, _both(overwrite_x, overwrite_w), ws.ptr, nb, None))
+    return dgx.numpy(), dgw.numpy()
+
+
 # ---- the four maps ---------------------------------------------------------------------------------------
 def deconv2d_ex(which, x, w, gz, OH, OW, padTop, padLeft, sy, sx, acc=None, overwrite=False):
     """DeConv2d at an explicit geometry: which 0 forward (gz unused), 1 gradient of x, 2 gradient of w; gradients are

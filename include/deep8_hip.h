@@ -266,6 +266,33 @@ int d8_deconv2d_grad_y_overwrite(int dtype, const void *x, int B, int IH, int IW
                                  int covered, int sy, int sx,
                                  void *scratch, size_t scratch_bytes, void *stream);
 
+/* Both gradients of a convolution from one call: what the _grad_x call followed by the _grad_y call of the same
+ * operator leave (Conv2d::backward / DeConv2d::backward run once per input, deep8/src/nodes/Conv2d.cpp:85-151,
+ * deep8/src/nodes/DeConv2d.cpp:74-126, each a cublasSgemm / cublasHgemm sequence of its own:
+ * deep8/src/math/Conv2d.cu:440-492 and :750-802, deep8/src/math/DeConv2d.cu:371-429 and :642-700).  The two are
+ * independent of each other; on a layer whose products each leave compute units idle they run as ONE launch, the
+ * workgroups of both side by side.  gw is bit for bit what the _grad_y call leaves; so is gx, except on small half
+ * layers where the product behind gx, cut into pieces when it runs alone, runs whole beside the other's workgroups:
+ * the same sums added in another order (equal within half rounding).  overwrite: bit 0 -- gx is
+ * written instead of added to, bit 1 -- gw likewise.  scratch: the larger of the scratch sizes of which = 1 and
+ * which = 2.                                                                                                      */
+int d8_conv2d_grad_xy(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
+                      const void *w, void *gw, int OC, int FH, int FW, const void *gz,
+                      int covered, int sy, int sx, int dy, int dx, int overwrite,
+                      void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_xy(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
+                        const void *w, void *gw, int OC, int FH, int FW, const void *gz,
+                        int covered, int sy, int sx, int overwrite,
+                        void *scratch, size_t scratch_bytes, void *stream);
+int d8_deconv2d_grad_xy_ex(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
+                           const void *w, void *gw, int OC, int FH, int FW, const void *gz,
+                           int OH, int OW, int padTop, int padLeft, int sy, int sx, int overwrite,
+                           void *scratch, size_t scratch_bytes, void *stream);
+
+/* Test and measurement aid: how many of the _grad_xy calls above have run as one launch since the library was
+ * loaded (no counterpart in the reference).                                                                       */
+unsigned long d8_conv_grad_pair_launches(void);
+
 /* ---- Add (broadcasting) and ReLu -----------------------------------------------------------
  * The element-wise steps that follow MatrixMultiply / Conv2d in a network (bias, activation).
  * Shapes are Deep8's 5-entry enlarged form [batch, d0, d1, d2, d3]: dims right-aligned, padded
