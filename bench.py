@@ -1094,7 +1094,8 @@ def tiled_phase_record(key, launches=8):
         t0 = r[:, 0].min()
         start, end = us(r[:, 0] - t0), us(r[:, 3] - t0)
         pro, loop, epi = us(r[:, 1] - r[:, 0]), us(r[:, 2] - r[:, 1]), us(r[:, 3] - r[:, 2])
-        band = r[:, 7] == 1
+        band = (r[:, 7] & 1) == 1
+        second = (r[:, 7] >> 1) == 1  # a launch of two products: the workgroups of the second (the gradient of x)
         key_cu = ((r[:, 6] >> 32) & 0xf) * 65536 + (r[:, 6] & 0xff00)  # XCD, and the SE / SH / CU bits of HW_ID
         cus = len(np.unique(key_cu))
         ghz = ((r[:, 5] - r[:, 4]) / np.maximum(loop * 1e3, 1e-9))[~band].mean()
@@ -1102,7 +1103,9 @@ def tiled_phase_record(key, launches=8):
         print("%s: %d workgroups on %d CUs (%d of them on the remainder band); first start to last store acknowledged "
               "%.1f us; the matrix pipe alone at the loop's own clock (%.2f GHz) would need %.1f us" % (
                   name, len(r), cus, band.sum(), end.max(), ghz, pipe_us), flush=True)
-        for label, m in (("tiles", ~band), ("band pieces", band)):
+        groups = ((("tiles", ~band), ("band pieces", band)) if not second.any() else
+                  (("filter-gradient pieces", ~second), ("input-gradient tiles", second)))
+        for label, m in groups:
             if not m.any():
                 continue
             print("  %s: start %.1f-%.1f us; prologue %.1f-%.1f (mean %.1f); K loop %.1f-%.1f (mean %.1f); epilogue "

@@ -85,7 +85,8 @@ struct GemmArgs {
     // measurement aid of the tiled kernels (d8_gemm_phase_record): when set, every workgroup writes eight 64-bit words
     // at index blockIdx.x + gridDim.x * blockIdx.z -- the chip's 100 MHz wall clock at its start, after its prologue,
     // after its K loop and after its last store was acknowledged, the shader clock at both ends of the loop, its
-    // placement (XCC_ID << 32 | HW_ID) and whether it worked on the remainder band
+    // placement (XCC_ID << 32 | HW_ID) and, in the last word, whether it worked on the remainder band (bit 0) and which
+    // product of a launch of two it belongs to (bit 1: gemm_tiled_pair_launch's gx)
     unsigned long long *phase_rec;
 };
 

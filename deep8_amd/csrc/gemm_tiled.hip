@@ -636,7 +636,7 @@ __device__ __forceinline__ void gemm_tiled_body(const GemmArgs &g, int tilesM, c
             rec[0] = st_w[0], rec[1] = st_w[1], rec[2] = st_w[2], rec[3] = st_w[3], rec[4] = st_c[0], rec[5] = st_c[1];
             // s_getreg_b32 of all 32 bits of hardware registers 20 (XCC_ID) and 4 (HW_ID: wave, SIMD, CU, SH, SE)
             rec[6] = ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
-            rec[7] = in_tail ? 1 : 0;
+            rec[7] = (in_tail ? 1 : 0) | (g.stamps << 1);  // (stamps: which product of a launch of two)
         }
     }
 }
@@ -765,10 +765,13 @@ static void grid_of(TileId t, const GemmArgs &g, int &tilesM, int &tilesN) {
 template <typename TX, typename TY>
 static int launch_pair_tiles(const GemmArgs &gx0, const GemmArgs &gy0, hipStream_t stream) {
     GemmArgs gx = gx0, gy = gy0;
-    gx.phase_rec = gy.phase_rec = nullptr;
     const int tMx = ceil_div(gx.M, TX::BM), tNx = ceil_div(gx.N, TX::BN), tMy = ceil_div(gy.M, TY::BM), tNy = ceil_div(gy.N, TY::BN);
     // the longer-running product first: gy's pieces, then gx's tiles
     const int ny = tMy * tNy, nzy = gy.batch * gy.splits, nx = tMx * tNx;
+    // phase records (a measurement aid): gy's workgroups first, then gx's, tagged 0 and 1
+    const bool rec = (size_t)(ny * nzy + nx) * 64 <= phase_rec_bytes;
+    gy.phase_rec = rec ? phase_rec_buf : nullptr, gy.stamps = 0;
+    gx.phase_rec = rec && phase_rec_buf ? phase_rec_buf + 8L * ny * nzy : nullptr, gx.stamps = 1;
     hipLaunchKernelGGL((gemm_tiled_pair_kernel<TY, TX>), dim3(ny * nzy + nx), dim3(TX::NT), 0, stream, gy, gx, tMy, tNy, ny, nzy, tMx, tNx, nx);
     D8_LAUNCH_CHECK();
     return 0;
