@@ -323,7 +323,7 @@ class ConvWorkload:
         self.gx = capi.DeviceArray((B, IH, IW, IC), dtype)
         self.gw = capi.DeviceArray((OC, FH, FW, IC), dtype)
         q = self.lib.d8_deconv2d_scratch_bytes if deconv else self.lib.d8_conv2d_scratch_bytes
-        self.ws_bytes = max(q(self.dt, w, B, IH, IW, IC, OC, FH, FW, *self.geo) for w in range(3))
+        self.ws_bytes = max(q(self.dt, w, B, IH, IW, IC, OC, FH, FW, *self.geo) for w in range(4))  # (3: both gradients from one call)
         self.ws = capi.DeviceArray((max(self.ws_bytes, 16),), np.uint8)
         os.environ.pop("D8_CONV_EXPLICIT", None)
         if deconv:
@@ -496,7 +496,7 @@ class DeconvLiteralWorkload:
         self.z = capi.DeviceArray((B, OH, OH, OC), np.float16)
         self.dx = capi.DeviceArray((B, IH, IH, IC), np.float16)
         self.dw = capi.DeviceArray((OC, F, F, IC), np.float16)
-        self.ws_bytes = max(self.lib.d8_deconv2d_scratch_bytes_ex(self.dt, wch, *self.shape, *self.filt, OH, OH, P, P, S, S) for wch in range(3))
+        self.ws_bytes = max(self.lib.d8_deconv2d_scratch_bytes_ex(self.dt, wch, *self.shape, *self.filt, OH, OH, P, P, S, S) for wch in range(4))
         self.ws = capi.DeviceArray((max(self.ws_bytes, 16),), np.uint8)
         M, N = B * IH * IH, OC * F * F
         self.flops = 3 * 2.0 * M * N * IC

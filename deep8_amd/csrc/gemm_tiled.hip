@@ -765,9 +765,12 @@ static void grid_of(TileId t, const GemmArgs &g, int &tilesM, int &tilesN) {
 template <typename TX, typename TY>
 static int launch_pair_tiles(const GemmArgs &gx0, const GemmArgs &gy0, hipStream_t stream) {
     GemmArgs gx = gx0, gy = gy0;
-    const int tMx = ceil_div(gx.M, TX::BM), tNx = ceil_div(gx.N, TX::BN), tMy = ceil_div(gy.M, TY::BM), tNy = ceil_div(gy.N, TY::BN);
+    // (gx may carry its remainder band as pieces of the same launch: GemmArgs::tail_m0)
+    const bool tail = gx.tail_splits > 0;
+    const int tMx = ceil_div(tail ? gx.tail_m0 : gx.M, TX::BM), tNx = ceil_div(gx.N, TX::BN), tMy = ceil_div(gy.M, TY::BM), tNy = ceil_div(gy.N, TY::BN);
+    const int extra = tail ? ceil_div(gx.M - gx.tail_m0, TX::BM) * tNx * gx.tail_splits : 0;
     // the longer-running product first: gy's pieces, then gx's tiles
-    const int ny = tMy * tNy, nzy = gy.batch * gy.splits, nx = tMx * tNx;
+    const int ny = tMy * tNy, nzy = gy.batch * gy.splits, nx = tMx * tNx + extra;
     // phase records (a measurement aid): gy's workgroups first, then gx's, tagged 0 and 1
     const bool rec = (size_t)(ny * nzy + nx) * 64 <= phase_rec_bytes;
     gy.phase_rec = rec ? phase_rec_buf : nullptr, gy.stamps = 0;
@@ -806,12 +809,13 @@ static int launch_pair(const GemmArgs &gx, const GemmArgs &gy, hipStream_t strea
 
 long gemm_tiled_pair_workgroups(int dtype, const GemmArgs &gx, const GemmArgs &gy) {
     TileId tx, ty;
-    if (gx.virt != VIRT_A_ROWS || gy.virt != VIRT_B_KROWS || gx.tail_splits || gy.tail_splits || gx.splits != 1 || gx.batch != 1 || gy.batch != 1)
+    if (gx.virt != VIRT_A_ROWS || gy.virt != VIRT_B_KROWS || gy.tail_splits || gx.splits != 1 || gx.batch != 1 || gy.batch != 1)
         return 0;
     if (!(dtype == D8_FLOAT16 ? pair_tiles<f16>(gx, gy, tx, ty) : pair_tiles<float>(gx, gy, tx, ty))) return 0;
     int mx, nx, my, ny;
     grid_of(tx, gx, mx, nx);
     grid_of(ty, gy, my, ny);
+    if (gx.tail_splits && tx != TILE_128x64) return 0;  // (a band is cut for 128-row tiles of a narrow output only)
     return (long)mx * nx + (long)my * ny * gy.splits;
 }
 

@@ -412,6 +412,9 @@ static PaddedScratch conv_padded_scratch(int dtype, int which, int M, int OC, in
 
 size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                int OC, int FH, int FW, int covered, int sy, int sx, int dy, int dx) {
+    if (which == 3)  // for d8_conv2d_grad_xy: both gradients' scratch side by side (they may share a launch)
+        return align256(d8_conv2d_scratch_bytes(dtype, 2, B, IH, IW, IC, OC, FH, FW, covered, sy, sx, dy, dx)) +
+               d8_conv2d_scratch_bytes(dtype, 1, B, IH, IW, IC, OC, FH, FW, covered, sy, sx, dy, dx);
     int g[4];
     if (check_conv("d8_conv2d_scratch_bytes", dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, dy, dx)) return 0;
     if (d8_conv2d_geometry(IH, IW, FH, FW, covered, sy, sx, dy, dx, g)) return 0;
@@ -680,6 +683,9 @@ static int check_deconv_out(const char *who, int B, const int *geo) {
 
 static size_t deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                      int OC, int FH, int FW, const int *geo, int sy, int sx) {
+    if (which == 3)  // for d8_deconv2d_grad_xy: both gradients' scratch side by side
+        return align256(deconv2d_scratch_bytes(dtype, 2, B, IH, IW, IC, OC, FH, FW, geo, sy, sx)) +
+               deconv2d_scratch_bytes(dtype, 1, B, IH, IW, IC, OC, FH, FW, geo, sy, sx);
     if (check_deconv_out("d8_deconv2d_scratch_bytes", B, geo)) return 0;
     const int M = B * IH * IW, T = FH * FW;
     GemmArgs ga;

@@ -281,8 +281,7 @@ void Conv2dGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, cons
     const ConvDims d = checkConv(x, y, z, CONV_ARGS);
     requireGPU(x);
     const int dt = dtypeOf(x);
-    const size_t need = std::max(d8_conv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS),
-                                 d8_conv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS));
+    const size_t need = d8_conv2d_scratch_bytes(dt, 3, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, CONV_ARGS);  // both gradients' scratch
     PoolScratch ws(x.device(), need);
     const int overwrite = (dx.takeZero() ? 1 : 0) | (dy.takeZero() ? 2 : 0);  // deferred zero fills: write instead of add
     D8_CHECK(d8_conv2d_grad_xy(dt, x.raw(), dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), dy.raw(), d.OC, d.FH, d.FW, dz.raw(), CONV_ARGS,
@@ -373,8 +372,7 @@ void DeConv2dGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, co
     const ConvDims d = checkDeConv(x, y, z, DECONV_ARGS);
     requireGPU(x);
     const int dt = dtypeOf(x);
-    const size_t need = std::max(d8_deconv2d_scratch_bytes(dt, 1, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS),
-                                 d8_deconv2d_scratch_bytes(dt, 2, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS));
+    const size_t need = d8_deconv2d_scratch_bytes(dt, 3, d.B, d.IH, d.IW, d.IC, d.OC, d.FH, d.FW, DECONV_ARGS);
     PoolScratch ws(x.device(), need);
     const int overwrite = (dx.takeZero() ? 1 : 0) | (dy.takeZero() ? 2 : 0);
     D8_CHECK(d8_deconv2d_grad_xy(dt, x.raw(), dx.raw(), d.B, d.IH, d.IW, d.IC, y.raw(), dy.raw(), d.OC, d.FH, d.FW, dz.raw(), DECONV_ARGS,

@@ -302,7 +302,7 @@ def conv2d_grad_xy(x, w, gz, covered=True, sy=1, sx=1, dy=1, dx=1, gx=None, gw=N
     gw = np.zeros(w.shape, x.dtype) if gw is None else _filt(gw)
     dx_, dw_, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
     dgx, dgw = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(gw)
-    nb = max(lib.d8_conv2d_scratch_bytes(dt, which, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx) for which in (1, 2))
+    nb = lib.d8_conv2d_scratch_bytes(dt, 3, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx, dy, dx)
     ws = _scratch(nb)
     check(lib.d8_conv2d_grad_xy(dt, dx_.ptr, dgx.ptr, B, IH, IW, IC, dw_.ptr, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
                                 sy, sx, dy, dx, _both(overwrite_x, overwrite_w), ws.ptr, nb, None))
@@ -322,12 +322,12 @@ def deconv2d_grad_xy(x, w, gz, covered=False, sy=1, sx=1, gx=None, gw=None, over
     dx_, dw_, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
     dgx, dgw = DeviceArray.from_numpy(gx), DeviceArray.from_numpy(gw)
     if geometry is None:
-        nb = max(lib.d8_deconv2d_scratch_bytes(dt, which, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx) for which in (1, 2))
+        nb = lib.d8_deconv2d_scratch_bytes(dt, 3, B, IH, IW, IC, OC, FH, FW, int(covered), sy, sx)
         ws = _scratch(nb)
         check(lib.d8_deconv2d_grad_xy(dt, dx_.ptr, dgx.ptr, B, IH, IW, IC, dw_.ptr, dgw.ptr, OC, FH, FW, dgz.ptr, int(covered),
                                       sy, sx, _both(overwrite_x, overwrite_w), ws.ptr, nb, None))
     else:
-        nb = max(lib.d8_deconv2d_scratch_bytes_ex(dt, which, B, IH, IW, IC, OC, FH, FW, *geometry, sy, sx) for which in (1, 2))
+        nb = lib.d8_deconv2d_scratch_bytes_ex(dt, 3, B, IH, IW, IC, OC, FH, FW, *geometry, sy, sx)
         ws = _scratch(nb)
         check(lib.d8_deconv2d_grad_xy_ex(dt, dx_.ptr, dgx.ptr, B, IH, IW, IC, dw_.ptr, dgw.ptr, OC, FH, FW, dgz.ptr, *geometry,
                                          sy, sx, _both(overwrite_x, overwrite_w), ws.ptr, nb, None))

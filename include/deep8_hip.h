@@ -195,6 +195,8 @@ int d8_conv2d_geometry(int IH, int IW, int FH, int FW, int covered,
                        int sy, int sx, int dy, int dx, int *out);
 int d8_deconv2d_geometry(int IH, int IW, int FH, int FW, int covered, int sy, int sx, int *out);
 
+/* which: 0 forward, 1 gradient of x, 2 gradient of the filter, 3 both gradients from one call (the _grad_xy entry
+ * points; the same for the DeConv2d queries) */
 size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int IC,
                                int OC, int FH, int FW, int covered, int sy, int sx, int dy, int dx);
 int d8_conv2d(int dtype, const void *x, int B, int IH, int IW, int IC,
@@ -274,8 +276,9 @@ int d8_deconv2d_grad_y_overwrite(int dtype, const void *x, int B, int IH, int IW
  * workgroups of both side by side.  gw is bit for bit what the _grad_y call leaves; so is gx, except on small half
  * layers where the product behind gx, cut into pieces when it runs alone, runs whole beside the other's workgroups:
  * the same sums added in another order (equal within half rounding).  overwrite: bit 0 -- gx is
- * written instead of added to, bit 1 -- gw likewise.  scratch: the larger of the scratch sizes of which = 1 and
- * which = 2.                                                                                                      */
+ * written instead of added to, bit 1 -- gw likewise.  scratch: the scratch query with which = 3 (room for both
+ * gradients' scratch side by side); with less, but at least the larger of which = 1 and which = 2, the call still
+ * works and large layers run as two launches.                                                                     */
 int d8_conv2d_grad_xy(int dtype, const void *x, void *gx, int B, int IH, int IW, int IC,
                       const void *w, void *gw, int OC, int FH, int FW, const void *gz,
                       int covered, int sy, int sx, int dy, int dx, int overwrite,

@@ -185,3 +185,29 @@ def test_deconv2d_both_gradients_at_an_explicit_geometry():
     assert lib.d8_conv_grad_pair_launches() == before + 1
     assert _same(gx, ops.deconv2d_ex(1, x, w, gz, *geo, sy, sx, gx0))
     assert _same(gw, ops.deconv2d_ex(2, x, w, gz, *geo, sy, sx, gw0, overwrite=True))
+
+
+def test_large_half_layer_shares_a_launch_when_the_scratch_has_room():
+    """benchmark configuration 4's layer in half (B32 56 x 56 x 64, 3 x 3): more workgroups than the chip holds at once,
+    and a gradient of x whose remainder band rides in its launch.  With the scratch of the which = 3 query both
+    gradients share a launch; with the larger of the two single queries they run apart; both leave the bits of the
+    two calls."""
+    from deep8_amd import capi, ops
+    from deep8_amd.capi import DeviceArray, check
+    lib = capi.init()
+    B, IH, IW, IC, OC, FH, FW = 32, 56, 56, 64, 64, 3, 3
+    a = (1, 1, 1, 1, 1)
+    dt = capi.FLOAT16
+    x, w, gz, gx0, gw0 = _data(rng(404), B, IH, IW, IC, OC, FH, FW, 56, 56, np.float16)
+    want_x = ops.conv2d_grad_x(x, w, gz, True, 1, 1, 1, 1, gx0)
+    want_w = ops.conv2d_grad_y(x, w, gz, True, 1, 1, 1, 1, gw0, overwrite=True)
+    dx_, dw_, dgz = DeviceArray.from_numpy(x), DeviceArray.from_numpy(w), DeviceArray.from_numpy(gz)
+    q = lambda which: lib.d8_conv2d_scratch_bytes(dt, which, B, IH, IW, IC, OC, FH, FW, *a)
+    assert q(3) >= q(1) + q(2) > max(q(1), q(2)) > 0
+    for nb, shared in ((q(3), 1), (max(q(1), q(2)), 0)):
+        ws = DeviceArray((nb,), np.uint8)
+        dgx, dgw = DeviceArray.from_numpy(gx0), DeviceArray.from_numpy(gw0)
+        before = lib.d8_conv_grad_pair_launches()
+        check(lib.d8_conv2d_grad_xy(dt, dx_.ptr, dgx.ptr, B, IH, IW, IC, dw_.ptr, dgw.ptr, OC, FH, FW, dgz.ptr, *a, 2, ws.ptr, nb, None))
+        assert lib.d8_conv_grad_pair_launches() - before == shared
+        assert _same(dgx.numpy(), want_x) and _same(dgw.numpy(), want_w), shared
