@@ -429,7 +429,7 @@ class ConvWorkload:
 
 class ConvBiasReluWorkload(ConvWorkload):
     """Configuration 4's layer as it sits in a network: Conv2d -> Add (per-channel bias) -> ReLu, forward and backward.
-    fused:   d8_conv2d_bias_relu | d8_bias_relu_grad, d8_conv2d_grad_x, d8_conv2d_grad_y          (4 calls)
+    fused:   d8_conv2d_bias_relu | d8_bias_relu_grad, d8_conv2d_grad_xy                           (3 calls)
     unfused: d8_conv2d, d8_add, d8_relu | d8_relu_grad, d8_add_grad, d8_conv2d_grad_x, d8_conv2d_grad_y   (7 calls, the
              reference's sequence: deep8/src/math/Add.cu:21-52, ReLu.cu:20-116)"""
 
@@ -468,8 +468,12 @@ class ConvBiasReluWorkload(ConvWorkload):
             check(L.d8_relu(self.dt, self.sum.ptr, self.z.ptr, n, None))
             check(L.d8_relu_grad_overwrite(self.dt, self.sum.ptr, self.dpre.ptr, self.gz.ptr, n, None))
             check(L.d8_add_grad_overwrite(self.dt, self.gb.ptr, self.bd, self.dpre.ptr, self.zd, self.rs.ptr, self.rs_bytes, None))
-        self._call(L.d8_conv2d_grad_x_overwrite, self.gx.ptr, self.w.ptr, self.dpre.ptr)
-        self._call(L.d8_conv2d_grad_y_overwrite, self.x.ptr, self.gw.ptr, self.dpre.ptr)
+        if self.fused:  # both gradients from one call, as the fused node issues them
+            check(L.d8_conv2d_grad_xy(self.dt, self.x.ptr, self.gx.ptr, B, IH, IW, IC, self.w.ptr, self.gw.ptr, OC, FH, FW, self.dpre.ptr,
+                                      *self.geo, 3, self.ws.ptr, self.ws_bytes, None))
+        else:
+            self._call(L.d8_conv2d_grad_x_overwrite, self.gx.ptr, self.w.ptr, self.dpre.ptr)
+            self._call(L.d8_conv2d_grad_y_overwrite, self.x.ptr, self.gw.ptr, self.dpre.ptr)
 
 
 class DeconvLiteralWorkload:

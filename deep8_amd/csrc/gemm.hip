@@ -626,10 +626,11 @@ bool gemm_tiled_run_pair(int dtype, GemmArgs &gx, GemmArgs &gy, void *workspace,
     // More workgroups than the chip holds at once (two per compute unit): in half the shared launch still gains
     // (3x3 Conv2d, B32: 56x56x64 49.9 -> 47.0 us, 14x14x256 46.0 -> 34.9, 56x56x64->128 74.2 -> 65.0; DeConv2d 4x4 s2
     // B64 14x14x256 60.7 -> 47.9), gx's remainder band riding along as it does alone.  In fp32, bound by the matrix
-    // pipe, it gains 2-4 % on some layers and loses 8-21 % on others (3x3 of 128 channels at 28x28): those stay apart.
-    const bool big = dtype == D8_FLOAT16;
+    // pipe, it gains 2-4 % where gx's output is narrow (fewer than 128 input channels: three workgroups of either
+    // product fit a compute unit; B32 56x56x64 135.4 -> 129.7 us) and loses 8-21 % on 3x3 layers of 128 channels at
+    // 28x28 (128 x 128 tiles in both products): there only a gx with a remainder band, i.e. a narrow one, pairs.
     const int head = balanced_rows(gx);
-    if (head && !big) return false;
+    const bool big = dtype == D8_FLOAT16 || head != 0;
     const size_t usable = (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0;
     const int BK = gemm_tiled_k_step(dtype);
     int tps = 0;

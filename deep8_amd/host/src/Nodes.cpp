@@ -491,9 +491,10 @@ void checkBiasShape(const Shape &bias, const Shape &out) {
                          "the bias needs one value per element of the output's last dimension");
 }
 
-// The backward pass shared by the two fused nodes: gate once, then the products `grads` asks for.
-template <typename Products>
-void fusedBackward(Function *f, const std::vector<const Tensor *> &values, Variable *out, const Products &products) {
+// The backward pass shared by the two fused nodes: gate once, then the products the inputs ask for -- both from one
+// Math call (`both`) when the two operands are different variables that each take a gradient, else one by one.
+template <typename Products, typename Both>
+void fusedBackward(Function *f, const std::vector<const Tensor *> &values, Variable *out, const Products &products, const Both &both) {
     Variable *bias = (Variable *)f->inputs[2];
     Tensor dpre = tensorLike(out->gradient);
     if (bias->updateGradient) {
@@ -501,6 +502,11 @@ void fusedBackward(Function *f, const std::vector<const Tensor *> &values, Varia
     } else {
         Tensor unused = tensorLike(bias->value);
         Math::BiasReLuGrad(out->value, out->gradient, dpre, unused);
+    }
+    Variable *a = (Variable *)f->inputs[0], *b = (Variable *)f->inputs[1];
+    if (a->updateGradient && b->updateGradient && a != b) {
+        both(values, out->value, dpre, a->gradient, b->gradient);
+        return;
     }
     for (size_t i = 0; i < 2; ++i) {
         Variable *in = (Variable *)f->inputs[i];
@@ -546,6 +552,8 @@ void MatrixMultiplyBiasReLu::backward() {
     std::vector<const Tensor *> values = gatherInputs(this, out);
     fusedBackward(this, values, out, [this](const std::vector<const Tensor *> &v, const Tensor *z, const Tensor *dz, size_t i, Tensor *g) {
         MatrixMultiply::backward(v, z, dz, i, g);
+    }, [](const std::vector<const Tensor *> &v, const Tensor &z, const Tensor &dz, Tensor &gx, Tensor &gy) {
+        Math::MatrixMultiplyGradXY(*v[0], gx, *v[1], gy, z, dz);
     });
 }
 
@@ -588,6 +596,8 @@ void Conv2dBiasReLu::backward() {
     std::vector<const Tensor *> values = gatherInputs(this, out);
     fusedBackward(this, values, out, [this](const std::vector<const Tensor *> &v, const Tensor *z, const Tensor *dz, size_t i, Tensor *g) {
         Conv2d::backward(v, z, dz, i, g);
+    }, [this](const std::vector<const Tensor *> &v, const Tensor &z, const Tensor &dz, Tensor &gx, Tensor &gw) {
+        Math::Conv2dGradXY(*v[0], gx, *v[1], gw, z, dz, covered, strideY, strideX, dilationY, dilationX);
     });
 }
 
