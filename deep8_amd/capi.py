@@ -76,6 +76,7 @@ SIGNATURES = {
     "d8_conv2d_scratch_bytes": (_Z, [_I] * 14),
     "d8_conv2d": (_I, [_I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P]),
     "d8_conv_grad_pair_launches": (ctypes.c_ulong, []),
+    "d8_matmul_grad_pair_launches": (ctypes.c_ulong, []),
     "d8_conv2d_grad_xy": (_I, [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P] + [_I] * 6 + [_P, _Z, _P]),
     "d8_deconv2d_grad_xy": (_I, [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P] + [_I] * 4 + [_P, _Z, _P]),
     "d8_deconv2d_grad_xy_ex": (_I, [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _P] + [_I] * 7 + [_P, _Z, _P]),

@@ -226,16 +226,15 @@ struct SmallOp<f16> {
     }
 };
 
+// (the work of workgroup (bx, by) of output b; part: 3 x 32 x 32 floats of LDS)
 template <typename T, bool TA, bool TB>
-__global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
+__device__ __forceinline__ void gemm_small_body(const GemmArgs &g, const int bx, const int by, const int b, float (*part)[32 * 32]) {
     typedef SmallOp<T> OP;
     constexpr int BT = 32, PER = OP::PER, KG = OP::KG, MAXC = OP::MAXC;
-    __shared__ float part[3][BT * BT];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
-    const int b = blockIdx.z;
-    const int gm = blockIdx.y * BT + l32, gn = blockIdx.x * BT + l32;  // this lane's row of A and column of B
+    const int gm = by * BT + l32, gn = bx * BT + l32;  // this lane's row of A and column of B
     const int kchunks = (g.K + KG - 1) / KG, total = g.red * kchunks;   // total <= 4 * MAXC (gemm_is_small)
 
     // a K-contiguous operand whose rows can be read 16 bytes at a time gives a lane its values in one load
@@ -282,7 +281,7 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
     if (wave == 0) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int row = (r >> 2) * 8 + lhi * 4 + (r & 3), m = blockIdx.y * BT + row;
+            const int row = (r >> 2) * 8 + lhi * 4 + (r & 3), m = by * BT + row;
             float v = acc[r];
 #pragma unroll
             for (int w = 0; w < 3; ++w) v += part[w][row * BT + l32];
@@ -292,6 +291,27 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
                 *c = (T)v;
             }
         }
+    }
+}
+
+template <typename T, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_small_kernel(GemmArgs g) {
+    __shared__ float part[3][32 * 32];
+    gemm_small_body<T, TA, TB>(g, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z, part);
+}
+
+// Two small products in one launch: the first n0 = nx0 * ny0 * batch workgroups are g0's grid (NT: the gradient of
+// a MatrixMultiply's first input), the rest g1's (TN: the gradient of its second).  Each of them is one load
+// latency and a few matrix instructions long; what a launch of its own costs on top is most of its time.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_small_pair_kernel(GemmArgs g0, GemmArgs g1, int nx0, int ny0, int n0, int nx1, int ny1) {
+    __shared__ float part[3][32 * 32];
+    int id = (int)blockIdx.x;
+    if (id < n0) {
+        gemm_small_body<T, false, true>(g0, id % nx0, (id / nx0) % ny0, id / (nx0 * ny0), part);
+    } else {
+        id -= n0;
+        gemm_small_body<T, true, false>(g1, id % nx1, (id / nx1) % ny1, id / (nx1 * ny1), part);
     }
 }
 
@@ -610,6 +630,26 @@ int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspa
     }
     if (int rc = gemm_tiled_run_whole(dtype, first, transA, transB, nullptr, 0, stream)) return rc;
     return gemm_tiled_run_whole(dtype, second, transA, transB, workspace, workspace_bytes, stream);
+}
+
+// The two gradients of a small MatrixMultiply (g0 = dZ . Y^T, NT; g1 = X^T . dZ, TN; both small in the sense of
+// gemm_is_small, neither Float64) as one launch.  False, with nothing launched, when they do not qualify.
+bool gemm_small_pair_run(int dtype, const GemmArgs &g0, int ta0, int tb0, const GemmArgs &g1, int ta1, int tb1, hipStream_t stream, int *rc) {
+    if (dtype == D8_FLOAT64 || ta0 || !tb0 || !ta1 || tb1) return false;
+    if (g0.virt != VIRT_NONE || g1.virt != VIRT_NONE || g0.K < 1 || g1.K < 1) return false;
+    if (!gemm_is_small(g0.M, g0.N, g0.K, g0.batch, g0.red) || !gemm_is_small(g1.M, g1.N, g1.K, g1.batch, g1.red)) return false;
+    const int nx0 = ceil_div(g0.N, 32), ny0 = ceil_div(g0.M, 32), nx1 = ceil_div(g1.N, 32), ny1 = ceil_div(g1.M, 32);
+    const long n0 = (long)nx0 * ny0 * g0.batch, n1 = (long)nx1 * ny1 * g1.batch;
+    if (n0 + n1 > 0x7fffffffL) return false;
+    GemmArgs a = g0, b = g1;
+    a.splits = b.splits = 1;
+    if (dtype == D8_FLOAT16)
+        hipLaunchKernelGGL((gemm_small_pair_kernel<f16>), dim3((unsigned)(n0 + n1)), dim3(256), 0, stream, a, b, nx0, ny0, (int)n0, nx1, ny1);
+    else
+        hipLaunchKernelGGL((gemm_small_pair_kernel<float>), dim3((unsigned)(n0 + n1)), dim3(256), 0, stream, a, b, nx0, ny0, (int)n0, nx1, ny1);
+    const hipError_t e = hipGetLastError();
+    *rc = e == hipSuccess ? 0 : fail((int)e, "kernel launch: %s", hipGetErrorString(e));
+    return true;
 }
 
 static std::atomic<unsigned long> pair_launches{0};  // d8_conv_grad_pair_launches

@@ -124,6 +124,10 @@ int gemm_wide_launch(const GemmArgs &g, int transA, int transB, hipStream_t stre
 int gemm_wide_pair_launch(const GemmArgs &g0, int transA0, int transB0, const GemmArgs &g1, int transA1, int transB1,
                           hipStream_t stream);
 
+// The two gradients of a small MatrixMultiply (NT then TN, both on the small-product kernel) as ONE launch; false, with
+// nothing launched, when they do not qualify.
+bool gemm_small_pair_run(int dtype, const GemmArgs &g0, int ta0, int tb0, const GemmArgs &g1, int ta1, int tb1, hipStream_t stream, int *rc);
+
 // fp64 kernel (64 x 64 or 128 x 128 tiles, v_mfma_f64_16x16x4_f64): any shape; plans its own split of the
 // reduction from g.ws / g.ws_bytes (double partial sums) and reduces.
 int gemm_f64_launch(const GemmArgs &g, int transA, int transB, hipStream_t stream);

@@ -5,6 +5,8 @@
 //   MatrixMultiply   deep8/src/math/MatrixMultiply.cu:21-57 (fwd), :193-232 (GradX), :381-420 (GradY)
 //   Conv2d           deep8/src/math/Conv2d.cu:145-196, :440-492, :750-802, pads :332-336
 //   DeConv2d         deep8/src/math/DeConv2d.cu:76-131, :371-429, :642-700, pads :99-100
+#include <atomic>
+
 #include "conv_maps.h"
 #include "gemm_args.h"
 
@@ -311,6 +313,9 @@ int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc,
     return run(dtype, mm_plan(2, x, xb, xr, xc, dy, yb, yr, yc, dz, 0.f), scratch, scratch_bytes, stream);
 }
 
+static std::atomic<unsigned long> matmul_pair_launches{0};
+unsigned long d8_matmul_grad_pair_launches(void) { return matmul_pair_launches.load(); }
+
 int d8_matmul_grad_xy(int dtype, const void *x, void *dx, int xb, int xr, int xc, const void *y, void *dy, int yb, int yr,
                       int yc, const void *dz, int overwrite, void *scratch, size_t scratch_bytes, void *stream) {
     if (int rc = check_mm("d8_matmul_grad_xy", dtype, xb, xr, xc, yb, yr, yc)) return rc;
@@ -329,8 +334,17 @@ int d8_matmul_grad_xy(int dtype, const void *x, void *dx, int xb, int xr, int xc
         const long ty = (long)ceil_div(gy.M, 256) * ceil_div(gy.N, 256) * gy.batch;
         const long most = (long)cu_count() * 3 / 4;
         if (!(wide && atoi(wide) == 0) && gx.red == 1 && gy.red == 1 && tx >= most && ty >= most && tx + ty < 0x3fffffffL &&
-            gemm_wide_eligible(gx, px.ta, px.tb) && gemm_wide_eligible(gy, py.ta, py.tb))
+            gemm_wide_eligible(gx, px.ta, px.tb) && gemm_wide_eligible(gy, py.ta, py.tb)) {
+            ++matmul_pair_launches;
             return gemm_wide_pair_launch(gx, px.ta, px.tb, gy, py.ta, py.tb, as_stream(stream));
+        }
+    }
+    {  // both products small: one launch of the small-product kernel's workgroups for both
+        int rc = 0;
+        if (gemm_small_pair_run(dtype, to_args(px), px.ta, px.tb, to_args(py), py.ta, py.tb, as_stream(stream), &rc)) {
+            ++matmul_pair_launches;
+            return rc;
+        }
     }
     if (int rc = run(dtype, px, scratch, scratch_bytes, stream)) return rc;
     return run(dtype, py, scratch, scratch_bytes, stream);

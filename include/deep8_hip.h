@@ -172,7 +172,8 @@ int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc,
  * of each other, so large Float16 ones run as ONE launch in which a workgroup goes from a tile of dx straight on
  * to a tile of dy; everything else is d8_matmul_grad_x followed by d8_matmul_grad_y.  The results are bit for bit
  * those of the two calls.  overwrite: bit 0 -- dx is written instead of added to, bit 1 -- dy likewise (the
- * _overwrite forms above).  scratch: the larger of d8_matmul_scratch_bytes(which = 1) and (which = 2).          */
+ * _overwrite forms above).  scratch: the larger of d8_matmul_scratch_bytes(which = 1) and (which = 2).  Two small
+ * products (each at most four 128 x 128 tiles over a reduction of at most 512) share a launch as well.         */
 int d8_matmul_grad_xy(int dtype, const void *x, void *dx, int xb, int xr, int xc,
                       const void *y, void *dy, int yb, int yr, int yc, const void *dz, int overwrite,
                       void *scratch, size_t scratch_bytes, void *stream);
@@ -295,6 +296,7 @@ int d8_deconv2d_grad_xy_ex(int dtype, const void *x, void *gx, int B, int IH, in
 /* Test and measurement aid: how many of the _grad_xy calls above have run as one launch since the library was
  * loaded (no counterpart in the reference).                                                                       */
 unsigned long d8_conv_grad_pair_launches(void);
+unsigned long d8_matmul_grad_pair_launches(void);  /* ... and of the d8_matmul_grad_xy calls */
 
 /* ---- Add (broadcasting) and ReLu -----------------------------------------------------------
  * The element-wise steps that follow MatrixMultiply / Conv2d in a network (bias, activation).

@@ -129,6 +129,35 @@ PAIRS = [
 ]
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("xs,ys,shared", [((1, 64, 128), (1, 128, 256), True),    # benchmark configuration 1
+                                          ((1, 33, 70), (1, 70, 50), True),       # ragged 32 x 32 tiles
+                                          ((3, 40, 64), (3, 64, 72), True),       # a batch of three small products
+                                          ((1, 64, 1024), (1, 1024, 256), False)])  # a reduction too long for the small-product kernel
+def test_small_matmul_gradients_share_a_launch(oracle_port, xs, ys, shared, dtype):
+    """two small products: d8_matmul_grad_xy runs them as one launch of the small-product kernel; integers bit for bit
+    against the oracle, and the bits of the two separate calls"""
+    from deep8_amd import capi, ops
+    lib = capi.init()
+    r = rng(sum(xs) + sum(ys) + 3)
+    c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
+    hi = 2 if dtype == np.float16 else 20
+    x, y = ints(r, xs, hi), ints(r, ys, hi)
+    dz = ints(r, (xs[0], xs[1], ys[2]), hi)
+    dx0, dy0 = ints(r, xs, hi), ints(r, ys, hi)
+    before = lib.d8_matmul_grad_pair_launches()
+    gx, gy = ops.matmul_grad_xy(c(x), c(y), c(dz), c(dx0), c(dy0), False, True)
+    assert lib.d8_matmul_grad_pair_launches() - before == (1 if shared else 0)
+    wx, wy = oracle_port.matmul_grad_x(x, y, dz, dx0), oracle_port.matmul_grad_y(x, y, dz)
+    assert dtype == np.float32 or max(np.abs(wx).max(), np.abs(wy).max()) < 2048
+    assert np.array_equal(f(gx), wx) and np.array_equal(f(gy), wy)
+    xr_, yr_, dzr = c(nrm(r, xs)), c(nrm(r, ys)), c(nrm(r, dz.shape))
+    gx, gy = ops.matmul_grad_xy(xr_, yr_, dzr, overwrite_x=True, overwrite_y=True)
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    assert np.array_equal(gx.view(bits), ops.matmul_grad_x(xr_, yr_, dzr, overwrite=True).view(bits))
+    assert np.array_equal(gy.view(bits), ops.matmul_grad_y(xr_, yr_, dzr, overwrite=True).view(bits))
+
+
 @pytest.mark.parametrize("xr,xc,yc", PAIRS)
 @pytest.mark.parametrize("overwrite", [True, False])
 def test_matmul_both_gradients_as_one_launch(xr, xc, yc, overwrite):
