@@ -69,7 +69,22 @@ def test_im2col_col2im_bit_exact(oracle_port, cfg, dtype):
         assert np.array_equal(f(g), w)
 
 
-@pytest.mark.parametrize("cfg", DECONV)
+# shapes for the gather maps' staged kernels: channel counts that move in 16-byte pieces, the filters the im2col kernel
+# with the in-register block transpose is built for (4 x 4, 3 x 3, 2 x 2) at strides 1, 2, 3, a 5 x 3 filter for the
+# kernel that walks filter windows, rows that are not a multiple of the workgroup, pads on and off
+DECONV_MAPS = [
+    (2, 6, 6, 16, 16, 2, 2, False, 2, 2),
+    (2, 9, 7, 8, 24, 3, 3, True, 2, 2),
+    (1, 10, 10, 8, 40, 4, 4, False, 1, 1),
+    (2, 5, 9, 8, 8, 4, 4, True, 3, 3),
+    (3, 7, 5, 8, 72, 3, 3, False, 1, 1),
+    (1, 6, 6, 8, 16, 5, 3, False, 2, 1),
+    (2, 28, 28, 16, 64, 4, 4, False, 2, 2),
+    (1, 3, 33, 8, 128, 2, 2, True, 2, 2),
+]
+
+
+@pytest.mark.parametrize("cfg", DECONV + DECONV_MAPS)
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_deconv_maps_bit_exact(oracle_port, cfg, dtype):
     from deep8_amd import ops
