@@ -55,7 +55,7 @@ TRAFFIC_ROWS = {
                                                        "relu_grad": [("relu_grad_kernel", 1)],
                                                        "bias_grad (sum over rows)": [("column_sum_kernel", 1), ("column_sum_finish", 1)]}),
     "p4": ("maxpool2d_b32_56x56x64.txt", {"maxpool2d": [("pool_forward_kernel", 1)], "maxpool2d_grad": [("pool_backward", 1)]}),
-    "k5": ("deconv_maps_half_b16_28x28_to_56x56x64_4x4s2.txt", {"deconv_im2col": [("deconv_im2col_windows_kernel", 1)],
+    "k5": ("deconv_maps_half_b16_28x28_to_56x56x64_4x4s2.txt", {"deconv_im2col": [("deconv_im2col_blocks_kernel", 1)],
                                                                  "deconv_col2im": [("deconv_col2im_lds_kernel", 1)]}),
     "i4": ("im2col_col2im_fp32_b32_56x56x64_3x3.txt", {"im2col": [("im2col_vec_kernel", 1)], "col2im": [("col2im_kernel", 1)]}),
 }

@@ -79,6 +79,7 @@ DECONV_MAPS = [
     (2, 5, 9, 8, 8, 4, 4, True, 3, 3),
     (3, 7, 5, 8, 72, 3, 3, False, 1, 1),
     (1, 6, 6, 8, 16, 5, 3, False, 2, 1),
+    (2, 6, 7, 8, 16, 4, 2, False, 2, 2),
     (2, 28, 28, 16, 64, 4, 4, False, 2, 2),
     (1, 3, 33, 8, 128, 2, 2, True, 2, 2),
 ]
