@@ -304,7 +304,7 @@ __global__ __launch_bounds__(256) void deconv_im2col_kernel(const T *__restrict_
 // channels of one output pixel, adds its taps from LDS into fp32 registers and, after the last fy, writes once.
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restrict__ zmat, T *__restrict__ z, MapGeom g, FastDiv by_C,
-                                                                FastDiv by_CV) {
+                                                                FastDiv by_CV, FastDiv by_sx) {
     extern __shared__ __attribute__((aligned(16))) unsigned char deconv_lds[];
     T *slab = (T *)deconv_lds;  // [IW][FW][C]
     typedef T VT __attribute__((ext_vector_type(VEC)));
@@ -324,6 +324,84 @@ __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restr
     for (int o = 0; o < MAXO; ++o)
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc[o][e] = 0.f;
+    // the taps of the slab now in LDS into this thread's sums
+    auto accumulate = [&]() {
+#pragma unroll
+        for (int o = 0; o < MAXO; ++o) {
+            const int q = threadIdx.x + 256 * o;
+            if (q < outs) {
+                const int ox = (int)div_by((unsigned)q, by_CV), cv = q - ox * CV;
+                for (int fx = 0; fx < g.FW; ++fx) {
+                    const int tx = ox - g.pl + fx;
+                    if (tx < 0) continue;
+                    const int ix = (int)div_by((unsigned)tx, by_sx);  // (a division by a multiplication: the stride is a run-time value)
+                    if (ix * g.sx != tx || ix >= g.IW) continue;
+                    const VT v = *(const VT *)(slab + (ix * g.FW + fx) * C + cv * VEC);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[o][e] += (float)v[e];
+                }
+            }
+        }
+    };
+    // which input row filter row fy reads for this output row, if any (uniform over the workgroup)
+    auto reaches = [&](int fy, int &iy) -> bool {
+        const int ty = oy - g.pt + fy;
+        if (ty < 0 || ty % g.sy) return false;
+        iy = ty / g.sy;
+        return iy < g.IH;
+    };
+    // a filter row of a channel is FW contiguous elements: fetched as one 8- or 16-byte piece where it is one
+    const bool row8 = g.FW * sizeof(T) == 8 && (taps * sizeof(T)) % 8 == 0 && ((size_t)zmat & 7) == 0;
+    const bool row16 = g.FW * sizeof(T) == 16 && (taps * sizeof(T)) % 16 == 0 && ((size_t)zmat & 15) == 0;
+    constexpr int U = 8;
+    if ((row8 || row16) && pairs <= 256 * U) {
+        // Every thread's pieces of a slab fit its registers: the next filter row's pieces are requested before the
+        // present slab is added up, so their way from memory runs under that work instead of after it.
+        u32x4v v[U];
+        auto fetch = [&](int fy, int iy) {
+            const unsigned char *base = (const unsigned char *)(zmat + ((long)b * g.IH + iy) * g.IW * N + (long)fy * g.FW);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int q = threadIdx.x + 256 * u;  // (ix * C + oc): its filter rows start q * taps elements in
+                if (q < pairs) {
+                    const unsigned char *p = base + (long)q * taps * sizeof(T);
+                    if (row16) {
+                        v[u] = *(const u32x4v *)p;
+                    } else {
+                        const uint2 w = *(const uint2 *)p;
+                        v[u] = u32x4v{w.x, w.y, 0u, 0u};
+                    }
+                }
+            }
+        };
+        int fy = 0, iy = 0;
+        while (fy < g.FH && !reaches(fy, iy)) ++fy;
+        if (fy < g.FH) fetch(fy, iy);
+        while (fy < g.FH) {
+            __syncthreads();  // the previous slab has been consumed
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int q = threadIdx.x + 256 * u;
+                if (q < pairs) {
+                    const int ix = (int)div_by((unsigned)q, by_C), oc = q - ix * C;
+                    T *d = slab + ix * g.FW * C + oc;
+#pragma unroll
+                    for (int fx = 0; fx < (int)(16 / sizeof(T)); ++fx) {
+                        if (fx < g.FW) {
+                            if constexpr (sizeof(T) == 4) ((unsigned *)d)[fx * C] = v[u][fx & 3];
+                            else ((unsigned short *)d)[fx * C] = (unsigned short)(v[u][(fx >> 1) & 3] >> (16 * (fx & 1)));
+                        }
+                    }
+                }
+            }
+            int nfy = fy + 1, niy = 0;
+            while (nfy < g.FH && !reaches(nfy, niy)) ++nfy;
+            if (nfy < g.FH) fetch(nfy, niy);
+            __syncthreads();
+            accumulate();
+            fy = nfy;
+        }
+    } else
     for (int fy = 0; fy < g.FH; ++fy) {
         const int ty = oy - g.pt + fy;
         if (ty < 0 || ty % g.sy) continue;  // (uniform over the workgroup)
@@ -331,9 +409,6 @@ __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restr
         if (iy >= g.IH) continue;
         __syncthreads();  // the previous slab has been consumed
         const T *src = zmat + ((long)b * g.IH + iy) * g.IW * N + (long)fy * g.FW;
-        // a filter row of a channel is FW contiguous elements: fetched as one 8- or 16-byte piece where it is one
-        const bool row8 = g.FW * sizeof(T) == 8 && (taps * sizeof(T)) % 8 == 0 && ((size_t)zmat & 7) == 0;
-        const bool row16 = g.FW * sizeof(T) == 16 && (taps * sizeof(T)) % 16 == 0 && ((size_t)zmat & 15) == 0;
         for (int q = threadIdx.x; q < pairs; q += 256) {
             const int ix = (int)div_by((unsigned)q, by_C), oc = q - ix * C;
             const T *p = src + (long)ix * N + (long)oc * taps;
@@ -353,22 +428,7 @@ __global__ __launch_bounds__(256) void deconv_col2im_lds_kernel(const T *__restr
             }
         }
         __syncthreads();
-#pragma unroll
-        for (int o = 0; o < MAXO; ++o) {
-            const int q = threadIdx.x + 256 * o;
-            if (q < outs) {
-                const int ox = (int)div_by((unsigned)q, by_CV), cv = q - ox * CV;
-                for (int fx = 0; fx < g.FW; ++fx) {
-                    const int tx = ox - g.pl + fx;
-                    if (tx < 0 || tx % g.sx) continue;
-                    const int ix = tx / g.sx;
-                    if (ix >= g.IW) continue;
-                    const VT v = *(const VT *)(slab + (ix * g.FW + fx) * C + cv * VEC);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) acc[o][e] += (float)v[e];
-                }
-            }
-        }
+        accumulate();
     }
     T *row = z + ((long)b * g.OH + oy) * g.OW * C;
 #pragma unroll
@@ -794,10 +854,10 @@ int d8_deconv_col2im(int dtype, const void *zmat, void *z,
         if (es <= 4 && OC % vec == 0 && aligned16(z) && lds <= 60 * 1024 && (long)OW * (OC / vec) <= 1024 && (long)B * OH < (1L << 31)) {
             if (es == 4)
                 hipLaunchKernelGGL((deconv_col2im_lds_kernel<float, 4>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const float *)zmat, (float *)z, g,
-                                   fast_div((unsigned)OC), fast_div((unsigned)(OC / vec)));
+                                   fast_div((unsigned)OC), fast_div((unsigned)(OC / vec)), fast_div((unsigned)sx));
             else
                 hipLaunchKernelGGL((deconv_col2im_lds_kernel<f16, 8>), dim3((B * OH + 7) & ~7), dim3(256), lds, s, (const f16 *)zmat, (f16 *)z, g,
-                                   fast_div((unsigned)OC), fast_div((unsigned)(OC / vec)));
+                                   fast_div((unsigned)OC), fast_div((unsigned)(OC / vec)), fast_div((unsigned)sx));
             D8_LAUNCH_CHECK();
             return 0;
         }
