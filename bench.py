@@ -183,7 +183,7 @@ class MatMulWorkload:
         self.z = capi.DeviceArray(self.zs, dtype)
         self.dx = capi.DeviceArray(xs, dtype)
         self.dy = capi.DeviceArray(ys, dtype)
-        nb = max(self.lib.d8_matmul_scratch_bytes(self.dt, w, *xs, *ys) for w in range(3))
+        nb = max(self.lib.d8_matmul_scratch_bytes(self.dt, w, *xs, *ys) for w in range(4))  # (3: both gradients from one call)
         self.ws_bytes = nb
         self.ws = capi.DeviceArray((max(nb, 16),), np.uint8)
         m, k, n = xs[1], xs[2], ys[2]

@@ -707,6 +707,32 @@ bool gemm_tiled_run_pair(int dtype, GemmArgs &gx, GemmArgs &gy, void *workspace,
     return true;
 }
 
+bool gemm_tiled_run_plain_pair(int dtype, GemmArgs &g0, int ta0, int tb0, GemmArgs &g1, int ta1, int tb1, void *workspace,
+                               size_t workspace_bytes, hipStream_t stream, int *rc) {
+    const bool off = getenv("D8_MATMUL_GRADS_APART") != nullptr;  // tuning and test aid (read at every call)
+    if (off || dtype == D8_FLOAT64 || ta0 || !tb0 || !ta1 || tb1) return false;
+    if (g0.virt != VIRT_NONE || g1.virt != VIRT_NONE || g0.K < 1 || g1.K < 1) return false;
+    if (!gemm_tiled_eligible(dtype, g0, ta0, tb0) || !gemm_tiled_eligible(dtype, g1, ta1, tb1)) return false;
+    if (gemm_is_small(g0.M, g0.N, g0.K, g0.batch, g0.red) || gemm_is_small(g1.M, g1.N, g1.K, g1.batch, g1.red)) return false;
+    if (balanced_rows(g0) || balanced_rows(g1)) return false;
+    const size_t usable = (workspace && ((size_t)workspace & 15) == 0) ? workspace_bytes : 0;
+    const int BK = gemm_tiled_k_step(dtype);
+    // each split as it would be alone, the partial sums of the two side by side in the workspace
+    g0.splits = plan_splits(BK, g0.M, g0.N, g0.K, g0.batch, g0.red, usable, &g0.tiles_per_split);
+    g1.splits = plan_splits(BK, g1.M, g1.N, g1.K, g1.batch, g1.red, usable, &g1.tiles_per_split);
+    const size_t need0 = g0.splits > 1 ? ((size_t)g0.splits * g0.batch * g0.M * g0.N * sizeof(float) + 255) & ~(size_t)255 : 0;
+    const size_t need1 = g1.splits > 1 ? (size_t)g1.splits * g1.batch * g1.M * g1.N * sizeof(float) : 0;
+    if (need0 + need1 > usable) return false;
+    g0.ws = (float *)workspace, g1.ws = (float *)((char *)workspace + need0);
+    g0.tail_splits = g1.tail_splits = 0;
+    const long wgs = gemm_tiled_plain_pair_workgroups(dtype, g0, g1);
+    if (wgs <= 0 || wgs > 2L * cu_count()) return false;
+    *rc = gemm_tiled_plain_pair_launch(dtype, g0, g1, stream);
+    if (*rc == 0 && g0.splits > 1) *rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(g0, stream) : launch_reduce<float>(g0, stream);
+    if (*rc == 0 && g1.splits > 1) *rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(g1, stream) : launch_reduce<float>(g1, stream);
+    return true;
+}
+
 bool gemm_fuses_store(int dtype, const GemmArgs &g, int transA, int transB) {
     // (a product beyond one launch's limits -- more than 448 outputs, more than 65535 * 128 rows -- is cut into several
     // by d8_gemm; the fused store stays out of that: the caller runs the product and one pass over its result)

@@ -110,6 +110,10 @@ int gemm_tiled_launch(int dtype, const GemmArgs &g, int transA, int transB, hipS
 // pair cannot run this way (the tiles the two products would choose have no common kernel, or one is cut into a band).
 long gemm_tiled_pair_workgroups(int dtype, const GemmArgs &gx, const GemmArgs &gy);
 int gemm_tiled_pair_launch(int dtype, const GemmArgs &gx, const GemmArgs &gy, hipStream_t stream);
+// The same for two real products: g0 NT, g1 TN (the two gradients of a MatrixMultiply), each batched or split as planned
+// (g.splits / tiles_per_split / ws set; the caller reduces).
+long gemm_tiled_plain_pair_workgroups(int dtype, const GemmArgs &g0, const GemmArgs &g1);
+int gemm_tiled_plain_pair_launch(int dtype, const GemmArgs &g0, const GemmArgs &g1, hipStream_t stream);
 // Where the next launches write their per-workgroup phase records (GemmArgs::phase_rec); null switches them off.
 void gemm_tiled_phase_record(void *records, size_t bytes);
 
@@ -146,6 +150,11 @@ int gemm_tiled_run(int dtype, GemmArgs &g, int transA, int transB, void *workspa
 // into the filter's) as one launch where that pays; false, with nothing launched, where it does not (the caller then
 // runs them one after the other).  The workspace is gy's.
 bool gemm_tiled_run_pair(int dtype, GemmArgs &gx, GemmArgs &gy, void *workspace, size_t workspace_bytes, hipStream_t stream, int *rc);
+// The two gradients of a mid-size MatrixMultiply (g0 = dZ . Y^T, NT; g1 = X^T . dZ, TN; both on the tiled kernels, all their
+// workgroups resident at once) as one launch plus their split reductions; false, with nothing launched, otherwise.
+// The workspace holds both products' partial sums side by side.
+bool gemm_tiled_run_plain_pair(int dtype, GemmArgs &g0, int ta0, int tb0, GemmArgs &g1, int ta1, int tb1, void *workspace,
+                               size_t workspace_bytes, hipStream_t stream, int *rc);
 // Workspace gemm_tiled_run may use for this shape.
 size_t gemm_tiled_workspace(int dtype, int M, int N, int K, int red, int virt = VIRT_NONE);
 // Whether a product whose B is a patch matrix (VIRT_B_KROWS) runs on 64 x 64 tiles: fewer than 128 rows, and the last

@@ -765,17 +765,17 @@ static void grid_of(TileId t, const GemmArgs &g, int &tilesM, int &tilesN) {
 template <typename TX, typename TY>
 static int launch_pair_tiles(const GemmArgs &gx0, const GemmArgs &gy0, hipStream_t stream) {
     GemmArgs gx = gx0, gy = gy0;
-    // (gx may carry its remainder band as pieces of the same launch: GemmArgs::tail_m0)
+    // (gx may carry its remainder band as pieces of the same launch: GemmArgs::tail_m0; then it has one layer)
     const bool tail = gx.tail_splits > 0;
     const int tMx = ceil_div(tail ? gx.tail_m0 : gx.M, TX::BM), tNx = ceil_div(gx.N, TX::BN), tMy = ceil_div(gy.M, TY::BM), tNy = ceil_div(gy.N, TY::BN);
     const int extra = tail ? ceil_div(gx.M - gx.tail_m0, TX::BM) * tNx * gx.tail_splits : 0;
     // the longer-running product first: gy's pieces, then gx's tiles
-    const int ny = tMy * tNy, nzy = gy.batch * gy.splits, nx = tMx * tNx + extra;
+    const int ny = tMy * tNy, nzy = gy.batch * gy.splits, nx = tMx * tNx + extra, nzx = tail ? 1 : gx.batch * gx.splits;
     // phase records (a measurement aid): gy's workgroups first, then gx's, tagged 0 and 1
-    const bool rec = (size_t)(ny * nzy + nx) * 64 <= phase_rec_bytes;
+    const bool rec = (size_t)(ny * nzy + nx * nzx) * 64 <= phase_rec_bytes;
     gy.phase_rec = rec ? phase_rec_buf : nullptr, gy.stamps = 0;
     gx.phase_rec = rec && phase_rec_buf ? phase_rec_buf + 8L * ny * nzy : nullptr, gx.stamps = 1;
-    hipLaunchKernelGGL((gemm_tiled_pair_kernel<TY, TX>), dim3(ny * nzy + nx), dim3(TX::NT), 0, stream, gy, gx, tMy, tNy, ny, nzy, tMx, tNx, nx);
+    hipLaunchKernelGGL((gemm_tiled_pair_kernel<TY, TX>), dim3(ny * nzy + nx * nzx), dim3(TX::NT), 0, stream, gy, gx, tMy, tNy, ny, nzy, tMx, tNx, nx);
     D8_LAUNCH_CHECK();
     return 0;
 }
@@ -805,6 +805,50 @@ static int launch_pair(const GemmArgs &gx, const GemmArgs &gy, hipStream_t strea
     if (tx == TILE_128x128) { D8_PAIR_Y(X1) }
     D8_PAIR_Y(X2)
 #undef D8_PAIR_Y
+}
+
+// ---- the same for two real products (no patch matrices): g0 is NT (a MatrixMultiply's gradient of its first input),
+// g1 is TN (the gradient of its second); either may be batched or split along its reduction (the caller reduces).
+template <typename E>
+static bool plain_pair_tiles(const GemmArgs &g0, const GemmArgs &g1, TileId &t0, TileId &t1) {
+    t0 = choose_tile<E, true, true>(g0), t1 = choose_tile<E, false, false>(g1);
+    const bool ok0 = t0 == TILE_64x128 || t0 == TILE_128x128 || t0 == TILE_128x64;
+    const bool ok1 = t1 == TILE_64x128 || t1 == TILE_128x128 || t1 == TILE_128x64;
+    constexpr int BK = 128 / (int)sizeof(E);
+    return ok0 && ok1 && g0.K % BK == 0 && g1.K % BK == 0;
+}
+
+template <typename E>
+static int launch_plain_pair(const GemmArgs &g0, const GemmArgs &g1, hipStream_t stream) {
+    TileId t0, t1;
+    if (!plain_pair_tiles<E>(g0, g1, t0, t1)) return fail(D8_ERR_ARGUMENT, "gemm_tiled_plain_pair_launch: no kernel for this pair of tiles");
+#define D8_PAIR_1(T0T)                                                                                              \
+    switch (t1) {                                                                                                   \
+        case TILE_128x128: return launch_pair_tiles<T0T, Tile<E, 128, 128, 2, 2, false, false>>(g0, g1, stream);    \
+        case TILE_64x128: return launch_pair_tiles<T0T, Tile<E, 64, 128, 2, 2, false, false>>(g0, g1, stream);      \
+        default: return launch_pair_tiles<T0T, Tile<E, 128, 64, 2, 2, false, false>>(g0, g1, stream);               \
+    }
+    typedef Tile<E, 64, 128, 2, 2, true, true> A0;
+    typedef Tile<E, 128, 128, 2, 2, true, true> A1;
+    typedef Tile<E, 128, 64, 2, 2, true, true> A2;
+    if (t0 == TILE_64x128) { D8_PAIR_1(A0) }
+    if (t0 == TILE_128x128) { D8_PAIR_1(A1) }
+    D8_PAIR_1(A2)
+#undef D8_PAIR_1
+}
+
+long gemm_tiled_plain_pair_workgroups(int dtype, const GemmArgs &g0, const GemmArgs &g1) {
+    TileId t0, t1;
+    if (g0.virt != VIRT_NONE || g1.virt != VIRT_NONE || g0.tail_splits || g1.tail_splits) return 0;
+    if (!(dtype == D8_FLOAT16 ? plain_pair_tiles<f16>(g0, g1, t0, t1) : plain_pair_tiles<float>(g0, g1, t0, t1))) return 0;
+    int m0, n0, m1, n1;
+    grid_of(t0, g0, m0, n0);
+    grid_of(t1, g1, m1, n1);
+    return (long)m0 * n0 * g0.batch * g0.splits + (long)m1 * n1 * g1.batch * g1.splits;
+}
+
+int gemm_tiled_plain_pair_launch(int dtype, const GemmArgs &g0, const GemmArgs &g1, hipStream_t stream) {
+    return dtype == D8_FLOAT16 ? launch_plain_pair<f16>(g0, g1, stream) : launch_plain_pair<float>(g0, g1, stream);
 }
 
 long gemm_tiled_pair_workgroups(int dtype, const GemmArgs &gx, const GemmArgs &gy) {

@@ -260,6 +260,8 @@ extern "C" {
 // ---------------------------------------------------------------------------------------------
 size_t d8_matmul_scratch_bytes(int dtype, int which, int xb, int xr, int xc, int yb, int yr, int yc) {
     if (check_mm("d8_matmul_scratch_bytes", dtype, xb, xr, xc, yb, yr, yc)) return 0;
+    if (which == 3)  // for d8_matmul_grad_xy: both gradients' scratch side by side (they may share a launch)
+        return align256(d8_matmul_scratch_bytes(dtype, 1, xb, xr, xc, yb, yr, yc)) + d8_matmul_scratch_bytes(dtype, 2, xb, xr, xc, yb, yr, yc);
     return gemm_ws(dtype, mm_plan(which, nullptr, xb, xr, xc, nullptr, yb, yr, yc, nullptr));
 }
 
@@ -342,6 +344,14 @@ int d8_matmul_grad_xy(int dtype, const void *x, void *dx, int xb, int xr, int xc
     {  // both products small: one launch of the small-product kernel's workgroups for both
         int rc = 0;
         if (gemm_small_pair_run(dtype, to_args(px), px.ta, px.tb, to_args(py), py.ta, py.tb, as_stream(stream), &rc)) {
+            ++matmul_pair_launches;
+            return rc;
+        }
+    }
+    {  // both on the tiled kernels with all their workgroups resident at once: one launch, then their split reductions
+        int rc = 0;
+        GemmArgs gx = to_args(px), gy = to_args(py);
+        if (gemm_tiled_run_plain_pair(dtype, gx, px.ta, px.tb, gy, py.ta, py.tb, scratch, scratch_bytes, as_stream(stream), &rc)) {
             ++matmul_pair_launches;
             return rc;
         }

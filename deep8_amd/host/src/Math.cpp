@@ -188,8 +188,7 @@ void MatrixMultiplyGradXY(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &
 void MatrixMultiplyGradXYGPU(const Tensor &x, Tensor &dx, const Tensor &y, Tensor &dy, const Tensor &, const Tensor &dz) {
     const MM d = mmDims(x, y);
     const int dt = dtypeOf(x);
-    const size_t need = std::max(d8_matmul_scratch_bytes(dt, 1, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc),
-                                 d8_matmul_scratch_bytes(dt, 2, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc));
+    const size_t need = d8_matmul_scratch_bytes(dt, 3, d.xb, d.xr, d.xc, d.yb, d.yr, d.yc);  // both gradients' scratch
     PoolScratch ws(x.device(), need);
     // a gradient whose zero fill is still deferred is written, not added to
     const int overwrite = (dx.takeZero() ? 1 : 0) | (dy.takeZero() ? 2 : 0);

@@ -116,7 +116,7 @@ def matmul_grad_xy(x, y, dz, dx=None, dy=None, overwrite_x=False, overwrite_y=Fa
     yb, yr, yc = _mat(y)
     x_, y_, dz_ = DeviceArray.from_numpy(x), DeviceArray.from_numpy(y), DeviceArray.from_numpy(dz)
     dx_, dy_ = DeviceArray.from_numpy(dx), DeviceArray.from_numpy(dy)
-    nb = max(lib.d8_matmul_scratch_bytes(dt, w, xb, xr, xc, yb, yr, yc) for w in (1, 2))
+    nb = lib.d8_matmul_scratch_bytes(dt, 3, xb, xr, xc, yb, yr, yc)
     ws = _scratch(nb) if nb else None
     check(lib.d8_matmul_grad_xy(dt, x_.ptr, dx_.ptr, xb, xr, xc, y_.ptr, dy_.ptr, yb, yr, yc, dz_.ptr,
                                 int(overwrite_x) | int(overwrite_y) << 1, ws.ptr if ws else None, nb, None))

@@ -145,7 +145,7 @@ int d8_deconv_im2col(int dtype, const void *dz, void *dzmat,
  * is not can only take the staged route, whose interim matrix is sizeof(T)*B*OH*OW*FH*FW*IC
  * (Conv2d) or sizeof(T)*B*IH*IW*OC*FH*FW (DeConv2d) bytes plus d8_gemm_workspace_bytes; with
  * less the call fails with D8_ERR_ARGUMENT and says so.                                       */
-size_t d8_matmul_scratch_bytes(int dtype, int which /*0 fwd, 1 gradX, 2 gradY*/,
+size_t d8_matmul_scratch_bytes(int dtype, int which /*0 fwd, 1 gradX, 2 gradY, 3 both gradients from one call*/,
                                int xb, int xr, int xc, int yb, int yr, int yc);
 int d8_matmul(int dtype, const void *x, int xb, int xr, int xc,
               const void *y, int yb, int yr, int yc, void *z,
@@ -172,8 +172,10 @@ int d8_matmul_grad_y_overwrite(int dtype, const void *x, int xb, int xr, int xc,
  * of each other, so large Float16 ones run as ONE launch in which a workgroup goes from a tile of dx straight on
  * to a tile of dy; everything else is d8_matmul_grad_x followed by d8_matmul_grad_y.  The results are bit for bit
  * those of the two calls.  overwrite: bit 0 -- dx is written instead of added to, bit 1 -- dy likewise (the
- * _overwrite forms above).  scratch: the larger of d8_matmul_scratch_bytes(which = 1) and (which = 2).  Two small
- * products (each at most four 128 x 128 tiles over a reduction of at most 512) share a launch as well.         */
+ * _overwrite forms above).  scratch: d8_matmul_scratch_bytes(which = 3), room for both gradients' scratch side by
+ * side; with less, but at least the larger of which = 1 and which = 2, the call still works (mid-size products
+ * then run as two launches).  Two small products (each at most four 128 x 128 tiles over a reduction of at most
+ * 512) share a launch as well, and so do two mid-size ones whose workgroups all fit the chip at once.          */
 int d8_matmul_grad_xy(int dtype, const void *x, void *dx, int xb, int xr, int xc,
                       const void *y, void *dy, int yb, int yr, int yc, const void *dz, int overwrite,
                       void *scratch, size_t scratch_bytes, void *stream);

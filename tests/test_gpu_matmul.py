@@ -130,28 +130,39 @@ PAIRS = [
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
-@pytest.mark.parametrize("xs,ys,shared", [((1, 64, 128), (1, 128, 256), True),    # benchmark configuration 1
-                                          ((1, 33, 70), (1, 70, 50), True),       # ragged 32 x 32 tiles
-                                          ((3, 40, 64), (3, 64, 72), True),       # a batch of three small products
-                                          ((1, 64, 1024), (1, 1024, 256), False)])  # a reduction too long for the small-product kernel
-def test_small_matmul_gradients_share_a_launch(oracle_port, xs, ys, shared, dtype):
-    """two small products: d8_matmul_grad_xy runs them as one launch of the small-product kernel; integers bit for bit
-    against the oracle, and the bits of the two separate calls"""
+@pytest.mark.parametrize("xs,ys,shared", [((1, 64, 128), (1, 128, 256), (True, True)),    # benchmark configuration 1
+                                          ((1, 33, 70), (1, 70, 50), (True, True)),       # ragged 32 x 32 tiles
+                                          ((3, 40, 64), (3, 64, 72), (True, True)),       # a batch of three small products
+                                          # a fully connected layer: the tiled kernels, both products split along their reductions
+                                          ((1, 64, 1024), (1, 1024, 256), (True, True)),
+                                          ((1, 256, 1024), (1, 1024, 1024), (True, True)),
+                                          ((4, 128, 256), (1, 256, 384), (True, True)),   # the second input shared by a batch: its gradient sums over it
+                                          ((1, 200, 264), (1, 264, 136), (False, False)),  # a reduction that is not a multiple of the K step
+                                          # more workgroups than the chip holds at once (and too few 256 x 256 tiles in dX for the large-output kernel's pair)
+                                          ((1, 4096, 2048), (1, 2048, 4096), (False, False))])
+def test_small_and_mid_size_matmul_gradients_share_a_launch(oracle_port, xs, ys, shared, dtype):
+    """d8_matmul_grad_xy runs two small products as one launch of the small-product kernel and two mid-size ones as
+    one launch of the tiled kernel (shared: whether in fp32, in half); integers bit for bit against the oracle, and
+    the bits of the two separate calls"""
+    shared = shared[0] if dtype == np.float32 else shared[1]
     from deep8_amd import capi, ops
     lib = capi.init()
     r = rng(sum(xs) + sum(ys) + 3)
     c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
     hi = 2 if dtype == np.float16 else 20
     x, y = ints(r, xs, hi), ints(r, ys, hi)
-    dz = ints(r, (xs[0], xs[1], ys[2]), hi)
+    dz = ints(r, (max(xs[0], ys[0]), xs[1], ys[2]), hi)
     dx0, dy0 = ints(r, xs, hi), ints(r, ys, hi)
+    if dtype == np.float16:  # thinned so that every sum stays exact in half
+        keep = min(1.0, 24.0 / np.sqrt(max(xs[1] * max(xs[0], ys[0]), xs[2], ys[2])))
+        x, dz = x * (r.random(x.shape) < keep), dz * (r.random(dz.shape) < keep)
     before = lib.d8_matmul_grad_pair_launches()
     gx, gy = ops.matmul_grad_xy(c(x), c(y), c(dz), c(dx0), c(dy0), False, True)
     assert lib.d8_matmul_grad_pair_launches() - before == (1 if shared else 0)
     wx, wy = oracle_port.matmul_grad_x(x, y, dz, dx0), oracle_port.matmul_grad_y(x, y, dz)
     assert dtype == np.float32 or max(np.abs(wx).max(), np.abs(wy).max()) < 2048
     assert np.array_equal(f(gx), wx) and np.array_equal(f(gy), wy)
-    xr_, yr_, dzr = c(nrm(r, xs)), c(nrm(r, ys)), c(nrm(r, dz.shape))
+    xr_, yr_, dzr = c(nrm(r, xs)), c(nrm(r, ys, 1 / 32.0)), c(nrm(r, dz.shape))
     gx, gy = ops.matmul_grad_xy(xr_, yr_, dzr, overwrite_x=True, overwrite_y=True)
     bits = np.uint16 if dtype == np.float16 else np.uint32
     assert np.array_equal(gx.view(bits), ops.matmul_grad_x(xr_, yr_, dzr, overwrite=True).view(bits))
