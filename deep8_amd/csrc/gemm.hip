@@ -326,11 +326,10 @@ static bool gemm_is_small(int M, int N, int K, int batch, int red) {
 // outputs; its 8 thread rows each add every 8th partial (16-byte loads), and the 8 sums meet in
 // LDS in a fixed order, so the result does not depend on scheduling.
 template <typename T>
-__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(GemmArgs g) {
-    __shared__ f32x4 part[8][32];
+__device__ __forceinline__ void gemm_split_reduce_body(const GemmArgs &g, const long block, f32x4 (*part)[32]) {
     const long mn = (long)g.M * g.N;
     const int lane = threadIdx.x & 31, row = threadIdx.x >> 5;
-    const long e = ((long)blockIdx.x * 32 + lane) * 4;  // first of this thread's 4 outputs (N % 4 == 0)
+    const long e = (block * 32 + lane) * 4;  // first of this thread's 4 outputs (N % 4 == 0)
     const bool live = e < mn * g.batch;
     const int b = live ? (int)(e / mn) : 0;
     const long r = e - (long)b * mn;
@@ -355,6 +354,20 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(GemmArgs g) {
             *c = (T)(g.relu && !(o > 0.f) ? 0.f : o);
         }
     }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(GemmArgs g) {
+    __shared__ f32x4 part[8][32];
+    gemm_split_reduce_body<T>(g, (long)blockIdx.x, part);
+}
+
+// The reductions of two products in one launch: the first blocks0 workgroups are g0's, the rest g1's.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_split_reduce_pair_kernel(GemmArgs g0, GemmArgs g1, unsigned blocks0) {
+    __shared__ f32x4 part[8][32];
+    if (blockIdx.x < blocks0) gemm_split_reduce_body<T>(g0, (long)blockIdx.x, part);
+    else gemm_split_reduce_body<T>(g1, (long)(blockIdx.x - blocks0), part);
 }
 
 // The same for N not a multiple of 4: a workgroup covers 32 outputs; its 8 thread rows each add every 8th
@@ -512,6 +525,29 @@ static int launch_reduce(const GemmArgs &g, hipStream_t stream) {
         hipLaunchKernelGGL((gemm_split_reduce_scalar_kernel<T>), dim3((unsigned)((total + 31) / 32)), dim3(256), 0, stream, g);
     }
     D8_LAUNCH_CHECK();
+    return 0;
+}
+
+// The reductions that follow a launch of two products (either may be unsplit): one launch for both where both take
+// the 16-byte form.
+static int launch_reduce_pair(int dtype, const GemmArgs &g0, const GemmArgs &g1, hipStream_t stream) {
+    const bool r0 = g0.splits > 1, r1 = g1.splits > 1;
+    auto vec = [](const GemmArgs &g) { return g.N % 4 == 0 && ((size_t)g.ws & 15) == 0; };
+    if (r0 && r1 && vec(g0) && vec(g1)) {
+        const long b0 = ((long)g0.M * g0.N * g0.batch / 4 + 31) / 32, b1 = ((long)g1.M * g1.N * g1.batch / 4 + 31) / 32;
+        if (b0 + b1 < 0x7fffffffL) {
+            if (dtype == D8_FLOAT16)
+                hipLaunchKernelGGL((gemm_split_reduce_pair_kernel<f16>), dim3((unsigned)(b0 + b1)), dim3(256), 0, stream, g0, g1, (unsigned)b0);
+            else
+                hipLaunchKernelGGL((gemm_split_reduce_pair_kernel<float>), dim3((unsigned)(b0 + b1)), dim3(256), 0, stream, g0, g1, (unsigned)b0);
+            D8_LAUNCH_CHECK();
+            return 0;
+        }
+    }
+    if (r0)
+        if (int rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(g0, stream) : launch_reduce<float>(g0, stream)) return rc;
+    if (r1)
+        if (int rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(g1, stream) : launch_reduce<float>(g1, stream)) return rc;
     return 0;
 }
 
@@ -702,8 +738,8 @@ bool gemm_tiled_run_pair(int dtype, GemmArgs &gx, GemmArgs &gy, void *workspace,
     if (wgs <= 0 || (wgs > 2L * cu_count() && !big)) return false;
     ++pair_launches;
     *rc = gemm_tiled_pair_launch(dtype, gx, gy, stream);
-    if (*rc == 0 && head) *rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(band, stream) : launch_reduce<float>(band, stream);
-    if (*rc == 0 && gy.splits > 1) *rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(gy, stream) : launch_reduce<float>(gy, stream);
+    if (!head) band.splits = 1;  // (no band: nothing of gx's to reduce)
+    if (*rc == 0) *rc = launch_reduce_pair(dtype, band, gy, stream);
     return true;
 }
 
@@ -728,8 +764,7 @@ bool gemm_tiled_run_plain_pair(int dtype, GemmArgs &g0, int ta0, int tb0, GemmAr
     const long wgs = gemm_tiled_plain_pair_workgroups(dtype, g0, g1);
     if (wgs <= 0 || wgs > 2L * cu_count()) return false;
     *rc = gemm_tiled_plain_pair_launch(dtype, g0, g1, stream);
-    if (*rc == 0 && g0.splits > 1) *rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(g0, stream) : launch_reduce<float>(g0, stream);
-    if (*rc == 0 && g1.splits > 1) *rc = dtype == D8_FLOAT16 ? launch_reduce<f16>(g1, stream) : launch_reduce<float>(g1, stream);
+    if (*rc == 0) *rc = launch_reduce_pair(dtype, g0, g1, stream);
     return true;
 }
 
