@@ -207,43 +207,60 @@ static bool conv_implicit_plan(int dtype, int which, const ConvShape &c, const v
     return implicit_eligible(dtype, g, ta, tb);
 }
 
-// Conv2d's gradient of x for a stride above 1 (dilation 1), input pixel by input pixel: the pixels of dx with
-// one residue (py, px) modulo the stride receive the taps fy = f0y + sy * j, f0y = (py + pt) mod sy, from
-// dz[b][y' + (py + pt - f0y) / sy - j][..] -- a stride-1 patch product with dilation -1 per class (OutClass),
-// all classes in one launch, nothing staged.
-static bool conv_classes_grad_x(int dtype, const ConvShape &c, const void *gx, const void *w, const void *gz, GemmArgs &g) {
+// Conv2d's gradient of x for a stride above 1, input pixel by input pixel: the pixels of dx with one residue (py, px)
+// modulo the stride receive the taps fy with fy * dy = py + pt (mod sy) -- fy = f0y + (sy / gcd(sy, dy)) * j -- from
+// dz[b][y' + (py + pt - f0y * dy) / sy - j * dy / gcd(sy, dy)][..]: a stride-1 patch product with a negative dilation
+// per class (OutClass), all classes in one launch, nothing staged.  A class that no tap reaches (a filter smaller
+// than the stride; a dilation that shares a factor with the stride, which leaves whole rows of x unread) gets no
+// product: *untouched tells the caller, who zero-fills dx before an overwriting call.
+static int gcd_of(int a, int b) { return b ? gcd_of(b, a % b) : a; }
+
+static bool conv_classes_grad_x(int dtype, const ConvShape &c, const void *gx, const void *w, const void *gz, GemmArgs &g, bool *untouched) {
+    *untouched = false;
     if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
-    if ((c.sy == 1 && c.sx == 1) || c.dy != 1 || c.dx != 1 || c.sy * c.sx > MAX_CLASSES) return false;
-    if (c.FH < c.sy || c.FW < c.sx || c.IH < c.sy || c.IW < c.sx) return false;  // every class needs a tap
+    if ((c.sy == 1 && c.sx == 1) || c.sy * c.sx > MAX_CLASSES) return false;
+    if (c.IH < c.sy || c.IW < c.sx) return false;
     if (!f64_grad_x_fills_tiles(dtype, c.IC)) return false;
     const long es = (long)dtype_bytes(dtype), T = (long)c.FH * c.FW;
     const long zbytes = (long)c.B * c.OH * c.OW * c.OC * es;
     if (zbytes >= (1L << 31) || (long)c.B * c.IH * c.IW * c.IC * es >= (1L << 31) || T * c.IC * c.OC * es >= (1L << 31))
         return false;
+    const int gy = gcd_of(c.sy, c.dy), gw = gcd_of(c.sx, c.dx), stepy = c.sy / gy, stepx = c.sx / gw;
     memset(&g, 0, sizeof(g));
-    g.pg = {c.OH, c.OW, c.OC, 0, 0, 0, 1, 1, -1, -1, 0, 0, 0, 0, (unsigned)zbytes};
+    g.pg = {c.OH, c.OW, c.OC, 0, 0, 0, 1, 1, -(c.dy / gy), -(c.dx / gw), 0, 0, 0, 0, (unsigned)zbytes};
     g.virt = VIRT_A_CLASSES;
     g.A = gz, g.B = w, g.C = (void *)gx;
     g.N = c.IC, g.K = c.OC;
-    g.ldb = (int)(T * c.IC), g.sB = (long)c.sx * c.IC, g.sB_row = (long)c.sy * c.FW * c.IC, g.ldc = c.IC;
+    g.ldb = (int)(T * c.IC), g.sB = (long)stepx * c.IC, g.sB_row = (long)stepy * c.FW * c.IC, g.ldc = c.IC;
     g.batch = 1, g.red = 1, g.splits = 1, g.beta = 1.f;
     g.out_H = c.IH, g.out_W = c.IW, g.out_sy = c.sy, g.out_sx = c.sx;
+    // the first tap f < n with f * d = v (mod s), or -1
+    auto first_tap = [](int v, int d, int s, int step, int n) {
+        for (int f = 0; f < step && f < n; ++f)
+            if ((((v - f * d) % s) + s) % s == 0) return f;
+        return -1;
+    };
     int largest = 0, smallest = 0x7fffffff, most_taps = 0;
     for (int py = 0; py < c.sy; ++py)
         for (int px = 0; px < c.sx; ++px) {
+            const int f0y = first_tap(py + c.pt, c.dy, c.sy, stepy, c.FH), f0x = first_tap(px + c.pl, c.dx, c.sx, stepx, c.FW);
+            if (f0y < 0 || f0x < 0) {
+                *untouched = true;
+                continue;
+            }
             OutClass &k = g.cls[g.ncls++];
             k.OH = (c.IH - py + c.sy - 1) / c.sy, k.OW = (c.IW - px + c.sx - 1) / c.sx;
             k.M = c.B * k.OH * k.OW;
-            const int f0y = (py + c.pt) % c.sy, f0x = (px + c.pl) % c.sx;
-            k.taps_w = (c.FW - f0x + c.sx - 1) / c.sx;
-            k.red = ((c.FH - f0y + c.sy - 1) / c.sy) * k.taps_w;
-            k.pt = -((py + c.pt - f0y) / c.sy), k.pl = -((px + c.pl - f0x) / c.sx);  // dz row = y' - j + (py + pt - f0y) / sy
+            k.taps_w = (c.FW - f0x + stepx - 1) / stepx;
+            k.red = ((c.FH - f0y + stepy - 1) / stepy) * k.taps_w;
+            k.pt = -((py + c.pt - f0y * c.dy) / c.sy), k.pl = -((px + c.pl - f0x * c.dx) / c.sx);  // (exact divisions)
             k.py = py, k.px = px;
             k.b_off = (unsigned)((f0y * c.FW + f0x) * c.IC);
             largest = k.M > largest ? k.M : largest;
             smallest = k.M < smallest ? k.M : smallest;
             most_taps = k.red > most_taps ? k.red : most_taps;
         }
+    if (g.ncls == 0) return false;
     g.tiles_per_split = most_taps * (c.OC / (dtype == D8_FLOAT64 ? 16 : gemm_tiled_k_step(dtype)) + 1);
     g.M = smallest;
     const bool ok = implicit_eligible(dtype, g, 0, 0);
@@ -448,7 +465,8 @@ size_t d8_conv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW, int 
     int ta, tb;
     if (conv_implicit_plan(dtype, which, cs, nullptr, nullptr, nullptr, ga, ta, tb))
         return implicit_workspace(dtype, ga);
-    if (which == 1 && conv_classes_grad_x(dtype, cs, nullptr, nullptr, nullptr, ga)) return 0;
+    bool untouched = false;
+    if (which == 1 && conv_classes_grad_x(dtype, cs, nullptr, nullptr, nullptr, ga, &untouched)) return 0;
     const size_t col = align256((size_t)M * K * dtype_bytes(dtype));
     const size_t plain = col + gemm_ws(dtype, conv_plan(which, M, K, OC, nullptr, nullptr, nullptr));
     if (const int pitch = conv_padded_pitch(dtype, K, OC)) {
@@ -528,7 +546,12 @@ static int d8_conv2d_grad_x_impl(int dtype, void *gx, int B, int IH, int IW, int
             ga.beta = beta;
             return implicit_run(dtype, ga, ta, tb, scratch, scratch_bytes, as_stream(stream));
         }
-        if (conv_classes_grad_x(dtype, cs, gx, w, gz, ga)) {
+        bool untouched = false;
+        if (conv_classes_grad_x(dtype, cs, gx, w, gz, ga, &untouched)) {
+            if (untouched && beta == 0.f) {  // pixels of dx that no tap reaches: zero, and the classes add to that
+                if (int rc = d8_fill(dtype, gx, (size_t)B * IH * IW * IC, 0.f, stream)) return rc;
+                beta = 1.f;
+            }
             ga.beta = beta;
             return implicit_run(dtype, ga, 0, 0, nullptr, 0, as_stream(stream));
         }

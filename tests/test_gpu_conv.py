@@ -466,8 +466,13 @@ CONV_DX_CLASSES = [
     ((4, 18, 18, 128, 64, 4, 4, True, 3, 3, 1, 1), True),
     ((2, 16, 16, 64, 64, 5, 3, True, 2, 1, 1, 1), True),     # stride 2 down, 1 across
     ((4, 16, 16, 64, 64, 2, 2, False, 2, 2, 1, 1), True),    # filter == stride: one tap per class
-    ((2, 16, 16, 64, 64, 3, 3, True, 2, 2, 2, 2), False),    # dilation: im2col route
-    ((2, 16, 16, 64, 64, 1, 1, True, 2, 2, 1, 1), False),    # filter smaller than the stride: classes without a tap
+    ((2, 16, 16, 64, 64, 3, 3, True, 2, 2, 2, 2), True),     # dilation 2 at stride 2: only even rows and columns of x are read at all
+    ((2, 16, 16, 64, 64, 1, 1, True, 2, 2, 1, 1), True),     # filter smaller than the stride: classes without a tap
+    ((2, 32, 32, 64, 32, 4, 4, True, 2, 2, 2, 2), True),     # Conv2dTest forwardCPU_float's geometry (fp32: 32 output channels are one K step)
+    ((2, 18, 17, 64, 64, 3, 3, True, 2, 2, 3, 3), True),     # dilation 3 at stride 2: every class has taps, two filter rows apart
+    ((3, 25, 25, 64, 64, 3, 3, False, 3, 3, 2, 2), True),    # stride 3, dilation 2, not covered
+    ((2, 40, 20, 64, 64, 5, 5, True, 4, 2, 2, 3), True),     # stride 4 x 2, dilation 2 x 3: a common factor down, none across
+    ((2, 24, 24, 64, 64, 3, 3, True, 6, 6, 1, 1), False),    # 36 classes: more than a launch takes
 ]
 
 
@@ -480,7 +485,7 @@ def test_conv2d_strided_gradient_of_x(oracle_port, monkeypatch, cfg, classes, dt
     a = (cov, sy, sx, dy, dx)
     OH, OW, _, _ = ops.conv2d_geometry(IH, IW, FH, FW, *a)
     nb = lib.d8_conv2d_scratch_bytes(capi.dtype_id(np.dtype(dtype)), 1, B, IH, IW, IC, OC, FH, FW, int(cov), sy, sx, dy, dx)
-    assert (nb == 0) == classes
+    assert (nb == 0) == (classes and OC % (64 if dtype == np.float16 else 32) == 0)  # (a K step stays inside one tap)
     r = rng(B + IH + OC + 95)
     c = (lambda v: h(v)) if dtype == np.float16 else (lambda v: v)
     hi = 3 if dtype == np.float16 else 20
