@@ -657,11 +657,12 @@ static bool deconv_implicit_grad_x(int dtype, int B, int IH, int IW, int IC, int
 // a stride-1 patch product over the taps that reach them (OutClass), all in one launch; nothing
 // is staged.  Needs a tap for every class (FH >= sy, FW >= sx) and tile-sized classes.
 static bool deconv_implicit_fwd(int dtype, int B, int IH, int IW, int IC, int OC, int FH, int FW, int sy, int sx,
-                                const int *geo, const void *x, const void *w, const void *z, GemmArgs &g) {
+                                const int *geo, const void *x, const void *w, const void *z, GemmArgs &g, bool *untouched) {
+    *untouched = false;
     if (getenv("D8_CONV_EXPLICIT") != nullptr) return false;
     const long es = (long)dtype_bytes(dtype), T = (long)FH * FW;
     const int OH = geo[0], OW = geo[1], pt = geo[2], pl = geo[3];
-    if (sy * sx > MAX_CLASSES || FH < sy || FW < sx || OH < sy || OW < sx) return false;
+    if (sy * sx > MAX_CLASSES || OH < sy || OW < sx) return false;
     const long xbytes = (long)B * IH * IW * IC * es;
     if (xbytes >= (1L << 31) || (long)B * OH * OW * OC * es >= (1L << 31) || T * IC * OC * es >= (1L << 31)) return false;
     memset(&g, 0, sizeof(g));
@@ -675,11 +676,15 @@ static bool deconv_implicit_fwd(int dtype, int B, int IH, int IW, int IC, int OC
     int largest = 0, smallest = 0x7fffffff, most_taps = 0;
     for (int py = 0; py < sy; ++py)
         for (int px = 0; px < sx; ++px) {
+            // taps fy with (py - pt + fy) a multiple of sy: fy = f0y + sy * j
+            const int f0y = (((pt - py) % sy) + sy) % sy, f0x = (((pl - px) % sx) + sx) % sx;
+            if (f0y >= FH || f0x >= FW) {  // a stride larger than the filter: output pixels that no tap writes (zero; the caller fills z)
+                *untouched = true;
+                continue;
+            }
             OutClass &c = g.cls[g.ncls++];
             c.OH = (OH - py + sy - 1) / sy, c.OW = (OW - px + sx - 1) / sx;
             c.M = B * c.OH * c.OW;
-            // taps fy with (py - pt + fy) a multiple of sy: fy = f0y + sy * j
-            const int f0y = (((pt - py) % sy) + sy) % sy, f0x = (((pl - px) % sx) + sx) % sx;
             const int nty = (FH - f0y + sy - 1) / sy, ntx = (FW - f0x + sx - 1) / sx;
             c.taps_w = ntx, c.red = nty * ntx;
             c.pt = -((py - pt + f0y) / sy), c.pl = -((px - pl + f0x) / sx);  // input row = y' + j + (py - pt + f0y) / sy
@@ -689,6 +694,7 @@ static bool deconv_implicit_fwd(int dtype, int B, int IH, int IW, int IC, int OC
             smallest = c.M < smallest ? c.M : smallest;
             most_taps = c.red > most_taps ? c.red : most_taps;
         }
+    if (g.ncls == 0) return false;
     g.tiles_per_split = most_taps * (IC / (dtype == D8_FLOAT64 ? 16 : gemm_tiled_k_step(dtype)) + 1);  // never the limit: a class walks all its taps
     g.M = smallest;
     const bool ok = implicit_eligible(dtype, g, 0, 1);
@@ -738,7 +744,8 @@ static size_t deconv2d_scratch_bytes(int dtype, int which, int B, int IH, int IW
     GemmArgs ga;
     if (which == 1 && deconv_implicit_grad_x(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
         return implicit_workspace(dtype, ga);
-    if (which == 0 && deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga)) return 0;
+    bool untouched = false;
+    if (which == 0 && deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga, &untouched)) return 0;
     if (which == 2 && deconv_implicit_grad_y(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, geo, nullptr, nullptr, nullptr, ga))
         return implicit_workspace(dtype, ga);
     const size_t mat = align256((size_t)M * T * OC * dtype_bytes(dtype));
@@ -770,8 +777,12 @@ static int deconv2d_impl(int dtype, const void *x, int B, int IH, int IW, int IC
     if (int rc = check_deconv_out("d8_deconv2d", B, g)) return rc;
     {
         GemmArgs ga;
-        if (deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, w, z, ga))
+        bool untouched = false;
+        if (deconv_implicit_fwd(dtype, B, IH, IW, IC, OC, FH, FW, sy, sx, g, x, w, z, ga, &untouched)) {
+            if (untouched)  // the pixels between the filter's footprints stay zero
+                if (int rc = d8_fill(dtype, z, (size_t)B * g[0] * g[1] * OC, 0.f, stream)) return rc;
             return implicit_run(dtype, ga, 0, 1, nullptr, 0, as_stream(stream));
+        }
     }
     if (int rc = need_scratch("d8_deconv2d", scratch, scratch_bytes, (size_t)M * T * OC * dtype_bytes(dtype), x, w, z)) return rc;
     const size_t ws = scratch_bytes > mat ? scratch_bytes - mat : 0;

@@ -366,7 +366,8 @@ DECONV_CLASSES = [
     ((3, 8, 8, 32, 64, 2, 2, False, 2, 2), True, False),    # 32 channels: one fp32 K step, too few for half
     ((1, 16, 16, 64, 64, 4, 4, False, 1, 1), True, True),   # stride 1: a single class with all 16 taps
     ((2, 16, 16, 64, 72, 4, 4, True, 4, 4), True, True),    # 16 classes of one tap each
-    ((2, 9, 8, 64, 64, 2, 2, False, 3, 3), False, False),   # stride > filter: some classes have no tap
+    ((2, 9, 8, 64, 64, 2, 2, False, 3, 3), True, True),     # stride > filter: some classes have no tap, their pixels stay zero
+    ((2, 9, 9, 64, 64, 1, 1, True, 2, 2), True, True),      # a 1 x 1 filter at stride 2: one class in four has a tap
     ((1, 6, 6, 64, 64, 4, 4, False, 2, 2), False, False),   # classes smaller than a tile
 ]
 
