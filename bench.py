@@ -48,6 +48,7 @@ EAGER_ZERO = False
 # of that row per launch; a list of alternatives is averaged).  None where the summary or a row is missing.
 TRAFFIC_ROWS = {
     "c3": ("gemm_wide_f16_matmul_4096_half.txt", [("gemm_wide_kernel", 1.0 / 3)]),           # NN, NT, TN averaged
+    "f1": ("gemm_tiled_pair_f16_matmul_1024_half.txt", [("2x2 waves, NN>", 1.0 / 3), ("gemm_tiled_pair_kernel", 1.0 / 3)]),  # fwd + the gradients' shared launch, per product
     "c4": ("conv2d_fp32_b32_56x56x64_3x3.txt", [("NT, A = patch rows", 1), ("gemm_split_reduce", 1)]),  # forward: one launch (remainder band included) + the band's reduction
     "c5": ("deconv2d_half_b16_28x28x128_4x4s2.txt", [("one class of output pixels", 1)]),    # forward: one launch over the classes
     "d3": ("gemm_f64_matmul_2048_double.txt", [("gemm_f64_kernel", 1.0 / 3)]),
@@ -195,7 +196,8 @@ class MatMulWorkload:
             if self.dtype == np.float64 else
             "gemm_wide_kernel (fp16, 256x256 tiles)" if wide else
             "gemm_%s_kernel<%s>" % ("small" if small else "tiled", "f16" if self.dtype == np.float16 else "f32"),
-            "one launch for fwd, one for dX and dY together" if wide else "one launch each for fwd, dX, dY")
+            "one launch for fwd, one for dX and dY together" if wide or small or zb * (-(-m // 128)) * (-(-k // 128)) + (-(-k // 128)) * (-(-n // 128)) <= 128
+            else "one launch each for fwd, dX, dY")
         es = self.dtype.itemsize
         nx, ny, nz = np.prod(xs), np.prod(ys), np.prod(self.zs)
         # fwd reads x,y writes z; dX reads dz,y and read-modify-writes dx; dY likewise
@@ -746,6 +748,13 @@ def make_workload(key):
     if key == "c2b":
         return MatMulWorkload("c2b: MatrixMultiply fwd+dX+dY fp32 A batch 32 [512x512], B batch 1 (shared)",
                               np.float32, (32, 512, 512), (1, 512, 512), U, 3)
+    if key in ("f1", "f1s"):  # a fully connected layer: x [1024 x 1024] . W [1024 x 1024], half / fp32
+        g = {"x": lambda r, s: r.standard_normal(s).astype(np.float32),
+             "y": lambda r, s: (r.standard_normal(s) / 32.0).astype(np.float32),
+             "dz": lambda r, s: r.standard_normal(s).astype(np.float32)}
+        return MatMulWorkload("%s: MatrixMultiply fwd+dX+dY %s [1024x1024]x[1024x1024] (a fully connected layer: both gradients "
+                              "in one launch of the tiled kernel)" % (key, "half" if key == "f1" else "fp32"),
+                              np.float16 if key == "f1" else np.float32, (1, 1024, 1024), (1, 1024, 1024), g, 13)
     if key == "c3":
         g = {"x": lambda r, s: (r.standard_normal(s) / 64.0).astype(np.float32),
              "y": lambda r, s: (r.standard_normal(s) / 64.0).astype(np.float32),
@@ -1272,7 +1281,7 @@ def main():
         out["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_others:
         others = {}
-        for key in ("c1", "c2a", "c2b", "c3", "c4", "c4h", "c4e", "c4e_unfused", "c4x", "i4", "k5", "c5", "c5l", "e4", "p4", "d3"):
+        for key in ("c1", "c2a", "c2b", "c3", "f1", "f1s", "c4", "c4h", "c4e", "c4e_unfused", "c4x", "i4", "k5", "c5", "c5l", "e4", "p4", "d3"):
             if key == a.workload:
                 continue
             del wl
